@@ -1,0 +1,182 @@
+/*
+ * omk_forest.h -- C ABI of the device-resident search forest (MI355X / gfx950).
+ *
+ * The library replaces the pointer tree of the reference (class MCTSNode,
+ * include/mcts/mcts_node.h:20-199) by per-node arrays in HBM and the inner loops of
+ * MCTSEngine::executeBatchedTreeSearch (src/mcts/mcts_engine_batch_tree_simple.cpp)
+ * by HIP kernels.  Each entry point names the reference code it stands for.
+ *
+ * Conventions
+ *   - every function returns an omk_status (0 = OK, negative = error); no C++
+ *     exception crosses this boundary; omk_last_error() gives the message of the
+ *     calling thread's last failure;
+ *   - handles are opaque and own their device memory; the caller owns every
+ *     host buffer it passes;
+ *   - pointers named h_* are host pointers, d_* are device pointers;
+ *   - all work of a forest is enqueued on one HIP stream (its own by default,
+ *     see omk_forest_set_stream); calls that return data to the host wait for it;
+ *   - one host thread drives a forest at a time.
+ *
+ * Node ids are int32 indices into the arrays; the children of node v are the ids
+ * child_begin[v] .. child_begin[v]+child_count[v]-1 (their order is the order of the
+ * reference's children_ vector, so "lowest index wins a tie" means the same thing).
+ */
+#ifndef OMK_FOREST_H
+#define OMK_FOREST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum omk_status {
+    OMK_OK = 0,
+    OMK_ERR_INVALID = -1,     /* bad argument                                   */
+    OMK_ERR_HIP = -2,         /* a HIP runtime call failed                      */
+    OMK_ERR_CAPACITY = -3,    /* larger than the handle was created for         */
+    OMK_ERR_STRUCTURE = -4,   /* the uploaded arrays do not describe a forest   */
+    OMK_ERR_UNSUPPORTED = -5, /* valid request this build has no kernel for     */
+    OMK_ERR_STATE = -6        /* call order (e.g. backup before any select)     */
+} omk_status;
+
+#define OMK_MAX_FANOUT 1024 /* children per node the selection kernels hold in registers */
+
+typedef struct omk_forest omk_forest;
+typedef struct omk_batch omk_batch;
+typedef struct omk_tt omk_tt;
+
+/* Host view of the per-node arrays: the flattened fields of MCTSNode
+ * (include/mcts/mcts_node.h:154-178). */
+typedef struct omk_soa_view {
+    int64_t n_nodes;
+    int32_t *N;                 /* visit_count_                                  */
+    float *W;                   /* value_sum_                                    */
+    float *P;                   /* prior_probability_                            */
+    int32_t *VL;                /* virtual_loss_count_                           */
+    int32_t *rN;                /* rave_count_      (NULL unless the forest has RAVE) */
+    float *rW;                  /* rave_value_sum_  (NULL unless the forest has RAVE) */
+    const int32_t *child_begin; /* children_: first child id                     */
+    const int32_t *child_count; /* children_.size(); 0 = isLeaf()                */
+    const int32_t *action;      /* action_ (NULL: the node id stands in)         */
+    const uint32_t *legal;      /* optional bit per node id (bit i of word i/32): 0 = the slot
+                                   holds no child and never takes part in a selection */
+    const uint64_t *hash;       /* optional position key of the node's state (getHash()) */
+} omk_soa_view;
+
+typedef struct omk_forest_desc {
+    int64_t capacity_nodes;
+    int32_t device;   /* HIP device ordinal */
+    int32_t has_rave; /* allocate rN / rW   */
+} omk_forest_desc;
+
+/* MCTSSettings fields read on this path (include/mcts/mcts_engine.h:81-112). */
+typedef struct omk_select_params {
+    float c_puct;         /* exploration_constant                                  */
+    int32_t virtual_loss; /* virtual_loss                                          */
+    int32_t use_rave;     /* use_rave: second scan of selectChild blends RAVE      */
+    float rave_k;         /* rave_constant                                         */
+    int32_t pw;           /* selection-time progressive widening: only the top
+                             ceil(sqrt(N_parent)) children by prior take part.
+                             Needs children stored in prior-descending order.      */
+} omk_select_params;
+
+/* Device pointers of a batch, for consumers that stay on the GPU. Level-major:
+ * the node of traversal t at depth d is d_paths[d * stride + t]. */
+typedef struct omk_batch_dev {
+    int32_t *d_paths;
+    int32_t *d_path_len; /* nodes on the path (selection steps + 1) */
+    int32_t *d_leaf;
+    float *d_values;
+    int32_t stride;
+    int32_t max_depth;
+    int32_t n_traversals;
+} omk_batch_dev;
+
+const char *omk_last_error(void);
+int omk_version(void);
+
+/* ---- forest: replaces the MCTSNode allocations (MCTSNode::create, mcts_node.cpp:68-75) ---- */
+int omk_forest_create(const omk_forest_desc *desc, omk_forest **out);
+int omk_forest_destroy(omk_forest *f);
+/* Use the caller's hipStream_t (NULL restores the forest's own stream). */
+int omk_forest_set_stream(omk_forest *f, void *hip_stream);
+/* Checks that the arrays describe a forest (ranges in bounds, every node the child of at
+ * most one parent, fan-out <= OMK_MAX_FANOUT) and copies them to the device. */
+int omk_forest_upload(omk_forest *f, const omk_soa_view *h_view);
+/* Copies N, W, P, VL (and rN, rW) back; structure pointers of the view are ignored. */
+int omk_forest_download(omk_forest *f, omk_soa_view *h_view);
+int omk_sync(omk_forest *f);
+
+/* ---- batch: the per-search buffers of executeBatchedTreeSearch
+ *      (leaf_nodes / paths / leaf_states, mcts_engine_batch_tree_simple.cpp:41-57) ---- */
+int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, omk_batch **out);
+int omk_batch_destroy(omk_batch *b);
+/* Traversal t starts at h_roots[t] (the reference: every simulation starts at root_,
+ * mcts_engine_batch_tree_simple.cpp:86-92).  Distinct roots must head disjoint trees. */
+int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n_traversals);
+int omk_batch_set_values(omk_batch *b, const float *h_values, int32_t n); /* NetworkOutput::value of each leaf */
+int omk_batch_device(omk_batch *b, omk_batch_dev *out);
+
+/* Phase 1 of executeBatchedTreeSearch (mcts_engine_batch_tree_simple.cpp:73-185): for
+ * every traversal, in traversal-index order semantics, descend while the node is expanded:
+ * MCTSNode::selectChild (mcts_node.cpp:90-236, with getCombinedValue :657-678 when use_rave),
+ * then addVirtualLoss(virtual_loss) on the selected child (mcts_node_virtual_loss.cpp:15-20).
+ * Results stay on the device (omk_batch_read / omk_batch_device). Asynchronous. */
+int omk_select_batch(omk_batch *b, const omk_select_params *params);
+
+/* Phase 3 (mcts_engine_batch_tree_simple.cpp:276-281) on the paths of the last select:
+ * leaf to root, MCTSNode::update(value) (mcts_node_virtual_loss.cpp:54-71), then
+ * revertVirtualLoss(virtual_loss) (:32-42), value = -value.  Asynchronous. */
+int omk_backup_batch(omk_batch *b, int32_t virtual_loss);
+/* removeVirtualLoss(virtual_loss) on every node of the paths of the last select. */
+int omk_revert_vl(omk_batch *b, int32_t virtual_loss);
+
+/* The same three node operations over caller-supplied device paths (level-major, node of
+ * traversal t at depth d = d_paths[d*stride+t], d < d_path_len[t]); atomics, any paths. */
+int omk_apply_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len, int32_t n,
+                       int32_t stride, int32_t max_len, int32_t virtual_loss);
+int omk_revert_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len, int32_t n,
+                        int32_t stride, int32_t max_len, int32_t virtual_loss);
+int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len,
+                     const float *d_values, int32_t n, int32_t stride, int32_t max_len, int32_t virtual_loss);
+
+/* Leaf gather (mcts_engine_batch_tree_simple.cpp:114,166-184): waits for the stream and
+ * returns, per traversal, the path (row of max_depth+1 ids, -1 padded), its length, the
+ * leaf node and the move list to replay on a clone of the root state (row of max_depth
+ * actions, -1 padded).  Any pointer may be NULL. */
+int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t *h_leaf, int32_t *h_actions);
+/* Traversals of the last select that stopped at max_depth on an expanded node. */
+int omk_batch_truncated(omk_batch *b, int32_t *h_count);
+
+/* ---- transposition table: the lookup/store call sites of
+ *      mcts_engine_batch_tree_simple.cpp:126,141 (PHMapTranspositionTable::store / lookup,
+ *      phmap_transposition_table.cpp:51-117) over an open-addressing table in HBM ---- */
+typedef struct omk_tt_slot {
+    uint64_t key; /* ~0 = empty */
+    int32_t node;
+    int32_t depth;
+} omk_tt_slot;
+
+int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out);
+int omk_tt_destroy(omk_tt *tt);
+int omk_tt_clear(omk_tt *tt);
+/* store(hash, node, depth) for n entries; a key already present keeps its first entry. */
+int omk_tt_insert(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, const int32_t *d_depths, int64_t n);
+/* lookup(hash, min_depth): d_out[i] = node or -1. */
+int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_depth, int32_t *d_out);
+/* lookup of the position key of every leaf of the last select: d_out[t] = node or -1. */
+int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_out);
+int omk_tt_upload(omk_tt *tt, const omk_tt_slot *h_slots);
+int omk_tt_download(omk_tt *tt, omk_tt_slot *h_slots);
+
+/* ---- device memory helpers for hosts without a HIP binding of their own ---- */
+int omk_dev_alloc(omk_forest *f, int64_t bytes, void **d_out);
+int omk_dev_free(omk_forest *f, void *d_ptr);
+int omk_dev_h2d(omk_forest *f, void *d_dst, const void *h_src, int64_t bytes);
+int omk_dev_d2h(omk_forest *f, void *h_dst, const void *d_src, int64_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

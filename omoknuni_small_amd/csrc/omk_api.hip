@@ -1,0 +1,618 @@
+// C ABI of libomk_forest.so: handles, host<->device transfers, structural validation,
+// and the launch glue of the selection / backup kernels.  Declarations and the reference
+// interfaces they replace: include/omk_forest.h.
+#include "../../include/omk_forest.h"
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "omk_internal.h"
+
+using namespace omk;
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess) return fail(OMK_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_));    \
+    } while (0)
+
+struct omk_forest {
+    int device = 0;
+    int64_t capacity = 0;
+    int64_t n_nodes = 0;
+    bool has_rave = false;
+    bool uploaded = false;
+    bool prior_sorted = false;
+    int max_fanout = 0;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    // device arrays
+    int2 *span = nullptr;
+    int32_t *N = nullptr, *VL = nullptr, *rN = nullptr, *action = nullptr;
+    float *W = nullptr, *P = nullptr, *rW = nullptr;
+    uint32_t *legal = nullptr;
+    uint64_t *hash = nullptr;
+    bool has_legal = false, has_action = false, has_hash = false;
+
+    ForestDev dev() const {
+        ForestDev d;
+        d.span = span;
+        d.N = N;
+        d.W = W;
+        d.P = P;
+        d.VL = VL;
+        d.rN = has_rave ? rN : nullptr;
+        d.rW = has_rave ? rW : nullptr;
+        d.legal = has_legal ? legal : nullptr;
+        d.action = has_action ? action : nullptr;
+        d.hash = has_hash ? hash : nullptr;
+        d.n_nodes = n_nodes;
+        return d;
+    }
+};
+
+struct omk_batch {
+    omk_forest *f = nullptr;
+    int32_t max_traversals = 0;
+    int32_t max_depth = 0;
+    int32_t stride = 0;
+    int32_t n = 0;          // traversals bound by set_roots
+    bool selected = false;  // paths of a select are on the device
+    int32_t *paths = nullptr, *path_len = nullptr, *leaf = nullptr;
+    float *values = nullptr;
+    Item *items0 = nullptr, *items[2] = {nullptr, nullptr};
+    int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
+    int32_t *sc_child = nullptr, *sc_occ = nullptr;
+    int32_t *counters = nullptr;  // [max_depth + 2] level counters, then 1 truncated counter
+    int32_t n_items0 = 0;
+    int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
+};
+
+struct omk_tt {
+    omk_forest *f = nullptr;
+    int log2_slots = 0;
+    TTSlot *slots = nullptr;
+    int *d_status = nullptr;
+};
+
+template <typename T>
+static hipError_t dalloc(T **p, int64_t count) {
+    return hipMalloc((void **)p, (size_t)std::max<int64_t>(count, 1) * sizeof(T));
+}
+
+static int use_device(const omk_forest *f) {
+    HIP_TRY(hipSetDevice(f->device));
+    return OMK_OK;
+}
+
+extern "C" {
+
+const char *omk_last_error(void) { return g_err; }
+int omk_version(void) { return 1; }
+
+int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
+    if (!desc || !out) return fail(OMK_ERR_INVALID, "omk_forest_create: null argument");
+    if (desc->capacity_nodes <= 0 || desc->capacity_nodes > 0x7FFFFFF0ll)
+        return fail(OMK_ERR_INVALID, "omk_forest_create: capacity_nodes %lld out of range",
+                    (long long)desc->capacity_nodes);
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (desc->device < 0 || desc->device >= count)
+        return fail(OMK_ERR_INVALID, "omk_forest_create: device %d of %d", desc->device, count);
+    omk_forest *f = new (std::nothrow) omk_forest();
+    if (!f) return fail(OMK_ERR_INVALID, "out of host memory");
+    f->device = desc->device;
+    f->capacity = desc->capacity_nodes;
+    f->has_rave = desc->has_rave != 0;
+    hipError_t e = hipSetDevice(f->device);
+    if (e == hipSuccess) e = hipStreamCreate(&f->own_stream);
+    const int64_t n = f->capacity;
+    if (e == hipSuccess) e = dalloc(&f->span, n);
+    if (e == hipSuccess) e = dalloc(&f->N, n);
+    if (e == hipSuccess) e = dalloc(&f->W, n);
+    if (e == hipSuccess) e = dalloc(&f->P, n);
+    if (e == hipSuccess) e = dalloc(&f->VL, n);
+    if (e == hipSuccess && f->has_rave) e = dalloc(&f->rN, n);
+    if (e == hipSuccess && f->has_rave) e = dalloc(&f->rW, n);
+    if (e != hipSuccess) {
+        int rc = fail(OMK_ERR_HIP, "omk_forest_create: %s", hipGetErrorString(e));
+        omk_forest_destroy(f);
+        return rc;
+    }
+    f->stream = f->own_stream;
+    *out = f;
+    return OMK_OK;
+}
+
+int omk_forest_destroy(omk_forest *f) {
+    if (!f) return OMK_OK;
+    (void)hipSetDevice(f->device);
+    if (f->own_stream) (void)hipStreamSynchronize(f->own_stream);
+    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->action, f->legal, f->hash};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    if (f->own_stream) (void)hipStreamDestroy(f->own_stream);
+    delete f;
+    return OMK_OK;
+}
+
+int omk_forest_set_stream(omk_forest *f, void *hip_stream) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_set_stream: null forest");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    f->stream = hip_stream ? (hipStream_t)hip_stream : f->own_stream;
+    return OMK_OK;
+}
+
+int omk_sync(omk_forest *f) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_sync: null forest");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    return OMK_OK;
+}
+
+// The selection kernels give every node to exactly one wavefront per batch; that is only
+// correct when every node is the child of at most one parent, so it is checked here, on
+// the host, before anything reaches the device (it also keeps every child range in
+// bounds, which is what protects the kernels from wild reads).
+static int validate(const omk_soa_view *v, int64_t n, int *max_fanout, bool *prior_sorted) {
+    std::vector<uint8_t> is_child((size_t)n, 0);
+    int mf = 0;
+    bool sorted = true;
+    for (int64_t i = 0; i < n; i++) {
+        int32_t cc = v->child_count[i];
+        if (cc == 0) continue;
+        int32_t cb = v->child_begin[i];
+        if (cc < 0) return fail(OMK_ERR_STRUCTURE, "node %lld: child_count %d < 0", (long long)i, cc);
+        if (cc > OMK_MAX_FANOUT)
+            return fail(OMK_ERR_STRUCTURE, "node %lld: child_count %d exceeds OMK_MAX_FANOUT %d", (long long)i, cc,
+                        OMK_MAX_FANOUT);
+        if (cb < 0 || (int64_t)cb + cc > n)
+            return fail(OMK_ERR_STRUCTURE, "node %lld: children [%d, %d) outside [0, %lld)", (long long)i, cb,
+                        cb + cc, (long long)n);
+        for (int32_t c = cb; c < cb + cc; c++) {
+            if (c == i) return fail(OMK_ERR_STRUCTURE, "node %lld is its own child", (long long)i);
+            if (is_child[(size_t)c]) return fail(OMK_ERR_STRUCTURE, "node %d has two parents", c);
+            is_child[(size_t)c] = 1;
+            if (sorted && c > cb && !(v->P[c - 1] >= v->P[c])) sorted = false;
+        }
+        mf = std::max(mf, (int)cc);
+    }
+    *max_fanout = mf;
+    *prior_sorted = sorted && v->legal == nullptr;
+    return OMK_OK;
+}
+
+int omk_forest_upload(omk_forest *f, const omk_soa_view *v) {
+    if (!f || !v) return fail(OMK_ERR_INVALID, "omk_forest_upload: null argument");
+    const int64_t n = v->n_nodes;
+    if (n <= 0 || n > f->capacity)
+        return fail(OMK_ERR_CAPACITY, "omk_forest_upload: %lld nodes, capacity %lld", (long long)n,
+                    (long long)f->capacity);
+    if (!v->N || !v->W || !v->P || !v->VL || !v->child_begin || !v->child_count)
+        return fail(OMK_ERR_INVALID, "omk_forest_upload: N, W, P, VL, child_begin, child_count are required");
+    if (f->has_rave && (!v->rN || !v->rW))
+        return fail(OMK_ERR_INVALID, "omk_forest_upload: the forest was created with RAVE, rN and rW are required");
+    int mf = 0;
+    bool sorted = false;
+    if (int rc = validate(v, n, &mf, &sorted)) return rc;
+    if (int rc = use_device(f)) return rc;
+
+    std::vector<int2> span((size_t)n);
+    for (int64_t i = 0; i < n; i++) {
+        span[(size_t)i].x = v->child_begin[i];
+        span[(size_t)i].y = v->child_count[i];
+    }
+    hipStream_t s = f->stream;
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipMemcpy(f->span, span.data(), (size_t)n * sizeof(int2), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(f->N, v->N, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(f->W, v->W, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(f->P, v->P, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(f->VL, v->VL, (size_t)n * 4, hipMemcpyHostToDevice));
+    if (f->has_rave) {
+        HIP_TRY(hipMemcpy(f->rN, v->rN, (size_t)n * 4, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(f->rW, v->rW, (size_t)n * 4, hipMemcpyHostToDevice));
+    }
+    f->has_action = v->action != nullptr;
+    if (f->has_action) {
+        if (!f->action) HIP_TRY(dalloc(&f->action, f->capacity));
+        HIP_TRY(hipMemcpy(f->action, v->action, (size_t)n * 4, hipMemcpyHostToDevice));
+    }
+    f->has_legal = v->legal != nullptr;
+    if (f->has_legal) {
+        if (!f->legal) HIP_TRY(dalloc(&f->legal, (f->capacity + 31) / 32));
+        HIP_TRY(hipMemcpy(f->legal, v->legal, (size_t)((n + 31) / 32) * 4, hipMemcpyHostToDevice));
+    }
+    f->has_hash = v->hash != nullptr;
+    if (f->has_hash) {
+        if (!f->hash) HIP_TRY(dalloc(&f->hash, f->capacity));
+        HIP_TRY(hipMemcpy(f->hash, v->hash, (size_t)n * 8, hipMemcpyHostToDevice));
+    }
+    f->n_nodes = n;
+    f->max_fanout = mf;
+    f->prior_sorted = sorted;
+    f->uploaded = true;
+    return OMK_OK;
+}
+
+int omk_forest_download(omk_forest *f, omk_soa_view *v) {
+    if (!f || !v) return fail(OMK_ERR_INVALID, "omk_forest_download: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_download: nothing uploaded");
+    if (v->n_nodes != f->n_nodes)
+        return fail(OMK_ERR_INVALID, "omk_forest_download: view has %lld nodes, forest %lld", (long long)v->n_nodes,
+                    (long long)f->n_nodes);
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    const size_t b = (size_t)f->n_nodes * 4;
+    if (v->N) HIP_TRY(hipMemcpy(v->N, f->N, b, hipMemcpyDeviceToHost));
+    if (v->W) HIP_TRY(hipMemcpy(v->W, f->W, b, hipMemcpyDeviceToHost));
+    if (v->P) HIP_TRY(hipMemcpy(v->P, f->P, b, hipMemcpyDeviceToHost));
+    if (v->VL) HIP_TRY(hipMemcpy(v->VL, f->VL, b, hipMemcpyDeviceToHost));
+    if (f->has_rave && v->rN) HIP_TRY(hipMemcpy(v->rN, f->rN, b, hipMemcpyDeviceToHost));
+    if (f->has_rave && v->rW) HIP_TRY(hipMemcpy(v->rW, f->rW, b, hipMemcpyDeviceToHost));
+    return OMK_OK;
+}
+
+// ---------------------------------------------------------------- batch
+
+int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, omk_batch **out) {
+    if (!f || !out) return fail(OMK_ERR_INVALID, "omk_batch_create: null argument");
+    if (max_traversals <= 0 || max_traversals > (1 << 24))
+        return fail(OMK_ERR_INVALID, "omk_batch_create: max_traversals %d out of range", max_traversals);
+    if (max_depth <= 0 || max_depth > 4096)
+        return fail(OMK_ERR_INVALID, "omk_batch_create: max_depth %d out of range", max_depth);
+    if (int rc = use_device(f)) return rc;
+    omk_batch *b = new (std::nothrow) omk_batch();
+    if (!b) return fail(OMK_ERR_INVALID, "out of host memory");
+    b->f = f;
+    b->max_traversals = max_traversals;
+    b->max_depth = max_depth;
+    b->stride = (max_traversals + 63) & ~63;
+    const int64_t B = b->stride;
+    hipError_t e = dalloc(&b->paths, B * (max_depth + 1));
+    if (e == hipSuccess) e = dalloc(&b->path_len, B);
+    if (e == hipSuccess) e = dalloc(&b->leaf, B);
+    if (e == hipSuccess) e = dalloc(&b->values, B);
+    if (e == hipSuccess) e = dalloc(&b->items0, B);
+    if (e == hipSuccess) e = dalloc(&b->items[0], B);
+    if (e == hipSuccess) e = dalloc(&b->items[1], B);
+    if (e == hipSuccess) e = dalloc(&b->seg0, B);
+    if (e == hipSuccess) e = dalloc(&b->seg[0], B);
+    if (e == hipSuccess) e = dalloc(&b->seg[1], B);
+    if (e == hipSuccess) e = dalloc(&b->sc_child, B);
+    if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
+    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3);
+    if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
+    if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
+    if (e == hipSuccess) e = hipMemset(b->values, 0, (size_t)B * 4);
+    if (e != hipSuccess) {
+        int rc = fail(OMK_ERR_HIP, "omk_batch_create: %s", hipGetErrorString(e));
+        omk_batch_destroy(b);
+        return rc;
+    }
+    *out = b;
+    return OMK_OK;
+}
+
+int omk_batch_destroy(omk_batch *b) {
+    if (!b) return OMK_OK;
+    (void)hipSetDevice(b->f->device);
+    (void)hipStreamSynchronize(b->f->stream);
+    void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items[0],  b->items[1],  b->seg0,
+                    b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions};
+    for (void *p : ptrs)
+        if (p) (void)hipFree(p);
+    delete b;
+    return OMK_OK;
+}
+
+int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
+    if (!b || !h_roots) return fail(OMK_ERR_INVALID, "omk_batch_set_roots: null argument");
+    if (n <= 0 || n > b->max_traversals)
+        return fail(OMK_ERR_CAPACITY, "omk_batch_set_roots: %d traversals, batch holds %d", n, b->max_traversals);
+    omk_forest *f = b->f;
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_batch_set_roots: upload the forest first");
+    for (int32_t t = 0; t < n; t++)
+        if (h_roots[t] < 0 || h_roots[t] >= f->n_nodes)
+            return fail(OMK_ERR_INVALID, "omk_batch_set_roots: root %d of traversal %d outside [0, %lld)", h_roots[t],
+                        t, (long long)f->n_nodes);
+    // level-0 work items: traversals grouped by root, ascending traversal index inside a group
+    std::vector<int32_t> order((size_t)n);
+    for (int32_t t = 0; t < n; t++) order[(size_t)t] = t;
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t c) { return h_roots[a] < h_roots[c]; });
+    std::vector<Item> items;
+    for (int32_t i = 0; i < n;) {
+        int32_t j = i;
+        while (j < n && h_roots[order[(size_t)j]] == h_roots[order[(size_t)i]]) j++;
+        Item it;
+        it.node = h_roots[order[(size_t)i]];
+        it.off = i;
+        it.m = j - i;
+        it.np = 0;
+        items.push_back(it);
+        i = j;
+    }
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    HIP_TRY(hipMemcpy(b->seg0, order.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(b->items0, items.data(), items.size() * sizeof(Item), hipMemcpyHostToDevice));
+    b->n_items0 = (int32_t)items.size();
+    b->n = n;
+    b->selected = false;
+    return OMK_OK;
+}
+
+int omk_batch_set_values(omk_batch *b, const float *h_values, int32_t n) {
+    if (!b || !h_values) return fail(OMK_ERR_INVALID, "omk_batch_set_values: null argument");
+    if (n <= 0 || n > b->max_traversals) return fail(OMK_ERR_CAPACITY, "omk_batch_set_values: %d values", n);
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(hipMemcpyAsync(b->values, h_values, (size_t)n * 4, hipMemcpyHostToDevice, b->f->stream));
+    HIP_TRY(hipStreamSynchronize(b->f->stream));
+    return OMK_OK;
+}
+
+int omk_batch_device(omk_batch *b, omk_batch_dev *out) {
+    if (!b || !out) return fail(OMK_ERR_INVALID, "omk_batch_device: null argument");
+    out->d_paths = b->paths;
+    out->d_path_len = b->path_len;
+    out->d_leaf = b->leaf;
+    out->d_values = b->values;
+    out->stride = b->stride;
+    out->max_depth = b->max_depth;
+    out->n_traversals = b->n;
+    return OMK_OK;
+}
+
+int omk_select_batch(omk_batch *b, const omk_select_params *p) {
+    if (!b || !p) return fail(OMK_ERR_INVALID, "omk_select_batch: null argument");
+    omk_forest *f = b->f;
+    if (!f->uploaded || b->n <= 0) return fail(OMK_ERR_STATE, "omk_select_batch: upload a forest and set roots first");
+    if (p->use_rave && !f->has_rave)
+        return fail(OMK_ERR_INVALID, "omk_select_batch: use_rave on a forest created without RAVE arrays");
+    if (p->pw && !f->prior_sorted)
+        return fail(OMK_ERR_UNSUPPORTED,
+                    "omk_select_batch: progressive widening needs children stored in prior-descending order "
+                    "and no legal mask");
+    if (int rc = use_device(f)) return rc;
+    SelectArgs a;
+    memset(&a, 0, sizeof(a));
+    a.counters = b->counters;
+    a.truncated = b->counters + b->max_depth + 2;
+    a.sc_child = b->sc_child;
+    a.sc_occ = b->sc_occ;
+    a.paths = b->paths;
+    a.path_len = b->path_len;
+    a.leaf = b->leaf;
+    a.stride = b->stride;
+    a.max_depth = b->max_depth;
+    a.vl = p->virtual_loss;
+    a.pw = p->pw;
+    a.c_puct = p->c_puct;
+    a.rave_k = p->rave_k;
+    BatchBuffers bb;
+    bb.items0 = b->items0;
+    bb.seg0 = b->seg0;
+    bb.n_items0 = b->n_items0;
+    bb.items[0] = b->items[0];
+    bb.items[1] = b->items[1];
+    bb.seg[0] = b->seg[0];
+    bb.seg[1] = b->seg[1];
+    bb.n_traversals = b->n;
+    HIP_TRY(launch_select(f->dev(), a, bb, f->max_fanout, p->use_rave != 0, f->stream));
+    b->selected = true;
+    return OMK_OK;
+}
+
+int omk_backup_batch(omk_batch *b, int32_t virtual_loss) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_backup_batch: null batch");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_backup_batch: no selected paths");
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(launch_backup(b->f->dev(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
+                          virtual_loss, b->f->stream));
+    return OMK_OK;
+}
+
+int omk_revert_vl(omk_batch *b, int32_t virtual_loss) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_revert_vl: null batch");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_revert_vl: no selected paths");
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(launch_revert_vl(b->f->dev(), b->paths, b->path_len, b->n, b->stride, b->max_depth + 1, virtual_loss,
+                             b->f->stream));
+    return OMK_OK;
+}
+
+static int check_paths_args(const char *who, omk_forest *f, const void *paths, const void *len, int32_t n,
+                            int32_t stride, int32_t max_len) {
+    if (!f || !paths || !len) return fail(OMK_ERR_INVALID, "%s: null argument", who);
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "%s: upload the forest first", who);
+    if (n < 0 || stride < n || max_len < 0 || max_len > 4097)
+        return fail(OMK_ERR_INVALID, "%s: n %d stride %d max_len %d", who, n, stride, max_len);
+    return use_device(f);
+}
+
+int omk_apply_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len, int32_t n, int32_t stride,
+                       int32_t max_len, int32_t virtual_loss) {
+    if (int rc = check_paths_args("omk_apply_vl_paths", f, d_paths, d_path_len, n, stride, max_len)) return rc;
+    HIP_TRY(launch_apply_vl(f->dev(), d_paths, d_path_len, n, stride, max_len, virtual_loss, f->stream));
+    return OMK_OK;
+}
+
+int omk_revert_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len, int32_t n, int32_t stride,
+                        int32_t max_len, int32_t virtual_loss) {
+    if (int rc = check_paths_args("omk_revert_vl_paths", f, d_paths, d_path_len, n, stride, max_len)) return rc;
+    HIP_TRY(launch_revert_vl(f->dev(), d_paths, d_path_len, n, stride, max_len, virtual_loss, f->stream));
+    return OMK_OK;
+}
+
+int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len, const float *d_values,
+                     int32_t n, int32_t stride, int32_t max_len, int32_t virtual_loss) {
+    if (int rc = check_paths_args("omk_backup_paths", f, d_paths, d_path_len, n, stride, max_len)) return rc;
+    if (!d_values) return fail(OMK_ERR_INVALID, "omk_backup_paths: null values");
+    HIP_TRY(launch_backup(f->dev(), d_paths, d_path_len, d_values, n, stride, max_len, virtual_loss, f->stream));
+    return OMK_OK;
+}
+
+int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t *h_leaf, int32_t *h_actions) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_batch_read: null batch");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_read: no selected paths");
+    omk_forest *f = b->f;
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    const int n = b->n, D = b->max_depth;
+    if (h_paths || h_actions)
+        HIP_TRY(launch_export(f->dev(), b->paths, b->path_len, n, b->stride, D, h_paths ? b->out_paths : nullptr,
+                              h_actions ? b->out_actions : nullptr, s));
+    if (h_paths) HIP_TRY(hipMemcpyAsync(h_paths, b->out_paths, (size_t)n * (D + 1) * 4, hipMemcpyDeviceToHost, s));
+    if (h_actions) HIP_TRY(hipMemcpyAsync(h_actions, b->out_actions, (size_t)n * D * 4, hipMemcpyDeviceToHost, s));
+    if (h_path_len) HIP_TRY(hipMemcpyAsync(h_path_len, b->path_len, (size_t)n * 4, hipMemcpyDeviceToHost, s));
+    if (h_leaf) HIP_TRY(hipMemcpyAsync(h_leaf, b->leaf, (size_t)n * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return OMK_OK;
+}
+
+int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
+    if (!b || !h_count) return fail(OMK_ERR_INVALID, "omk_batch_truncated: null argument");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_truncated: no selected paths");
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(hipMemcpyAsync(h_count, b->counters + b->max_depth + 2, 4, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipStreamSynchronize(b->f->stream));
+    return OMK_OK;
+}
+
+// ---------------------------------------------------------------- transposition table
+
+int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out) {
+    if (!f || !out) return fail(OMK_ERR_INVALID, "omk_tt_create: null argument");
+    if (log2_slots < 4 || log2_slots > 30) return fail(OMK_ERR_INVALID, "omk_tt_create: log2_slots %d", log2_slots);
+    if (int rc = use_device(f)) return rc;
+    omk_tt *tt = new (std::nothrow) omk_tt();
+    if (!tt) return fail(OMK_ERR_INVALID, "out of host memory");
+    tt->f = f;
+    tt->log2_slots = log2_slots;
+    hipError_t e = dalloc(&tt->slots, 1ll << log2_slots);
+    if (e == hipSuccess) e = dalloc(&tt->d_status, 2);
+    if (e != hipSuccess) {
+        int rc = fail(OMK_ERR_HIP, "omk_tt_create: %s", hipGetErrorString(e));
+        omk_tt_destroy(tt);
+        return rc;
+    }
+    *out = tt;
+    return omk_tt_clear(tt);
+}
+
+int omk_tt_destroy(omk_tt *tt) {
+    if (!tt) return OMK_OK;
+    (void)hipSetDevice(tt->f->device);
+    (void)hipStreamSynchronize(tt->f->stream);
+    if (tt->slots) (void)hipFree(tt->slots);
+    if (tt->d_status) (void)hipFree(tt->d_status);
+    delete tt;
+    return OMK_OK;
+}
+
+int omk_tt_clear(omk_tt *tt) {
+    if (!tt) return fail(OMK_ERR_INVALID, "omk_tt_clear: null table");
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(launch_tt_clear(tt->slots, tt->log2_slots, tt->f->stream));
+    return OMK_OK;
+}
+
+int omk_tt_insert(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, const int32_t *d_depths, int64_t n) {
+    if (!tt || !d_keys || !d_nodes) return fail(OMK_ERR_INVALID, "omk_tt_insert: null argument");
+    if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_insert: n %lld", (long long)n);
+    if (int rc = use_device(tt->f)) return rc;
+    hipStream_t s = tt->f->stream;
+    int status[2] = {0, 0};
+    HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
+    HIP_TRY(launch_tt_insert(tt->slots, tt->log2_slots, d_keys, d_nodes, d_depths, n, tt->d_status, s));
+    HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (status[1]) return fail(OMK_ERR_INVALID, "omk_tt_insert: %d keys equal the empty marker ~0", status[1]);
+    if (status[0]) return fail(OMK_ERR_CAPACITY, "omk_tt_insert: table full, %d entries dropped", status[0]);
+    return OMK_OK;
+}
+
+int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_depth, int32_t *d_out) {
+    if (!tt || !d_keys || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe: null argument");
+    if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_probe: n %lld", (long long)n);
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, n, min_depth, d_out, tt->f->stream));
+    return OMK_OK;
+}
+
+int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_out) {
+    if (!tt || !b || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe_leaves: null argument");
+    if (tt->f != b->f) return fail(OMK_ERR_INVALID, "omk_tt_probe_leaves: table and batch belong to different forests");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: no selected paths");
+    if (!b->f->has_hash) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: the forest was uploaded without position keys");
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->n, min_depth, d_out,
+                            tt->f->stream));
+    return OMK_OK;
+}
+
+int omk_tt_upload(omk_tt *tt, const omk_tt_slot *h_slots) {
+    if (!tt || !h_slots) return fail(OMK_ERR_INVALID, "omk_tt_upload: null argument");
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(hipStreamSynchronize(tt->f->stream));
+    HIP_TRY(hipMemcpy(tt->slots, h_slots, sizeof(TTSlot) << tt->log2_slots, hipMemcpyHostToDevice));
+    return OMK_OK;
+}
+
+int omk_tt_download(omk_tt *tt, omk_tt_slot *h_slots) {
+    if (!tt || !h_slots) return fail(OMK_ERR_INVALID, "omk_tt_download: null argument");
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(hipStreamSynchronize(tt->f->stream));
+    HIP_TRY(hipMemcpy(h_slots, tt->slots, sizeof(TTSlot) << tt->log2_slots, hipMemcpyDeviceToHost));
+    return OMK_OK;
+}
+
+// ---------------------------------------------------------------- device memory helpers
+
+int omk_dev_alloc(omk_forest *f, int64_t bytes, void **d_out) {
+    if (!f || !d_out || bytes < 0) return fail(OMK_ERR_INVALID, "omk_dev_alloc: bad argument");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipMalloc(d_out, (size_t)std::max<int64_t>(bytes, 1)));
+    return OMK_OK;
+}
+
+int omk_dev_free(omk_forest *f, void *d_ptr) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_dev_free: null forest");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    if (d_ptr) HIP_TRY(hipFree(d_ptr));
+    return OMK_OK;
+}
+
+int omk_dev_h2d(omk_forest *f, void *d_dst, const void *h_src, int64_t bytes) {
+    if (!f || !d_dst || !h_src || bytes < 0) return fail(OMK_ERR_INVALID, "omk_dev_h2d: bad argument");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipMemcpyAsync(d_dst, h_src, (size_t)bytes, hipMemcpyHostToDevice, f->stream));
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    return OMK_OK;
+}
+
+int omk_dev_d2h(omk_forest *f, void *h_dst, const void *d_src, int64_t bytes) {
+    if (!f || !h_dst || !d_src || bytes < 0) return fail(OMK_ERR_INVALID, "omk_dev_d2h: bad argument");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipMemcpyAsync(h_dst, d_src, (size_t)bytes, hipMemcpyDeviceToHost, f->stream));
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    return OMK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,242 @@
+// Virtual-loss apply / revert, value backup, leaf gather export and the transposition
+// table probes: the scattered read-modify-write side of the search step.
+//
+// Node operations restated from the reference (src/mcts/mcts_node_virtual_loss.cpp):
+//   addVirtualLoss(a)     :15-20   if a > 0: VL += a
+//   removeVirtualLoss(a)  :32-42   if a > 0: old = VL; VL -= a; if old < a: VL = 0
+//   update(v)             :54-71   N += 1; W += v; if VL > 0: VL -= 1
+// and the backup loop src/mcts/mcts_engine_batch_tree_simple.cpp:276-281
+//   for node in reversed(path): update(v); removeVirtualLoss(a); v = -v
+//
+// Counter algebra used below.  One backup visit maps VL = x to
+//   a > 0 :  max(0, x - (a+1))      (x <= 0 gives 0 as well)
+//   a <= 0:  x > 0 ? x - 1 : x
+// and one revert maps x to max(0, x - a).  Each is a "subtract, clamp at zero" map, so m
+// visits in ANY order give max(0, x - k*m): the result of the serial reference does not
+// depend on the order, and "atomic subtract, then atomic max with 0 if the old value was
+// too small" reaches it without a lock (after the first clamp fires the value never
+// rises above 0 again, and the last operation on the address is always a clamp or a
+// subtract that stayed non-negative).
+#include "omk_internal.h"
+
+namespace omk {
+
+__device__ __forceinline__ void vl_sub_clamp(int32_t *addr, int k) {
+    int old = atomicSub(addr, k);
+    if (old < k) atomicMax(addr, 0);
+}
+
+// x > 0 ? max(0, x - k) : x   (update() without a following revert)
+__device__ __forceinline__ void vl_dec_if_positive(int32_t *addr, int k) {
+    int old = *(volatile int32_t *)addr;
+    while (old > 0) {
+        int want = old > k ? old - k : 0;
+        int prev = atomicCAS(addr, old, want);
+        if (prev == old) break;
+        old = prev;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_apply_vl(ForestDev f, const int32_t *paths, const int32_t *path_len, int n,
+                                                  int stride, int vl) {
+    int t = blockIdx.x * 256 + threadIdx.x;
+    int d = blockIdx.y + 1;  // the root of a path never receives virtual loss
+    if (t >= n || d >= path_len[t]) return;
+    atomicAdd(f.VL + paths[(size_t)d * stride + t], vl);
+}
+
+__global__ __launch_bounds__(256) void k_revert_vl(ForestDev f, const int32_t *paths, const int32_t *path_len, int n,
+                                                   int stride, int vl) {
+    int t = blockIdx.x * 256 + threadIdx.x;
+    int d = blockIdx.y;
+    bool act = t < n && d < path_len[t];
+    int node = act ? paths[(size_t)d * stride + t] : -1;
+    uint64_t mask = __ballot(act);
+    if (mask == 0ull) return;
+    int leader = __ffsll((long long)mask) - 1;
+    int node0 = __builtin_amdgcn_readlane(node, leader);
+    if (__ballot(act && node != node0) == 0ull) {
+        // the whole wave sits on one node (top of a single tree): one combined operation
+        if ((int)(threadIdx.x & 63) == leader) vl_sub_clamp(f.VL + node0, vl * __popcll(mask));
+        return;
+    }
+    if (act) vl_sub_clamp(f.VL + node, vl);
+}
+
+__global__ __launch_bounds__(256) void k_backup(ForestDev f, const int32_t *paths, const int32_t *path_len,
+                                                const float *values, int n, int stride, int vl) {
+    int t = blockIdx.x * 256 + threadIdx.x;
+    int d = blockIdx.y;
+    int len = t < n ? path_len[t] : 0;
+    bool act = d < len;
+    int node = act ? paths[(size_t)d * stride + t] : -1;
+    float v = 0.0f;
+    if (act) {
+        v = values[t];
+        if ((len - 1 - d) & 1) v = -v;  // the leaf receives +value, every ply up flips it
+    }
+    uint64_t mask = __ballot(act);
+    if (mask == 0ull) return;
+    int leader = __ffsll((long long)mask) - 1;
+    int node0 = __builtin_amdgcn_readlane(node, leader);
+    bool same = __ballot(act && node != node0) == 0ull;
+    if (same) {
+        float sum = wave_sum_f32(v);
+        if ((int)(threadIdx.x & 63) == leader) {
+            int cnt = __popcll(mask);
+            atomicAdd(f.N + node0, cnt);
+            unsafeAtomicAdd(f.W + node0, sum);
+            if (vl > 0) vl_sub_clamp(f.VL + node0, (vl + 1) * cnt);
+            else vl_dec_if_positive(f.VL + node0, cnt);
+        }
+        return;
+    }
+    if (act) {
+        atomicAdd(f.N + node, 1);
+        unsafeAtomicAdd(f.W + node, v);
+        if (vl > 0) vl_sub_clamp(f.VL + node, vl + 1);
+        else vl_dec_if_positive(f.VL + node, 1);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_export(ForestDev f, const int32_t *paths, const int32_t *path_len, int n,
+                                                int stride, int max_depth, int32_t *out_paths,
+                                                int32_t *out_actions) {
+    int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int row = max_depth + 1;
+    if (g >= (int64_t)n * row) return;
+    int t = (int)(g / row);
+    int d = (int)(g - (int64_t)t * row);
+    int len = path_len[t];
+    int node = d < len ? paths[(size_t)d * stride + t] : -1;
+    if (out_paths) out_paths[g] = node;
+    if (out_actions && d >= 1) {
+        int act = -1;
+        if (node >= 0) act = f.action ? f.action[node] : node;
+        out_actions[(int64_t)t * max_depth + d - 1] = act;
+    }
+}
+
+hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                           int max_len, int vl, hipStream_t s) {
+    if (vl <= 0 || n <= 0 || max_len <= 1) return hipSuccess;
+    hipLaunchKernelGGL(k_apply_vl, dim3((n + 255) / 256, max_len - 1), dim3(256), 0, s, f, paths, path_len, n,
+                       stride, vl);
+    return hipGetLastError();
+}
+
+hipError_t launch_revert_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                            int max_len, int vl, hipStream_t s) {
+    if (vl <= 0 || n <= 0 || max_len <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_revert_vl, dim3((n + 255) / 256, max_len), dim3(256), 0, s, f, paths, path_len, n, stride,
+                       vl);
+    return hipGetLastError();
+}
+
+hipError_t launch_backup(const ForestDev &f, const int32_t *paths, const int32_t *path_len, const float *values,
+                         int n, int stride, int max_len, int vl, hipStream_t s) {
+    if (n <= 0 || max_len <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_backup, dim3((n + 255) / 256, max_len), dim3(256), 0, s, f, paths, path_len, values, n,
+                       stride, vl);
+    return hipGetLastError();
+}
+
+hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                         int max_depth, int32_t *out_paths, int32_t *out_actions, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    int64_t total = (int64_t)n * (max_depth + 1);
+    hipLaunchKernelGGL(k_export, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, f, paths, path_len, n,
+                       stride, max_depth, out_paths, out_actions);
+    return hipGetLastError();
+}
+
+// ---- open-addressing transposition table: 16-byte slots, linear probing ----
+
+constexpr unsigned long long kTTEmpty = ~0ull;
+
+__device__ __forceinline__ uint64_t tt_home(uint64_t key, int log2_slots) {
+    return (key * 0x9E3779B97F4A7C15ull) >> (64 - log2_slots);
+}
+
+__global__ __launch_bounds__(256) void k_tt_clear(TTSlot *slots, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    TTSlot e;
+    e.key = kTTEmpty;
+    e.node = -1;
+    e.depth = 0;
+    slots[i] = e;
+}
+
+// d_status[0] counts entries that found no slot, d_status[1] keys equal to the empty marker
+__global__ __launch_bounds__(256) void k_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys,
+                                                   const int32_t *nodes, const int32_t *depths, int64_t n,
+                                                   int *d_status) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    unsigned long long key = keys[i];
+    if (key == kTTEmpty) {
+        atomicAdd(d_status + 1, 1);
+        return;
+    }
+    uint64_t mask = (1ull << log2_slots) - 1ull;
+    uint64_t s = tt_home(key, log2_slots);
+    for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+        unsigned long long prev = atomicCAS(&slots[s].key, kTTEmpty, key);
+        if (prev == kTTEmpty) {
+            slots[s].node = nodes[i];
+            slots[s].depth = depths ? depths[i] : 0;
+            return;
+        }
+        if (prev == key) return;  // already present: the first entry stays
+    }
+    atomicAdd(d_status, 1);
+}
+
+__global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys,
+                                                  const int32_t *leaf, const uint64_t *node_hash, int64_t n,
+                                                  int min_depth, int32_t *out) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    unsigned long long key = keys ? keys[i] : node_hash[leaf[i]];
+    int found = -1;
+    if (key != kTTEmpty) {
+        uint64_t mask = (1ull << log2_slots) - 1ull;
+        uint64_t s = tt_home(key, log2_slots);
+        for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+            // one 16-byte load per slot touched
+            uint4 raw = *reinterpret_cast<const uint4 *>(slots + s);
+            unsigned long long k = ((unsigned long long)raw.y << 32) | raw.x;
+            if (k == key) {
+                if ((int)raw.w >= min_depth) found = (int)raw.z;
+                break;
+            }
+            if (k == kTTEmpty) break;
+        }
+    }
+    out[i] = found;
+}
+
+hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s) {
+    int64_t n = 1ll << log2_slots;
+    hipLaunchKernelGGL(k_tt_clear, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
+                           const uint64_t *node_hash, int64_t n, int min_depth, int32_t *out, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_tt_probe, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, log2_slots, keys, leaf,
+                       node_hash, n, min_depth, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
+                            const int32_t *depths, int64_t n, int *d_status, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_tt_insert, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, log2_slots, keys,
+                       nodes, depths, n, d_status);
+    return hipGetLastError();
+}
+
+}  // namespace omk

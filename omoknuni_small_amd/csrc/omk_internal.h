@@ -1,0 +1,89 @@
+// Internal declarations shared by the translation units of libomk_forest.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "omk_device.h"
+
+namespace omk {
+
+// Per-node arrays in HBM (structure of arrays; siblings are contiguous in every array).
+struct ForestDev {
+    const int2 *span;  // (child_begin, child_count); child_count 0 = not expanded
+    int32_t *N;
+    float *W;
+    const float *P;
+    int32_t *VL;
+    const int32_t *rN;
+    const float *rW;
+    const uint32_t *legal;  // nullptr = every slot holds a child
+    const int32_t *action;  // nullptr = node id
+    const uint64_t *hash;   // nullptr = none
+    int64_t n_nodes;
+};
+
+// A node together with the traversals that reached it: seg[off .. off+m) holds their
+// indices in ascending order.  np is the node's visit count as read by the parent's wave.
+struct Item {
+    int32_t node;
+    int32_t off;
+    int32_t m;
+    int32_t np;
+};
+
+struct SelectArgs {
+    const Item *items_in;
+    Item *items_out;
+    int32_t *counters;  // counters[d] = number of items of level d
+    const int32_t *seg_in;
+    int32_t *seg_out;
+    int32_t *sc_child;  // per visitor: chosen child index
+    int32_t *sc_occ;    // per visitor: how many earlier visitors of the item chose the same child
+    int32_t *paths;     // level-major [max_depth+1][stride]
+    int32_t *path_len;
+    int32_t *leaf;
+    int32_t *truncated;
+    int32_t stride;
+    int32_t max_depth;
+    int32_t vl;
+    int32_t pw;
+    float c_puct;
+    float rave_k;
+};
+
+struct BatchBuffers {
+    Item *items0;  // level-0 items, built by set_roots
+    int32_t *seg0;
+    int32_t n_items0;
+    Item *items[2];
+    int32_t *seg[2];
+    int32_t n_traversals;
+};
+
+hipError_t launch_select(const ForestDev &f, SelectArgs a, const BatchBuffers &b, int max_fanout, bool rave,
+                         hipStream_t s);
+
+hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                           int max_len, int vl, hipStream_t s);
+hipError_t launch_revert_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                            int max_len, int vl, hipStream_t s);
+hipError_t launch_backup(const ForestDev &f, const int32_t *paths, const int32_t *path_len, const float *values,
+                         int n, int stride, int max_len, int vl, hipStream_t s);
+// row-major copies for the host: paths [n][max_depth+1], actions [n][max_depth], -1 padded
+hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                         int max_depth, int32_t *out_paths, int32_t *out_actions, hipStream_t s);
+
+struct TTSlot {
+    unsigned long long key;
+    int32_t node;
+    int32_t depth;
+};
+hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s);
+// d_status[0] += entries that found no free slot, d_status[1] += keys equal to the empty marker
+hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
+                            const int32_t *depths, int64_t n, int *d_status, hipStream_t s);
+hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
+                           const uint64_t *node_hash, int64_t n, int min_depth, int32_t *out, hipStream_t s);
+
+}  // namespace omk

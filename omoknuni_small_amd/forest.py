@@ -1,0 +1,349 @@
+"""Host-side mirror of the C ABI in include/omk_forest.h.
+
+The classes follow the phases of the reference's MCTSEngine::executeBatchedTreeSearch
+(src/mcts/mcts_engine_batch_tree_simple.cpp): Batch.select() is phase 1 (selectChild +
+applyVirtualLoss down to a leaf), Batch.read() is the leaf gather, Batch.backup() is
+phase 3 (update + revertVirtualLoss, sign flipped per ply).  Every call goes through
+libomk_forest.so; there is no host fallback, and loading fails loudly when the library
+has not been built.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+i32p = C.POINTER(C.c_int32)
+f32p = C.POINTER(C.c_float)
+u32p = C.POINTER(C.c_uint32)
+u64p = C.POINTER(C.c_uint64)
+
+EXPORTS = [
+    "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream",
+    "omk_forest_upload", "omk_forest_download", "omk_sync", "omk_batch_create", "omk_batch_destroy",
+    "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
+    "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
+    "omk_batch_truncated", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
+    "omk_dev_d2h",
+]
+
+TT_SLOT = np.dtype([("key", "<u8"), ("node", "<i4"), ("depth", "<i4")])
+
+
+class OmkError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("omk status %d: %s" % (code, message))
+        self.code = code
+
+
+class _SoaView(C.Structure):
+    _fields_ = [("n_nodes", C.c_int64), ("N", i32p), ("W", f32p), ("P", f32p), ("VL", i32p), ("rN", i32p),
+                ("rW", f32p), ("child_begin", i32p), ("child_count", i32p), ("action", i32p), ("legal", u32p),
+                ("hash", u64p)]
+
+
+class _ForestDesc(C.Structure):
+    _fields_ = [("capacity_nodes", C.c_int64), ("device", C.c_int32), ("has_rave", C.c_int32)]
+
+
+class SelectParams(C.Structure):
+    """MCTSSettings fields read on this path (reference include/mcts/mcts_engine.h:81-112)."""
+    _fields_ = [("c_puct", C.c_float), ("virtual_loss", C.c_int32), ("use_rave", C.c_int32),
+                ("rave_k", C.c_float), ("pw", C.c_int32)]
+
+    def __init__(self, c_puct=1.4, virtual_loss=3, use_rave=False, rave_k=3000.0, pw=False):
+        super().__init__(c_puct, int(virtual_loss), int(bool(use_rave)), rave_k, int(bool(pw)))
+
+
+class _BatchDev(C.Structure):
+    _fields_ = [("d_paths", C.c_void_p), ("d_path_len", C.c_void_p), ("d_leaf", C.c_void_p),
+                ("d_values", C.c_void_p), ("stride", C.c_int32), ("max_depth", C.c_int32),
+                ("n_traversals", C.c_int32)]
+
+
+def library_path():
+    return os.path.join(_HERE, "libomk_forest.so")
+
+
+def load_library():
+    """Loads libomk_forest.so; raises when it is missing rather than falling back to anything."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    so = library_path()
+    if not os.path.exists(so):
+        raise OSError("%s is missing: build it with `python -m omoknuni_small_amd.build` "
+                      "(there is no host fallback for the HIP path)" % so)
+    L = C.CDLL(so)
+    L.omk_last_error.restype = C.c_char_p
+    for name in EXPORTS:
+        if name != "omk_last_error":
+            getattr(L, name).restype = C.c_int
+    _LIB = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise OmkError(rc, load_library().omk_last_error().decode())
+
+
+def _ptr(a, ty):
+    return a.ctypes.data_as(ty) if a is not None else ty()
+
+
+def _arr(x, dtype):
+    return None if x is None else np.ascontiguousarray(x, dtype=dtype)
+
+
+class Forest:
+    """Device-resident forest: the per-node arrays that replace the MCTSNode pointer tree."""
+
+    def __init__(self, capacity_nodes, device=0, has_rave=False):
+        self._lib = load_library()
+        self._h = C.c_void_p()
+        self.has_rave = bool(has_rave)
+        self.n_nodes = 0
+        desc = _ForestDesc(int(capacity_nodes), int(device), int(self.has_rave))
+        _check(self._lib.omk_forest_create(C.byref(desc), C.byref(self._h)))
+
+    @classmethod
+    def from_soa(cls, soa, device=0):
+        f = cls(len(soa["N"]), device=device, has_rave=soa.get("rN") is not None)
+        f.upload(soa)
+        return f
+
+    def close(self):
+        if self._h:
+            self._lib.omk_forest_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_stream(self, hip_stream):
+        _check(self._lib.omk_forest_set_stream(self._h, C.c_void_p(hip_stream or 0)))
+
+    def sync(self):
+        _check(self._lib.omk_sync(self._h))
+
+    def upload(self, soa):
+        keep = dict(N=_arr(soa["N"], np.int32), W=_arr(soa["W"], np.float32), P=_arr(soa["P"], np.float32),
+                    VL=_arr(soa["VL"], np.int32), rN=_arr(soa.get("rN"), np.int32), rW=_arr(soa.get("rW"), np.float32),
+                    child_begin=_arr(soa["child_begin"], np.int32), child_count=_arr(soa["child_count"], np.int32),
+                    action=_arr(soa.get("action"), np.int32), legal=_arr(soa.get("legal"), np.uint32),
+                    hash=_arr(soa.get("hash"), np.uint64))
+        n = len(keep["N"])
+        for k in ("W", "P", "VL", "child_begin", "child_count", "rN", "rW", "action", "hash"):
+            if keep[k] is not None and len(keep[k]) != n:
+                raise ValueError("array %s has %d entries, N has %d" % (k, len(keep[k]), n))
+        if keep["legal"] is not None and len(keep["legal"]) * 32 < n:
+            raise ValueError("legal mask shorter than the node count")
+        v = _SoaView(n, _ptr(keep["N"], i32p), _ptr(keep["W"], f32p), _ptr(keep["P"], f32p), _ptr(keep["VL"], i32p),
+                     _ptr(keep["rN"], i32p), _ptr(keep["rW"], f32p), _ptr(keep["child_begin"], i32p),
+                     _ptr(keep["child_count"], i32p), _ptr(keep["action"], i32p), _ptr(keep["legal"], u32p),
+                     _ptr(keep["hash"], u64p))
+        _check(self._lib.omk_forest_upload(self._h, C.byref(v)))
+        self.n_nodes = n
+
+    def download(self):
+        """Returns dict(N, W, P, VL[, rN, rW]) as numpy arrays."""
+        n = self.n_nodes
+        out = dict(N=np.empty(n, np.int32), W=np.empty(n, np.float32), P=np.empty(n, np.float32),
+                   VL=np.empty(n, np.int32))
+        if self.has_rave:
+            out["rN"] = np.empty(n, np.int32)
+            out["rW"] = np.empty(n, np.float32)
+        v = _SoaView(n, _ptr(out["N"], i32p), _ptr(out["W"], f32p), _ptr(out["P"], f32p), _ptr(out["VL"], i32p),
+                     _ptr(out.get("rN"), i32p), _ptr(out.get("rW"), f32p), i32p(), i32p(), i32p(), u32p(), u64p())
+        _check(self._lib.omk_forest_download(self._h, C.byref(v)))
+        return out
+
+    # device memory helpers (for callers without their own HIP binding)
+    def dev_alloc(self, nbytes):
+        p = C.c_void_p()
+        _check(self._lib.omk_dev_alloc(self._h, int(nbytes), C.byref(p)))
+        return p.value
+
+    def dev_free(self, ptr):
+        _check(self._lib.omk_dev_free(self._h, C.c_void_p(ptr)))
+
+    def h2d(self, dptr, arr):
+        arr = np.ascontiguousarray(arr)
+        _check(self._lib.omk_dev_h2d(self._h, C.c_void_p(dptr), arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+
+    def d2h(self, arr, dptr):
+        assert arr.flags["C_CONTIGUOUS"]
+        _check(self._lib.omk_dev_d2h(self._h, arr.ctypes.data_as(C.c_void_p), C.c_void_p(dptr), arr.nbytes))
+
+    # the three node operations over caller-supplied device paths (level-major)
+    def apply_vl_paths(self, d_paths, d_len, n, stride, max_len, vl):
+        _check(self._lib.omk_apply_vl_paths(self._h, C.c_void_p(d_paths), C.c_void_p(d_len), int(n), int(stride),
+                                            int(max_len), int(vl)))
+
+    def revert_vl_paths(self, d_paths, d_len, n, stride, max_len, vl):
+        _check(self._lib.omk_revert_vl_paths(self._h, C.c_void_p(d_paths), C.c_void_p(d_len), int(n), int(stride),
+                                             int(max_len), int(vl)))
+
+    def backup_paths(self, d_paths, d_len, d_values, n, stride, max_len, vl):
+        _check(self._lib.omk_backup_paths(self._h, C.c_void_p(d_paths), C.c_void_p(d_len), C.c_void_p(d_values),
+                                          int(n), int(stride), int(max_len), int(vl)))
+
+
+class Batch:
+    """The per-search buffers of executeBatchedTreeSearch: paths, leaves, leaf values."""
+
+    def __init__(self, forest, max_traversals, max_depth):
+        self._lib = load_library()
+        self.forest = forest
+        self.max_traversals = int(max_traversals)
+        self.max_depth = int(max_depth)
+        self.n = 0
+        self._h = C.c_void_p()
+        _check(self._lib.omk_batch_create(forest._h, self.max_traversals, self.max_depth, C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            self._lib.omk_batch_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_roots(self, roots):
+        roots = np.ascontiguousarray(roots, dtype=np.int32)
+        _check(self._lib.omk_batch_set_roots(self._h, _ptr(roots, i32p), len(roots)))
+        self.n = len(roots)
+
+    def set_values(self, values):
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        _check(self._lib.omk_batch_set_values(self._h, _ptr(values, f32p), len(values)))
+
+    def select(self, params):
+        _check(self._lib.omk_select_batch(self._h, C.byref(params)))
+
+    def backup(self, virtual_loss):
+        _check(self._lib.omk_backup_batch(self._h, int(virtual_loss)))
+
+    def revert_vl(self, virtual_loss):
+        _check(self._lib.omk_revert_vl(self._h, int(virtual_loss)))
+
+    def read(self):
+        """Leaf gather: (paths [n, max_depth+1], path_len [n], leaf [n], actions [n, max_depth])."""
+        n, D = self.n, self.max_depth
+        paths = np.empty((n, D + 1), np.int32)
+        plen = np.empty(n, np.int32)
+        leaf = np.empty(n, np.int32)
+        actions = np.empty((n, D), np.int32)
+        _check(self._lib.omk_batch_read(self._h, _ptr(paths, i32p), _ptr(plen, i32p), _ptr(leaf, i32p),
+                                        _ptr(actions, i32p)))
+        return paths, plen, leaf, actions
+
+    def truncated(self):
+        c = C.c_int32()
+        _check(self._lib.omk_batch_truncated(self._h, C.byref(c)))
+        return c.value
+
+    def device(self):
+        d = _BatchDev()
+        _check(self._lib.omk_batch_device(self._h, C.byref(d)))
+        return d
+
+
+class TranspositionTable:
+    """Open-addressing table in HBM standing in for PHMapTranspositionTable store/lookup."""
+
+    def __init__(self, forest, log2_slots):
+        self._lib = load_library()
+        self.forest = forest
+        self.log2 = int(log2_slots)
+        self._h = C.c_void_p()
+        _check(self._lib.omk_tt_create(forest._h, self.log2, C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            self._lib.omk_tt_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def clear(self):
+        _check(self._lib.omk_tt_clear(self._h))
+
+    def insert_dev(self, d_keys, d_nodes, d_depths, n):
+        _check(self._lib.omk_tt_insert(self._h, C.c_void_p(d_keys), C.c_void_p(d_nodes), C.c_void_p(d_depths or 0),
+                                       int(n)))
+
+    def probe_dev(self, d_keys, n, d_out, min_depth=0):
+        _check(self._lib.omk_tt_probe(self._h, C.c_void_p(d_keys), int(n), int(min_depth), C.c_void_p(d_out)))
+
+    def probe_leaves_dev(self, batch, d_out, min_depth=0):
+        _check(self._lib.omk_tt_probe_leaves(self._h, batch._h, int(min_depth), C.c_void_p(d_out)))
+
+    def insert(self, keys, nodes, depths=None):
+        f = self.forest
+        keys = np.ascontiguousarray(keys, np.uint64)
+        nodes = np.ascontiguousarray(nodes, np.int32)
+        n = len(keys)
+        dk, dn = f.dev_alloc(n * 8), f.dev_alloc(n * 4)
+        dd = 0
+        try:
+            f.h2d(dk, keys)
+            f.h2d(dn, nodes)
+            if depths is not None:
+                dd = f.dev_alloc(n * 4)
+                f.h2d(dd, np.ascontiguousarray(depths, np.int32))
+            self.insert_dev(dk, dn, dd, n)
+        finally:
+            for p in (dk, dn, dd):
+                if p:
+                    f.dev_free(p)
+
+    def probe(self, keys, min_depth=0):
+        f = self.forest
+        keys = np.ascontiguousarray(keys, np.uint64)
+        n = len(keys)
+        out = np.empty(n, np.int32)
+        dk, do = f.dev_alloc(n * 8), f.dev_alloc(n * 4)
+        try:
+            f.h2d(dk, keys)
+            self.probe_dev(dk, n, do, min_depth)
+            f.d2h(out, do)
+        finally:
+            f.dev_free(dk)
+            f.dev_free(do)
+        return out
+
+    def probe_leaves(self, batch, min_depth=0):
+        f = self.forest
+        out = np.empty(batch.n, np.int32)
+        do = f.dev_alloc(batch.n * 4)
+        try:
+            self.probe_leaves_dev(batch, do, min_depth)
+            f.d2h(out, do)
+        finally:
+            f.dev_free(do)
+        return out
+
+    def upload(self, slots):
+        slots = np.ascontiguousarray(slots, dtype=TT_SLOT)
+        assert len(slots) == 1 << self.log2
+        _check(self._lib.omk_tt_upload(self._h, slots.ctypes.data_as(C.c_void_p)))
+
+    def download(self):
+        slots = np.empty(1 << self.log2, dtype=TT_SLOT)
+        _check(self._lib.omk_tt_download(self._h, slots.ctypes.data_as(C.c_void_p)))
+        return slots

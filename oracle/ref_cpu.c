@@ -1,0 +1,320 @@
+/*
+ * ref_cpu.c -- see ref_cpu.h.  TEST INFRASTRUCTURE ONLY: the checker and the
+ * timed CPU baseline, never part of the shipped path.
+ *
+ * Build: gcc -O2 -std=c11 -ffp-contract=off -fno-fast-math -fPIC -shared
+ */
+#include "ref_cpu.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+static inline int is_legal(const ref_tree *t, int32_t id) {
+    return t->legal == NULL || ((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u);
+}
+
+/* mcts_node.cpp:657-678 -- blend of the Monte-Carlo mean and the RAVE mean.
+ * Virtual loss is not part of it. */
+float ref_combined_value(const ref_tree *t, int32_t node, float rave_k) {
+    int visits = t->N[node];
+    int rave_visits = t->rN ? t->rN[node] : 0;
+    if (visits == 0 && rave_visits == 0) {
+        return 0.0f;
+    }
+    float mcts_value = visits > 0 ? t->W[node] / (float)visits : 0.0f;
+    float rave_value = rave_visits > 0 ? (t->rW ? t->rW[node] : 0.0f) / (float)rave_visits : 0.0f;
+    /* "3 * visits + rave_constant": the product is an int, the sum a float */
+    int three_v = (int)(3u * (uint32_t)visits);
+    float beta = sqrtf(rave_k / ((float)three_v + rave_k));
+    float a = (1.0f - beta) * mcts_value;
+    float b = beta * rave_value;
+    return a + b;
+}
+
+/* mcts_node.cpp:143-160 (first loop) and :196-214 (second loop). */
+void ref_child_scores(const ref_tree *t, int32_t parent, int32_t child, const ref_params *p,
+                      float *score_first, float *score_second) {
+    /* mcts_node.cpp:94-95: the parent's raw visit count, no virtual loss */
+    float exploration_param = p->c_puct * sqrtf((float)t->N[parent]);
+
+    int child_visits = t->N[child];
+    float child_value = t->W[child];
+    int virtual_losses = t->VL[child];
+    int effective_visits = (int)((uint32_t)child_visits + (uint32_t)virtual_losses);
+    float effective_value = child_value - (float)virtual_losses;
+
+    float exploitation = effective_visits > 0 ? effective_value / (float)effective_visits : 0.0f;
+    /* first loop divides by the float sum 1.0f + ev */
+    float prod = t->P[child] * exploration_param;
+    float exploration = prod / (1.0f + (float)effective_visits);
+    *score_first = exploitation + exploration;
+
+    /* second loop divides by the int sum 1 + ev, and swaps in the RAVE blend */
+    float exploitation2 = p->use_rave ? ref_combined_value(t, child, p->rave_k) : exploitation;
+    int one_plus = (int)(1u + (uint32_t)effective_visits);
+    float exploration2 = prod / (float)one_plus;
+    *score_second = exploitation2 + exploration2;
+}
+
+/* smallest k >= 1 with k*k >= n */
+int32_t ref_ceil_sqrt(int32_t n) {
+    if (n <= 1) return 1;
+    int64_t k = (int64_t)sqrt((double)n);
+    while (k * k < (int64_t)n) k++;
+    while ((k - 1) * (k - 1) >= (int64_t)n) k--;
+    return (int32_t)k;
+}
+
+/* Progressive-widening eligibility: child takes part iff fewer than k legal siblings
+ * beat it by (prior descending, index ascending). */
+static void pw_eligible(const ref_tree *t, int32_t cb, int32_t cc, int32_t k, uint8_t *elig) {
+    int sorted = 1;
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_legal(t, cb + i)) { sorted = 0; break; }
+        if (i > 0 && !(t->P[cb + i - 1] >= t->P[cb + i])) { sorted = 0; break; }
+    }
+    if (sorted) { /* prior-descending storage: the first k children */
+        for (int32_t i = 0; i < cc; i++) elig[i] = (uint8_t)(i < k);
+        return;
+    }
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_legal(t, cb + i)) { elig[i] = 0; continue; }
+        int32_t rank = 0;
+        float pi = t->P[cb + i];
+        for (int32_t j = 0; j < cc; j++) {
+            if (j == i || !is_legal(t, cb + j)) continue;
+            float pj = t->P[cb + j];
+            if (pj > pi || (pj == pi && j < i)) rank++;
+        }
+        elig[i] = (uint8_t)(rank < k);
+    }
+}
+
+/* mcts_node.cpp:90-236.  The pending-evaluation flags of the reference node are always
+ * clear on this path (they are set by evaluator plumbing that is not part of it), so
+ * every skip on them is a no-op.  Returns the chosen child's node id, or -1. */
+int32_t ref_select_child(const ref_tree *t, int32_t node, const ref_params *p, ref_select_info *info) {
+    const int32_t cb = t->child_begin[node];
+    const int32_t cc = t->child_count[node];
+    float best_score = -INFINITY;
+    int32_t best = -1;
+    int32_t ncand = 0;
+
+    uint8_t stack_elig[512];
+    uint8_t *elig = NULL;
+    if (p->pw && cc > 0) {
+        elig = cc <= 512 ? stack_elig : (uint8_t *)malloc((size_t)cc);
+        pw_eligible(t, cb, cc, ref_ceil_sqrt(t->N[node]), elig);
+    }
+#define TAKES_PART(i) (is_legal(t, cb + (i)) && (!elig || elig[i]))
+
+    /* first loop: plain PUCT, keep the first strict maximum */
+    for (int32_t i = 0; i < cc; i++) {
+        if (!TAKES_PART(i)) continue;
+        float s1, s2;
+        ref_child_scores(t, node, cb + i, p, &s1, &s2);
+        if (s1 > best_score) { best_score = s1; best = i; }
+        ncand++;
+    }
+    if (best < 0 && ncand > 0) {
+        /* mcts_node.cpp:173-181: no score beat -inf (all NaN or -inf): least visited, first minimum */
+        int min_visits = INT32_MAX;
+        for (int32_t i = 0; i < cc; i++) {
+            if (!TAKES_PART(i)) continue;
+            if (t->N[cb + i] < min_visits) { min_visits = t->N[cb + i]; best = i; }
+        }
+    } else if (best >= 0) {
+        /* mcts_node.cpp:184-220: second scan over the same children, best_score carried over */
+        for (int32_t i = 0; i < cc; i++) {
+            if (!TAKES_PART(i)) continue;
+            float s1, s2;
+            ref_child_scores(t, node, cb + i, p, &s1, &s2);
+            if (s2 > best_score) { best_score = s2; best = i; }
+        }
+    }
+
+    if (info) {
+        /* best candidate of any other child, over both scans */
+        float second = -INFINITY;
+        for (int32_t i = 0; i < cc; i++) {
+            if (i == best || !TAKES_PART(i)) continue;
+            float s1, s2;
+            ref_child_scores(t, node, cb + i, p, &s1, &s2);
+            if (s1 > second) second = s1;
+            if (s2 > second) second = s2;
+        }
+        info->best = best_score;
+        info->second = second;
+        info->n_candidates = ncand;
+        float m = fmaxf(fabsf(best_score), fabsf(second));
+        info->near_tie = (best >= 0 && ncand > 1 && isfinite(second) && isfinite(best_score) &&
+                          fabsf(best_score - second) <= 1e-6f * m) ? 1 : 0;
+    }
+#undef TAKES_PART
+    if (elig && elig != stack_elig) free(elig);
+    return best < 0 ? -1 : cb + best;
+}
+
+/* mcts_node_virtual_loss.cpp:15-20 */
+void ref_add_vl(ref_tree *t, int32_t node, int32_t amount) {
+    if (amount > 0) {
+        t->VL[node] = (int32_t)((uint32_t)t->VL[node] + (uint32_t)amount);
+    }
+}
+
+/* mcts_node_virtual_loss.cpp:22-30 */
+void ref_remove_vl1(ref_tree *t, int32_t node) {
+    int current = t->VL[node];
+    t->VL[node] = (int32_t)((uint32_t)current - 1u);
+    if (current <= 0) {
+        t->VL[node] = 0;
+    }
+}
+
+/* mcts_node_virtual_loss.cpp:32-42 */
+void ref_remove_vl(ref_tree *t, int32_t node, int32_t amount) {
+    if (amount <= 0) return;
+    int current = t->VL[node];
+    t->VL[node] = (int32_t)((uint32_t)current - (uint32_t)amount);
+    if (current < amount) {
+        t->VL[node] = 0;
+    }
+}
+
+/* mcts_node_virtual_loss.cpp:54-71 -- note the trailing removal of one virtual loss */
+void ref_update(ref_tree *t, int32_t node, float value) {
+    t->N[node] = (int32_t)((uint32_t)t->N[node] + 1u);
+    t->W[node] = t->W[node] + value;
+    if (t->VL[node] > 0) {
+        ref_remove_vl1(t, node);
+    }
+}
+
+/* mcts_engine_batch_tree_simple.cpp:73-185 run by one thread, traversals in index order:
+ * descend while the node is expanded, select, add virtual loss to the selected child
+ * (never to the root), record it. */
+int ref_select_batch(ref_tree *t, const int32_t *roots, int32_t B, const ref_params *p,
+                     int32_t *paths, int32_t *path_len, int32_t *leaf, int32_t *near_tie_depth) {
+    const int32_t stride = p->max_depth + 1;
+    for (int32_t i = 0; i < B; i++) {
+        int32_t *path = paths + (int64_t)i * stride;
+        for (int32_t d = 0; d < stride; d++) path[d] = -1;
+        int32_t current = roots[i];
+        if (current < 0 || current >= t->n_nodes) return -1;
+        int32_t len = 0;
+        path[len++] = current;
+        if (near_tie_depth) near_tie_depth[i] = -1;
+        while (t->child_count[current] > 0 && len <= p->max_depth) {
+            ref_select_info info;
+            int32_t best = ref_select_child(t, current, p, near_tie_depth ? &info : NULL);
+            if (best < 0) break;
+            if (near_tie_depth && info.near_tie && near_tie_depth[i] < 0) near_tie_depth[i] = len - 1;
+            ref_add_vl(t, best, p->virtual_loss);
+            current = best;
+            path[len++] = current;
+        }
+        path_len[i] = len;
+        leaf[i] = current;
+    }
+    return 0;
+}
+
+void ref_apply_vl_paths(ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B,
+                        int32_t stride, int32_t amount) {
+    for (int32_t i = 0; i < B; i++)
+        for (int32_t d = 1; d < path_len[i]; d++) ref_add_vl(t, paths[(int64_t)i * stride + d], amount);
+}
+
+void ref_revert_vl_paths(ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B,
+                         int32_t stride, int32_t amount) {
+    for (int32_t i = 0; i < B; i++)
+        for (int32_t d = path_len[i] - 1; d >= 0; d--) ref_remove_vl(t, paths[(int64_t)i * stride + d], amount);
+}
+
+/* mcts_engine_batch_tree_simple.cpp:276-281, results in index order: leaf to root,
+ * update, revert, flip the sign for the opponent. */
+void ref_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *path_len,
+                      const float *values, int32_t B, int32_t stride, int32_t amount) {
+    for (int32_t i = 0; i < B; i++) {
+        float value = values[i];
+        for (int32_t d = path_len[i] - 1; d >= 0; d--) {
+            int32_t node = paths[(int64_t)i * stride + d];
+            ref_update(t, node, value);
+            ref_remove_vl(t, node, amount);
+            value = -value;
+        }
+    }
+}
+
+/* mcts_engine_batch_tree_simple.cpp:114,174-178: the recorded move of every selected child */
+void ref_gather_actions(const ref_tree *t, const int32_t *paths, const int32_t *path_len,
+                        int32_t B, int32_t stride, int32_t *actions) {
+    const int32_t astride = stride - 1;
+    for (int32_t i = 0; i < B; i++) {
+        for (int32_t d = 0; d < astride; d++) {
+            int32_t v = -1;
+            if (d + 1 < path_len[i]) {
+                int32_t node = paths[(int64_t)i * stride + d + 1];
+                v = t->action ? t->action[node] : node;
+            }
+            actions[(int64_t)i * astride + d] = v;
+        }
+    }
+}
+
+/* ---- open-addressing transposition table ---- */
+
+#define REF_TT_EMPTY (~(uint64_t)0)
+
+static inline uint64_t tt_home(uint64_t key, int32_t log2_slots) {
+    return (key * 0x9E3779B97F4A7C15ull) >> (64 - log2_slots);
+}
+
+void ref_tt_clear(ref_tt_slot *slots, int32_t log2_slots) {
+    uint64_t n = (uint64_t)1 << log2_slots;
+    for (uint64_t i = 0; i < n; i++) {
+        slots[i].key = REF_TT_EMPTY;
+        slots[i].node = -1;
+        slots[i].depth = 0;
+    }
+}
+
+int ref_tt_insert(ref_tt_slot *slots, int32_t log2_slots, uint64_t key, int32_t node, int32_t depth) {
+    if (key == REF_TT_EMPTY) return -2;
+    uint64_t mask = ((uint64_t)1 << log2_slots) - 1;
+    uint64_t s = tt_home(key, log2_slots);
+    for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+        if (slots[s].key == key) return 1;
+        if (slots[s].key == REF_TT_EMPTY) {
+            slots[s].key = key;
+            slots[s].node = node;
+            slots[s].depth = depth;
+            return 0;
+        }
+    }
+    return -1;
+}
+
+int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_t *keys, int64_t n,
+                     int32_t min_depth, int32_t *out_node) {
+    uint64_t mask = ((uint64_t)1 << log2_slots) - 1;
+    int64_t hits = 0;
+    for (int64_t i = 0; i < n; i++) {
+        uint64_t key = keys[i];
+        int32_t found = -1;
+        if (key != REF_TT_EMPTY) {
+            uint64_t s = tt_home(key, log2_slots);
+            for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+                if (slots[s].key == key) {
+                    if (slots[s].depth >= min_depth) found = slots[s].node;
+                    break;
+                }
+                if (slots[s].key == REF_TT_EMPTY) break;
+            }
+        }
+        out_node[i] = found;
+        if (found >= 0) hits++;
+    }
+    return hits;
+}

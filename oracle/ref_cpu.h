@@ -1,0 +1,124 @@
+/*
+ * ref_cpu -- CPU restatement of the reference's tree-search arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is the checker the HIP path is compared
+ * against and the timed CPU baseline.  Nothing in the shipped library may
+ * call, link or load it; only tests, the smoke check and the benchmark's
+ * cpu_baseline leg do.
+ *
+ * Every function restates one piece of the reference (paths relative to the
+ * reference checkout):
+ *   ref_select_child      src/mcts/mcts_node.cpp:90-236   (MCTSNode::selectChild)
+ *   ref_combined_value    src/mcts/mcts_node.cpp:657-678  (MCTSNode::getCombinedValue)
+ *   ref_add_vl            src/mcts/mcts_node_virtual_loss.cpp:15-20
+ *   ref_remove_vl1        src/mcts/mcts_node_virtual_loss.cpp:22-30
+ *   ref_remove_vl         src/mcts/mcts_node_virtual_loss.cpp:32-42
+ *   ref_update            src/mcts/mcts_node_virtual_loss.cpp:54-71
+ *   ref_select_batch      src/mcts/mcts_engine_batch_tree_simple.cpp:73-185 (one thread, i ascending)
+ *   ref_backup_batch      src/mcts/mcts_engine_batch_tree_simple.cpp:242-282 (i ascending)
+ *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
+ *                         src/mcts/phmap_transposition_table.cpp:51-117
+ *
+ * The node record of include/mcts/mcts_node.h:160-178 is flattened into
+ * arrays indexed by node id; the children of a node are the contiguous id
+ * range [child_begin, child_begin + child_count).
+ *
+ * Pinned by: the reference's own unit-test facts (tests/mcts/mcts_node_test.cpp:237-313,
+ * tests/mcts/virtual_loss_test.cpp:42-69,160-224,282-308), the recorded known-answer
+ * table of the compiled reference node class (tests/golden/kat_reference.json), closed
+ * forms and a double-precision brute force (tests/test_oracle_*.py).
+ *
+ * PARITY UNPINNED (no reference behaviour exists to pin them; defined here):
+ *   - the progressive-widening eligibility filter (pw != 0): top ceil(sqrt(N_parent))
+ *     children by prior, ties to the lower child index;
+ *   - the open-addressing transposition table (the reference delegates to the
+ *     absent third-party parallel-hashmap v1.3.8); checked against a brute-force map.
+ *
+ * Must be compiled with -ffp-contract=off and without -ffast-math: the reference
+ * translation unit is built for baseline x86-64 (no FMA), IEEE binary32, round to nearest.
+ */
+#ifndef OMK_ORACLE_REF_CPU_H
+#define OMK_ORACLE_REF_CPU_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ref_tree {
+    int64_t n_nodes;
+    int32_t *N;                 /* visit_count_            */
+    float *W;                   /* value_sum_              */
+    float *P;                   /* prior_probability_      */
+    int32_t *VL;                /* virtual_loss_count_     */
+    int32_t *rN;                /* rave_count_     (NULL = all zero) */
+    float *rW;                  /* rave_value_sum_ (NULL = all zero) */
+    const int32_t *child_begin; /* first child id          */
+    const int32_t *child_count; /* 0 = not expanded (isLeaf) */
+    const int32_t *action;      /* action_ (may be NULL)   */
+    const uint32_t *legal;      /* bit per node id, 1 = the slot holds a child; NULL = all */
+} ref_tree;
+
+typedef struct ref_params {
+    float c_puct;         /* MCTSSettings::exploration_constant */
+    int32_t virtual_loss; /* MCTSSettings::virtual_loss         */
+    int32_t use_rave;     /* MCTSSettings::use_rave             */
+    float rave_k;         /* MCTSSettings::rave_constant        */
+    int32_t pw;           /* selection-time progressive widening (0 = off) */
+    int32_t max_depth;    /* bound on selection steps per traversal (buffer size; the reference has none) */
+} ref_params;
+
+/* Scores of the winning candidate and of the best candidate belonging to a different child. */
+typedef struct ref_select_info {
+    float best;
+    float second;
+    int32_t n_candidates; /* children that took part */
+    int32_t near_tie;     /* |best-second| <= 1e-6 * max(|best|,|second|) */
+} ref_select_info;
+
+float ref_combined_value(const ref_tree *t, int32_t node, float rave_k);
+/* The two per-child scores of selectChild: first loop and second loop. */
+void ref_child_scores(const ref_tree *t, int32_t parent, int32_t child, const ref_params *p,
+                      float *score_first, float *score_second);
+int32_t ref_ceil_sqrt(int32_t n);
+int32_t ref_select_child(const ref_tree *t, int32_t node, const ref_params *p, ref_select_info *info);
+
+void ref_add_vl(ref_tree *t, int32_t node, int32_t amount);
+void ref_remove_vl1(ref_tree *t, int32_t node);
+void ref_remove_vl(ref_tree *t, int32_t node, int32_t amount);
+void ref_update(ref_tree *t, int32_t node, float value);
+
+/* paths: [B][max_depth+1] node ids (row per traversal), unused entries -1.
+ * near_tie_depth (may be NULL): first selection step of the traversal with a near tie, else -1. */
+int ref_select_batch(ref_tree *t, const int32_t *roots, int32_t B, const ref_params *p,
+                     int32_t *paths, int32_t *path_len, int32_t *leaf, int32_t *near_tie_depth);
+void ref_apply_vl_paths(ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B,
+                        int32_t stride, int32_t amount);
+void ref_revert_vl_paths(ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B,
+                         int32_t stride, int32_t amount);
+void ref_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *path_len,
+                      const float *values, int32_t B, int32_t stride, int32_t amount);
+/* Leaf gather: the move list replayed on the root state, actions[B][max_depth], unused -1. */
+void ref_gather_actions(const ref_tree *t, const int32_t *paths, const int32_t *path_len,
+                        int32_t B, int32_t stride, int32_t *actions);
+
+/* Open-addressing table: 2^log2_slots slots of 16 bytes, linear probing,
+ * home slot = (key * 0x9E3779B97F4A7C15) >> (64 - log2_slots), empty key = ~0. */
+typedef struct ref_tt_slot {
+    uint64_t key;
+    int32_t node;
+    int32_t depth;
+} ref_tt_slot;
+
+void ref_tt_clear(ref_tt_slot *slots, int32_t log2_slots);
+/* 0 stored, 1 key already present (first entry kept), -1 table full, -2 reserved key */
+int ref_tt_insert(ref_tt_slot *slots, int32_t log2_slots, uint64_t key, int32_t node, int32_t depth);
+/* out_node[i] = node stored under keys[i] with depth >= min_depth, else -1; returns hits */
+int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_t *keys, int64_t n,
+                     int32_t min_depth, int32_t *out_node);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

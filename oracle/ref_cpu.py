@@ -1,0 +1,207 @@
+"""ctypes binding of the CPU checker (libref_cpu.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests, by the smoke check and by the
+benchmark's cpu_baseline leg, never by the shipped package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+i32p = C.POINTER(C.c_int32)
+f32p = C.POINTER(C.c_float)
+u32p = C.POINTER(C.c_uint32)
+u64p = C.POINTER(C.c_uint64)
+
+
+class _Tree(C.Structure):
+    _fields_ = [("n_nodes", C.c_int64), ("N", i32p), ("W", f32p), ("P", f32p), ("VL", i32p),
+                ("rN", i32p), ("rW", f32p), ("child_begin", i32p), ("child_count", i32p),
+                ("action", i32p), ("legal", u32p)]
+
+
+class _Params(C.Structure):
+    _fields_ = [("c_puct", C.c_float), ("virtual_loss", C.c_int32), ("use_rave", C.c_int32),
+                ("rave_k", C.c_float), ("pw", C.c_int32), ("max_depth", C.c_int32)]
+
+
+class _Info(C.Structure):
+    _fields_ = [("best", C.c_float), ("second", C.c_float), ("n_candidates", C.c_int32),
+                ("near_tie", C.c_int32)]
+
+
+TT_SLOT = np.dtype([("key", "<u8"), ("node", "<i4"), ("depth", "<i4")])
+
+
+def build(force=False):
+    so = os.path.join(_HERE, "libref_cpu.so")
+    if force or not os.path.exists(so):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "libref_cpu.so"])
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        L = C.CDLL(build())
+        L.ref_combined_value.restype = C.c_float
+        L.ref_combined_value.argtypes = [C.POINTER(_Tree), C.c_int32, C.c_float]
+        L.ref_child_scores.argtypes = [C.POINTER(_Tree), C.c_int32, C.c_int32, C.POINTER(_Params), f32p, f32p]
+        L.ref_ceil_sqrt.restype = C.c_int32
+        L.ref_ceil_sqrt.argtypes = [C.c_int32]
+        L.ref_select_child.restype = C.c_int32
+        L.ref_select_child.argtypes = [C.POINTER(_Tree), C.c_int32, C.POINTER(_Params), C.POINTER(_Info)]
+        for name in ("ref_add_vl", "ref_remove_vl"):
+            getattr(L, name).argtypes = [C.POINTER(_Tree), C.c_int32, C.c_int32]
+            getattr(L, name).restype = None
+        L.ref_remove_vl1.argtypes = [C.POINTER(_Tree), C.c_int32]
+        L.ref_remove_vl1.restype = None
+        L.ref_update.argtypes = [C.POINTER(_Tree), C.c_int32, C.c_float]
+        L.ref_update.restype = None
+        L.ref_select_batch.restype = C.c_int
+        L.ref_select_batch.argtypes = [C.POINTER(_Tree), i32p, C.c_int32, C.POINTER(_Params), i32p, i32p, i32p, i32p]
+        for name in ("ref_apply_vl_paths", "ref_revert_vl_paths"):
+            getattr(L, name).argtypes = [C.POINTER(_Tree), i32p, i32p, C.c_int32, C.c_int32, C.c_int32]
+            getattr(L, name).restype = None
+        L.ref_backup_batch.argtypes = [C.POINTER(_Tree), i32p, i32p, f32p, C.c_int32, C.c_int32, C.c_int32]
+        L.ref_backup_batch.restype = None
+        L.ref_gather_actions.argtypes = [C.POINTER(_Tree), i32p, i32p, C.c_int32, C.c_int32, i32p]
+        L.ref_gather_actions.restype = None
+        L.ref_tt_clear.argtypes = [C.c_void_p, C.c_int32]
+        L.ref_tt_clear.restype = None
+        L.ref_tt_insert.argtypes = [C.c_void_p, C.c_int32, C.c_uint64, C.c_int32, C.c_int32]
+        L.ref_tt_insert.restype = C.c_int
+        L.ref_tt_probe.argtypes = [C.c_void_p, C.c_int32, u64p, C.c_int64, C.c_int32, i32p]
+        L.ref_tt_probe.restype = C.c_int64
+        _LIB = L
+    return _LIB
+
+
+def _ptr(a, ty):
+    return a.ctypes.data_as(ty) if a is not None else ty()
+
+
+def make_params(c_puct=1.4, virtual_loss=3, use_rave=False, rave_k=3000.0, pw=False, max_depth=32):
+    return _Params(c_puct, int(virtual_loss), int(bool(use_rave)), rave_k, int(bool(pw)), int(max_depth))
+
+
+class RefTree:
+    """Owns private copies of the per-node arrays and runs the checker on them."""
+
+    def __init__(self, N, W, P, VL, child_begin, child_count, action=None, rN=None, rW=None, legal=None):
+        n = len(N)
+        self.n = n
+        self.N = np.ascontiguousarray(N, dtype=np.int32).copy()
+        self.W = np.ascontiguousarray(W, dtype=np.float32).copy()
+        self.P = np.ascontiguousarray(P, dtype=np.float32).copy()
+        self.VL = np.ascontiguousarray(VL, dtype=np.int32).copy()
+        self.child_begin = np.ascontiguousarray(child_begin, dtype=np.int32).copy()
+        self.child_count = np.ascontiguousarray(child_count, dtype=np.int32).copy()
+        self.action = None if action is None else np.ascontiguousarray(action, dtype=np.int32).copy()
+        self.rN = None if rN is None else np.ascontiguousarray(rN, dtype=np.int32).copy()
+        self.rW = None if rW is None else np.ascontiguousarray(rW, dtype=np.float32).copy()
+        self.legal = None if legal is None else np.ascontiguousarray(legal, dtype=np.uint32).copy()
+        for a in (self.W, self.P, self.VL, self.child_begin, self.child_count):
+            assert len(a) == n
+        if self.legal is not None:
+            assert len(self.legal) * 32 >= n
+        self._c = _Tree(n, _ptr(self.N, i32p), _ptr(self.W, f32p), _ptr(self.P, f32p), _ptr(self.VL, i32p),
+                        _ptr(self.rN, i32p), _ptr(self.rW, f32p), _ptr(self.child_begin, i32p),
+                        _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p))
+
+    @classmethod
+    def from_soa(cls, soa):
+        """soa: mapping with the keys of omoknuni_small_amd.synth (N, W, P, VL, child_begin, ...)."""
+        return cls(soa["N"], soa["W"], soa["P"], soa["VL"], soa["child_begin"], soa["child_count"],
+                   action=soa.get("action"), rN=soa.get("rN"), rW=soa.get("rW"), legal=soa.get("legal"))
+
+    # -- single-node operations -------------------------------------------------
+    def select_child(self, node, params, with_info=False):
+        info = _Info()
+        r = lib().ref_select_child(C.byref(self._c), int(node), C.byref(params), C.byref(info))
+        if with_info:
+            return r, dict(best=info.best, second=info.second, n_candidates=info.n_candidates,
+                           near_tie=bool(info.near_tie))
+        return r
+
+    def child_scores(self, parent, child, params):
+        a, b = C.c_float(), C.c_float()
+        lib().ref_child_scores(C.byref(self._c), int(parent), int(child), C.byref(params), C.byref(a), C.byref(b))
+        return np.float32(a.value), np.float32(b.value)
+
+    def combined_value(self, node, rave_k):
+        return np.float32(lib().ref_combined_value(C.byref(self._c), int(node), rave_k))
+
+    def add_vl(self, node, amount):
+        lib().ref_add_vl(C.byref(self._c), int(node), int(amount))
+
+    def remove_vl(self, node, amount=None):
+        if amount is None:
+            lib().ref_remove_vl1(C.byref(self._c), int(node))
+        else:
+            lib().ref_remove_vl(C.byref(self._c), int(node), int(amount))
+
+    def update(self, node, value):
+        lib().ref_update(C.byref(self._c), int(node), float(value))
+
+    # -- batched operations -----------------------------------------------------
+    def select_batch(self, roots, params, near_ties=True):
+        roots = np.ascontiguousarray(roots, dtype=np.int32)
+        B = len(roots)
+        stride = params.max_depth + 1
+        paths = np.empty((B, stride), dtype=np.int32)
+        path_len = np.empty(B, dtype=np.int32)
+        leaf = np.empty(B, dtype=np.int32)
+        nt = np.empty(B, dtype=np.int32) if near_ties else None
+        rc = lib().ref_select_batch(C.byref(self._c), _ptr(roots, i32p), B, C.byref(params), _ptr(paths, i32p),
+                                    _ptr(path_len, i32p), _ptr(leaf, i32p), _ptr(nt, i32p))
+        if rc != 0:
+            raise ValueError("ref_select_batch: bad root")
+        return paths, path_len, leaf, nt
+
+    def _paths_args(self, paths, path_len):
+        paths = np.ascontiguousarray(paths, dtype=np.int32)
+        path_len = np.ascontiguousarray(path_len, dtype=np.int32)
+        return paths, path_len, paths.shape[0], paths.shape[1]
+
+    def apply_vl_paths(self, paths, path_len, amount):
+        paths, path_len, B, stride = self._paths_args(paths, path_len)
+        lib().ref_apply_vl_paths(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), B, stride, int(amount))
+
+    def revert_vl_paths(self, paths, path_len, amount):
+        paths, path_len, B, stride = self._paths_args(paths, path_len)
+        lib().ref_revert_vl_paths(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), B, stride, int(amount))
+
+    def backup_batch(self, paths, path_len, values, amount):
+        paths, path_len, B, stride = self._paths_args(paths, path_len)
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        assert len(values) == B
+        lib().ref_backup_batch(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), _ptr(values, f32p),
+                               B, stride, int(amount))
+
+    def gather_actions(self, paths, path_len):
+        paths, path_len, B, stride = self._paths_args(paths, path_len)
+        out = np.empty((B, stride - 1), dtype=np.int32)
+        lib().ref_gather_actions(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), B, stride, _ptr(out, i32p))
+        return out
+
+
+class RefTT:
+    def __init__(self, log2_slots):
+        self.log2 = int(log2_slots)
+        self.slots = np.empty(1 << self.log2, dtype=TT_SLOT)
+        lib().ref_tt_clear(self.slots.ctypes.data, self.log2)
+
+    def insert(self, key, node, depth=0):
+        return lib().ref_tt_insert(self.slots.ctypes.data, self.log2, int(key), int(node), int(depth))
+
+    def probe(self, keys, min_depth=0):
+        keys = np.ascontiguousarray(keys, dtype=np.uint64)
+        out = np.empty(len(keys), dtype=np.int32)
+        hits = lib().ref_tt_probe(self.slots.ctypes.data, self.log2, _ptr(keys, u64p), len(keys), int(min_depth),
+                                  _ptr(out, i32p))
+        return out, int(hits)
