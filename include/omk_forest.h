@@ -101,6 +101,8 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out);
 int omk_forest_destroy(omk_forest *f);
 /* Use the caller's hipStream_t (NULL restores the forest's own stream). */
 int omk_forest_set_stream(omk_forest *f, void *hip_stream);
+/* The hipStream_t the forest's work is enqueued on (to record events on it). */
+int omk_forest_get_stream(omk_forest *f, void **hip_stream_out);
 /* Checks that the arrays describe a forest (ranges in bounds, every node the child of at
  * most one parent, fan-out <= OMK_MAX_FANOUT) and copies them to the device. */
 int omk_forest_upload(omk_forest *f, const omk_soa_view *h_view);

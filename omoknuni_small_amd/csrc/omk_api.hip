@@ -158,6 +158,12 @@ int omk_forest_set_stream(omk_forest *f, void *hip_stream) {
     return OMK_OK;
 }
 
+int omk_forest_get_stream(omk_forest *f, void **hip_stream_out) {
+    if (!f || !hip_stream_out) return fail(OMK_ERR_INVALID, "omk_forest_get_stream: null argument");
+    *hip_stream_out = (void *)f->stream;
+    return OMK_OK;
+}
+
 int omk_sync(omk_forest *f) {
     if (!f) return fail(OMK_ERR_INVALID, "omk_sync: null forest");
     if (int rc = use_device(f)) return rc;

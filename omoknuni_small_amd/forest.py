@@ -21,7 +21,7 @@ u32p = C.POINTER(C.c_uint32)
 u64p = C.POINTER(C.c_uint64)
 
 EXPORTS = [
-    "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream",
+    "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
@@ -129,6 +129,11 @@ class Forest:
 
     def set_stream(self, hip_stream):
         _check(self._lib.omk_forest_set_stream(self._h, C.c_void_p(hip_stream or 0)))
+
+    def get_stream(self):
+        s = C.c_void_p()
+        _check(self._lib.omk_forest_get_stream(self._h, C.byref(s)))
+        return s.value or 0
 
     def sync(self):
         _check(self._lib.omk_sync(self._h))
