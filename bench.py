@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the tree-search hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of concurrent traversals of a seeded
+synthetic forest: batched PUCT selection with virtual loss down to the leaves, then the
+backup of one value per leaf (update + revert virtual loss, sign flipped per ply), plus
+the leaf-key table probes on the workload that has them.  Everything a step touches is
+resident in HBM before the timed region starts; nothing returns to the host inside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0..c4]
+
+Prints ONE JSON line.  `value` is traversals per second over whole steps (every
+traversal is selected AND backed up inside the timed region).  `roofline` prices the
+selection kernel against HBM bandwidth with algorithmic bytes (what one selection step
+has to read: the statistics of the children that take part, the node header, the legal
+mask bits, the virtual-loss update), measured with HIP events on the stream the kernels
+run on.  `cpu_baseline` times the CPU checker (a restatement of the reference's serial
+selection / backup loops) on the host cores of the same machine, on a bounded number of
+steps of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+class HipEvents:
+    """hipEvent timing on a given stream through the HIP runtime the library itself uses."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+
+    def _ok(self, rc, what):
+        if rc != 0:
+            raise RuntimeError("%s failed with hipError %d" % (what, rc))
+
+    def create(self):
+        ev = C.c_void_p()
+        self._ok(self.hip.hipEventCreate(C.byref(ev)), "hipEventCreate")
+        return ev
+
+    def record(self, ev, stream):
+        self._ok(self.hip.hipEventRecord(ev, C.c_void_p(stream)), "hipEventRecord")
+
+    def elapsed_ms(self, a, b):
+        self._ok(self.hip.hipEventSynchronize(b), "hipEventSynchronize")
+        ms = C.c_float()
+        self._ok(self.hip.hipEventElapsedTime(C.byref(ms), a, b), "hipEventElapsedTime")
+        return float(ms.value)
+
+    def device_sync(self):
+        self._ok(self.hip.hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+
+def legal_children_per_node(soa):
+    """Number of children of every node that a selection at it has to read."""
+    cb, cc = soa["child_begin"].astype(np.int64), soa["child_count"].astype(np.int64)
+    n = len(cc)
+    if soa.get("legal") is None:
+        return cc.copy()
+    bits = np.unpackbits(soa["legal"].view(np.uint8), bitorder="little")[:n].astype(np.int64)
+    cs = np.concatenate([[0], np.cumsum(bits)])
+    return cs[np.minimum(cb + cc, n)] - cs[np.minimum(cb, n)]
+
+
+def algorithmic_bytes(soa, meta, paths, plen, N_now):
+    """Bytes one step has to move, by the per-unit model:
+    selection step at a node with L participating children of F slots:
+        L*16 (N, W, P, VL)  [+ L*8 RAVE]  + ceil(F/8) mask bytes (dense slots only)
+        + 16 (child range, N_parent, flags) + 8 (virtual-loss update of the chosen child)
+    backup of a path node: 24 (N, W, VL read-modify-write), + 4 per leaf value + 4 per path entry."""
+    L = legal_children_per_node(soa)
+    cc = soa["child_count"].astype(np.int64)
+    per_child = 24 if meta.get("has_rave") else 16
+    n_t, row = paths.shape
+    d_idx = np.arange(row)[None, :]
+    sel_mask = d_idx < (plen[:, None] - 1)  # a selection happens at every path node but the leaf
+    nodes = paths[sel_mask]
+    Lsel = L[nodes]
+    if meta.get("pw"):
+        k = np.ceil(np.sqrt(np.maximum(N_now[nodes].astype(np.float64), 1.0))).astype(np.int64)
+        Lsel = np.minimum(Lsel, np.maximum(k, 1))
+    mask_bytes = (cc[nodes] + 7) // 8 if soa.get("legal") is not None else 0
+    sel = int((Lsel * per_child + mask_bytes + 24).sum()) + int(4 * plen.sum())
+    bak = int(24 * plen.sum() + 4 * n_t + 4 * plen.sum())
+    return sel, bak, int(sel_mask.sum())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=["c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--seed", type=int, default=2025)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--scale", type=float, default=1.0, help="scale nodes_per_tree (debugging only)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (independent trees would shard by tree id with no "
+              "exchange); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import omoknuni_small_amd as omk
+    from omoknuni_small_amd import synth
+
+    kw = {}
+    if args.scale != 1.0:
+        kw["nodes_per_tree"] = max(1000, int(synth.CONFIGS[args.workload]["nodes_per_tree"] * args.scale))
+    t0 = time.time()
+    soa, roots, meta = synth.generate(args.workload, seed=args.seed, **kw)
+    gen_s = time.time() - t0
+    B = int(meta["n_traversals"])
+    D = int(meta["max_depth"])
+    vl = int(meta["virtual_loss"])
+    troots = synth.traversal_roots(roots, B)
+    values = np.random.default_rng(args.seed + 1).uniform(-1, 1, B).astype(np.float32)
+    params = omk.SelectParams(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                              rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")))
+
+    forest = omk.Forest.from_soa(soa)
+    batch = omk.Batch(forest, B, D)
+    batch.set_roots(troots)
+    batch.set_values(values)
+    tt = None
+    d_probe = 0
+    if meta.get("tt_log2"):
+        tt = omk.TranspositionTable(forest, int(meta["tt_log2"]))
+        n_ins = 1 << (int(meta["tt_log2"]) - 1)  # 50 % load
+        ids = np.linspace(0, meta["n_nodes"] - 1, n_ins).astype(np.int64)
+        ids = np.unique(ids)
+        tt.insert(soa["hash"][ids], ids.astype(np.int32))
+        d_probe = forest.dev_alloc(B * 4)
+
+    def step():
+        batch.select(params)
+        if tt is not None:
+            tt.probe_leaves_dev(batch, d_probe)
+        batch.backup(vl)
+
+    ev = HipEvents()
+    stream = forest.get_stream()
+    for _ in range(args.warmup):
+        step()
+    forest.sync()
+    ev.device_sync()
+
+    K = args.steps
+    e_sel0 = [ev.create() for _ in range(K)]
+    e_sel1 = [ev.create() for _ in range(K)]
+    e_end = [ev.create() for _ in range(K)]
+    t_wall0 = time.perf_counter()
+    for i in range(K):
+        ev.record(e_sel0[i], stream)
+        batch.select(params)
+        ev.record(e_sel1[i], stream)
+        if tt is not None:
+            tt.probe_leaves_dev(batch, d_probe)
+        batch.backup(vl)
+        ev.record(e_end[i], stream)
+    forest.sync()
+    ev.device_sync()
+    wall_s = time.perf_counter() - t_wall0
+    total_ms = ev.elapsed_ms(e_sel0[0], e_end[K - 1])
+    sel_ms = sum(ev.elapsed_ms(e_sel0[i], e_sel1[i]) for i in range(K))
+    bak_ms = sum(ev.elapsed_ms(e_sel1[i], e_end[i]) for i in range(K))
+
+    # the byte model is evaluated on the paths of one more (untimed) step
+    batch.select(params)
+    paths, plen, leaf, _ = batch.read()
+    N_now = forest.download()["N"]
+    batch.backup(vl)
+    forest.sync()
+    sel_bytes, bak_bytes, n_sel_steps = algorithmic_bytes(soa, meta, paths, plen, N_now)
+    launches_per_select = D + 2  # one reset + one launch per level
+    sel_ms_step = sel_ms / K
+    bak_ms_step = bak_ms / K
+    achieved = sel_bytes / (sel_ms_step * 1e-3) / 1e9
+
+    out = {
+        "metric": "PUCT traversals/s (selection with virtual loss + value backup per step)",
+        "value": B * K / (total_ms * 1e-3),
+        "unit": "traversals/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": args.warmup,
+        "ms_per_step": total_ms / K,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: %d tree(s) x %d nodes, %d traversals per step, depth <= %d, c_puct %.2f, virtual loss %d%s%s%s"
+                        % (args.workload, meta["n_trees"], meta["nodes_per_tree"], B, D, meta["c_puct"], vl,
+                           ", RAVE k=%g" % meta["rave_k"] if meta.get("has_rave") else "",
+                           ", progressive widening" if meta.get("pw") else "",
+                           ", 2^%d-slot table probes" % meta["tt_log2"] if meta.get("tt_log2") else ""),
+            "traversals_per_step": B,
+            "seed": args.seed,
+            "mean_path_nodes": float(plen.mean()),
+            "selection_steps_per_step": n_sel_steps,
+        },
+        "select_traversals_per_s": B / (sel_ms_step * 1e-3),
+        "backups_per_s": B / (bak_ms_step * 1e-3),
+        "select_ms_per_step": sel_ms_step,
+        "backup_ms_per_step": bak_ms_step,
+        "wall_ms_per_step": wall_s * 1e3 / K,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "k_select_level",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "algorithmic_bytes_per_step": sel_bytes,
+            "launches_per_step": launches_per_select,
+            "avg_launch_us": sel_ms_step * 1e3 / launches_per_select,
+            "backup_algorithmic_bytes_per_step": bak_bytes,
+            "backup_achieved": bak_bytes / (bak_ms_step * 1e-3) / 1e9,
+        },
+        "generate_s": gen_s,
+    }
+
+    if args.cpu_seconds > 0:
+        from oracle import ref_cpu as R
+        ref = R.RefTree.from_soa(soa)
+        rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                           rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+        rtt = None
+        done = 0
+        sel_s = bak_s = 0.0
+        t_start = time.perf_counter()
+        while done < 2 or (time.perf_counter() - t_start) < args.cpu_seconds:
+            a = time.perf_counter()
+            rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
+            b = time.perf_counter()
+            ref.backup_batch(rpaths, rlen, values, vl)
+            c = time.perf_counter()
+            sel_s += b - a
+            bak_s += c - b
+            done += 1
+            if done >= K + args.warmup:
+                break
+        out["cpu_baseline"] = {
+            "value": B * done / (sel_s + bak_s),
+            "unit": "traversals/s",
+            "cores": 1,
+            "kind": "port",
+            "sample": "%d steps of the same workload (same forest, roots and leaf values) through the "
+                      "serial CPU restatement of selectChild / applyVirtualLoss / update / revertVirtualLoss" % done,
+            "select_traversals_per_s": B * done / sel_s,
+            "backups_per_s": B * done / bak_s,
+            "host_cores_visible": os.cpu_count(),
+        }
+        del rtt
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
