@@ -47,6 +47,8 @@ struct omk_forest {
     uint32_t *legal = nullptr;
     uint64_t *hash = nullptr;
     bool has_legal = false, has_action = false, has_hash = false;
+    int children = 0;       // live batches and tables created on this forest
+    bool released = false;  // omk_forest_destroy was called while children were alive
 
     ForestDev dev() const {
         ForestDev d;
@@ -74,7 +76,7 @@ struct omk_batch {
     bool selected = false;  // paths of a select are on the device
     int32_t *paths = nullptr, *path_len = nullptr, *leaf = nullptr;
     float *values = nullptr;
-    Item *items0 = nullptr, *items[2] = {nullptr, nullptr};
+    Item *items0 = nullptr, *items_q = nullptr;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
     int32_t *counters = nullptr;  // [max_depth + 2] level counters, then 1 truncated counter
@@ -95,7 +97,9 @@ static hipError_t dalloc(T **p, int64_t count) {
 }
 
 static int use_device(const omk_forest *f) {
+    if (f->released) return fail(OMK_ERR_STATE, "the forest of this handle has been destroyed");
     HIP_TRY(hipSetDevice(f->device));
+    (void)hipGetLastError();  // launches are checked with hipGetLastError: start from a clean slate
     return OMK_OK;
 }
 
@@ -138,15 +142,30 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
     return OMK_OK;
 }
 
-int omk_forest_destroy(omk_forest *f) {
-    if (!f) return OMK_OK;
+static void forest_free(omk_forest *f) {
     (void)hipSetDevice(f->device);
     if (f->own_stream) (void)hipStreamSynchronize(f->own_stream);
     void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->action, f->legal, f->hash};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     if (f->own_stream) (void)hipStreamDestroy(f->own_stream);
+    (void)hipGetLastError();
     delete f;
+}
+
+// Batches and tables point into their forest: the memory goes when the last of them has.
+static void forest_child_gone(omk_forest *f) {
+    if (--f->children == 0 && f->released) forest_free(f);
+}
+
+int omk_forest_destroy(omk_forest *f) {
+    if (!f) return OMK_OK;
+    if (f->released) return fail(OMK_ERR_STATE, "omk_forest_destroy: called twice");
+    if (f->children > 0) {
+        f->released = true;
+        return OMK_OK;
+    }
+    forest_free(f);
     return OMK_OK;
 }
 
@@ -282,10 +301,14 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
         return fail(OMK_ERR_INVALID, "omk_batch_create: max_traversals %d out of range", max_traversals);
     if (max_depth <= 0 || max_depth > 4096)
         return fail(OMK_ERR_INVALID, "omk_batch_create: max_depth %d out of range", max_depth);
+    if ((int64_t)max_traversals * (max_depth + 1) > (1ll << 28))
+        return fail(OMK_ERR_CAPACITY, "omk_batch_create: max_traversals x (max_depth+1) = %lld exceeds 2^28",
+                    (long long)max_traversals * (max_depth + 1));
     if (int rc = use_device(f)) return rc;
     omk_batch *b = new (std::nothrow) omk_batch();
     if (!b) return fail(OMK_ERR_INVALID, "out of host memory");
     b->f = f;
+    f->children++;
     b->max_traversals = max_traversals;
     b->max_depth = max_depth;
     b->stride = (max_traversals + 63) & ~63;
@@ -295,8 +318,7 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->leaf, B);
     if (e == hipSuccess) e = dalloc(&b->values, B);
     if (e == hipSuccess) e = dalloc(&b->items0, B);
-    if (e == hipSuccess) e = dalloc(&b->items[0], B);
-    if (e == hipSuccess) e = dalloc(&b->items[1], B);
+    if (e == hipSuccess) e = dalloc(&b->items_q, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->seg0, B);
     if (e == hipSuccess) e = dalloc(&b->seg[0], B);
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
@@ -319,10 +341,12 @@ int omk_batch_destroy(omk_batch *b) {
     if (!b) return OMK_OK;
     (void)hipSetDevice(b->f->device);
     (void)hipStreamSynchronize(b->f->stream);
-    void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items[0],  b->items[1],  b->seg0,
+    void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
+    (void)hipGetLastError();
+    forest_child_gone(b->f);
     delete b;
     return OMK_OK;
 }
@@ -397,6 +421,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     if (int rc = use_device(f)) return rc;
     SelectArgs a;
     memset(&a, 0, sizeof(a));
+    a.items0 = b->items0;
+    a.seg0 = b->seg0;
+    a.items_q = b->items_q;
+    a.seg[0] = b->seg[0];
+    a.seg[1] = b->seg[1];
     a.counters = b->counters;
     a.truncated = b->counters + b->max_depth + 2;
     a.sc_child = b->sc_child;
@@ -410,16 +439,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.pw = p->pw;
     a.c_puct = p->c_puct;
     a.rave_k = p->rave_k;
-    BatchBuffers bb;
-    bb.items0 = b->items0;
-    bb.seg0 = b->seg0;
-    bb.n_items0 = b->n_items0;
-    bb.items[0] = b->items[0];
-    bb.items[1] = b->items[1];
-    bb.seg[0] = b->seg[0];
-    bb.seg[1] = b->seg[1];
-    bb.n_traversals = b->n;
-    HIP_TRY(launch_select(f->dev(), a, bb, f->max_fanout, p->use_rave != 0, f->stream));
+    HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n, f->max_fanout, p->use_rave != 0, f->stream));
     b->selected = true;
     return OMK_OK;
 }
@@ -509,6 +529,7 @@ int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out) {
     omk_tt *tt = new (std::nothrow) omk_tt();
     if (!tt) return fail(OMK_ERR_INVALID, "out of host memory");
     tt->f = f;
+    f->children++;
     tt->log2_slots = log2_slots;
     hipError_t e = dalloc(&tt->slots, 1ll << log2_slots);
     if (e == hipSuccess) e = dalloc(&tt->d_status, 2);
@@ -527,6 +548,8 @@ int omk_tt_destroy(omk_tt *tt) {
     (void)hipStreamSynchronize(tt->f->stream);
     if (tt->slots) (void)hipFree(tt->slots);
     if (tt->d_status) (void)hipFree(tt->d_status);
+    (void)hipGetLastError();
+    forest_child_gone(tt->f);
     delete tt;
     return OMK_OK;
 }

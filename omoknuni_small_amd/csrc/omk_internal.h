@@ -33,14 +33,14 @@ struct Item {
 };
 
 struct SelectArgs {
-    const Item *items_in;
-    Item *items_out;
-    int32_t *counters;  // counters[d] = number of items of level d
-    const int32_t *seg_in;
-    int32_t *seg_out;
-    int32_t *sc_child;  // per visitor: chosen child index
-    int32_t *sc_occ;    // per visitor: how many earlier visitors of the item chose the same child
-    int32_t *paths;     // level-major [max_depth+1][stride]
+    const Item *items0;    // level-0 items, built when the roots are set
+    const int32_t *seg0;   // their visitor lists
+    Item *items_q;         // queue of level L >= 1 at items_q + (L-1)*stride
+    int32_t *counters;     // counters[L] = number of items of level L
+    int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
+    int32_t *sc_child;     // per visitor: chosen child index
+    int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child
+    int32_t *paths;        // level-major [max_depth+1][stride]
     int32_t *path_len;
     int32_t *leaf;
     int32_t *truncated;
@@ -52,17 +52,8 @@ struct SelectArgs {
     float rave_k;
 };
 
-struct BatchBuffers {
-    Item *items0;  // level-0 items, built by set_roots
-    int32_t *seg0;
-    int32_t n_items0;
-    Item *items[2];
-    int32_t *seg[2];
-    int32_t n_traversals;
-};
-
-hipError_t launch_select(const ForestDev &f, SelectArgs a, const BatchBuffers &b, int max_fanout, bool rave,
-                         hipStream_t s);
+hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals, int max_fanout,
+                         bool rave, hipStream_t s);
 
 hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                            int max_len, int vl, hipStream_t s);
