@@ -79,7 +79,7 @@ struct omk_batch {
     Item *items0 = nullptr, *items_q = nullptr;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
-    int32_t *counters = nullptr;  // [max_depth + 2] level counters, then 1 truncated counter
+    int32_t *counters = nullptr;  // [max_depth + 2] level counters, 1 truncated counter, 8 work statistics
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
 };
@@ -324,7 +324,7 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, B);
     if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
-    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3);
+    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3 + 8);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
     if (e == hipSuccess) e = hipMemset(b->values, 0, (size_t)B * 4);
@@ -428,6 +428,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.seg[1] = b->seg[1];
     a.counters = b->counters;
     a.truncated = b->counters + b->max_depth + 2;
+    a.stats = b->counters + b->max_depth + 3;
     a.sc_child = b->sc_child;
     a.sc_occ = b->sc_occ;
     a.paths = b->paths;
@@ -516,6 +517,15 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_truncated: no selected paths");
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipMemcpyAsync(h_count, b->counters + b->max_depth + 2, 4, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipStreamSynchronize(b->f->stream));
+    return OMK_OK;
+}
+
+int omk_batch_stats(omk_batch *b, int32_t *h_stats8) {
+    if (!b || !h_stats8) return fail(OMK_ERR_INVALID, "omk_batch_stats: null argument");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_stats: no selected paths");
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + b->max_depth + 3, 32, hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }

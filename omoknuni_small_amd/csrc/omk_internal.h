@@ -44,6 +44,7 @@ struct SelectArgs {
     int32_t *path_len;
     int32_t *leaf;
     int32_t *truncated;
+    int32_t *stats;        // optional 8 counters describing how the work was done (nullptr = off)
     int32_t stride;
     int32_t max_depth;
     int32_t vl;

@@ -13,8 +13,9 @@
 // on register-resident statistics: score, DPP arg-max with lowest-index tie-break, bump
 // the chosen child's virtual loss, next visitor.  That reproduces the serial order
 // exactly.  The visitors are then partitioned by chosen child (stable, so still in
-// traversal order); the wavefront keeps the largest part and walks on with it, the other
-// parts become work items of the next level's launch.
+// traversal order) into the work items of the next level's launch; a group that stays
+// together (every visitor chose the same child) and a lone visitor are walked on by the
+// same wavefront without waiting for that launch.
 //
 // Playing the visitors of a crowded node one at a time is a chain of dependent wave
 // reductions.  The score a child will have after j more visits depends on nothing but j,
@@ -194,7 +195,7 @@ struct Dominant {
     int K;
 };
 
-// Where the walk goes on after a multi-visitor node: the child that received most visitors.
+// Where the walk goes on after a multi-visitor node whose visitors all chose one child.
 struct Continuation {
     int node;
     int off;
@@ -204,8 +205,8 @@ struct Continuation {
 
 // All visitors of a multi-visitor item, in order.  Records the chosen child of every
 // visitor, bumps virtual loss, partitions the visitors by child into seg_out, writes the
-// next path entry, appends one item per visited child (except the kept one) to the next
-// level's queue.  Returns false when no child takes part in the selection.
+// next path entry, appends one item per visited child to the next level's queue (none when
+// all visitors chose the same child: then the caller walks on with them).  Returns false when no child takes part in the selection.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              const int32_t *seg_in, int32_t *seg_out, int off, int m, int depth,
@@ -239,12 +240,15 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     int done = 0;
     int backoff = 0;
     int fails = 0;
+    int recent0 = -1, recent1 = -1;  // the last two children settled one at a time
+    int st_rounds = 0, st_settled = 0, st_single = 0, st_viol = 0, st_none = 0;
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
 
     while (done < m) {
         if (dom.K > 0 && backoff == 0 && m - done >= 4) {
             // ---- look-ahead round ----
             const int K = dom.K;
+            st_rounds++;
             const int logE = K <= 1 ? 6 : (K == 2 ? 5 : 4);
             const int E = 1 << logE;
             const int g = lane >> logE;
@@ -265,16 +269,15 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                     scnt = dom.cnt[gg];
                 }
             }
-            uint32_t ek = 0u, epos = 0xFFFFFFFFu;
+            uint32_t ek = 0u, epos = 0xFFFFFFFFu, ek1 = 0u, ek2 = 0u;
             if (slot) {
                 int vlj = (int)((uint32_t)svl + (uint32_t)o * uvl);
-                uint32_t k1, k2;
-                child_keys<RAVE>(sn, sw, sp, vlj, srn, srw, c.ep, a.rave_k, k1, k2);
-                if (k2 > k1) {
-                    ek = k2;
+                child_keys<RAVE>(sn, sw, sp, vlj, srn, srw, c.ep, a.rave_k, ek1, ek2);
+                if (ek2 > ek1) {
+                    ek = ek2;
                     epos = (uint32_t)(R * kWave + sc);
                 } else {
-                    ek = k1;
+                    ek = ek1;
                     epos = (uint32_t)sc;
                 }
             }
@@ -283,6 +286,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             uint32_t ppos = (uint32_t)__shfl_up((int)epos, 1, kWave);
             bool viol = slot && o > 0 && ek != 0u && (pk == 0u || ek > pk || (ek == pk && epos < ppos));
             bool ok = __ballot(viol) == 0ull;
+            if (!ok) st_viol++;
             int settled = 0;
             if (ok) {
                 // bound: best head of every other child, and the last evaluated entry of each list
@@ -299,20 +303,39 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                 if (accm != 0ull) {
                     // rank in the merged order: own offset + entries of the other lists that come first
                     int rank = o;
-                    for (int gg = 0; gg < K; gg++) {
-                        int lo = 0, hi = E;
+                    if (K > 1) {
+                        // binary searches in the other lists, advanced together so that their
+                        // cross-lane reads overlap
+                        int lo[4], hi[4];
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++) {
+                            lo[gg] = 0;
+                            hi[gg] = E;
+                        }
                         for (int s = 0; s <= logE; s++) {
-                            int mid = (lo + hi) >> 1;
-                            int src = (gg << logE) + (mid < E ? mid : E - 1);
-                            uint32_t mk = (uint32_t)__shfl((int)ek, src, kWave);
-                            uint32_t mpos = (uint32_t)__shfl((int)epos, src, kWave);
-                            bool before = mk != 0u && (mk > ek || (mk == ek && mpos < epos));
-                            if (lo < hi) {
-                                if (before) lo = mid + 1;
-                                else hi = mid;
+                            uint32_t mk[4], mpos[4];
+#pragma unroll
+                            for (int gg = 0; gg < 4; gg++) {
+                                if (gg < K) {
+                                    int mid = (lo[gg] + hi[gg]) >> 1;
+                                    int src = (gg << logE) + (mid < E ? mid : E - 1);
+                                    mk[gg] = (uint32_t)__shfl((int)ek, src, kWave);
+                                    mpos[gg] = (uint32_t)__shfl((int)epos, src, kWave);
+                                }
+                            }
+#pragma unroll
+                            for (int gg = 0; gg < 4; gg++) {
+                                if (gg < K && lo[gg] < hi[gg]) {
+                                    int mid = (lo[gg] + hi[gg]) >> 1;
+                                    bool before = mk[gg] != 0u && (mk[gg] > ek || (mk[gg] == ek && mpos[gg] < epos));
+                                    if (before) lo[gg] = mid + 1;
+                                    else hi[gg] = mid;
+                                }
                             }
                         }
-                        if (gg != g) rank += lo;
+#pragma unroll
+                        for (int gg = 0; gg < 4; gg++)
+                            if (gg < K && gg != g) rank += lo[gg];
                     }
                     const int remaining = m - done;
                     const bool valid = acc && rank < remaining;
@@ -329,13 +352,19 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                                 dom.vl[gg] = (int)((uint32_t)dom.vl[gg] + (uint32_t)ag * uvl);
                                 dom.cnt[gg] += ag;
                                 int ch = dom.child[gg];
+                                // the new head of this child was looked ahead at offset ag
+                                // (the last entry of a list is never settled, so ag < E)
+                                const int hl = (gg << logE) + ag;
+                                uint32_t nk1 = (uint32_t)__builtin_amdgcn_readlane((int)ek1, hl);
+                                uint32_t nk2 = (uint32_t)__builtin_amdgcn_readlane((int)ek2, hl);
                                 if (lane == (ch & 63)) {
 #pragma unroll
                                     for (int r = 0; r < R; r++) {
                                         if (r == (ch >> 6)) {
                                             cnt[r] += ag;
                                             k.vl[r] = (int)((uint32_t)k.vl[r] + (uint32_t)ag * uvl);
-                                            score_round<R, RAVE>(k, r, c.ep, a.rave_k);
+                                            k.k1[r] = nk1;
+                                            k.k2[r] = nk2;
                                         }
                                     }
                                 }
@@ -387,9 +416,11 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             }
             if (settled > 0) {
                 done += settled;
+                st_settled += settled;
                 fails = 0;
                 continue;
             }
+            if (ok) st_none++;
             fails = fails < 5 ? fails + 1 : 5;
             backoff = 1 << fails;
         }
@@ -397,6 +428,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         // ---- one visitor ----
         int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
         if (i < 0) return false;  // no child takes part: uniform, and then for every visitor
+        st_single++;
         int tn = 0, tvl = 0, trn = 0, tcnt = 0;
         float tw = 0.0f, tp = 0.0f, trw = 0.0f;
         if (lane == (i & 63)) {
@@ -451,7 +483,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                     dom.stale[gg] = 0;
                 }
             }
-        } else {
+        } else if (i == recent0 || i == recent1) {
             int slot_g = dom.K;
             if (dom.K >= 4) {
                 slot_g = 0;
@@ -495,8 +527,18 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             }
             if (lane == ol) dmask |= 1u << (i >> 6);
         }
+        recent1 = recent0;
+        recent0 = i;
     }
 
+    if (a.stats && lane == 0) {
+        atomicAdd(a.stats + 0, 1);
+        atomicAdd(a.stats + 1, st_rounds);
+        atomicAdd(a.stats + 2, st_settled);
+        atomicAdd(a.stats + 3, st_single);
+        atomicAdd(a.stats + 4, st_viol);
+        atomicAdd(a.stats + 5, st_none);
+    }
     // the child with most visitors (lowest index on ties) is where this wavefront walks on
     uint32_t lmax = 0u;
 #pragma unroll
@@ -506,7 +548,9 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
 #pragma unroll
     for (int r = R - 1; r >= 0; r--)
         if ((uint32_t)cnt[r] == gmax) lidx = (uint32_t)(r * kWave + lane);
-    const int keep = (int)wave_min_u32(lidx);
+    // walking on is only worth it when the group stays together: a split group is handed to
+    // the next level's launch whole, so that its parts are played side by side
+    const int keep = gmax == (uint32_t)m ? (int)wave_min_u32(lidx) : -1;
 
     // exclusive prefix of the visit counts in child order -> segment of every child
     int carry = 0;
@@ -548,10 +592,13 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         path_next[t] = c.cb + i;
         seg_out[off + s_offs[i] + a.sc_occ[off + j]] = t;
     }
-    next.node = c.cb + keep;
-    next.off = off + s_offs[keep];
-    next.m = (int)gmax;
-    next.np = __builtin_amdgcn_readlane(keep_np, keep & 63);
+    next.node = -1;
+    if (keep >= 0) {
+        next.node = c.cb + keep;
+        next.off = off + s_offs[keep];
+        next.m = (int)gmax;
+        next.np = __builtin_amdgcn_readlane(keep_np, keep & 63);
+    }
     // the next step of the walk reads seg_out and reuses s_offs
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
@@ -599,6 +646,7 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
             if (c.cc > 0 && depth >= a.max_depth && lane == 0) atomicAdd(a.truncated, m);
             return;
         }
+        if (next.node < 0) return;
         node = next.node;
         off = next.off;
         m = next.m;
@@ -628,6 +676,7 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
         }
         int child = c.cb + i;
         if (lane == 0) {
+            if (a.stats) atomicAdd(a.stats + 6, 1);
             if (a.vl > 0) atomicAdd(f.VL + child, a.vl);
             a.paths[(size_t)(d + 1) * a.stride + t] = child;
         }
@@ -637,10 +686,11 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
     }
 }
 
-__global__ void k_select_reset(int *counters, int n_counters, int n_items0, int *truncated) {
+__global__ void k_select_reset(int *counters, int n_counters, int n_items0, int *truncated, int *stats) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n_counters) counters[i] = (i == 0) ? n_items0 : 0;
     if (i == 0) *truncated = 0;
+    if (stats && i < 8) stats[i] = 0;
 }
 
 template <int RMAX, bool RAVE>
@@ -654,7 +704,7 @@ static hipError_t launch_levels(const ForestDev &f, const SelectArgs &a, int n_t
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals, int max_fanout,
                          bool rave, hipStream_t s) {
     hipLaunchKernelGGL(k_select_reset, dim3((a.max_depth + 2 + 63) / 64), dim3(64), 0, s, a.counters,
-                       a.max_depth + 2, n_items0, a.truncated);
+                       a.max_depth + 2, n_items0, a.truncated, a.stats);
 #define OMK_DISPATCH(RM) \
     return rave ? launch_levels<RM, true>(f, a, n_traversals, s) : launch_levels<RM, false>(f, a, n_traversals, s)
     if (max_fanout <= 64) { OMK_DISPATCH(1); }
