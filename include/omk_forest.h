@@ -151,9 +151,10 @@ int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t 
 /* Traversals of the last select that stopped at max_depth on an expanded node. */
 int omk_batch_truncated(omk_batch *b, int32_t *h_count);
 /* How the last select did its work, 8 counters: [0] multi-visitor nodes processed,
- * [1] look-ahead rounds, [2] visitors settled by look-ahead, [3] visitors settled one at a
- * time, [4] rounds abandoned because a child's scores rose, [5] rounds that settled nothing,
- * [6] single-visitor selection steps, [7] unused. */
+ * [1] of these settled by the parallel water-level path, [2] visitors settled by it,
+ * [3] visitors settled one at a time, [4] nodes replayed one visitor at a time because the
+ * parallel path's exactness checks did not hold, [5] unused, [6] single-visitor selection
+ * steps, [7] unused. */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats8);
 
 /* ---- transposition table: the lookup/store call sites of

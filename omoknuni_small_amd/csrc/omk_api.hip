@@ -79,6 +79,7 @@ struct omk_batch {
     Item *items0 = nullptr, *items_q = nullptr;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
+    int32_t *sort_buf[4] = {nullptr, nullptr, nullptr, nullptr};
     int32_t *counters = nullptr;  // [max_depth + 2] level counters, 1 truncated counter, 8 work statistics
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
@@ -324,6 +325,8 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, B);
     if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
+    for (int i = 0; i < 4; i++)
+        if (e == hipSuccess) e = dalloc(&b->sort_buf[i], B);
     if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3 + 8);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
@@ -342,7 +345,8 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipSetDevice(b->f->device);
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
-                    b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions};
+                    b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
+                    b->sort_buf[0], b->sort_buf[1], b->sort_buf[2], b->sort_buf[3]};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -431,6 +435,10 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.stats = b->counters + b->max_depth + 3;
     a.sc_child = b->sc_child;
     a.sc_occ = b->sc_occ;
+    a.sort_key[0] = b->sort_buf[0];
+    a.sort_key[1] = b->sort_buf[1];
+    a.sort_pay[0] = b->sort_buf[2];
+    a.sort_pay[1] = b->sort_buf[3];
     a.paths = b->paths;
     a.path_len = b->path_len;
     a.leaf = b->leaf;

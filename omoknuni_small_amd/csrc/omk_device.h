@@ -49,6 +49,21 @@ __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
     return umin32(umin32(a, b), umin32(c, d));
 }
 
+// Sum over the 64 lanes: xor butterfly inside each row of 16 (quad swaps, half-row mirror,
+// row mirror leave the row total in every lane), the four row totals added on the scalar unit.
+__device__ __forceinline__ int wave_sum_i32(int x) {
+    uint32_t v = (uint32_t)x;
+    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_mov<0x141>(v);  // row_half_mirror
+    v += dpp_mov<0x140>(v);  // row_mirror
+    uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
+    uint32_t b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
+    uint32_t d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return (int)(a + b + c + d);
+}
+
 // Inclusive prefix sum over the 64 lanes (used once per multi-visitor node, not per pick).
 __device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
 #pragma unroll

@@ -40,6 +40,8 @@ struct SelectArgs {
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
     int32_t *sc_child;     // per visitor: chosen child index
     int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child
+    int32_t *sort_key[2];  // per visitor: ping-pong buffers of the winner-order sort
+    int32_t *sort_pay[2];
     int32_t *paths;        // level-major [max_depth+1][stride]
     int32_t *path_len;
     int32_t *leaf;

@@ -8,28 +8,34 @@
 // How.  During this phase only virtual-loss counters change, and the counter of a child
 // matters only to selections made at its parent.  On a tree, the traversals that reach a
 // node all come through its parent.  So a work item is (node, the list of traversals that
-// reached it, in traversal-index order); ONE 64-lane wavefront owns the item, loads the
-// children once (coalesced, one child per lane per round) and plays the visitors in order
-// on register-resident statistics: score, DPP arg-max with lowest-index tie-break, bump
-// the chosen child's virtual loss, next visitor.  That reproduces the serial order
-// exactly.  The visitors are then partitioned by chosen child (stable, so still in
-// traversal order) into the work items of the next level's launch; a group that stays
-// together (every visitor chose the same child) and a lone visitor are walked on by the
-// same wavefront without waiting for that launch.
+// reached it, in traversal-index order); ONE 64-lane wavefront owns the item and loads the
+// children once (coalesced, one child per lane per round).  The visitors are then
+// partitioned by chosen child (stable, so still in traversal order) into the work items
+// of the next level's launch; a group that stays together (every visitor chose the same
+// child) and a lone visitor are walked on by the same wavefront.
 //
-// Playing the visitors of a crowded node one at a time is a chain of dependent wave
-// reductions.  The score a child will have after j more visits depends on nothing but j,
-// so the lanes evaluate AHEAD: the next E scores of each of the (up to four) children that
-// have been winning.  As long as each child's scores do not increase, the serial winner
-// sequence is the merge of these descending lists, and every looked-ahead score that
-// beats (a) the best score of every other child and (b) the last looked-ahead score of
-// each list is certain to be played before anything not evaluated yet.  One round thus
-// settles up to 64 visitors with two reductions and a binary-search merge; a round that
-// settles nothing falls back to the one-visitor step, so the result never depends on the
-// speculation, only the speed does.
+// Which child each visitor chooses:
+//  * few visitors: they are played one after another on register-resident statistics --
+//    score, DPP arg-max with lowest-index tie-break, bump the chosen child's virtual loss,
+//    next visitor.  That is the serial order itself.
+//  * many visitors ("water level"): the score child i shows to its j-th visitor of this
+//    batch depends on nothing but j.  If every child's scores do not increase with j, the
+//    serial winner sequence is the merge of these descending lists, i.e. the m best
+//    entries (i, j) in the order (score descending, candidate position ascending, j
+//    ascending).  A bisection on the score threshold finds how many entries each child
+//    contributes, all m entries are evaluated in parallel, a stable radix sort puts them
+//    in winner order.  Nothing is assumed: afterwards the wavefront checks, on the exact
+//    binary32 values, (i) that every child's taken entries and its first untaken entry do
+//    not increase and (ii) that the last taken entry still comes before every child's
+//    first untaken one.  Under (i) and (ii) the serial loop provably produces exactly
+//    this sequence; if either fails the node is replayed one visitor at a time.
 #include "omk_internal.h"
 
 namespace omk {
+
+constexpr int kRunMin = 4;                // visitors from which the one-winner check is tried
+constexpr int kWaterLevelMin = 32;        // visitors from which the parallel path is tried
+constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in the sort payload
 
 // Register-resident statistics of the children a lane is responsible for: child index
 // i = r * 64 + lane for round r.
@@ -44,6 +50,19 @@ struct Kids {
     uint32_t k1[R];
     uint32_t k2[R];
     bool part[R];
+};
+
+// Per-wavefront scratch in LDS.
+template <int R>
+struct WaveLds {
+    int offs[R * kWave];  // exclusive prefix of the visit counts in child order
+    int st_n[R * kWave];
+    float st_w[R * kWave];
+    float st_p[R * kWave];
+    int st_vl[R * kWave];
+    int st_rn[R * kWave];
+    float st_rw[R * kWave];
+    int hist[256];
 };
 
 template <int R, bool RAVE>
@@ -79,19 +98,17 @@ __device__ __forceinline__ void score_round(Kids<R, RAVE> &k, int r, float ep, f
 
 // Best candidate of this lane in the order (key descending, position ascending); the
 // candidates of the second scan sit at positions R*64 + i, after all of the first scan.
-// Children whose bit is set in skip are left out.
 template <int R, bool RAVE>
-__device__ __forceinline__ void lane_best(const Kids<R, RAVE> &k, int lane, uint32_t skip, uint32_t &bk,
-                                          uint32_t &bpos) {
+__device__ __forceinline__ void lane_best(const Kids<R, RAVE> &k, int lane, uint32_t &bk, uint32_t &bpos) {
     bk = 0u;
     bpos = 0xFFFFFFFFu;
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        if (k.k1[r] > bk && !((skip >> r) & 1u)) { bk = k.k1[r]; bpos = (uint32_t)(r * kWave + lane); }
+        if (k.k1[r] > bk) { bk = k.k1[r]; bpos = (uint32_t)(r * kWave + lane); }
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        if (k.k2[r] > bk && !((skip >> r) & 1u)) { bk = k.k2[r]; bpos = (uint32_t)(R * kWave + r * kWave + lane); }
+        if (k.k2[r] > bk) { bk = k.k2[r]; bpos = (uint32_t)(R * kWave + r * kWave + lane); }
     }
 }
 
@@ -168,7 +185,7 @@ __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArg
 #pragma unroll
     for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep, a.rave_k);
     uint32_t bk, bpos;
-    lane_best<R, RAVE>(k, lane, 0u, bk, bpos);
+    lane_best<R, RAVE>(k, lane, bk, bpos);
     int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
     if (i < 0) return -1;
     int nsel = 0;
@@ -180,20 +197,456 @@ __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArg
     return i;
 }
 
-// The children that have been winning lately, with a wave-uniform copy of their current
-// statistics so that any lane can evaluate their future scores.
-struct Dominant {
-    int child[4];
-    int n[4];
-    float w[4];
-    float p[4];
-    int vl[4];  // current counter, picks of this item included
-    int rn[4];
-    float rw[4];
-    int cnt[4];  // picks of this item so far
-    int stale[4];
-    int K;
-};
+// Key and candidate position child `child` shows to its j-th visitor of this batch.
+template <int R, bool RAVE>
+__device__ __forceinline__ void entry_key(int n, float w, float p, int vl0, int rn, float rw, float ep,
+                                          float rave_k, uint32_t uvl, int j, int child, uint32_t &key,
+                                          uint32_t &pos) {
+    int vlj = (int)((uint32_t)vl0 + (uint32_t)j * uvl);
+    uint32_t k1, k2;
+    child_keys<RAVE>(n, w, p, vlj, rn, rw, ep, rave_k, k1, k2);
+    if (k2 > k1) {
+        key = k2;
+        pos = (uint32_t)(R * kWave + child);
+    } else {
+        key = k1;
+        pos = (uint32_t)child;
+    }
+}
+
+// true when candidate (ka, pa) is played strictly before candidate (kb, pb)
+__device__ __forceinline__ bool comes_before(uint32_t ka, uint32_t pa, uint32_t kb, uint32_t pb) {
+    return ka > kb || (ka == kb && pa < pb);
+}
+
+__device__ __forceinline__ void wave_sync_memory() {
+    // Orders this wavefront's LDS / global writes before its own later reads from other
+    // lanes.  One wavefront's memory operations reach the cache in program order, so this
+    // only has to stop the compiler from moving them across.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The visitors of a crowded node, all at once (see the file header).  On success cnt[r]
+// holds the visitors of every child and sc_child / sc_occ hold (child, visit number) of
+// every visitor; returns false, having changed nothing that matters, when the node has to
+// be replayed one visitor at a time.
+template <int R, bool RAVE>
+__device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
+                                            uint32_t bk, uint32_t bpos, int off, int m, WaveLds<R> &lds,
+                                            int (&cnt)[R]) {
+    constexpr int F = R * kWave;
+    const uint32_t uvl = (uint32_t)a.vl;
+    if (m > kWaterLevelMaxJ) return false;
+
+    // ---- 1. threshold T* = largest key with at least m entries at or above it ----
+    uint32_t hi_key, hi_pos;
+    wave_best(bk, bpos, hi_key, hi_pos);
+    if (hi_key == 0u) return false;
+    const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
+    // the best child alone has m entries at or above the key of its m-th visit
+    uint32_t lo_key = 0u;
+    {
+        uint32_t kk = 0u, pp = 0u;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (r == (best >> 6))
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, m - 1,
+                                   best, kk, pp);
+        }
+        lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
+    }
+    if (lo_key == 0u) lo_key = 1u;
+    if (lo_key > hi_key) return false;  // scores rose along the best child's list
+
+    int cl[R], ch[R];
+    uint32_t head[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        head[r] = umax32(k.k1[r], k.k2[r]);
+        cl[r] = 0;
+        ch[r] = head[r] != 0u ? m : 0;
+    }
+    // Invariant: count(lo) >= m > count(hi), cl = per-child counts at hi, ch = at lo.  After
+    // every probe the bracket end that moved is snapped to the nearest key that actually
+    // occurs, so the search ends after about log2(distinct keys in the bracket) probes.
+    uint32_t lo = lo_key, hi = hi_key + 1u;
+    bool first = true;
+    int probes = 0;
+    while (first || hi - lo > 1u) {
+        if (++probes > 80) return false;
+        const uint32_t T = first ? lo : lo + ((hi - lo) >> 1);
+        int ct[R];
+        int sum = 0;
+        uint32_t below = 0u;             // largest key below T among the first entries below T
+        uint32_t above = 0xFFFFFFFFu;    // smallest key at or above T among the last entries at or above T
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int lo_c = cl[r], hi_c = ch[r];
+            if (head[r] < T) hi_c = 0;  // a list that starts below T has nothing above it
+            if (lo_c > hi_c) lo_c = hi_c;
+            uint32_t k_in = 0xFFFFFFFFu, k_out = 0u;  // keys seen at the boundary while searching
+            int j_in = -1, j_out = -1;
+            while (lo_c < hi_c) {
+                int t = (lo_c + hi_c + 1) >> 1;
+                uint32_t kk, pp;
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, t - 1,
+                                   r * kWave + lane, kk, pp);
+                if (kk >= T) {
+                    lo_c = t;
+                    k_in = kk;
+                    j_in = t - 1;
+                } else {
+                    hi_c = t - 1;
+                    k_out = kk;
+                    j_out = t - 1;
+                }
+            }
+            ct[r] = lo_c;
+            sum = sum + lo_c > m ? m : sum + lo_c;
+            if (head[r] != 0u) {
+                // last entry at or above T and first entry below T of this child
+                if (lo_c > 0) {
+                    if (j_in != lo_c - 1) {
+                        if (lo_c == 1) {
+                            k_in = head[r];
+                        } else {
+                            uint32_t pp;
+                            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
+                                               lo_c - 1, r * kWave + lane, k_in, pp);
+                        }
+                    }
+                    above = umin32(above, k_in);
+                }
+                if (lo_c < m) {
+                    if (j_out != lo_c) {
+                        if (lo_c == 0) {
+                            k_out = head[r];
+                        } else {
+                            uint32_t pp;
+                            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
+                                               lo_c, r * kWave + lane, k_out, pp);
+                        }
+                    }
+                    if (k_out < T) below = umax32(below, k_out);
+                }
+            }
+        }
+        const int total = wave_sum_i32(sum);  // at most 64 * m
+        if (first) {
+            if (total < m) return false;
+            first = false;
+        }
+        if (total >= m) {
+            uint32_t snap = wave_min_u32(above);
+            lo = (snap != 0xFFFFFFFFu && snap >= T && snap < hi) ? snap : T;
+#pragma unroll
+            for (int r = 0; r < R; r++) ch[r] = ct[r];
+        } else {
+            uint32_t snap = wave_max_u32(below);
+            hi = (snap + 1u > lo && snap < T) ? snap + 1u : T;
+#pragma unroll
+            for (int r = 0; r < R; r++) cl[r] = ct[r];
+        }
+    }
+    // now cl = entries above T*, ch = entries at or above T*
+
+    // ---- 2. entries at exactly T* are handed out in child order until m is reached ----
+    int above = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) above = above + cl[r] > m ? m : above + cl[r];
+    int rem = m - wave_sum_i32(above);
+    if (rem < 0) return false;
+    int cv[R];
+    int carry = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        int e = ch[r] - cl[r];
+        if (e < 0) e = 0;
+        if (e > rem) e = rem;
+        int inc = wave_inclusive_sum(e, lane);
+        long long excl = (long long)carry + inc - e;
+        long long left = (long long)rem - excl;
+        int take = left <= 0 ? 0 : (left < e ? (int)left : e);
+        cv[r] = cl[r] + take;
+        int tot = __builtin_amdgcn_readlane(inc, 63);
+        carry = carry + tot > m ? m : carry + tot;
+    }
+    int csum = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) csum = csum + cv[r] > m + 1 ? m + 1 : csum + cv[r];
+    if (wave_sum_i32(csum) != m) return false;
+
+    // ---- 3. evaluate the m entries, in (child, visit) order; first untaken entries ----
+    carry = 0;
+    uint32_t uk[R], upos[R];  // first untaken entry of every child of this lane
+    bool bad = false;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        int inc = wave_inclusive_sum(cv[r], lane);
+        int i = r * kWave + lane;
+        lds.offs[i] = carry + inc - cv[r];
+        lds.st_n[i] = k.n[r];
+        lds.st_w[i] = k.w[r];
+        lds.st_p[i] = k.p[r];
+        lds.st_vl[i] = k.vl[r];
+        if (RAVE) {
+            lds.st_rn[i] = k.rn[r];
+            lds.st_rw[i] = k.rw[r];
+        }
+        carry += __builtin_amdgcn_readlane(inc, 63);
+        uk[r] = 0u;
+        upos[r] = 0xFFFFFFFFu;
+        if (k.part[r]) {
+            uint32_t kk, pp;
+            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, cv[r], i, kk,
+                               pp);
+            uk[r] = kk;
+            upos[r] = pp;
+            if (cv[r] > 0) {
+                // the last taken entry of the child must not come after its first untaken one
+                uint32_t lk, lp;
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
+                                   cv[r] - 1, i, lk, lp);
+                if (lk == 0u || comes_before(kk, pp, lk, lp)) bad = true;
+            }
+        }
+    }
+    wave_sync_memory();
+
+    uint32_t *keyA = (uint32_t *)a.sort_key[0] + off, *keyB = (uint32_t *)a.sort_key[1] + off;
+    uint32_t *payA = (uint32_t *)a.sort_pay[0] + off, *payB = (uint32_t *)a.sort_pay[1] + off;
+    uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
+    uint32_t prev_key63 = 0u, prev_pos63 = 0u;
+    int prev_child63 = -1;
+    for (int base = 0; base < m; base += kWave) {
+        const int q = base + lane;
+        const bool in = q < m;
+        int child = -1;
+        uint32_t kk = 0u, pp = 0u;
+        if (in) {
+            // last child whose segment starts at or before q
+            int lo_i = 0, hi_i = F;
+            while (hi_i - lo_i > 1) {
+                int mid = (lo_i + hi_i) >> 1;
+                if (lds.offs[mid] <= q) lo_i = mid;
+                else hi_i = mid;
+            }
+            child = lo_i;
+            const int j = q - lds.offs[child];
+            entry_key<R, RAVE>(lds.st_n[child], lds.st_w[child], lds.st_p[child], lds.st_vl[child],
+                               RAVE ? lds.st_rn[child] : 0, RAVE ? lds.st_rw[child] : 0.0f, c.ep, a.rave_k, uvl, j,
+                               child, kk, pp);
+            keyA[q] = ~kk;
+            payA[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)j;
+            kmin = umin32(kmin, ~kk);
+            kmax = umax32(kmax, ~kk);
+            if (kk == 0u) bad = true;
+        }
+        // within a child the entries must not increase
+        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+        uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+        int pchild = __shfl_up(child, 1, kWave);
+        if (lane == 0) {
+            pk = prev_key63;
+            ppos = prev_pos63;
+            pchild = prev_child63;
+        }
+        if (in && pchild == child && comes_before(kk, pp, pk, ppos)) bad = true;
+        prev_key63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+        prev_pos63 = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+        prev_child63 = __builtin_amdgcn_readlane(child, 63);
+    }
+    if (__ballot(bad) != 0ull) return false;
+    kmin = wave_min_u32(kmin);
+    kmax = wave_max_u32(kmax);
+
+    // ---- 4. stable radix sort by key (descending score), only over the bits that differ ----
+    const uint32_t diff = kmin ^ kmax;
+    const int nbits = diff == 0u ? 0 : 32 - __clz((int)diff);
+    uint32_t *srcK = keyA, *srcP = payA, *dstK = keyB, *dstP = payB;
+    for (int sh = 0; sh < nbits; sh += 8) {
+        wave_sync_memory();
+#pragma unroll
+        for (int t = 0; t < 4; t++) lds.hist[lane * 4 + t] = 0;
+        wave_sync_memory();
+        for (int q = lane; q < m; q += kWave) atomicAdd(&lds.hist[(srcK[q] >> sh) & 255u], 1);
+        wave_sync_memory();
+        int h0 = lds.hist[lane * 4 + 0], h1 = lds.hist[lane * 4 + 1], h2 = lds.hist[lane * 4 + 2],
+            h3 = lds.hist[lane * 4 + 3];
+        int lsum = h0 + h1 + h2 + h3;
+        int excl = wave_inclusive_sum(lsum, lane) - lsum;
+        wave_sync_memory();
+        lds.hist[lane * 4 + 0] = excl;
+        lds.hist[lane * 4 + 1] = excl + h0;
+        lds.hist[lane * 4 + 2] = excl + h0 + h1;
+        lds.hist[lane * 4 + 3] = excl + h0 + h1 + h2;
+        wave_sync_memory();
+        for (int base = 0; base < m; base += kWave) {
+            const int q = base + lane;
+            const bool in = q < m;
+            uint32_t kk = in ? srcK[q] : 0u;
+            uint32_t pay = in ? srcP[q] : 0u;
+            uint32_t d = (kk >> sh) & 255u;
+            // lanes of this chunk with the same digit
+            uint64_t same = __ballot(in);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                uint64_t bal = __ballot(in && ((d >> b) & 1u));
+                same &= ((d >> b) & 1u) ? bal : ~bal;
+            }
+            int rank = __popcll(same & ((1ull << lane) - 1ull));
+            int count = __popcll(same);
+            int basepos = in ? lds.hist[d] : 0;
+            if (in) {
+                dstK[basepos + rank] = kk;
+                dstP[basepos + rank] = pay;
+            }
+            wave_sync_memory();
+            if (in && rank == 0) lds.hist[d] = basepos + count;
+            wave_sync_memory();
+        }
+        uint32_t *tk = srcK;
+        srcK = dstK;
+        dstK = tk;
+        uint32_t *tp = srcP;
+        srcP = dstP;
+        dstP = tp;
+    }
+    wave_sync_memory();
+
+    // ---- 5. winner order: check ties across children and the last taken entry, emit ----
+    uint32_t pk63 = 0u, ppay63 = 0u;
+    bool have_prev = false;
+    for (int base = 0; base < m; base += kWave) {
+        const int q = base + lane;
+        const bool in = q < m;
+        uint32_t kk = in ? srcK[q] : 0u;
+        uint32_t pay = in ? srcP[q] : 0u;
+        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+        uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
+        bool hp = lane > 0 || have_prev;
+        if (lane == 0) {
+            pk = pk63;
+            ppay = ppay63;
+        }
+        if (in) {
+            const int child = (int)((pay >> 21) & 1023u);
+            const int j = (int)(pay & 0x1FFFFFu);
+            a.sc_child[off + q] = child;
+            a.sc_occ[off + q] = j;
+            if (hp) {
+                if (pk > kk) bad = true;  // not sorted
+                if (pk == kk) {
+                    const uint32_t pchild = (ppay >> 21) & 1023u;
+                    const uint32_t ppos_ = pchild + ((ppay >> 31) ? (uint32_t)F : 0u);
+                    const uint32_t pos_ = (uint32_t)child + ((pay >> 31) ? (uint32_t)F : 0u);
+                    if (pchild != (uint32_t)child && ppos_ > pos_) bad = true;
+                }
+            }
+        }
+        pk63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+        ppay63 = (uint32_t)__builtin_amdgcn_readlane((int)pay, 63);
+        have_prev = true;
+    }
+    {
+        // the last taken entry must come before every other child's first untaken entry
+        // (its own child's next entry was checked in step 3)
+        const uint32_t lk = ~srcK[m - 1];
+        const uint32_t lpay = srcP[m - 1];
+        const uint32_t lchild = (lpay >> 21) & 1023u;
+        const uint32_t lpos = lchild + ((lpay >> 31) ? (uint32_t)F : 0u);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (uk[r] != 0u && (uint32_t)(r * kWave + lane) != lchild && !comes_before(lk, lpos, uk[r], upos[r]))
+                bad = true;
+        }
+    }
+    if (__ballot(bad) != 0ull) return false;
+#pragma unroll
+    for (int r = 0; r < R; r++) cnt[r] = cv[r];
+    return true;
+}
+
+// The commonest crowded node: one child wins every time.  That is the case exactly when
+// the score it shows to the last visitor still comes before the first score of every
+// other child and its own scores never increase on the way; both are checked on the exact
+// values (m evaluations spread over the lanes).  Returns false when it is not that case.
+template <int R, bool RAVE>
+__device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
+                                           uint32_t bk, uint32_t bpos, int off, int m, int (&cnt)[R]) {
+    constexpr int F = R * kWave;
+    const uint32_t uvl = (uint32_t)a.vl;
+    uint32_t hi_key, hi_pos;
+    wave_best(bk, bpos, hi_key, hi_pos);
+    if (hi_key == 0u) return false;
+    const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
+    // statistics of the best child, wave-uniform
+    int tn = 0, tvl = 0, trn = 0;
+    float tw = 0.0f, tp = 0.0f, trw = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (r == (best >> 6)) {
+            tn = k.n[r];
+            tw = k.w[r];
+            tp = k.p[r];
+            tvl = k.vl[r];
+            trn = k.rn[r];
+            trw = k.rw[r];
+        }
+    }
+    const int bl = best & 63;
+    const int bn = __builtin_amdgcn_readlane(tn, bl);
+    const float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), bl));
+    const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), bl));
+    const int bvl = __builtin_amdgcn_readlane(tvl, bl);
+    const int brn = __builtin_amdgcn_readlane(trn, bl);
+    const float brw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(trw), bl));
+    // best first candidate of all other children
+    uint32_t ok = 0u, opos = 0xFFFFFFFFu;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (r * kWave + lane != best && k.k1[r] > ok) { ok = k.k1[r]; opos = (uint32_t)(r * kWave + lane); }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (r * kWave + lane != best && k.k2[r] > ok) { ok = k.k2[r]; opos = (uint32_t)(F + r * kWave + lane); }
+    }
+    uint32_t sk, spos;
+    wave_best(ok, opos, sk, spos);
+    // the last visitor's entry decides; then every entry is checked
+    uint32_t lk, lp;
+    entry_key<R, RAVE>(bn, bw, bp, bvl, brn, brw, c.ep, a.rave_k, uvl, m - 1, best, lk, lp);
+    if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) return false;
+    bool bad = false;
+    uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
+    for (int base = 0; base < m; base += kWave) {
+        const int j = base + lane;
+        uint32_t kk = 0u, pp = 0xFFFFFFFFu;
+        if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, brn, brw, c.ep, a.rave_k, uvl, j, best, kk, pp);
+        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+        uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+        if (lane == 0) {
+            pk = carry_k;
+            ppos = carry_p;
+        }
+        if (j < m && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad = true;
+        carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+        carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+    }
+    if (__ballot(bad) != 0ull) return false;
+    for (int j = lane; j < m; j += kWave) {
+        a.sc_child[off + j] = best;
+        a.sc_occ[off + j] = j;
+    }
+    if (lane == bl) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (r == (best >> 6)) cnt[r] = m;
+    }
+    return true;
+}
 
 // Where the walk goes on after a multi-visitor node whose visitors all chose one child.
 struct Continuation {
@@ -203,14 +656,15 @@ struct Continuation {
     int np;
 };
 
-// All visitors of a multi-visitor item, in order.  Records the chosen child of every
-// visitor, bumps virtual loss, partitions the visitors by child into seg_out, writes the
-// next path entry, appends one item per visited child to the next level's queue (none when
-// all visitors chose the same child: then the caller walks on with them).  Returns false when no child takes part in the selection.
+// All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
+// virtual loss, partitions the visitors by child into seg_out, writes the next path
+// entry, appends one item per visited child to the next level's queue (none when all
+// visitors chose the same child: then the caller walks on with them).  Returns false when
+// no child takes part in the selection.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              const int32_t *seg_in, int32_t *seg_out, int off, int m, int depth,
-                                             int *s_offs, Continuation &next) {
+                                             WaveLds<R> &lds, Continuation &next) {
     Kids<R, RAVE> k;
     int cnt[R];
     load_kids<R, RAVE>(f, c.cb, c.nelig, lane, k);
@@ -220,326 +674,60 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         cnt[r] = 0;
     }
     uint32_t bk, bpos;
-    lane_best<R, RAVE>(k, lane, 0u, bk, bpos);
-
-    Dominant dom;
-    dom.K = 0;
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        dom.child[g] = -1;
-        dom.n[g] = 0;
-        dom.w[g] = 0.0f;
-        dom.p[g] = 0.0f;
-        dom.vl[g] = 0;
-        dom.rn[g] = 0;
-        dom.rw[g] = 0.0f;
-        dom.cnt[g] = 0;
-        dom.stale[g] = 0;
-    }
-    uint32_t dmask = 0u;  // bit r: child r*64+lane is in the dominant set
-    int done = 0;
-    int backoff = 0;
-    int fails = 0;
-    int recent0 = -1, recent1 = -1;  // the last two children settled one at a time
-    int st_rounds = 0, st_settled = 0, st_single = 0, st_viol = 0, st_none = 0;
+    lane_best<R, RAVE>(k, lane, bk, bpos);
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
 
-    while (done < m) {
-        if (dom.K > 0 && backoff == 0 && m - done >= 4) {
-            // ---- look-ahead round ----
-            const int K = dom.K;
-            st_rounds++;
-            const int logE = K <= 1 ? 6 : (K == 2 ? 5 : 4);
-            const int E = 1 << logE;
-            const int g = lane >> logE;
-            const int o = lane & (E - 1);
-            const bool slot = g < K;
-            int sc = -1, sn = 0, svl = 0, srn = 0, scnt = 0;
-            float sw = 0.0f, sp = 0.0f, srw = 0.0f;
-#pragma unroll
-            for (int gg = 0; gg < 4; gg++) {
-                if (g == gg) {
-                    sc = dom.child[gg];
-                    sn = dom.n[gg];
-                    sw = dom.w[gg];
-                    sp = dom.p[gg];
-                    svl = dom.vl[gg];
-                    srn = dom.rn[gg];
-                    srw = dom.rw[gg];
-                    scnt = dom.cnt[gg];
+    bool settled = false;
+    int st_replay = 0;
+    if (m >= kRunMin && a.vl > 0) settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, cnt);
+    if (!settled && m >= kWaterLevelMin && a.vl > 0) {
+        settled = water_level<R, RAVE>(a, c, lane, k, bk, bpos, off, m, lds, cnt);
+        if (!settled) st_replay = 1;
+    }
+    if (!settled) {
+        // one visitor after the other
+        for (int done = 0; done < m; done++) {
+            int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
+            if (i < 0) return false;  // no child takes part: uniform, and then for every visitor
+            if (a.vl <= 0) {
+                // no virtual loss: nothing changes between visitors, they all follow the first
+                for (int j = lane; j < m; j += kWave) {
+                    a.sc_child[off + j] = i;
+                    a.sc_occ[off + j] = j;
                 }
-            }
-            uint32_t ek = 0u, epos = 0xFFFFFFFFu, ek1 = 0u, ek2 = 0u;
-            if (slot) {
-                int vlj = (int)((uint32_t)svl + (uint32_t)o * uvl);
-                child_keys<RAVE>(sn, sw, sp, vlj, srn, srw, c.ep, a.rave_k, ek1, ek2);
-                if (ek2 > ek1) {
-                    ek = ek2;
-                    epos = (uint32_t)(R * kWave + sc);
-                } else {
-                    ek = ek1;
-                    epos = (uint32_t)sc;
+                if (lane == (i & 63)) {
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                        if (r == (i >> 6)) cnt[r] = m;
                 }
-            }
-            // each list must not increase in the order (key descending, position ascending)
-            uint32_t pk = (uint32_t)__shfl_up((int)ek, 1, kWave);
-            uint32_t ppos = (uint32_t)__shfl_up((int)epos, 1, kWave);
-            bool viol = slot && o > 0 && ek != 0u && (pk == 0u || ek > pk || (ek == pk && epos < ppos));
-            bool ok = __ballot(viol) == 0ull;
-            if (!ok) st_viol++;
-            int settled = 0;
-            if (ok) {
-                // bound: best head of every other child, and the last evaluated entry of each list
-                uint32_t ck, cpos;
-                lane_best<R, RAVE>(k, lane, dmask, ck, cpos);
-                if (slot && o == E - 1 && ek != 0u && (ek > ck || (ek == ck && epos < cpos))) {
-                    ck = ek;
-                    cpos = epos;
-                }
-                uint32_t tk, tpos;
-                wave_best(ck, cpos, tk, tpos);
-                bool acc = slot && ek != 0u && (ek > tk || (ek == tk && epos < tpos));
-                uint64_t accm = __ballot(acc);
-                if (accm != 0ull) {
-                    // rank in the merged order: own offset + entries of the other lists that come first
-                    int rank = o;
-                    if (K > 1) {
-                        // binary searches in the other lists, advanced together so that their
-                        // cross-lane reads overlap
-                        int lo[4], hi[4];
-#pragma unroll
-                        for (int gg = 0; gg < 4; gg++) {
-                            lo[gg] = 0;
-                            hi[gg] = E;
-                        }
-                        for (int s = 0; s <= logE; s++) {
-                            uint32_t mk[4], mpos[4];
-#pragma unroll
-                            for (int gg = 0; gg < 4; gg++) {
-                                if (gg < K) {
-                                    int mid = (lo[gg] + hi[gg]) >> 1;
-                                    int src = (gg << logE) + (mid < E ? mid : E - 1);
-                                    mk[gg] = (uint32_t)__shfl((int)ek, src, kWave);
-                                    mpos[gg] = (uint32_t)__shfl((int)epos, src, kWave);
-                                }
-                            }
-#pragma unroll
-                            for (int gg = 0; gg < 4; gg++) {
-                                if (gg < K && lo[gg] < hi[gg]) {
-                                    int mid = (lo[gg] + hi[gg]) >> 1;
-                                    bool before = mk[gg] != 0u && (mk[gg] > ek || (mk[gg] == ek && mpos[gg] < epos));
-                                    if (before) lo[gg] = mid + 1;
-                                    else hi[gg] = mid;
-                                }
-                            }
-                        }
-#pragma unroll
-                        for (int gg = 0; gg < 4; gg++)
-                            if (gg < K && gg != g) rank += lo[gg];
-                    }
-                    const int remaining = m - done;
-                    const bool valid = acc && rank < remaining;
-                    if (valid) {
-                        a.sc_child[off + done + rank] = sc;
-                        a.sc_occ[off + done + rank] = scnt + o;
-                    }
-#pragma unroll
-                    for (int gg = 0; gg < 4; gg++) {
-                        if (gg < K) {
-                            int ag = __popcll(__ballot(valid && g == gg));
-                            if (ag > 0) {
-                                dom.stale[gg] = 0;
-                                dom.vl[gg] = (int)((uint32_t)dom.vl[gg] + (uint32_t)ag * uvl);
-                                dom.cnt[gg] += ag;
-                                int ch = dom.child[gg];
-                                // the new head of this child was looked ahead at offset ag
-                                // (the last entry of a list is never settled, so ag < E)
-                                const int hl = (gg << logE) + ag;
-                                uint32_t nk1 = (uint32_t)__builtin_amdgcn_readlane((int)ek1, hl);
-                                uint32_t nk2 = (uint32_t)__builtin_amdgcn_readlane((int)ek2, hl);
-                                if (lane == (ch & 63)) {
-#pragma unroll
-                                    for (int r = 0; r < R; r++) {
-                                        if (r == (ch >> 6)) {
-                                            cnt[r] += ag;
-                                            k.vl[r] = (int)((uint32_t)k.vl[r] + (uint32_t)ag * uvl);
-                                            k.k1[r] = nk1;
-                                            k.k2[r] = nk2;
-                                        }
-                                    }
-                                }
-                            } else {
-                                dom.stale[gg]++;
-                            }
-                        }
-                    }
-                    lane_best<R, RAVE>(k, lane, 0u, bk, bpos);
-                    int A = __popcll(accm);
-                    settled = A < remaining ? A : remaining;
-                    // lists that stopped winning leave the set (more look-ahead for the others):
-                    // the last list moves into the freed place
-#pragma unroll
-                    for (int gg = 3; gg >= 0; gg--) {
-                        if (gg < dom.K && dom.stale[gg] >= 2) {
-                            int ch = dom.child[gg];
-                            if (lane == (ch & 63)) dmask &= ~(1u << (ch >> 6));
-                            const int last = dom.K - 1;
-                            int mc = -1, mn = 0, mvl = 0, mrn = 0, mcnt = 0, mst = 0;
-                            float mw = 0.0f, mp = 0.0f, mrw = 0.0f;
-#pragma unroll
-                            for (int q = 0; q < 4; q++) {
-                                if (q == last) {
-                                    mc = dom.child[q];
-                                    mn = dom.n[q];
-                                    mw = dom.w[q];
-                                    mp = dom.p[q];
-                                    mvl = dom.vl[q];
-                                    mrn = dom.rn[q];
-                                    mrw = dom.rw[q];
-                                    mcnt = dom.cnt[q];
-                                    mst = dom.stale[q];
-                                }
-                            }
-                            dom.child[gg] = mc;
-                            dom.n[gg] = mn;
-                            dom.w[gg] = mw;
-                            dom.p[gg] = mp;
-                            dom.vl[gg] = mvl;
-                            dom.rn[gg] = mrn;
-                            dom.rw[gg] = mrw;
-                            dom.cnt[gg] = mcnt;
-                            dom.stale[gg] = mst;
-                            dom.K = last;
-                        }
-                    }
-                }
-            }
-            if (settled > 0) {
-                done += settled;
-                st_settled += settled;
-                fails = 0;
-                continue;
-            }
-            if (ok) st_none++;
-            fails = fails < 5 ? fails + 1 : 5;
-            backoff = 1 << fails;
-        }
-
-        // ---- one visitor ----
-        int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
-        if (i < 0) return false;  // no child takes part: uniform, and then for every visitor
-        st_single++;
-        int tn = 0, tvl = 0, trn = 0, tcnt = 0;
-        float tw = 0.0f, tp = 0.0f, trw = 0.0f;
-        if (lane == (i & 63)) {
-            int occ = 0;
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                if (r == (i >> 6)) {
-                    occ = cnt[r];
-                    cnt[r] = occ + 1;
-                    k.vl[r] = (int)((uint32_t)k.vl[r] + uvl);
-                    score_round<R, RAVE>(k, r, c.ep, a.rave_k);
-                    tn = k.n[r];
-                    tw = k.w[r];
-                    tp = k.p[r];
-                    tvl = k.vl[r];
-                    trn = k.rn[r];
-                    trw = k.rw[r];
-                    tcnt = cnt[r];
-                }
-            }
-            lane_best<R, RAVE>(k, lane, 0u, bk, bpos);
-            a.sc_child[off + done] = i;
-            a.sc_occ[off + done] = occ;
-        }
-        done++;
-        if (a.vl <= 0) {
-            // no virtual loss: nothing changes between visitors, they all follow the first
-            for (int j = done + lane; j < m; j += kWave) {
-                a.sc_child[off + j] = i;
-                a.sc_occ[off + j] = j;
+                break;
             }
             if (lane == (i & 63)) {
+                int occ = 0;
 #pragma unroll
-                for (int r = 0; r < R; r++)
-                    if (r == (i >> 6)) cnt[r] = m;
-            }
-            done = m;
-            break;
-        }
-        if (backoff > 0) backoff--;
-        // keep the dominant set current
-        int found = -1;
-#pragma unroll
-        for (int gg = 0; gg < 4; gg++)
-            if (gg < dom.K && dom.child[gg] == i) found = gg;
-        if (found >= 0) {
-#pragma unroll
-            for (int gg = 0; gg < 4; gg++) {
-                if (gg == found) {
-                    dom.vl[gg] = (int)((uint32_t)dom.vl[gg] + uvl);
-                    dom.cnt[gg] += 1;
-                    dom.stale[gg] = 0;
-                }
-            }
-        } else if (i == recent0 || i == recent1) {
-            int slot_g = dom.K;
-            if (dom.K >= 4) {
-                slot_g = 0;
-                int worst = dom.stale[0];
-#pragma unroll
-                for (int gg = 1; gg < 4; gg++) {
-                    if (dom.stale[gg] >= worst) {
-                        worst = dom.stale[gg];
-                        slot_g = gg;
+                for (int r = 0; r < R; r++) {
+                    if (r == (i >> 6)) {
+                        occ = cnt[r];
+                        cnt[r] = occ + 1;
+                        k.vl[r] = (int)((uint32_t)k.vl[r] + uvl);
+                        score_round<R, RAVE>(k, r, c.ep, a.rave_k);
                     }
                 }
-                int ev = -1;
-#pragma unroll
-                for (int gg = 0; gg < 4; gg++)
-                    if (gg == slot_g) ev = dom.child[gg];
-                if (lane == (ev & 63)) dmask &= ~(1u << (ev >> 6));
-            } else {
-                dom.K++;
+                lane_best<R, RAVE>(k, lane, bk, bpos);
+                a.sc_child[off + done] = i;
+                a.sc_occ[off + done] = occ;
             }
-            const int ol = i & 63;
-            int xn = __builtin_amdgcn_readlane(tn, ol);
-            float xw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), ol));
-            float xp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ol));
-            int xvl = __builtin_amdgcn_readlane(tvl, ol);
-            int xrn = __builtin_amdgcn_readlane(trn, ol);
-            float xrw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(trw), ol));
-            int xcnt = __builtin_amdgcn_readlane(tcnt, ol);
-#pragma unroll
-            for (int gg = 0; gg < 4; gg++) {
-                if (gg == slot_g) {
-                    dom.child[gg] = i;
-                    dom.n[gg] = xn;
-                    dom.w[gg] = xw;
-                    dom.p[gg] = xp;
-                    dom.vl[gg] = xvl;
-                    dom.rn[gg] = xrn;
-                    dom.rw[gg] = xrw;
-                    dom.cnt[gg] = xcnt;
-                    dom.stale[gg] = 0;
-                }
-            }
-            if (lane == ol) dmask |= 1u << (i >> 6);
         }
-        recent1 = recent0;
-        recent0 = i;
     }
-
     if (a.stats && lane == 0) {
         atomicAdd(a.stats + 0, 1);
-        atomicAdd(a.stats + 1, st_rounds);
-        atomicAdd(a.stats + 2, st_settled);
-        atomicAdd(a.stats + 3, st_single);
-        atomicAdd(a.stats + 4, st_viol);
-        atomicAdd(a.stats + 5, st_none);
+        atomicAdd(a.stats + 1, settled ? 1 : 0);
+        atomicAdd(a.stats + 2, settled ? m : 0);
+        atomicAdd(a.stats + 3, settled ? 0 : m);
+        atomicAdd(a.stats + 4, st_replay);
     }
-    // the child with most visitors (lowest index on ties) is where this wavefront walks on
+
+    // a group that stays together is walked on by this wavefront
     uint32_t lmax = 0u;
 #pragma unroll
     for (int r = 0; r < R; r++) lmax = umax32(lmax, (uint32_t)cnt[r]);
@@ -548,8 +736,6 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
 #pragma unroll
     for (int r = R - 1; r >= 0; r--)
         if ((uint32_t)cnt[r] == gmax) lidx = (uint32_t)(r * kWave + lane);
-    // walking on is only worth it when the group stays together: a split group is handed to
-    // the next level's launch whole, so that its parts are played side by side
     const int keep = gmax == (uint32_t)m ? (int)wave_min_u32(lidx) : -1;
 
     // exclusive prefix of the visit counts in child order -> segment of every child
@@ -560,7 +746,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         int inc = wave_inclusive_sum(cnt[r], lane);
         int excl = carry + inc - cnt[r];
         int i = r * kWave + lane;
-        s_offs[i] = excl;
+        lds.offs[i] = excl;
         if (i == keep) keep_np = k.n[r];
         uint64_t has = __ballot(cnt[r] > 0 && i != keep);
         int nnew = __popcll(has);
@@ -581,34 +767,29 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
         carry += __builtin_amdgcn_readlane(inc, 63);
     }
-    // make this wave's LDS and scratch writes visible to its own other lanes
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    wave_sync_memory();
     int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
     for (int j = lane; j < m; j += kWave) {
         int t = seg_in[off + j];
         int i = a.sc_child[off + j];
         path_next[t] = c.cb + i;
-        seg_out[off + s_offs[i] + a.sc_occ[off + j]] = t;
+        seg_out[off + lds.offs[i] + a.sc_occ[off + j]] = t;
     }
     next.node = -1;
     if (keep >= 0) {
         next.node = c.cb + keep;
-        next.off = off + s_offs[keep];
+        next.off = off + lds.offs[keep];
         next.m = (int)gmax;
         next.np = __builtin_amdgcn_readlane(keep_np, keep & 63);
     }
-    // the next step of the walk reads seg_out and reuses s_offs
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // the next step of the walk reads seg_out and reuses the LDS scratch
+    wave_sync_memory();
     return true;
 }
 
 template <int RMAX, bool RAVE>
 __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a, int level) {
-    __shared__ int s_offs_all[4][RMAX * kWave];
+    __shared__ WaveLds<RMAX> s_lds[4];
     const int lane = threadIdx.x & 63;
     const int wib = threadIdx.x >> 6;
     const int wave = blockIdx.x * 4 + wib;
@@ -623,19 +804,20 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
         for (int j = lane; j < m; j += kWave) a.paths[a.seg0[off + j]] = node;
     }
 
-    // walk with a group of visitors while there is more than one
+    // walk with a group of visitors while it stays together
     while (m > 1) {
         const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
         int32_t *seg_out = a.seg[depth & 1];
         NodeCtx c = node_ctx(f, a, node, np);
         bool descended = false;
         Continuation next;
+        next.node = -1;
         if (c.cc > 0 && depth < a.max_depth) {
-            int *s_offs = s_offs_all[wib];
             if (c.cc <= kWave)
-                descended = select_group<1, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_offs, next);
+                descended = select_group<1, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth,
+                                                  reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
             else
-                descended = select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_offs, next);
+                descended = select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_lds[wib], next);
         }
         if (!descended) {
             for (int j = lane; j < m; j += kWave) {

@@ -261,8 +261,8 @@ class Batch:
     def stats(self):
         out = np.zeros(8, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
-        keys = ("group_nodes", "lookahead_rounds", "settled_by_lookahead", "settled_one_by_one",
-                "rounds_scores_rose", "rounds_settled_nothing", "single_visitor_steps")
+        keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
+                "replayed_nodes", "unused5", "single_visitor_steps")
         return dict(zip(keys, map(int, out)))
 
     def device(self):
