@@ -150,12 +150,12 @@ int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_pat
 int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t *h_leaf, int32_t *h_actions);
 /* Traversals of the last select that stopped at max_depth on an expanded node. */
 int omk_batch_truncated(omk_batch *b, int32_t *h_count);
-/* How the last select did its work, 8 counters: [0] multi-visitor nodes processed,
- * [1] of these settled by the parallel water-level path, [2] visitors settled by it,
- * [3] visitors settled one at a time, [4] nodes replayed one visitor at a time because the
- * parallel path's exactness checks did not hold, [5] unused, [6] single-visitor selection
- * steps, [7] unused. */
-int omk_batch_stats(omk_batch *b, int32_t *h_stats8);
+/* How the last select did its work, 16 counters: [0] multi-visitor nodes processed,
+ * [1] of these settled by the parallel paths, [2] visitors settled by them, [3] visitors
+ * settled one at a time, [4] nodes replayed one visitor at a time because the parallel
+ * path's exactness checks did not hold, [5] threshold probes, [6] single-visitor selection
+ * steps, [7] unused, [8..15] per-phase cycle counts in measurement builds (else 0). */
+int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
 
 /* ---- transposition table: the lookup/store call sites of
  *      mcts_engine_batch_tree_simple.cpp:126,141 (PHMapTranspositionTable::store / lookup,

@@ -76,10 +76,10 @@ struct omk_batch {
     bool selected = false;  // paths of a select are on the device
     int32_t *paths = nullptr, *path_len = nullptr, *leaf = nullptr;
     float *values = nullptr;
-    Item *items0 = nullptr, *items_q = nullptr;
+    Item *items0 = nullptr, *items_q = nullptr, *singles0 = nullptr, *singles_q = nullptr;
+    int32_t n_singles0 = 0;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
-    int32_t *sort_buf[4] = {nullptr, nullptr, nullptr, nullptr};
     int32_t *counters = nullptr;  // [max_depth + 2] level counters, 1 truncated counter, 8 work statistics
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
@@ -320,14 +320,14 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->values, B);
     if (e == hipSuccess) e = dalloc(&b->items0, B);
     if (e == hipSuccess) e = dalloc(&b->items_q, B * (max_depth + 1));
+    if (e == hipSuccess) e = dalloc(&b->singles0, B);
+    if (e == hipSuccess) e = dalloc(&b->singles_q, B);
     if (e == hipSuccess) e = dalloc(&b->seg0, B);
     if (e == hipSuccess) e = dalloc(&b->seg[0], B);
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, B);
     if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
-    for (int i = 0; i < 4; i++)
-        if (e == hipSuccess) e = dalloc(&b->sort_buf[i], B);
-    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3 + 8);
+    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3 + 16 + 1);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
     if (e == hipSuccess) e = hipMemset(b->values, 0, (size_t)B * 4);
@@ -346,7 +346,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->sort_buf[0], b->sort_buf[1], b->sort_buf[2], b->sort_buf[3]};
+                    b->singles0, b->singles_q};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -369,23 +369,33 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
     std::vector<int32_t> order((size_t)n);
     for (int32_t t = 0; t < n; t++) order[(size_t)t] = t;
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t c) { return h_roots[a] < h_roots[c]; });
-    std::vector<Item> items;
+    std::vector<Item> items, singles;
     for (int32_t i = 0; i < n;) {
         int32_t j = i;
         while (j < n && h_roots[order[(size_t)j]] == h_roots[order[(size_t)i]]) j++;
         Item it;
         it.node = h_roots[order[(size_t)i]];
-        it.off = i;
-        it.m = j - i;
         it.np = 0;
-        items.push_back(it);
+        if (j - i > 1) {
+            it.off = i;
+            it.m = j - i;
+            items.push_back(it);
+        } else {
+            it.off = order[(size_t)i];  // the traversal itself
+            it.m = 0;                   // depth
+            singles.push_back(it);
+        }
         i = j;
     }
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     HIP_TRY(hipMemcpy(b->seg0, order.data(), (size_t)n * 4, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(b->items0, items.data(), items.size() * sizeof(Item), hipMemcpyHostToDevice));
+    if (!items.empty())
+        HIP_TRY(hipMemcpy(b->items0, items.data(), items.size() * sizeof(Item), hipMemcpyHostToDevice));
+    if (!singles.empty())
+        HIP_TRY(hipMemcpy(b->singles0, singles.data(), singles.size() * sizeof(Item), hipMemcpyHostToDevice));
     b->n_items0 = (int32_t)items.size();
+    b->n_singles0 = (int32_t)singles.size();
     b->n = n;
     b->selected = false;
     return OMK_OK;
@@ -433,12 +443,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.counters = b->counters;
     a.truncated = b->counters + b->max_depth + 2;
     a.stats = b->counters + b->max_depth + 3;
+    a.n_singles = b->counters + b->max_depth + 19;
+    a.singles0 = b->singles0;
+    a.singles_q = b->singles_q;
     a.sc_child = b->sc_child;
     a.sc_occ = b->sc_occ;
-    a.sort_key[0] = b->sort_buf[0];
-    a.sort_key[1] = b->sort_buf[1];
-    a.sort_pay[0] = b->sort_buf[2];
-    a.sort_pay[1] = b->sort_buf[3];
     a.paths = b->paths;
     a.path_len = b->path_len;
     a.leaf = b->leaf;
@@ -448,7 +457,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.pw = p->pw;
     a.c_puct = p->c_puct;
     a.rave_k = p->rave_k;
-    HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n, f->max_fanout, p->use_rave != 0, f->stream));
+    HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n_singles0, b->n, f->max_fanout, p->use_rave != 0, f->stream));
     b->selected = true;
     return OMK_OK;
 }
@@ -529,11 +538,12 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     return OMK_OK;
 }
 
-int omk_batch_stats(omk_batch *b, int32_t *h_stats8) {
+int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
+    int32_t *h_stats8 = h_stats16;
     if (!b || !h_stats8) return fail(OMK_ERR_INVALID, "omk_batch_stats: null argument");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_stats: no selected paths");
     if (int rc = use_device(b->f)) return rc;
-    HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + b->max_depth + 3, 32, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + b->max_depth + 3, 64, hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }

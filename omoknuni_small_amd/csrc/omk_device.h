@@ -64,14 +64,28 @@ __device__ __forceinline__ int wave_sum_i32(int x) {
     return (int)(a + b + c + d);
 }
 
-// Inclusive prefix sum over the 64 lanes (used once per multi-visitor node, not per pick).
-__device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        int o = __shfl_up(v, d, kWave);
-        if (lane >= d) v += o;
-    }
-    return v;
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov_zero(uint32_t v) {
+    // lanes whose source lane does not exist receive 0
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+
+// Inclusive prefix sum over the 64 lanes: log-step scan inside each row of 16 with row
+// shifts, then the totals of the rows below are added from the scalar unit.
+__device__ __forceinline__ int wave_inclusive_sum(int x, int lane) {
+    uint32_t v = (uint32_t)x;
+    v += dpp_mov_zero<0x111>(v);  // row_shr:1
+    v += dpp_mov_zero<0x112>(v);  // row_shr:2
+    v += dpp_mov_zero<0x114>(v);  // row_shr:4
+    v += dpp_mov_zero<0x118>(v);  // row_shr:8
+    uint32_t t0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 15);
+    uint32_t t1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 31);
+    uint32_t t2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 47);
+    const int row = lane >> 4;
+    uint32_t add = row >= 1 ? t0 : 0u;
+    add += row >= 2 ? t1 : 0u;
+    add += row >= 3 ? t2 : 0u;
+    return (int)(v + add);
 }
 
 __device__ __forceinline__ float wave_sum_f32(float v) {
@@ -103,27 +117,29 @@ __device__ __forceinline__ float combined_value(int visits, float w, int rave_vi
 
 // Keys of the two candidates a child contributes: its score in the first scan of
 // selectChild and its score in the second scan.  The second differs from the first only
-// through the RAVE blend or, without RAVE, when 1 + ev is not exact in binary32; a second
-// score equal to the first can never win (strict comparison, first scan comes first), so
-// it is reported as 0.
+// through the RAVE blend q2 (getCombinedValue: it does not depend on virtual loss, so the
+// caller computes it once per child) or, without RAVE, when 1 + ev is not exact in
+// binary32; a second score equal to the first can never win (strict comparison, first
+// scan comes first), so it is reported as 0.  While |ev| < 2^24 the divisors 1.0f + ev
+// (first scan) and float(1 + ev) (second scan) are the same number, so one division
+// serves both.
 template <bool RAVE>
-__device__ __forceinline__ void child_keys(int n, float w, float p, int vl, int rn, float rw, float ep,
-                                           float rave_k, uint32_t &k1, uint32_t &k2) {
+__device__ __forceinline__ void child_keys(int n, float w, float p, int vl, float q2, float ep, uint32_t &k1,
+                                           uint32_t &k2) {
     int ev = (int)((uint32_t)n + (uint32_t)vl);
     float evalue = w - (float)vl;
     float q = ev > 0 ? evalue / (float)ev : 0.0f;
     float prod = p * ep;
-    float s1 = q + prod / (1.0f + (float)ev);
-    k1 = score_key(s1);
+    float u1 = prod / (1.0f + (float)ev);
+    k1 = score_key(q + u1);
+    const bool exact = ev < (1 << 24) && ev > -(1 << 24);
     if (RAVE) {
-        float q2 = combined_value(n, w, rn, rw, rave_k);
-        int one_plus = (int)(1u + (uint32_t)ev);
-        float s2 = q2 + prod / (float)one_plus;
-        k2 = score_key(s2);
-    } else if (ev >= (1 << 24) || ev <= -(1 << 24)) {
-        int one_plus = (int)(1u + (uint32_t)ev);
-        float s2 = q + prod / (float)one_plus;
-        k2 = score_key(s2);
+        float u2 = u1;
+        if (!exact) u2 = prod / (float)(int)(1u + (uint32_t)ev);
+        k2 = score_key(q2 + u2);
+    } else if (!exact) {
+        float u2 = prod / (float)(int)(1u + (uint32_t)ev);
+        k2 = score_key(q + u2);
     } else {
         k2 = 0u;
     }

@@ -33,15 +33,16 @@ struct Item {
 };
 
 struct SelectArgs {
-    const Item *items0;    // level-0 items, built when the roots are set
+    const Item *items0;    // level-0 items with several visitors, built when the roots are set
     const int32_t *seg0;   // their visitor lists
+    const Item *singles0;  // traversals alone at their root: (node, traversal, depth 0, -)
+    Item *singles_q;       // single visitors: (node, traversal, depth, N of the node)
+    int32_t *n_singles;
     Item *items_q;         // queue of level L >= 1 at items_q + (L-1)*stride
     int32_t *counters;     // counters[L] = number of items of level L
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
     int32_t *sc_child;     // per visitor: chosen child index
     int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child
-    int32_t *sort_key[2];  // per visitor: ping-pong buffers of the winner-order sort
-    int32_t *sort_pay[2];
     int32_t *paths;        // level-major [max_depth+1][stride]
     int32_t *path_len;
     int32_t *leaf;
@@ -55,8 +56,8 @@ struct SelectArgs {
     float rave_k;
 };
 
-hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals, int max_fanout,
-                         bool rave, hipStream_t s);
+hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
+                         int max_fanout, bool rave, hipStream_t s);
 
 hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                            int max_len, int vl, hipStream_t s);

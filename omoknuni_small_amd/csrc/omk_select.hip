@@ -22,20 +22,50 @@
 //    batch depends on nothing but j.  If every child's scores do not increase with j, the
 //    serial winner sequence is the merge of these descending lists, i.e. the m best
 //    entries (i, j) in the order (score descending, candidate position ascending, j
-//    ascending).  A bisection on the score threshold finds how many entries each child
-//    contributes, all m entries are evaluated in parallel, a stable radix sort puts them
-//    in winner order.  Nothing is assumed: afterwards the wavefront checks, on the exact
-//    binary32 values, (i) that every child's taken entries and its first untaken entry do
-//    not increase and (ii) that the last taken entry still comes before every child's
-//    first untaken one.  Under (i) and (ii) the serial loop provably produces exactly
-//    this sequence; if either fails the node is replayed one visitor at a time.
+//    ascending).  In batches of up to 2048 entries: a bisection on the score threshold
+//    finds how many entries each child contributes, the entries are evaluated in parallel
+//    into LDS, a stable radix sort puts them in winner order.  Nothing is assumed:
+//    afterwards the wavefront checks, on the exact binary32 values, (i) that every child's
+//    taken entries and its first untaken entry do not increase and (ii) that the last
+//    taken entry still comes before every child's first untaken one.  Under (i) and (ii)
+//    the serial loop provably produces exactly this sequence; if either fails the node is
+//    replayed one visitor at a time.
+//
+// Two kernels: the multi-visitor kernel (LDS heavy, one launch per tree level) and the
+// single-visitor walk (no LDS, high occupancy, one launch): a visitor that is alone at a
+// node stays alone to its leaf, so it needs no level synchronisation at all.
+#include <algorithm>
+
 #include "omk_internal.h"
 
 namespace omk {
 
 constexpr int kRunMin = 4;                // visitors from which the one-winner check is tried
-constexpr int kWaterLevelMin = 32;        // visitors from which the parallel path is tried
+constexpr int kWaterLevelMin = 24;        // visitors from which the parallel path is tried
 constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in the sort payload
+constexpr int kBatchCap = 2048;           // entries put in winner order at a time (LDS resident)
+constexpr int kDigitBits = 10;            // radix digit of that sort
+constexpr int kBins = 1 << kDigitBits;
+constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
+
+// Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
+// multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
+#ifdef OMK_PHASE_TIMERS
+#define OMK_T0() long long t_phase_ = clock64()
+#define OMK_TICK(slot)                                                              \
+    do {                                                                            \
+        long long now_ = clock64();                                                 \
+        if (a.stats && lane == 0) atomicAdd(a.stats + (slot), (int)((now_ - t_phase_) >> 4)); \
+        t_phase_ = now_;                                                            \
+    } while (0)
+#else
+#define OMK_T0() \
+    do {         \
+    } while (0)
+#define OMK_TICK(slot) \
+    do {               \
+    } while (0)
+#endif
 
 // Register-resident statistics of the children a lane is responsible for: child index
 // i = r * 64 + lane for round r.
@@ -45,28 +75,31 @@ struct Kids {
     float w[R];
     float p[R];
     int vl[R];
-    int rn[R];
-    float rw[R];
+    float q2[R];  // RAVE blend of the child (second scan), constant during the selection
     uint32_t k1[R];
     uint32_t k2[R];
     bool part[R];
 };
 
-// Per-wavefront scratch in LDS.
+// Per-wavefront scratch in LDS of the multi-visitor kernel.
 template <int R>
 struct WaveLds {
     int offs[R * kWave];  // exclusive prefix of the visit counts in child order
-    int st_n[R * kWave];
+    int st_n[R * kWave];  // statistics of every child, readable by any lane
     float st_w[R * kWave];
     float st_p[R * kWave];
     int st_vl[R * kWave];
-    int st_rn[R * kWave];
-    float st_rw[R * kWave];
-    int hist[256];
+    float st_q2[R * kWave];
+    int st_j0[R * kWave];  // visits already settled / visit count, by phase
+    int hist[kBins];
+    uint32_t key[kBatchCap];  // entries of the batch being ordered
+    uint32_t pay[kBatchCap];
+    uint16_t idx[2][kBatchCap];
 };
 
 template <int R, bool RAVE>
-__device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig, int lane, Kids<R, RAVE> &k) {
+__device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
+                                          Kids<R, RAVE> &k) {
 #pragma unroll
     for (int r = 0; r < R; r++) {
         int i = r * kWave + lane;
@@ -78,20 +111,19 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
         k.w[r] = in ? f.W[id] : 0.0f;
         k.p[r] = in ? f.P[id] : 0.0f;
         k.vl[r] = in ? f.VL[id] : 0;
+        k.q2[r] = 0.0f;
         if (RAVE) {
-            k.rn[r] = in ? f.rN[id] : 0;
-            k.rw[r] = in ? f.rW[id] : 0.0f;
-        } else {
-            k.rn[r] = 0;
-            k.rw[r] = 0.0f;
+            int rn = in ? f.rN[id] : 0;
+            float rw = in ? f.rW[id] : 0.0f;
+            k.q2[r] = combined_value(k.n[r], k.w[r], rn, rw, rave_k);
         }
     }
 }
 
 template <int R, bool RAVE>
-__device__ __forceinline__ void score_round(Kids<R, RAVE> &k, int r, float ep, float rave_k) {
+__device__ __forceinline__ void score_round(Kids<R, RAVE> &k, int r, float ep) {
     uint32_t a = 0u, b = 0u;
-    if (k.part[r]) child_keys<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], ep, rave_k, a, b);
+    if (k.part[r]) child_keys<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], ep, a, b);
     k.k1[r] = a;
     k.k2[r] = b;
 }
@@ -181,9 +213,9 @@ template <int R, bool RAVE>
 __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              int &np_child) {
     Kids<R, RAVE> k;
-    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, k);
+    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, a.rave_k, k);
 #pragma unroll
-    for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep, a.rave_k);
+    for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep);
     uint32_t bk, bpos;
     lane_best<R, RAVE>(k, lane, bk, bpos);
     int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
@@ -197,14 +229,14 @@ __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArg
     return i;
 }
 
-// Key and candidate position child `child` shows to its j-th visitor of this batch.
+// Key and candidate position child `child` shows to the visitor that finds its counter at
+// vl0 + j * uvl.
 template <int R, bool RAVE>
-__device__ __forceinline__ void entry_key(int n, float w, float p, int vl0, int rn, float rw, float ep,
-                                          float rave_k, uint32_t uvl, int j, int child, uint32_t &key,
-                                          uint32_t &pos) {
+__device__ __forceinline__ void entry_key(int n, float w, float p, int vl0, float q2, float ep, uint32_t uvl, int j,
+                                          int child, uint32_t &key, uint32_t &pos) {
     int vlj = (int)((uint32_t)vl0 + (uint32_t)j * uvl);
     uint32_t k1, k2;
-    child_keys<RAVE>(n, w, p, vlj, rn, rw, ep, rave_k, k1, k2);
+    child_keys<RAVE>(n, w, p, vlj, q2, ep, k1, k2);
     if (k2 > k1) {
         key = k2;
         pos = (uint32_t)(R * kWave + child);
@@ -228,344 +260,438 @@ __device__ __forceinline__ void wave_sync_memory() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// The visitors of a crowded node, all at once (see the file header).  On success cnt[r]
+// The visitors of a crowded node in batches (see the file header).  On success cnt[r]
 // holds the visitors of every child and sc_child / sc_occ hold (child, visit number) of
-// every visitor; returns false, having changed nothing that matters, when the node has to
-// be replayed one visitor at a time.
+// every visitor; returns false when the node has to be replayed one visitor at a time
+// (the caller's statistics are untouched either way).
 template <int R, bool RAVE>
 __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
-                                            uint32_t bk, uint32_t bpos, int off, int m, WaveLds<R> &lds,
-                                            int (&cnt)[R]) {
+                                            int off, int m, WaveLds<R> &lds, int (&cnt)[R]) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     if (m > kWaterLevelMaxJ) return false;
 
-    // ---- 1. threshold T* = largest key with at least m entries at or above it ----
-    uint32_t hi_key, hi_pos;
-    wave_best(bk, bpos, hi_key, hi_pos);
-    if (hi_key == 0u) return false;
-    const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
-    // the best child alone has m entries at or above the key of its m-th visit
-    uint32_t lo_key = 0u;
-    {
-        uint32_t kk = 0u, pp = 0u;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            if (r == (best >> 6))
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, m - 1,
-                                   best, kk, pp);
-        }
-        lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
-    }
-    if (lo_key == 0u) lo_key = 1u;
-    if (lo_key > hi_key) return false;  // scores rose along the best child's list
-
-    int cl[R], ch[R];
-    uint32_t head[R];
+    int tk[R];                      // visits settled so far, per child
+    uint32_t headk[R], headp[R];    // the entry each child shows next
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        head[r] = umax32(k.k1[r], k.k2[r]);
-        cl[r] = 0;
-        ch[r] = head[r] != 0u ? m : 0;
-    }
-    // Invariant: count(lo) >= m > count(hi), cl = per-child counts at hi, ch = at lo.  After
-    // every probe the bracket end that moved is snapped to the nearest key that actually
-    // occurs, so the search ends after about log2(distinct keys in the bracket) probes.
-    uint32_t lo = lo_key, hi = hi_key + 1u;
-    bool first = true;
-    int probes = 0;
-    while (first || hi - lo > 1u) {
-        if (++probes > 80) return false;
-        const uint32_t T = first ? lo : lo + ((hi - lo) >> 1);
-        int ct[R];
-        int sum = 0;
-        uint32_t below = 0u;             // largest key below T among the first entries below T
-        uint32_t above = 0xFFFFFFFFu;    // smallest key at or above T among the last entries at or above T
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            int lo_c = cl[r], hi_c = ch[r];
-            if (head[r] < T) hi_c = 0;  // a list that starts below T has nothing above it
-            if (lo_c > hi_c) lo_c = hi_c;
-            uint32_t k_in = 0xFFFFFFFFu, k_out = 0u;  // keys seen at the boundary while searching
-            int j_in = -1, j_out = -1;
-            while (lo_c < hi_c) {
-                int t = (lo_c + hi_c + 1) >> 1;
-                uint32_t kk, pp;
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, t - 1,
-                                   r * kWave + lane, kk, pp);
-                if (kk >= T) {
-                    lo_c = t;
-                    k_in = kk;
-                    j_in = t - 1;
-                } else {
-                    hi_c = t - 1;
-                    k_out = kk;
-                    j_out = t - 1;
-                }
-            }
-            ct[r] = lo_c;
-            sum = sum + lo_c > m ? m : sum + lo_c;
-            if (head[r] != 0u) {
-                // last entry at or above T and first entry below T of this child
-                if (lo_c > 0) {
-                    if (j_in != lo_c - 1) {
-                        if (lo_c == 1) {
-                            k_in = head[r];
-                        } else {
-                            uint32_t pp;
-                            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
-                                               lo_c - 1, r * kWave + lane, k_in, pp);
-                        }
-                    }
-                    above = umin32(above, k_in);
-                }
-                if (lo_c < m) {
-                    if (j_out != lo_c) {
-                        if (lo_c == 0) {
-                            k_out = head[r];
-                        } else {
-                            uint32_t pp;
-                            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
-                                               lo_c, r * kWave + lane, k_out, pp);
-                        }
-                    }
-                    if (k_out < T) below = umax32(below, k_out);
-                }
-            }
-        }
-        const int total = wave_sum_i32(sum);  // at most 64 * m
-        if (first) {
-            if (total < m) return false;
-            first = false;
-        }
-        if (total >= m) {
-            uint32_t snap = wave_min_u32(above);
-            lo = (snap != 0xFFFFFFFFu && snap >= T && snap < hi) ? snap : T;
-#pragma unroll
-            for (int r = 0; r < R; r++) ch[r] = ct[r];
+        const int i = r * kWave + lane;
+        tk[r] = 0;
+        if (k.k2[r] > k.k1[r]) {
+            headk[r] = k.k2[r];
+            headp[r] = (uint32_t)(F + i);
         } else {
-            uint32_t snap = wave_max_u32(below);
-            hi = (snap + 1u > lo && snap < T) ? snap + 1u : T;
-#pragma unroll
-            for (int r = 0; r < R; r++) cl[r] = ct[r];
+            headk[r] = k.k1[r];
+            headp[r] = (uint32_t)i;
         }
-    }
-    // now cl = entries above T*, ch = entries at or above T*
-
-    // ---- 2. entries at exactly T* are handed out in child order until m is reached ----
-    int above = 0;
-#pragma unroll
-    for (int r = 0; r < R; r++) above = above + cl[r] > m ? m : above + cl[r];
-    int rem = m - wave_sum_i32(above);
-    if (rem < 0) return false;
-    int cv[R];
-    int carry = 0;
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        int e = ch[r] - cl[r];
-        if (e < 0) e = 0;
-        if (e > rem) e = rem;
-        int inc = wave_inclusive_sum(e, lane);
-        long long excl = (long long)carry + inc - e;
-        long long left = (long long)rem - excl;
-        int take = left <= 0 ? 0 : (left < e ? (int)left : e);
-        cv[r] = cl[r] + take;
-        int tot = __builtin_amdgcn_readlane(inc, 63);
-        carry = carry + tot > m ? m : carry + tot;
-    }
-    int csum = 0;
-#pragma unroll
-    for (int r = 0; r < R; r++) csum = csum + cv[r] > m + 1 ? m + 1 : csum + cv[r];
-    if (wave_sum_i32(csum) != m) return false;
-
-    // ---- 3. evaluate the m entries, in (child, visit) order; first untaken entries ----
-    carry = 0;
-    uint32_t uk[R], upos[R];  // first untaken entry of every child of this lane
-    bool bad = false;
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        int inc = wave_inclusive_sum(cv[r], lane);
-        int i = r * kWave + lane;
-        lds.offs[i] = carry + inc - cv[r];
         lds.st_n[i] = k.n[r];
         lds.st_w[i] = k.w[r];
         lds.st_p[i] = k.p[r];
-        lds.st_vl[i] = k.vl[r];
-        if (RAVE) {
-            lds.st_rn[i] = k.rn[r];
-            lds.st_rw[i] = k.rw[r];
+        lds.st_q2[i] = k.q2[r];
+    }
+
+    OMK_T0();
+    for (int done = 0; done < m;) {
+        const int need = m - done < kBatchCap ? m - done : kBatchCap;
+
+        // ---- 1. threshold T* = largest key with at least `need` unsettled entries at or above it ----
+        uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (headk[r] != 0u && comes_before(headk[r], headp[r], lbk, lbp)) {
+                lbk = headk[r];
+                lbp = headp[r];
+            }
+        uint32_t hi_key, hi_pos;
+        wave_best(lbk, lbp, hi_key, hi_pos);
+        if (hi_key == 0u) return false;
+        const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
+        // the best child alone has `need` entries at or above the key of its need-th next visit
+        uint32_t lo_key = 0u;
+        {
+            uint32_t kk = 0u, pp = 0u;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (r == (best >> 6))
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl,
+                                       tk[r] + need - 1, best, kk, pp);
+            }
+            lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
         }
-        carry += __builtin_amdgcn_readlane(inc, 63);
-        uk[r] = 0u;
-        upos[r] = 0xFFFFFFFFu;
-        if (k.part[r]) {
-            uint32_t kk, pp;
-            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl, cv[r], i, kk,
-                               pp);
-            uk[r] = kk;
-            upos[r] = pp;
-            if (cv[r] > 0) {
-                // the last taken entry of the child must not come after its first untaken one
-                uint32_t lk, lp;
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.rn[r], k.rw[r], c.ep, a.rave_k, uvl,
-                                   cv[r] - 1, i, lk, lp);
-                if (lk == 0u || comes_before(kk, pp, lk, lp)) bad = true;
+        if (lo_key == 0u) lo_key = 1u;
+        if (lo_key > hi_key) return false;  // scores rose along the best child's list
+
+        // Only children whose next entry reaches the lower bound can contribute to this batch.
+        // They are listed densely (one per lane and round) so that the probes below cost
+        // one evaluation round per 64 ACTIVE children instead of one per 64 children.
+        int n_act = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int i = r * kWave + lane;
+            const bool act = headk[r] != 0u && headk[r] >= lo_key;
+            const uint64_t am = __ballot(act);
+            if (act) lds.idx[1][n_act + __popcll(am & ((1ull << lane) - 1ull))] = (uint16_t)i;
+            n_act += __popcll(am);
+            lds.key[i] = headk[r];  // key of the child's next entry
+            lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
+            lds.pay[i] = 0u;        // result: entries above T*
+            lds.idx[0][i] = 0;      // result: entries at or above T*
+        }
+        wave_sync_memory();
+        const int rounds = (n_act + kWave - 1) / kWave;
+        // statistics of this lane's active children
+        int an[R], avl[R], ac[R];
+        float aw[R], ap[R], aq2[R];
+        uint32_t ahead[R];
+        int cl[R], ch[R];  // counts of the batch at hi / at lo, relative to the settled visits
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            ac[r] = -1;
+            an[r] = 0;
+            avl[r] = 0;
+            aw[r] = ap[r] = aq2[r] = 0.0f;
+            ahead[r] = 0u;
+            cl[r] = ch[r] = 0;
+            if (r < rounds && r * kWave + lane < n_act) {
+                const int ci = (int)lds.idx[1][r * kWave + lane];
+                ac[r] = ci;
+                an[r] = lds.st_n[ci];
+                aw[r] = lds.st_w[ci];
+                ap[r] = lds.st_p[ci];
+                avl[r] = lds.st_vl[ci];
+                aq2[r] = lds.st_q2[ci];
+                ahead[r] = lds.key[ci];
+                ch[r] = need;
             }
         }
-    }
-    wave_sync_memory();
-
-    uint32_t *keyA = (uint32_t *)a.sort_key[0] + off, *keyB = (uint32_t *)a.sort_key[1] + off;
-    uint32_t *payA = (uint32_t *)a.sort_pay[0] + off, *payB = (uint32_t *)a.sort_pay[1] + off;
-    uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
-    uint32_t prev_key63 = 0u, prev_pos63 = 0u;
-    int prev_child63 = -1;
-    for (int base = 0; base < m; base += kWave) {
-        const int q = base + lane;
-        const bool in = q < m;
-        int child = -1;
-        uint32_t kk = 0u, pp = 0u;
-        if (in) {
-            // last child whose segment starts at or before q
-            int lo_i = 0, hi_i = F;
-            while (hi_i - lo_i > 1) {
-                int mid = (lo_i + hi_i) >> 1;
-                if (lds.offs[mid] <= q) lo_i = mid;
-                else hi_i = mid;
+        // Invariant: count(lo) >= need > count(hi), cl = per-child counts at hi, ch = at lo.
+        // After every probe the bracket end that moved is snapped to the nearest key that
+        // actually occurs, so the search ends after about log2(distinct keys in it) probes.
+        uint32_t lo = lo_key, hi = hi_key + 1u;
+        bool first = true;
+        int probes = 0;
+        while (first || hi - lo > 1u) {
+            if (++probes > 80) return false;
+            const uint32_t T = first ? lo : lo + ((hi - lo) >> 1);
+            int ct[R];
+            int sum = 0;
+            uint32_t below = 0u;           // largest key below T among the first entries below T
+            uint32_t above = 0xFFFFFFFFu;  // smallest key among the last entries at or above T
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                ct[r] = 0;
+                if (r < rounds) {
+                    int lo_c = cl[r], hi_c = ch[r];
+                    if (ahead[r] < T) hi_c = 0;  // a list that starts below T has nothing above it
+                    if (lo_c > hi_c) lo_c = hi_c;
+                    uint32_t k_in = 0xFFFFFFFFu, k_out = 0u;  // keys seen at the boundary while searching
+                    int j_in = -1, j_out = -1;
+                    while (lo_c < hi_c) {
+                        int t = (lo_c + hi_c + 1) >> 1;
+                        uint32_t kk, pp;
+                        entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, t - 1, ac[r], kk, pp);
+                        if (kk >= T) {
+                            lo_c = t;
+                            k_in = kk;
+                            j_in = t - 1;
+                        } else {
+                            hi_c = t - 1;
+                            k_out = kk;
+                            j_out = t - 1;
+                        }
+                    }
+                    ct[r] = lo_c;
+                    sum += lo_c;
+                    if (ac[r] >= 0) {
+                        // last entry at or above T and first entry below T of this child
+                        if (lo_c > 0) {
+                            if (j_in != lo_c - 1) {
+                                if (lo_c == 1) {
+                                    k_in = ahead[r];
+                                } else {
+                                    uint32_t pp;
+                                    entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, lo_c - 1, ac[r],
+                                                       k_in, pp);
+                                }
+                            }
+                            above = umin32(above, k_in);
+                        }
+                        if (lo_c < need) {
+                            if (j_out != lo_c) {
+                                if (lo_c == 0) {
+                                    k_out = ahead[r];
+                                } else {
+                                    uint32_t pp;
+                                    entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, lo_c, ac[r], k_out,
+                                                       pp);
+                                }
+                            }
+                            if (k_out < T) below = umax32(below, k_out);
+                        }
+                    }
+                }
             }
-            child = lo_i;
-            const int j = q - lds.offs[child];
-            entry_key<R, RAVE>(lds.st_n[child], lds.st_w[child], lds.st_p[child], lds.st_vl[child],
-                               RAVE ? lds.st_rn[child] : 0, RAVE ? lds.st_rw[child] : 0.0f, c.ep, a.rave_k, uvl, j,
-                               child, kk, pp);
-            keyA[q] = ~kk;
-            payA[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)j;
-            kmin = umin32(kmin, ~kk);
-            kmax = umax32(kmax, ~kk);
-            if (kk == 0u) bad = true;
+            const int total = wave_sum_i32(sum);  // at most 64 * R * need
+            if (first) {
+                if (total < need) return false;
+                first = false;
+            }
+            if (total >= need) {
+                uint32_t snap = wave_min_u32(above);
+                lo = (snap != 0xFFFFFFFFu && snap >= T && snap < hi) ? snap : T;
+#pragma unroll
+                for (int r = 0; r < R; r++) ch[r] = ct[r];
+            } else {
+                uint32_t snap = wave_max_u32(below);
+                hi = (snap + 1u > lo && snap < T) ? snap + 1u : T;
+#pragma unroll
+                for (int r = 0; r < R; r++) cl[r] = ct[r];
+            }
         }
-        // within a child the entries must not increase
-        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-        uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
-        int pchild = __shfl_up(child, 1, kWave);
-        if (lane == 0) {
-            pk = prev_key63;
-            ppos = prev_pos63;
-            pchild = prev_child63;
+        // hand the counts back to the lanes that own the children
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (ac[r] >= 0) {
+                lds.pay[ac[r]] = (uint32_t)cl[r];
+                lds.idx[0][ac[r]] = (uint16_t)ch[r];
+            }
         }
-        if (in && pchild == child && comes_before(kk, pp, pk, ppos)) bad = true;
-        prev_key63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-        prev_pos63 = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
-        prev_child63 = __builtin_amdgcn_readlane(child, 63);
-    }
-    if (__ballot(bad) != 0ull) return false;
-    kmin = wave_min_u32(kmin);
-    kmax = wave_max_u32(kmax);
-
-    // ---- 4. stable radix sort by key (descending score), only over the bits that differ ----
-    const uint32_t diff = kmin ^ kmax;
-    const int nbits = diff == 0u ? 0 : 32 - __clz((int)diff);
-    uint32_t *srcK = keyA, *srcP = payA, *dstK = keyB, *dstP = payB;
-    for (int sh = 0; sh < nbits; sh += 8) {
         wave_sync_memory();
 #pragma unroll
-        for (int t = 0; t < 4; t++) lds.hist[lane * 4 + t] = 0;
-        wave_sync_memory();
-        for (int q = lane; q < m; q += kWave) atomicAdd(&lds.hist[(srcK[q] >> sh) & 255u], 1);
-        wave_sync_memory();
-        int h0 = lds.hist[lane * 4 + 0], h1 = lds.hist[lane * 4 + 1], h2 = lds.hist[lane * 4 + 2],
-            h3 = lds.hist[lane * 4 + 3];
-        int lsum = h0 + h1 + h2 + h3;
-        int excl = wave_inclusive_sum(lsum, lane) - lsum;
-        wave_sync_memory();
-        lds.hist[lane * 4 + 0] = excl;
-        lds.hist[lane * 4 + 1] = excl + h0;
-        lds.hist[lane * 4 + 2] = excl + h0 + h1;
-        lds.hist[lane * 4 + 3] = excl + h0 + h1 + h2;
-        wave_sync_memory();
-        for (int base = 0; base < m; base += kWave) {
-            const int q = base + lane;
-            const bool in = q < m;
-            uint32_t kk = in ? srcK[q] : 0u;
-            uint32_t pay = in ? srcP[q] : 0u;
-            uint32_t d = (kk >> sh) & 255u;
-            // lanes of this chunk with the same digit
-            uint64_t same = __ballot(in);
-#pragma unroll
-            for (int b = 0; b < 8; b++) {
-                uint64_t bal = __ballot(in && ((d >> b) & 1u));
-                same &= ((d >> b) & 1u) ? bal : ~bal;
-            }
-            int rank = __popcll(same & ((1ull << lane) - 1ull));
-            int count = __popcll(same);
-            int basepos = in ? lds.hist[d] : 0;
-            if (in) {
-                dstK[basepos + rank] = kk;
-                dstP[basepos + rank] = pay;
-            }
-            wave_sync_memory();
-            if (in && rank == 0) lds.hist[d] = basepos + count;
-            wave_sync_memory();
+        for (int r = 0; r < R; r++) {
+            const int i = r * kWave + lane;
+            cl[r] = tk[r] + (int)lds.pay[i];
+            ch[r] = tk[r] + (int)lds.idx[0][i];
         }
-        uint32_t *tk = srcK;
-        srcK = dstK;
-        dstK = tk;
-        uint32_t *tp = srcP;
-        srcP = dstP;
-        dstP = tp;
-    }
-    wave_sync_memory();
+        wave_sync_memory();
+        // now cl = settled + entries above T*, ch = settled + entries at or above T*
+        OMK_TICK(8);
+        if (a.stats && lane == 0) atomicAdd(a.stats + 5, probes);
 
-    // ---- 5. winner order: check ties across children and the last taken entry, emit ----
-    uint32_t pk63 = 0u, ppay63 = 0u;
-    bool have_prev = false;
-    for (int base = 0; base < m; base += kWave) {
-        const int q = base + lane;
-        const bool in = q < m;
-        uint32_t kk = in ? srcK[q] : 0u;
-        uint32_t pay = in ? srcP[q] : 0u;
-        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-        uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
-        bool hp = lane > 0 || have_prev;
-        if (lane == 0) {
-            pk = pk63;
-            ppay = ppay63;
+        // ---- 2. entries at exactly T* are handed out in child order until `need` is reached ----
+        int above_n = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) above_n += cl[r] - tk[r];
+        const int rem = need - wave_sum_i32(above_n);
+        if (rem < 0) return false;
+        int cv[R];
+        int carry = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int e = ch[r] - cl[r];
+            if (e < 0) e = 0;
+            if (e > rem) e = rem;
+            int inc = wave_inclusive_sum(e, lane);
+            int excl = carry + inc - e;
+            int left = rem - excl;
+            int take = left <= 0 ? 0 : (left < e ? left : e);
+            cv[r] = cl[r] + take;
+            carry += __builtin_amdgcn_readlane(inc, 63);
         }
-        if (in) {
-            const int child = (int)((pay >> 21) & 1023u);
-            const int j = (int)(pay & 0x1FFFFFu);
-            a.sc_child[off + q] = child;
-            a.sc_occ[off + q] = j;
-            if (hp) {
-                if (pk > kk) bad = true;  // not sorted
-                if (pk == kk) {
-                    const uint32_t pchild = (ppay >> 21) & 1023u;
-                    const uint32_t ppos_ = pchild + ((ppay >> 31) ? (uint32_t)F : 0u);
-                    const uint32_t pos_ = (uint32_t)child + ((pay >> 31) ? (uint32_t)F : 0u);
-                    if (pchild != (uint32_t)child && ppos_ > pos_) bad = true;
+        int csum = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) csum += cv[r] - tk[r];
+        if (wave_sum_i32(csum) != need) return false;
+
+        // ---- 3. evaluate the batch in (child, visit) order; first untaken entries ----
+        carry = 0;
+        uint32_t uk[R], upos[R];  // first untaken entry of every child of this lane
+        bool bad = false;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int nr = cv[r] - tk[r];
+            int inc = wave_inclusive_sum(nr, lane);
+            int i = r * kWave + lane;
+            lds.offs[i] = carry + inc - nr;
+            lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
+            lds.st_j0[i] = tk[r];
+            carry += __builtin_amdgcn_readlane(inc, 63);
+            uk[r] = 0u;
+            upos[r] = 0xFFFFFFFFu;
+            if (k.part[r]) {
+                if (nr == 0) {
+                    uk[r] = headk[r];
+                    upos[r] = headp[r];
+                } else {
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, cv[r], i,
+                                       uk[r], upos[r]);
+                    // the last taken entry of the child must not come after its first untaken one
+                    uint32_t lk, lp;
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl,
+                                       cv[r] - 1, i, lk, lp);
+                    if (lk == 0u || comes_before(uk[r], upos[r], lk, lp)) bad = true;
                 }
             }
         }
-        pk63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-        ppay63 = (uint32_t)__builtin_amdgcn_readlane((int)pay, 63);
-        have_prev = true;
-    }
-    {
-        // the last taken entry must come before every other child's first untaken entry
-        // (its own child's next entry was checked in step 3)
-        const uint32_t lk = ~srcK[m - 1];
-        const uint32_t lpay = srcP[m - 1];
-        const uint32_t lchild = (lpay >> 21) & 1023u;
-        const uint32_t lpos = lchild + ((lpay >> 31) ? (uint32_t)F : 0u);
+        wave_sync_memory();
+
+        uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
+        uint32_t prev_key63 = 0u, prev_pos63 = 0u;
+        int prev_child63 = -1;
+        for (int base = 0; base < need; base += kWave) {
+            const int q = base + lane;
+            const bool in = q < need;
+            int child = -1;
+            uint32_t kk = 0u, pp = 0u;
+            if (in) {
+                // last child whose segment starts at or before q
+                int lo_i = 0, hi_i = F;
+                while (hi_i - lo_i > 1) {
+                    int mid = (lo_i + hi_i) >> 1;
+                    if (lds.offs[mid] <= q) lo_i = mid;
+                    else hi_i = mid;
+                }
+                child = lo_i;
+                const int jl = q - lds.offs[child];
+                entry_key<R, RAVE>(lds.st_n[child], lds.st_w[child], lds.st_p[child], lds.st_vl[child],
+                                   lds.st_q2[child], c.ep, uvl, jl, child, kk, pp);
+                lds.key[q] = ~kk;
+                lds.pay[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) |
+                             (uint32_t)(lds.st_j0[child] + jl);
+                kmin = umin32(kmin, ~kk);
+                kmax = umax32(kmax, ~kk);
+                if (kk == 0u) bad = true;
+            }
+            // within a child the entries must not increase
+            uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+            uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+            int pchild = __shfl_up(child, 1, kWave);
+            if (lane == 0) {
+                pk = prev_key63;
+                ppos = prev_pos63;
+                pchild = prev_child63;
+            }
+            if (in && pchild == child && comes_before(kk, pp, pk, ppos)) bad = true;
+            prev_key63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+            prev_pos63 = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+            prev_child63 = __builtin_amdgcn_readlane(child, 63);
+        }
+        if (__ballot(bad) != 0ull) return false;
+        kmin = wave_min_u32(kmin);
+        kmax = wave_max_u32(kmax);
+        OMK_TICK(9);
+
+        // ---- 4. stable radix sort of the batch by key, over the bits that differ, in LDS ----
+        const uint32_t diff = kmin ^ kmax;
+        const int nbits = diff == 0u ? 0 : 32 - __clz((int)diff);
+        int cur = -1;  // -1: identity order, else lds.idx[cur]
+        for (int sh = 0; sh < nbits; sh += kDigitBits) {
+            wave_sync_memory();
+#pragma unroll
+            for (int t = 0; t < kBins / kWave; t++) lds.hist[t * kWave + lane] = 0;
+            wave_sync_memory();
+            for (int q = lane; q < need; q += kWave) {
+                const int i = cur < 0 ? q : (int)lds.idx[cur][q];
+                atomicAdd(&lds.hist[(lds.key[i] >> sh) & (uint32_t)(kBins - 1)], 1);
+            }
+            wave_sync_memory();
+            {
+                // exclusive scan of the bins: lane owns bins [16*lane, 16*lane+16)
+                int h[kBins / kWave];
+                int lsum = 0;
+#pragma unroll
+                for (int t = 0; t < kBins / kWave; t++) {
+                    h[t] = lds.hist[lane * (kBins / kWave) + t];
+                    lsum += h[t];
+                }
+                int run = wave_inclusive_sum(lsum, lane) - lsum;
+                wave_sync_memory();
+#pragma unroll
+                for (int t = 0; t < kBins / kWave; t++) {
+                    lds.hist[lane * (kBins / kWave) + t] = run;
+                    run += h[t];
+                }
+            }
+            wave_sync_memory();
+            const int nxt = cur == 0 ? 1 : 0;
+            for (int base = 0; base < need; base += kWave) {
+                const int q = base + lane;
+                const bool in = q < need;
+                const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
+                const uint32_t d = in ? (lds.key[i] >> sh) & (uint32_t)(kBins - 1) : 0u;
+                // lanes of this chunk with the same digit
+                uint64_t same = __ballot(in);
+#pragma unroll
+                for (int b = 0; b < kDigitBits; b++) {
+                    uint64_t bal = __ballot(in && ((d >> b) & 1u));
+                    same &= ((d >> b) & 1u) ? bal : ~bal;
+                }
+                const int rank = __popcll(same & ((1ull << lane) - 1ull));
+                const int count = __popcll(same);
+                const int basepos = in ? lds.hist[d] : 0;
+                if (in) lds.idx[nxt][basepos + rank] = (uint16_t)i;
+                wave_sync_memory();
+                if (in && rank == 0) lds.hist[d] = basepos + count;
+                wave_sync_memory();
+            }
+            cur = nxt;
+        }
+        wave_sync_memory();
+
+        OMK_TICK(10);
+        // ---- 5. winner order of the batch: check ties across children, emit ----
+        uint32_t pk63 = 0u, ppay63 = 0u;
+        bool have_prev = false;
+        for (int base = 0; base < need; base += kWave) {
+            const int q = base + lane;
+            const bool in = q < need;
+            const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
+            uint32_t kk = in ? lds.key[i] : 0u;
+            uint32_t pay = in ? lds.pay[i] : 0u;
+            uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+            uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
+            bool hp = lane > 0 || have_prev;
+            if (lane == 0) {
+                pk = pk63;
+                ppay = ppay63;
+            }
+            if (in) {
+                const int child = (int)((pay >> 21) & 1023u);
+                const int j = (int)(pay & 0x1FFFFFu);
+                a.sc_child[off + done + q] = child;
+                a.sc_occ[off + done + q] = j;
+                if (hp) {
+                    if (pk > kk) bad = true;  // not sorted
+                    if (pk == kk) {
+                        const uint32_t pchild = (ppay >> 21) & 1023u;
+                        const uint32_t ppos_ = pchild + ((ppay >> 31) ? (uint32_t)F : 0u);
+                        const uint32_t pos_ = (uint32_t)child + ((pay >> 31) ? (uint32_t)F : 0u);
+                        if (pchild != (uint32_t)child && ppos_ > pos_) bad = true;
+                    }
+                }
+            }
+            pk63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+            ppay63 = (uint32_t)__builtin_amdgcn_readlane((int)pay, 63);
+            have_prev = true;
+        }
+        {
+            // the last taken entry must come before every other child's first untaken entry
+            // (its own child's next entry was checked in step 3)
+            const int il = cur < 0 ? need - 1 : (int)lds.idx[cur][need - 1];
+            const uint32_t lk = ~lds.key[il];
+            const uint32_t lpay = lds.pay[il];
+            const uint32_t lchild = (lpay >> 21) & 1023u;
+            const uint32_t lpos = lchild + ((lpay >> 31) ? (uint32_t)F : 0u);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (uk[r] != 0u && (uint32_t)(r * kWave + lane) != lchild &&
+                    !comes_before(lk, lpos, uk[r], upos[r]))
+                    bad = true;
+            }
+        }
+        if (__ballot(bad) != 0ull) return false;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if (uk[r] != 0u && (uint32_t)(r * kWave + lane) != lchild && !comes_before(lk, lpos, uk[r], upos[r]))
-                bad = true;
+            tk[r] = cv[r];
+            headk[r] = uk[r];
+            headp[r] = upos[r];
         }
+        done += need;
+        wave_sync_memory();
+        OMK_TICK(11);
     }
-    if (__ballot(bad) != 0ull) return false;
 #pragma unroll
-    for (int r = 0; r < R; r++) cnt[r] = cv[r];
+    for (int r = 0; r < R; r++) cnt[r] = tk[r];
     return true;
 }
 
@@ -583,8 +709,8 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
     if (hi_key == 0u) return false;
     const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
     // statistics of the best child, wave-uniform
-    int tn = 0, tvl = 0, trn = 0;
-    float tw = 0.0f, tp = 0.0f, trw = 0.0f;
+    int tn = 0, tvl = 0;
+    float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         if (r == (best >> 6)) {
@@ -592,8 +718,7 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
             tw = k.w[r];
             tp = k.p[r];
             tvl = k.vl[r];
-            trn = k.rn[r];
-            trw = k.rw[r];
+            tq2 = k.q2[r];
         }
     }
     const int bl = best & 63;
@@ -601,8 +726,7 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
     const float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), bl));
     const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), bl));
     const int bvl = __builtin_amdgcn_readlane(tvl, bl);
-    const int brn = __builtin_amdgcn_readlane(trn, bl);
-    const float brw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(trw), bl));
+    const float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), bl));
     // best first candidate of all other children
     uint32_t ok = 0u, opos = 0xFFFFFFFFu;
 #pragma unroll
@@ -617,14 +741,14 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
     wave_best(ok, opos, sk, spos);
     // the last visitor's entry decides; then every entry is checked
     uint32_t lk, lp;
-    entry_key<R, RAVE>(bn, bw, bp, bvl, brn, brw, c.ep, a.rave_k, uvl, m - 1, best, lk, lp);
+    entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, m - 1, best, lk, lp);
     if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) return false;
     bool bad = false;
     uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
     for (int base = 0; base < m; base += kWave) {
         const int j = base + lane;
         uint32_t kk = 0u, pp = 0xFFFFFFFFu;
-        if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, brn, brw, c.ep, a.rave_k, uvl, j, best, kk, pp);
+        if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, j, best, kk, pp);
         uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
         uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
         if (lane == 0) {
@@ -658,30 +782,33 @@ struct Continuation {
 
 // All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
 // virtual loss, partitions the visitors by child into seg_out, writes the next path
-// entry, appends one item per visited child to the next level's queue (none when all
-// visitors chose the same child: then the caller walks on with them).  Returns false when
-// no child takes part in the selection.
+// entry; children with several visitors become items of the next level's queue, children
+// with one visitor go to the single-visitor queue (none when all visitors chose the same
+// child: then the caller walks on with them).  Returns false when no child takes part in
+// the selection.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              const int32_t *seg_in, int32_t *seg_out, int off, int m, int depth,
                                              WaveLds<R> &lds, Continuation &next) {
+    OMK_T0();
     Kids<R, RAVE> k;
     int cnt[R];
-    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, k);
+    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, a.rave_k, k);
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        score_round<R, RAVE>(k, r, c.ep, a.rave_k);
+        score_round<R, RAVE>(k, r, c.ep);
         cnt[r] = 0;
     }
     uint32_t bk, bpos;
     lane_best<R, RAVE>(k, lane, bk, bpos);
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
+    OMK_TICK(12);
 
     bool settled = false;
     int st_replay = 0;
     if (m >= kRunMin && a.vl > 0) settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, cnt);
     if (!settled && m >= kWaterLevelMin && a.vl > 0) {
-        settled = water_level<R, RAVE>(a, c, lane, k, bk, bpos, off, m, lds, cnt);
+        settled = water_level<R, RAVE>(a, c, lane, k, off, m, lds, cnt);
         if (!settled) st_replay = 1;
     }
     if (!settled) {
@@ -710,7 +837,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                         occ = cnt[r];
                         cnt[r] = occ + 1;
                         k.vl[r] = (int)((uint32_t)k.vl[r] + uvl);
-                        score_round<R, RAVE>(k, r, c.ep, a.rave_k);
+                        score_round<R, RAVE>(k, r, c.ep);
                     }
                 }
                 lane_best<R, RAVE>(k, lane, bk, bpos);
@@ -719,6 +846,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             }
         }
     }
+    OMK_TICK(13);
     if (a.stats && lane == 0) {
         atomicAdd(a.stats + 0, 1);
         atomicAdd(a.stats + 1, settled ? 1 : 0);
@@ -747,14 +875,16 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         int excl = carry + inc - cnt[r];
         int i = r * kWave + lane;
         lds.offs[i] = excl;
+        lds.st_j0[i] = cnt[r];
+        lds.st_n[i] = k.n[r];
         if (i == keep) keep_np = k.n[r];
-        uint64_t has = __ballot(cnt[r] > 0 && i != keep);
+        uint64_t has = __ballot(cnt[r] > 1 && i != keep);
         int nnew = __popcll(has);
         if (nnew > 0) {
             int slot0 = 0;
             if (lane == 0) slot0 = atomicAdd(a.counters + depth + 1, nnew);
             slot0 = __builtin_amdgcn_readfirstlane(slot0);
-            if (cnt[r] > 0 && i != keep) {
+            if (cnt[r] > 1 && i != keep) {
                 int slot = slot0 + __popcll(has & ((1ull << lane) - 1ull));
                 Item it;
                 it.node = c.cb + i;
@@ -769,11 +899,33 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     }
     wave_sync_memory();
     int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
-    for (int j = lane; j < m; j += kWave) {
-        int t = seg_in[off + j];
-        int i = a.sc_child[off + j];
-        path_next[t] = c.cb + i;
-        seg_out[off + lds.offs[i] + a.sc_occ[off + j]] = t;
+    for (int base = 0; base < m; base += kWave) {
+        const int j = base + lane;
+        const bool in = j < m;
+        int t = 0, i = 0;
+        bool lone = false;
+        if (in) {
+            t = seg_in[off + j];
+            i = a.sc_child[off + j];
+            path_next[t] = c.cb + i;
+            seg_out[off + lds.offs[i] + a.sc_occ[off + j]] = t;
+            lone = lds.st_j0[i] == 1;
+        }
+        // a visitor that is now alone goes to the single-visitor walk
+        uint64_t lm = __ballot(lone);
+        if (lm != 0ull) {
+            int s0 = 0;
+            if (lane == 0) s0 = atomicAdd(a.n_singles, __popcll(lm));
+            s0 = __builtin_amdgcn_readfirstlane(s0);
+            if (lone) {
+                Item it;
+                it.node = c.cb + i;
+                it.off = t;
+                it.m = depth + 1;
+                it.np = lds.st_n[i];
+                a.singles_q[s0 + __popcll(lm & ((1ull << lane) - 1ull))] = it;
+            }
+        }
     }
     next.node = -1;
     if (keep >= 0) {
@@ -784,15 +936,17 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     }
     // the next step of the walk reads seg_out and reuses the LDS scratch
     wave_sync_memory();
+    OMK_TICK(14);
     return true;
 }
 
+// Multi-visitor items of one tree level; a group that stays together is walked on.
 template <int RMAX, bool RAVE>
-__global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a, int level) {
-    __shared__ WaveLds<RMAX> s_lds[4];
+__global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev f, SelectArgs a, int level) {
+    __shared__ WaveLds<RMAX> s_lds[kGroupWaves];
     const int lane = threadIdx.x & 63;
     const int wib = threadIdx.x >> 6;
-    const int wave = blockIdx.x * 4 + wib;
+    const int wave = blockIdx.x * kGroupWaves + wib;
     if (wave >= a.counters[level]) return;
     const Item it = level == 0 ? a.items0[wave] : a.items_q[(size_t)(level - 1) * a.stride + wave];
     int node = it.node;
@@ -803,9 +957,7 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
     if (level == 0) {
         for (int j = lane; j < m; j += kWave) a.paths[a.seg0[off + j]] = node;
     }
-
-    // walk with a group of visitors while it stays together
-    while (m > 1) {
+    for (;;) {
         const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
         int32_t *seg_out = a.seg[depth & 1];
         NodeCtx c = node_ctx(f, a, node, np);
@@ -835,11 +987,23 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
         np = next.np;
         depth++;
     }
+}
 
-    // single visitor: the rest of the path is private to it
-    const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
-    const int t = seg_in[off];
-    int d = depth;
+// Single visitors: the rest of the path is private to the visitor, one wavefront walks it.
+template <int RMAX, bool RAVE>
+__global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave >= *a.n_singles) return;
+    const Item it = a.singles_q[wave];
+    int node = it.node;
+    const int t = it.off;
+    int d = it.m;
+    int np = it.np;
+    if (d == 0) {
+        np = f.N[node];
+        if (lane == 0) a.paths[t] = node;
+    }
     for (;;) {
         NodeCtx c = node_ctx(f, a, node, np);
         int i = -1;
@@ -868,27 +1032,40 @@ __global__ __launch_bounds__(256) void k_select_level(ForestDev f, SelectArgs a,
     }
 }
 
-__global__ void k_select_reset(int *counters, int n_counters, int n_items0, int *truncated, int *stats) {
+// Level counters, statistics, and the single-visitor queue seeded with the traversals
+// that are alone at their root.
+__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n_counters) counters[i] = (i == 0) ? n_items0 : 0;
-    if (i == 0) *truncated = 0;
-    if (stats && i < 8) stats[i] = 0;
+    if (i < a.max_depth + 2) a.counters[i] = (i == 0) ? n_items0 : 0;
+    if (i == 0) {
+        *a.truncated = 0;
+        *a.n_singles = n_singles0;
+    }
+    if (a.stats && i < 16) a.stats[i] = 0;
+    if (i < n_singles0) a.singles_q[i] = a.singles0[i];
 }
 
 template <int RMAX, bool RAVE>
-static hipError_t launch_levels(const ForestDev &f, const SelectArgs &a, int n_traversals, hipStream_t s) {
-    const int grid = (n_traversals + 3) / 4;
-    for (int level = 0; level <= a.max_depth; level++)
-        hipLaunchKernelGGL((k_select_level<RMAX, RAVE>), dim3(grid), dim3(256), 0, s, f, a, level);
+static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals,
+                                 hipStream_t s) {
+    if (n_items0 > 0) {
+        // an item has at least two visitors
+        const int grid = (n_traversals / 2 + kGroupWaves - 1) / kGroupWaves;
+        for (int level = 0; level <= a.max_depth; level++)
+            hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid > 0 ? grid : 1), dim3(kGroupWaves * kWave), 0,
+                               s, f, a, level);
+    }
+    hipLaunchKernelGGL((k_select_singles<RMAX, RAVE>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
     return hipGetLastError();
 }
 
-hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals, int max_fanout,
-                         bool rave, hipStream_t s) {
-    hipLaunchKernelGGL(k_select_reset, dim3((a.max_depth + 2 + 63) / 64), dim3(64), 0, s, a.counters,
-                       a.max_depth + 2, n_items0, a.truncated, a.stats);
-#define OMK_DISPATCH(RM) \
-    return rave ? launch_levels<RM, true>(f, a, n_traversals, s) : launch_levels<RM, false>(f, a, n_traversals, s)
+hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
+                         int max_fanout, bool rave, hipStream_t s) {
+    const int n_reset = std::max(std::max(a.max_depth + 2, 8), n_singles0);
+    hipLaunchKernelGGL(k_select_reset, dim3((n_reset + 255) / 256), dim3(256), 0, s, a, n_items0, n_singles0);
+#define OMK_DISPATCH(RM)                                                           \
+    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, s)        \
+                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, s)
     if (max_fanout <= 64) { OMK_DISPATCH(1); }
     if (max_fanout <= 256) { OMK_DISPATCH(4); }
     if (max_fanout <= 384) { OMK_DISPATCH(6); }

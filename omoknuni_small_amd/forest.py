@@ -259,10 +259,11 @@ class Batch:
         return c.value
 
     def stats(self):
-        out = np.zeros(8, np.int32)
+        out = np.zeros(16, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
-                "replayed_nodes", "unused5", "single_visitor_steps")
+                "replayed_nodes", "threshold_probes", "single_visitor_steps", "unused7", "cyc_threshold",
+                "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "unused15")
         return dict(zip(keys, map(int, out)))
 
     def device(self):
