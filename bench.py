@@ -104,6 +104,9 @@ def main():
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--scale", type=float, default=1.0, help="scale nodes_per_tree (debugging only)")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="only run the plain copy kernel over this many MiB, 10 times (to scale profiler "
+                         "traffic counters by) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (independent trees would shard by tree id with no "
@@ -112,6 +115,17 @@ def main():
 
     import omoknuni_small_amd as omk
     from omoknuni_small_amd import synth
+
+    if args.copy_calibration > 0:
+        nbytes = args.copy_calibration << 20
+        f = omk.Forest(16)
+        src, dst = f.dev_alloc(nbytes), f.dev_alloc(nbytes)
+        f.h2d(src, np.zeros(nbytes // 4, np.uint32))
+        for _ in range(10):
+            f.dev_copy(dst, src, nbytes)
+        f.sync()
+        print(json.dumps({"copy_calibration_bytes_each_way": nbytes, "launches": 10}))
+        return
 
     kw = {}
     if args.scale != 1.0:
@@ -174,6 +188,16 @@ def main():
     sel_ms = sum(ev.elapsed_ms(e_sel0[i], e_sel1[i]) for i in range(K))
     bak_ms = sum(ev.elapsed_ms(e_sel1[i], e_end[i]) for i in range(K))
 
+    # outside the timed region: three plain copies of 64 MiB, the known-size kernel that a
+    # profiler run of this command scales its traffic counters by
+    cal_bytes = 64 << 20
+    d_src, d_dst = forest.dev_alloc(cal_bytes), forest.dev_alloc(cal_bytes)
+    for _ in range(3):
+        forest.dev_copy(d_dst, d_src, cal_bytes)
+    forest.sync()
+    forest.dev_free(d_src)
+    forest.dev_free(d_dst)
+
     # the byte model is evaluated on the paths of one more (untimed) step
     batch.select(params)
     paths, plen, leaf, _ = batch.read()
@@ -181,10 +205,22 @@ def main():
     batch.backup(vl)
     forest.sync()
     sel_bytes, bak_bytes, n_sel_steps = algorithmic_bytes(soa, meta, paths, plen, N_now)
-    launches_per_select = D + 2  # one reset + one launch per level
+    # selection = 1 reset + (D+1) launches of the multi-visitor kernel (when any traversals share a
+    # root) + 1 launch of the single-visitor kernel; the roofline is quoted per launch of the kernel
+    # that carries the work, with the whole selection phase as its time
+    has_groups = len(np.unique(troots)) < B
+    dominant = "k_select_groups" if has_groups else "k_select_singles"
+    launches_per_select = (D + 1) if has_groups else 1
     sel_ms_step = sel_ms / K
     bak_ms_step = bak_ms / K
     achieved = sel_bytes / (sel_ms_step * 1e-3) / 1e9
+    traffic = None
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tfile):
+        with open(tfile) as fh:
+            tj = json.load(fh)
+        if args.workload in tj and args.scale == 1.0:
+            traffic = tj[args.workload].get("selection_bytes_per_launch")
 
     out = {
         "metric": "PUCT traversals/s (selection with virtual loss + value backup per step)",
@@ -217,12 +253,12 @@ def main():
         "wall_ms_per_step": wall_s * 1e3 / K,
         "roofline": {
             "bound": "hbm",
-            "kernel": "k_select_level",
+            "kernel": dominant,
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": traffic,
             "algorithmic_bytes_per_step": sel_bytes,
             "launches_per_step": launches_per_select,
             "avg_launch_us": sel_ms_step * 1e3 / launches_per_select,

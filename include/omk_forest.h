@@ -183,6 +183,9 @@ int omk_dev_alloc(omk_forest *f, int64_t bytes, void **d_out);
 int omk_dev_free(omk_forest *f, void *d_ptr);
 int omk_dev_h2d(omk_forest *f, void *d_dst, const void *h_src, int64_t bytes);
 int omk_dev_d2h(omk_forest *f, void *h_dst, const void *d_src, int64_t bytes);
+/* Device-to-device copy by a plain kernel (bytes a multiple of 4), asynchronous.  It moves
+ * exactly `bytes` in and `bytes` out, which is what profiler traffic counters are scaled by. */
+int omk_dev_copy(omk_forest *f, void *d_dst, const void *d_src, int64_t bytes);
 
 #ifdef __cplusplus
 }

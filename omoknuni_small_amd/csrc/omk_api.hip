@@ -656,6 +656,13 @@ int omk_dev_free(omk_forest *f, void *d_ptr) {
     return OMK_OK;
 }
 
+int omk_dev_copy(omk_forest *f, void *d_dst, const void *d_src, int64_t bytes) {
+    if (!f || !d_dst || !d_src || bytes < 0 || (bytes & 3)) return fail(OMK_ERR_INVALID, "omk_dev_copy: bad argument");
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(launch_copy_words(d_dst, d_src, bytes / 4, f->stream));
+    return OMK_OK;
+}
+
 int omk_dev_h2d(omk_forest *f, void *d_dst, const void *h_src, int64_t bytes) {
     if (!f || !d_dst || !h_src || bytes < 0) return fail(OMK_ERR_INVALID, "omk_dev_h2d: bad argument");
     if (int rc = use_device(f)) return rc;

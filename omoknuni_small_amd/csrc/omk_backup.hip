@@ -117,6 +117,22 @@ __global__ __launch_bounds__(256) void k_export(ForestDev f, const int32_t *path
     }
 }
 
+// plain copy of 4-byte words: the known-size kernel that hardware traffic counters are scaled by
+__global__ __launch_bounds__(256) void k_copy_words(uint32_t *dst, const uint32_t *src, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for (; i < n; i += step) dst[i] = src[i];
+}
+
+hipError_t launch_copy_words(void *dst, const void *src, int64_t n_words, hipStream_t s) {
+    if (n_words <= 0) return hipSuccess;
+    int64_t blocks = (n_words + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(k_copy_words, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t *)dst, (const uint32_t *)src,
+                       n_words);
+    return hipGetLastError();
+}
+
 hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                            int max_len, int vl, hipStream_t s) {
     if (vl <= 0 || n <= 0 || max_len <= 1) return hipSuccess;

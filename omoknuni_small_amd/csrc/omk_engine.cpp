@@ -1,0 +1,102 @@
+// See omk_engine.h.  Plain host C++: links against libomk_forest.so, includes no HIP header.
+#include "omk_engine.h"
+
+#include <algorithm>
+
+namespace omk {
+
+ForestEngine::ForestEngine(InferenceFunction inference_fn, const MCTSSettings &settings, int64_t capacity_nodes,
+                           int device, bool has_rave)
+    : inference_fn_(std::move(inference_fn)), settings_(settings), has_rave_(has_rave) {
+    omk_forest_desc desc;
+    desc.capacity_nodes = capacity_nodes;
+    desc.device = device;
+    desc.has_rave = has_rave ? 1 : 0;
+    check(omk_forest_create(&desc, &forest_), "omk_forest_create");
+}
+
+ForestEngine::~ForestEngine() {
+    if (batch_) omk_batch_destroy(batch_);
+    if (forest_) omk_forest_destroy(forest_);
+}
+
+void ForestEngine::check(int status, const char *what) const {
+    if (status != OMK_OK) throw std::runtime_error(std::string(what) + ": " + omk_last_error());
+}
+
+void ForestEngine::uploadTree(const omk_soa_view &view) { check(omk_forest_upload(forest_, &view), "omk_forest_upload"); }
+
+void ForestEngine::downloadStatistics(omk_soa_view &view) {
+    check(omk_forest_download(forest_, &view), "omk_forest_download");
+}
+
+void ForestEngine::ensureBatch(int n) {
+    if (batch_ && n <= batch_capacity_) return;
+    if (batch_) {
+        omk_batch_destroy(batch_);
+        batch_ = nullptr;
+    }
+    batch_capacity_ = std::max(n, settings_.batch_size);
+    check(omk_batch_create(forest_, batch_capacity_, settings_.max_depth, &batch_), "omk_batch_create");
+}
+
+void ForestEngine::selectLeafBatch(int32_t root, int batch_size, std::vector<LeafItem> &leaves) {
+    h_roots_.assign((size_t)batch_size, root);
+    selectLeafBatch(h_roots_, leaves);
+}
+
+void ForestEngine::selectLeafBatch(const std::vector<int32_t> &roots, std::vector<LeafItem> &leaves) {
+    const int n = (int)roots.size();
+    if (n <= 0) throw std::runtime_error("selectLeafBatch: empty batch");
+    ensureBatch(n);
+    check(omk_batch_set_roots(batch_, roots.data(), n), "omk_batch_set_roots");
+    omk_select_params p;
+    p.c_puct = settings_.exploration_constant;
+    p.virtual_loss = settings_.virtual_loss;
+    p.use_rave = (settings_.use_rave && has_rave_) ? 1 : 0;
+    p.rave_k = settings_.rave_constant;
+    p.pw = settings_.use_progressive_widening ? 1 : 0;
+    check(omk_select_batch(batch_, &p), "omk_select_batch");
+    const int D = settings_.max_depth;
+    h_paths_.resize((size_t)n * (D + 1));
+    h_len_.resize((size_t)n);
+    h_leaf_.resize((size_t)n);
+    h_actions_.resize((size_t)n * D);
+    check(omk_batch_read(batch_, h_paths_.data(), h_len_.data(), h_leaf_.data(), h_actions_.data()), "omk_batch_read");
+    leaves.clear();
+    leaves.resize((size_t)n);
+    for (int i = 0; i < n; i++) {
+        LeafItem &it = leaves[(size_t)i];
+        const int len = h_len_[(size_t)i];
+        it.node = h_leaf_[(size_t)i];
+        it.path.assign(h_paths_.begin() + (size_t)i * (D + 1), h_paths_.begin() + (size_t)i * (D + 1) + len);
+        it.move_sequence.assign(h_actions_.begin() + (size_t)i * D, h_actions_.begin() + (size_t)i * D + (len - 1));
+    }
+    last_n_ = n;
+}
+
+void ForestEngine::backPropagateBatch(const std::vector<float> &leaf_values) {
+    if ((int)leaf_values.size() != last_n_) throw std::runtime_error("backPropagateBatch: one value per selected leaf");
+    check(omk_batch_set_values(batch_, leaf_values.data(), last_n_), "omk_batch_set_values");
+    check(omk_backup_batch(batch_, settings_.virtual_loss), "omk_backup_batch");
+}
+
+int ForestEngine::executeBatchedTreeSearch(int32_t root) {
+    int completed = 0;
+    std::vector<LeafItem> leaves;
+    std::vector<float> values;
+    while (completed < settings_.num_simulations) {
+        const int n = std::min(settings_.batch_size, settings_.num_simulations - completed);
+        selectLeafBatch(root, n, leaves);
+        std::vector<NetworkOutput> out = inference_fn_(leaves);
+        if (out.size() != leaves.size()) throw std::runtime_error("inference function returned a short batch");
+        values.resize(out.size());
+        for (size_t i = 0; i < out.size(); i++) values[i] = out[i].value;
+        backPropagateBatch(values);
+        completed += n;
+    }
+    check(omk_sync(forest_), "omk_sync");
+    return completed;
+}
+
+}  // namespace omk

@@ -1,0 +1,92 @@
+// Host-side C++ adapter above the C ABI (include/omk_forest.h): the leaf-selection and
+// batch-collection interface of the reference's MCTSEngine for the device-resident forest.
+//
+// It mirrors, phase by phase, MCTSEngine::executeBatchedTreeSearch
+// (reference src/mcts/mcts_engine_batch_tree_simple.cpp:14-301):
+//   selectLeafBatch      phase 1 (:73-185) + leaf gather (:166-206): one LeafItem per simulation
+//   InferenceFunction    phase 2 (:212-236): the evaluator, called once per batch
+//   backPropagateBatch   phase 3 (:276-281): update + revertVirtualLoss, sign flipped per ply
+// The reference hands the evaluator cloned game states; here a LeafItem carries the leaf
+// node and the move list to replay on a clone of the root state (what :170-178 does), so
+// game rules stay on the host, untouched.
+//
+// Errors of the C ABI surface as std::runtime_error carrying omk_last_error(), which is what
+// MCTSEngine::search logs and rethrows (reference src/mcts/mcts_engine_main.cpp:343-355).
+#pragma once
+
+#include <cstdint>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/omk_forest.h"
+
+namespace omk {
+
+// reference include/mcts/evaluation_types.h:14-17
+struct NetworkOutput {
+    std::vector<float> policy;
+    float value = 0.0f;
+};
+
+// The fields of MCTSSettings this path reads (reference include/mcts/mcts_engine.h:55-120).
+struct MCTSSettings {
+    int num_simulations = 800;
+    int batch_size = 256;
+    float exploration_constant = 1.4f;
+    int virtual_loss = 3;
+    bool use_rave = true;
+    float rave_constant = 3000.0f;
+    bool use_progressive_widening = false;  // selection-time eligibility filter, see omk_select_params::pw
+    int max_depth = 64;                     // longest path the batch buffers hold
+};
+
+// What PendingEvaluation{node, state, path} (reference include/mcts/evaluation_types.h:49-73)
+// becomes when the tree lives on the device.
+struct LeafItem {
+    int32_t node = -1;                  // the leaf
+    std::vector<int32_t> path;          // root .. leaf node ids
+    std::vector<int32_t> move_sequence; // actions to replay on a clone of the root state
+};
+
+using InferenceFunction = std::function<std::vector<NetworkOutput>(const std::vector<LeafItem> &)>;
+
+class ForestEngine {
+   public:
+    ForestEngine(InferenceFunction inference_fn, const MCTSSettings &settings, int64_t capacity_nodes, int device = 0,
+                 bool has_rave = false);
+    ~ForestEngine();
+    ForestEngine(const ForestEngine &) = delete;
+    ForestEngine &operator=(const ForestEngine &) = delete;
+
+    void uploadTree(const omk_soa_view &view);
+    void downloadStatistics(omk_soa_view &view);
+
+    // One batch: every simulation starts at `root` (reference :86-92).
+    void selectLeafBatch(int32_t root, int batch_size, std::vector<LeafItem> &leaves);
+    // Simulation i starts at roots[i]: independent trees searched side by side.
+    void selectLeafBatch(const std::vector<int32_t> &roots, std::vector<LeafItem> &leaves);
+    void backPropagateBatch(const std::vector<float> &leaf_values);
+
+    // The whole loop of executeBatchedTreeSearch without the expansion step: batches of
+    // settings.batch_size until num_simulations are done.  Returns simulations run.
+    int executeBatchedTreeSearch(int32_t root);
+
+    const MCTSSettings &settings() const { return settings_; }
+
+   private:
+    void check(int status, const char *what) const;
+    void ensureBatch(int n);
+
+    InferenceFunction inference_fn_;
+    MCTSSettings settings_;
+    omk_forest *forest_ = nullptr;
+    omk_batch *batch_ = nullptr;
+    int batch_capacity_ = 0;
+    int last_n_ = 0;
+    bool has_rave_ = false;
+    std::vector<int32_t> h_paths_, h_len_, h_leaf_, h_actions_, h_roots_;
+};
+
+}  // namespace omk

@@ -69,6 +69,8 @@ hipError_t launch_backup(const ForestDev &f, const int32_t *paths, const int32_t
 hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                          int max_depth, int32_t *out_paths, int32_t *out_actions, hipStream_t s);
 
+hipError_t launch_copy_words(void *dst, const void *src, int64_t n_words, hipStream_t s);
+
 struct TTSlot {
     unsigned long long key;
     int32_t node;

@@ -11,8 +11,9 @@
 // reached it, in traversal-index order); ONE 64-lane wavefront owns the item and loads the
 // children once (coalesced, one child per lane per round).  The visitors are then
 // partitioned by chosen child (stable, so still in traversal order) into the work items
-// of the next level's launch; a group that stays together (every visitor chose the same
-// child) and a lone visitor are walked on by the same wavefront.
+// of the next level's launch; the wavefront walks on itself with a group that stays together
+// (or, for small groups, with a part that holds at least three quarters of it), and lone
+// visitors go to the single-visitor walk.
 //
 // Which child each visitor chooses:
 //  * few visitors: they are played one after another on register-resident statistics --
@@ -47,10 +48,16 @@ constexpr int kBatchCap = 2048;           // entries put in winner order at a ti
 constexpr int kDigitBits = 10;            // radix digit of that sort
 constexpr int kBins = 1 << kDigitBits;
 constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
+constexpr int kWalkOnSmall = 32;          // groups up to this size walk on with their dominant part
 
 // Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
 // multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
 #ifdef OMK_PHASE_TIMERS
+#define OMK_FAIL(code)                                                      \
+    do {                                                                    \
+        if (a.stats && lane == 0) atomicExch(a.stats + 7, (code));          \
+        return false;                                                       \
+    } while (0)
 #define OMK_T0() long long t_phase_ = clock64()
 #define OMK_TICK(slot)                                                              \
     do {                                                                            \
@@ -59,6 +66,7 @@ constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-v
         t_phase_ = now_;                                                            \
     } while (0)
 #else
+#define OMK_FAIL(code) return false
 #define OMK_T0() \
     do {         \
     } while (0)
@@ -93,7 +101,8 @@ struct WaveLds {
     int st_j0[R * kWave];  // visits already settled / visit count, by phase
     int hist[kBins];
     uint32_t key[kBatchCap];  // entries of the batch being ordered
-    uint32_t pay[kBatchCap];
+    uint32_t pay[kBatchCap];   // per child: entries of the batch
+    uint32_t pay2[kBatchCap];  // per entry: pass flag, child, visit number
     uint16_t idx[2][kBatchCap];
 };
 
@@ -260,19 +269,61 @@ __device__ __forceinline__ void wave_sync_memory() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Inverse of score_key for real keys: the score a key stands for.
+__device__ __forceinline__ float key_score(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
+}
+
+// ESTIMATE of how many of a child's next entries score at least tau, from the closed form
+// of the score as a function of x = N + VL:  s1(x) = (W+N)/x - 1 + c/(1+x)  (c = P * ep) and,
+// with RAVE, s2(x) = q2 + c/(1+x).  Fast approximate arithmetic on purpose: the result only
+// seeds the exact search, which tests the two entries around it.
+template <bool RAVE>
+__device__ __forceinline__ int predict_count(int n, float w, float p, int vl, float q2, float ep, uint32_t uvl,
+                                             float tau, int cap) {
+    const float x0 = (float)n + (float)vl;
+    const float A = w + (float)n;
+    const float cc = p * ep;
+    const float inv_step = __frcp_rn((float)uvl);
+    float xs = -1.0f;  // largest x with score >= tau
+    const float a2 = tau + 1.0f;
+    if (a2 > 1e-12f) {
+        const float b2 = a2 - A - cc;
+        const float disc = b2 * b2 + 4.0f * a2 * A;
+        if (disc >= 0.0f) xs = (-b2 + __fsqrt_rn(disc)) * __frcp_rn(2.0f * a2);
+    } else {
+        xs = 3.0e38f;
+    }
+    if (RAVE) {
+        const float d = tau - q2;
+        float x2 = d > 1e-12f ? cc * __frcp_rn(d) - 1.0f : 3.0e38f;
+        xs = fmaxf(xs, x2);
+    }
+    float cnt = floorf((xs - x0) * inv_step) + 1.0f;
+    if (!(cnt > 0.0f)) return 0;
+    return cnt >= (float)cap ? cap : (int)cnt;
+}
+
 // The visitors of a crowded node in batches (see the file header).  On success cnt[r]
 // holds the visitors of every child and sc_child / sc_occ hold (child, visit number) of
 // every visitor; returns false when the node has to be replayed one visitor at a time
 // (the caller's statistics are untouched either way).
+//
+// One batch: pick a score threshold (estimated so that about `target` unsettled entries
+// lie at or above it), count EXACTLY how many entries of every child lie at or above it
+// (estimate, then test the two entries around the estimate), evaluate these entries into
+// LDS, sort them, and keep the first `remaining` of them when this is the last batch.
+// The threshold does not have to be anything in particular: whatever it is, the entries at
+// or above it are played before every entry below it, provided the checks hold.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
                                             int off, int m, WaveLds<R> &lds, int (&cnt)[R]) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
-    if (m > kWaterLevelMaxJ) return false;
+    if (m > kWaterLevelMaxJ) OMK_FAIL(1);
 
-    int tk[R];                      // visits settled so far, per child
-    uint32_t headk[R], headp[R];    // the entry each child shows next
+    int tk[R];                    // visits settled so far, per child
+    uint32_t headk[R], headp[R];  // the entry each child shows next
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int i = r * kWave + lane;
@@ -292,9 +343,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
 
     OMK_T0();
     for (int done = 0; done < m;) {
-        const int need = m - done < kBatchCap ? m - done : kBatchCap;
+        const int remaining = m - done;
 
-        // ---- 1. threshold T* = largest key with at least `need` unsettled entries at or above it ----
+        // ---- 1. threshold and exact per-child counts ----
         uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -304,26 +355,28 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             }
         uint32_t hi_key, hi_pos;
         wave_best(lbk, lbp, hi_key, hi_pos);
-        if (hi_key == 0u) return false;
+        if (hi_key == 0u) OMK_FAIL(2);
         const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
-        // the best child alone has `need` entries at or above the key of its need-th next visit
+        const int want = remaining < kBatchCap ? remaining : kBatchCap;
+        // lower bound of any useful threshold: the best child alone has `want` entries at or
+        // above the key of its want-th next visit
         uint32_t lo_key = 0u;
         {
             uint32_t kk = 0u, pp = 0u;
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 if (r == (best >> 6))
-                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl,
-                                       tk[r] + need - 1, best, kk, pp);
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk[r] + want - 1, best, kk,
+                                       pp);
             }
             lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
         }
         if (lo_key == 0u) lo_key = 1u;
-        if (lo_key > hi_key) return false;  // scores rose along the best child's list
+        if (lo_key > hi_key) OMK_FAIL(3);  // scores rose along the best child's list
 
-        // Only children whose next entry reaches the lower bound can contribute to this batch.
-        // They are listed densely (one per lane and round) so that the probes below cost
-        // one evaluation round per 64 ACTIVE children instead of one per 64 children.
+        // Only children whose next entry reaches the lower bound can contribute.  They are
+        // listed densely (one per lane and round), so that the work below costs one round per
+        // 64 ACTIVE children instead of one per 64 children.
         int n_act = 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -334,16 +387,14 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             n_act += __popcll(am);
             lds.key[i] = headk[r];  // key of the child's next entry
             lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
-            lds.pay[i] = 0u;        // result: entries above T*
-            lds.idx[0][i] = 0;      // result: entries at or above T*
+            lds.st_j0[i] = tk[r];
+            lds.pay[i] = 0u;  // result: entries of the batch
         }
         wave_sync_memory();
         const int rounds = (n_act + kWave - 1) / kWave;
-        // statistics of this lane's active children
         int an[R], avl[R], ac[R];
         float aw[R], ap[R], aq2[R];
         uint32_t ahead[R];
-        int cl[R], ch[R];  // counts of the batch at hi / at lo, relative to the settled visits
 #pragma unroll
         for (int r = 0; r < R; r++) {
             ac[r] = -1;
@@ -351,7 +402,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             avl[r] = 0;
             aw[r] = ap[r] = aq2[r] = 0.0f;
             ahead[r] = 0u;
-            cl[r] = ch[r] = 0;
             if (r < rounds && r * kWave + lane < n_act) {
                 const int ci = (int)lds.idx[1][r * kWave + lane];
                 ac[r] = ci;
@@ -361,179 +411,139 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 avl[r] = lds.st_vl[ci];
                 aq2[r] = lds.st_q2[ci];
                 ahead[r] = lds.key[ci];
-                ch[r] = need;
             }
         }
-        // Invariant: count(lo) >= need > count(hi), cl = per-child counts at hi, ch = at lo.
-        // After every probe the bracket end that moved is snapped to the nearest key that
-        // actually occurs, so the search ends after about log2(distinct keys in it) probes.
-        uint32_t lo = lo_key, hi = hi_key + 1u;
-        bool first = true;
-        int probes = 0;
-        while (first || hi - lo > 1u) {
-            if (++probes > 80) return false;
-            const uint32_t T = first ? lo : lo + ((hi - lo) >> 1);
-            int ct[R];
+        // the estimate is off by about one entry per active child: aim a margin above what is
+        // needed when this can be the last batch, a margin below the capacity otherwise
+        const int margin = n_act + 8;
+        const bool can_finish = remaining + 2 * margin <= kBatchCap;
+        int target = can_finish ? remaining + margin : kBatchCap - margin;
+        if (target < 1) OMK_FAIL(4);
+        int ct[R];
+        int total = 0;
+        int tries = 0;
+        int capped_child = -1, capped_last = 0;
+        for (;;) {
+            if (++tries > 6) OMK_FAIL(5);
+            // bisection on the score with the estimated counts only (no exact evaluation)
+            float flo = key_score(lo_key), fhi = key_score(hi_key);
+            for (int it = 0; it < 22; it++) {
+                const float mid = 0.5f * (flo + fhi);
+                int est = 0;
+#pragma unroll
+                for (int r = 0; r < R; r++)
+                    if (r < rounds && ac[r] >= 0)
+                        est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, kBatchCap);
+                if (wave_sum_i32(est) >= target) flo = mid;
+                else fhi = mid;
+            }
+            uint32_t T = score_key(flo);
+            if (T < lo_key) T = lo_key;
+            if (T > hi_key) T = hi_key;
+            const float tau = key_score(T);
+            // exact count of every active child at T: test the two entries around the estimate
             int sum = 0;
-            uint32_t below = 0u;           // largest key below T among the first entries below T
-            uint32_t above = 0xFFFFFFFFu;  // smallest key among the last entries at or above T
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 ct[r] = 0;
-                if (r < rounds) {
-                    int lo_c = cl[r], hi_c = ch[r];
-                    if (ahead[r] < T) hi_c = 0;  // a list that starts below T has nothing above it
-                    if (lo_c > hi_c) lo_c = hi_c;
-                    uint32_t k_in = 0xFFFFFFFFu, k_out = 0u;  // keys seen at the boundary while searching
-                    int j_in = -1, j_out = -1;
+                if (r < rounds && ac[r] >= 0 && ahead[r] >= T) {
+                    int lo_c = 1, hi_c = kBatchCap + 1;  // the next entry itself is at or above T
+                    int g = predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, tau, kBatchCap);
+                    g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
+                    uint32_t kk, pp;
+                    if (g > lo_c) {
+                        entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, g - 1, ac[r], kk, pp);
+                        if (kk >= T) lo_c = g;
+                        else hi_c = g - 1;
+                    }
+                    if (lo_c == g && g < hi_c) {
+                        entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, g, ac[r], kk, pp);
+                        if (kk >= T) lo_c = g + 1;
+                        else hi_c = g;
+                    }
                     while (lo_c < hi_c) {
                         int t = (lo_c + hi_c + 1) >> 1;
-                        uint32_t kk, pp;
                         entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, t - 1, ac[r], kk, pp);
-                        if (kk >= T) {
-                            lo_c = t;
-                            k_in = kk;
-                            j_in = t - 1;
-                        } else {
-                            hi_c = t - 1;
-                            k_out = kk;
-                            j_out = t - 1;
-                        }
+                        if (kk >= T) lo_c = t;
+                        else hi_c = t - 1;
                     }
                     ct[r] = lo_c;
                     sum += lo_c;
-                    if (ac[r] >= 0) {
-                        // last entry at or above T and first entry below T of this child
-                        if (lo_c > 0) {
-                            if (j_in != lo_c - 1) {
-                                if (lo_c == 1) {
-                                    k_in = ahead[r];
-                                } else {
-                                    uint32_t pp;
-                                    entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, lo_c - 1, ac[r],
-                                                       k_in, pp);
-                                }
-                            }
-                            above = umin32(above, k_in);
-                        }
-                        if (lo_c < need) {
-                            if (j_out != lo_c) {
-                                if (lo_c == 0) {
-                                    k_out = ahead[r];
-                                } else {
-                                    uint32_t pp;
-                                    entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, lo_c, ac[r], k_out,
-                                                       pp);
-                                }
-                            }
-                            if (k_out < T) below = umax32(below, k_out);
-                        }
-                    }
                 }
             }
-            const int total = wave_sum_i32(sum);  // at most 64 * R * need
-            if (first) {
-                if (total < need) return false;
-                first = false;
-            }
-            if (total >= need) {
-                uint32_t snap = wave_min_u32(above);
-                lo = (snap != 0xFFFFFFFFu && snap >= T && snap < hi) ? snap : T;
+            total = wave_sum_i32(sum);  // at most 64 * R * (capacity + 1)
+            if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
+            // A batch that does not fit is cut at the child with most entries (typically one
+            // whose score hardly moves with virtual loss): it contributes fewer entries now,
+            // and the batch is later cut right after its last one.
+            capped_child = -1;
+            capped_last = 0;
+            if (total > kBatchCap) {
+                int mx = 0, mi = -1;
 #pragma unroll
-                for (int r = 0; r < R; r++) ch[r] = ct[r];
-            } else {
-                uint32_t snap = wave_max_u32(below);
-                hi = (snap + 1u > lo && snap < T) ? snap + 1u : T;
+                for (int r = 0; r < R; r++)
+                    if (ct[r] > mx) {
+                        mx = ct[r];
+                        mi = ac[r];
+                    }
+                const uint32_t gmx = wave_max_u32((uint32_t)mx);
+                const int who = (int)wave_min_u32((uint32_t)mx == gmx ? (uint32_t)mi : 0xFFFFFFFFu);
+                const int excess = total - kBatchCap;
+                if ((int)gmx <= excess) {
+                    target -= excess + margin;  // no single child absorbs it: aim higher instead
+                    if (target < 1) target = 1;
+                    continue;
+                }
 #pragma unroll
-                for (int r = 0; r < R; r++) cl[r] = ct[r];
+                for (int r = 0; r < R; r++)
+                    if (ac[r] == who) ct[r] -= excess;
+                capped_child = who;
+                total = kBatchCap;
             }
+            if (can_finish && total < remaining) {
+                target += (remaining - total) + margin;  // not enough to finish: aim lower
+                if (target > kBatchCap) OMK_FAIL(6);
+                continue;
+            }
+            if (total < 1) OMK_FAIL(7);
+            break;
         }
         // hand the counts back to the lanes that own the children
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            if (ac[r] >= 0) {
-                lds.pay[ac[r]] = (uint32_t)cl[r];
-                lds.idx[0][ac[r]] = (uint16_t)ch[r];
-            }
-        }
+        for (int r = 0; r < R; r++)
+            if (ac[r] >= 0) lds.pay[ac[r]] = (uint32_t)ct[r];
         wave_sync_memory();
+        int nb[R];  // entries of every own child in this batch
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int i = r * kWave + lane;
-            cl[r] = tk[r] + (int)lds.pay[i];
-            ch[r] = tk[r] + (int)lds.idx[0][i];
-        }
+        for (int r = 0; r < R; r++) nb[r] = (int)lds.pay[r * kWave + lane];
+        if (capped_child >= 0) capped_last = lds.st_j0[capped_child] + (int)lds.pay[capped_child] - 1;
         wave_sync_memory();
-        // now cl = settled + entries above T*, ch = settled + entries at or above T*
         OMK_TICK(8);
-        if (a.stats && lane == 0) atomicAdd(a.stats + 5, probes);
 
-        // ---- 2. entries at exactly T* are handed out in child order until `need` is reached ----
-        int above_n = 0;
-#pragma unroll
-        for (int r = 0; r < R; r++) above_n += cl[r] - tk[r];
-        const int rem = need - wave_sum_i32(above_n);
-        if (rem < 0) return false;
-        int cv[R];
+        // ---- 2. evaluate the batch in (child, visit) order ----
         int carry = 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            int e = ch[r] - cl[r];
-            if (e < 0) e = 0;
-            if (e > rem) e = rem;
-            int inc = wave_inclusive_sum(e, lane);
-            int excl = carry + inc - e;
-            int left = rem - excl;
-            int take = left <= 0 ? 0 : (left < e ? left : e);
-            cv[r] = cl[r] + take;
+            int inc = wave_inclusive_sum(nb[r], lane);
+            lds.offs[r * kWave + lane] = carry + inc - nb[r];
             carry += __builtin_amdgcn_readlane(inc, 63);
-        }
-        int csum = 0;
-#pragma unroll
-        for (int r = 0; r < R; r++) csum += cv[r] - tk[r];
-        if (wave_sum_i32(csum) != need) return false;
-
-        // ---- 3. evaluate the batch in (child, visit) order; first untaken entries ----
-        carry = 0;
-        uint32_t uk[R], upos[R];  // first untaken entry of every child of this lane
-        bool bad = false;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int nr = cv[r] - tk[r];
-            int inc = wave_inclusive_sum(nr, lane);
-            int i = r * kWave + lane;
-            lds.offs[i] = carry + inc - nr;
-            lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
-            lds.st_j0[i] = tk[r];
-            carry += __builtin_amdgcn_readlane(inc, 63);
-            uk[r] = 0u;
-            upos[r] = 0xFFFFFFFFu;
-            if (k.part[r]) {
-                if (nr == 0) {
-                    uk[r] = headk[r];
-                    upos[r] = headp[r];
-                } else {
-                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, cv[r], i,
-                                       uk[r], upos[r]);
-                    // the last taken entry of the child must not come after its first untaken one
-                    uint32_t lk, lp;
-                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl,
-                                       cv[r] - 1, i, lk, lp);
-                    if (lk == 0u || comes_before(uk[r], upos[r], lk, lp)) bad = true;
-                }
-            }
         }
         wave_sync_memory();
-
+        bool bad = false;
+        bool any_first = false, any_second = false;  // candidates of the first / second scan present
         uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
-        uint32_t prev_key63 = 0u, prev_pos63 = 0u;
-        int prev_child63 = -1;
-        for (int base = 0; base < need; base += kWave) {
-            const int q = base + lane;
-            const bool in = q < need;
-            int child = -1;
-            uint32_t kk = 0u, pp = 0u;
-            if (in) {
+        {
+            // every lane evaluates a contiguous run of `per` entries (odd, so that the LDS
+            // writes of the lanes fall into different banks)
+            const int per = ((total + kWave - 1) / kWave) | 1;
+            int q = lane * per;
+            const int q_end = q + per < total ? q + per : total;
+            int child = 0, seg_end = 0;
+            int sn = 0, svl = 0, sj0 = 0;
+            float sw = 0.0f, sp = 0.0f, sq2 = 0.0f;
+            uint32_t pk = 0u, ppos = 0u;
+            bool have = false;
+            if (q < q_end) {
                 // last child whose segment starts at or before q
                 int lo_i = 0, hi_i = F;
                 while (hi_i - lo_i > 1) {
@@ -542,47 +552,78 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     else hi_i = mid;
                 }
                 child = lo_i;
+                seg_end = lds.offs[child] + (int)lds.pay[child];
+            }
+            bool fresh = true;
+            uint32_t firstk = 0u, firstp = 0u;
+            int firstchild = -1, firstj = 0;
+            for (; q < q_end; q++) {
+                while (q >= seg_end) {  // next child with entries
+                    child++;
+                    seg_end = lds.offs[child] + (int)lds.pay[child];
+                    fresh = true;
+                }
+                if (fresh) {
+                    sn = lds.st_n[child];
+                    sw = lds.st_w[child];
+                    sp = lds.st_p[child];
+                    svl = lds.st_vl[child];
+                    sq2 = lds.st_q2[child];
+                    sj0 = lds.st_j0[child];
+                    fresh = false;
+                    have = false;
+                }
                 const int jl = q - lds.offs[child];
-                entry_key<R, RAVE>(lds.st_n[child], lds.st_w[child], lds.st_p[child], lds.st_vl[child],
-                                   lds.st_q2[child], c.ep, uvl, jl, child, kk, pp);
+                uint32_t kk, pp;
+                entry_key<R, RAVE>(sn, sw, sp, svl, sq2, c.ep, uvl, jl, child, kk, pp);
                 lds.key[q] = ~kk;
-                lds.pay[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) |
-                             (uint32_t)(lds.st_j0[child] + jl);
+                lds.pay2[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)(sj0 + jl);
                 kmin = umin32(kmin, ~kk);
                 kmax = umax32(kmax, ~kk);
+                if (pp >= (uint32_t)F) any_second = true;
+                else any_first = true;
                 if (kk == 0u) bad = true;
+                // within a child the entries must not increase
+                if (have && comes_before(kk, pp, pk, ppos)) bad = true;
+                if (firstchild < 0) {
+                    firstk = kk;
+                    firstp = pp;
+                    firstchild = child;
+                    firstj = jl;
+                }
+                pk = kk;
+                ppos = pp;
+                have = true;
             }
-            // within a child the entries must not increase
-            uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-            uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
-            int pchild = __shfl_up(child, 1, kWave);
-            if (lane == 0) {
-                pk = prev_key63;
-                ppos = prev_pos63;
-                pchild = prev_child63;
-            }
-            if (in && pchild == child && comes_before(kk, pp, pk, ppos)) bad = true;
-            prev_key63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-            prev_pos63 = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
-            prev_child63 = __builtin_amdgcn_readlane(child, 63);
+            // the run of the previous lane may end inside the same child: check the seam
+            uint32_t lk = (uint32_t)__shfl_up((int)pk, 1, kWave);
+            uint32_t lp = (uint32_t)__shfl_up((int)ppos, 1, kWave);
+            if (lane > 0 && firstchild >= 0 && firstj > 0 && comes_before(firstk, firstp, lk, lp)) bad = true;
         }
-        if (__ballot(bad) != 0ull) return false;
+        if (__ballot(bad) != 0ull) OMK_FAIL(8);
         kmin = wave_min_u32(kmin);
         kmax = wave_max_u32(kmax);
+        wave_sync_memory();
         OMK_TICK(9);
 
-        // ---- 4. stable radix sort of the batch by key, over the bits that differ, in LDS ----
+        // ---- 3. stable radix sort of the batch, in LDS ----
+        // Order wanted: key descending, then candidate position ascending, then visit number.
+        // The entries start in (child, visit) order; least significant digit first, a 1-bit
+        // pass on the scan kind (only when both kinds occur: candidates of the first scan sit
+        // before those of the second) and then the key digits, over the bits that differ.
         const uint32_t diff = kmin ^ kmax;
         const int nbits = diff == 0u ? 0 : 32 - __clz((int)diff);
+        const bool mixed = __ballot(any_first) != 0ull && __ballot(any_second) != 0ull;
         int cur = -1;  // -1: identity order, else lds.idx[cur]
-        for (int sh = 0; sh < nbits; sh += kDigitBits) {
+        for (int sh = mixed ? -kDigitBits : 0; sh < nbits; sh += kDigitBits) {
             wave_sync_memory();
 #pragma unroll
             for (int t = 0; t < kBins / kWave; t++) lds.hist[t * kWave + lane] = 0;
             wave_sync_memory();
-            for (int q = lane; q < need; q += kWave) {
+            for (int q = lane; q < total; q += kWave) {
                 const int i = cur < 0 ? q : (int)lds.idx[cur][q];
-                atomicAdd(&lds.hist[(lds.key[i] >> sh) & (uint32_t)(kBins - 1)], 1);
+                const uint32_t d = sh < 0 ? lds.pay2[i] >> 31 : (lds.key[i] >> sh) & (uint32_t)(kBins - 1);
+                atomicAdd(&lds.hist[d], 1);
             }
             wave_sync_memory();
             {
@@ -604,11 +645,12 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             }
             wave_sync_memory();
             const int nxt = cur == 0 ? 1 : 0;
-            for (int base = 0; base < need; base += kWave) {
+            for (int base = 0; base < total; base += kWave) {
                 const int q = base + lane;
-                const bool in = q < need;
+                const bool in = q < total;
                 const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
-                const uint32_t d = in ? (lds.key[i] >> sh) & (uint32_t)(kBins - 1) : 0u;
+                const uint32_t d =
+                    !in ? 0u : (sh < 0 ? lds.pay2[i] >> 31 : (lds.key[i] >> sh) & (uint32_t)(kBins - 1));
                 // lanes of this chunk with the same digit
                 uint64_t same = __ballot(in);
 #pragma unroll
@@ -627,17 +669,33 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             cur = nxt;
         }
         wave_sync_memory();
-
         OMK_TICK(10);
-        // ---- 5. winner order of the batch: check ties across children, emit ----
+
+        // ---- 4. winner order: keep what is needed, check ties across children, emit ----
+        int keep = total < remaining ? total : remaining;
+        if (capped_child >= 0) {
+            // position of the capped child's last evaluated entry in the sorted batch
+            uint32_t qcut = 0xFFFFFFFFu;
+            const uint32_t want_pay = ((uint32_t)capped_child << 21) | (uint32_t)capped_last;
+            for (int q = lane; q < total; q += kWave) {
+                const int i = cur < 0 ? q : (int)lds.idx[cur][q];
+                if ((lds.pay2[i] & 0x7FFFFFFFu) == want_pay) qcut = umin32(qcut, (uint32_t)q);
+            }
+            qcut = wave_min_u32(qcut);
+            if (qcut == 0xFFFFFFFFu) OMK_FAIL(10);
+            if ((int)qcut + 1 < keep) keep = (int)qcut + 1;
+        }
+#pragma unroll
+        for (int t = 0; t < kBins / kWave; t++) lds.hist[t * kWave + lane] = 0;  // visits per child after this batch
+        wave_sync_memory();
         uint32_t pk63 = 0u, ppay63 = 0u;
         bool have_prev = false;
-        for (int base = 0; base < need; base += kWave) {
+        for (int base = 0; base < total; base += kWave) {
             const int q = base + lane;
-            const bool in = q < need;
+            const bool in = q < total;
             const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
             uint32_t kk = in ? lds.key[i] : 0u;
-            uint32_t pay = in ? lds.pay[i] : 0u;
+            uint32_t pay = in ? lds.pay2[i] : 0u;
             uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
             uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
             bool hp = lane > 0 || have_prev;
@@ -648,8 +706,13 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (in) {
                 const int child = (int)((pay >> 21) & 1023u);
                 const int j = (int)(pay & 0x1FFFFFu);
-                a.sc_child[off + done + q] = child;
-                a.sc_occ[off + done + q] = j;
+                if (q < keep) {
+                    a.sc_child[off + done + q] = child;
+                    a.sc_occ[off + done + q] = j;
+                    atomicMax(&lds.hist[child], j + 1);
+                }
+                // the order of the whole batch is checked, kept or not: what is dropped must
+                // come after what is kept
                 if (hp) {
                     if (pk > kk) bad = true;  // not sorted
                     if (pk == kk) {
@@ -664,29 +727,44 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             ppay63 = (uint32_t)__builtin_amdgcn_readlane((int)pay, 63);
             have_prev = true;
         }
+        wave_sync_memory();
         {
-            // the last taken entry must come before every other child's first untaken entry
-            // (its own child's next entry was checked in step 3)
-            const int il = cur < 0 ? need - 1 : (int)lds.idx[cur][need - 1];
+            // The last kept entry must come before every child's first unevaluated entry (a
+            // child with dropped entries is covered by the order check above), and that entry
+            // must not come before the child's own last evaluated one.
+            const int il = cur < 0 ? keep - 1 : (int)lds.idx[cur][keep - 1];
             const uint32_t lk = ~lds.key[il];
-            const uint32_t lpay = lds.pay[il];
+            const uint32_t lpay = lds.pay2[il];
             const uint32_t lchild = (lpay >> 21) & 1023u;
             const uint32_t lpos = lchild + ((lpay >> 31) ? (uint32_t)F : 0u);
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                if (uk[r] != 0u && (uint32_t)(r * kWave + lane) != lchild &&
-                    !comes_before(lk, lpos, uk[r], upos[r]))
-                    bad = true;
+                const int i = r * kWave + lane;
+                const int settled = lds.hist[i] > tk[r] ? lds.hist[i] : tk[r];
+                uint32_t uk = headk[r], up = headp[r];
+                if (k.part[r] && nb[r] > 0) {
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk[r] + nb[r], i, uk, up);
+                    uint32_t ek, ep2;
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk[r] + nb[r] - 1, i, ek,
+                                       ep2);
+                    if (ek == 0u || comes_before(uk, up, ek, ep2)) bad = true;
+                }
+                if (k.part[r] && uk != 0u && (uint32_t)i != lchild && !comes_before(lk, lpos, uk, up)) bad = true;
+                // the child's next entry after this batch
+                if (k.part[r] && settled > tk[r]) {
+                    if (settled == tk[r] + nb[r]) {
+                        headk[r] = uk;
+                        headp[r] = up;
+                    } else {
+                        entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, settled, i, headk[r],
+                                           headp[r]);
+                    }
+                }
+                tk[r] = settled;
             }
         }
-        if (__ballot(bad) != 0ull) return false;
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            tk[r] = cv[r];
-            headk[r] = uk[r];
-            headp[r] = upos[r];
-        }
-        done += need;
+        if (__ballot(bad) != 0ull) OMK_FAIL(9);
+        done += keep;
         wave_sync_memory();
         OMK_TICK(11);
     }
@@ -855,7 +933,6 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         atomicAdd(a.stats + 4, st_replay);
     }
 
-    // a group that stays together is walked on by this wavefront
     uint32_t lmax = 0u;
 #pragma unroll
     for (int r = 0; r < R; r++) lmax = umax32(lmax, (uint32_t)cnt[r]);
@@ -864,7 +941,11 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
 #pragma unroll
     for (int r = R - 1; r >= 0; r--)
         if ((uint32_t)cnt[r] == gmax) lidx = (uint32_t)(r * kWave + lane);
-    const int keep = gmax == (uint32_t)m ? (int)wave_min_u32(lidx) : -1;
+    // Walk on when the group stays together, or when it is small and most of it does (the rest
+    // goes to the queues); a large group that splits is handed to the next level's launch
+    // whole, so that its parts are played side by side.
+    const bool walk_on = gmax == (uint32_t)m || (m <= kWalkOnSmall && gmax * 4u >= (uint32_t)m * 3u);
+    const int keep = walk_on ? (int)wave_min_u32(lidx) : -1;
 
     // exclusive prefix of the visit counts in child order -> segment of every child
     int carry = 0;

@@ -27,7 +27,7 @@ EXPORTS = [
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_truncated", "omk_batch_stats", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
-    "omk_dev_d2h",
+    "omk_dev_d2h", "omk_dev_copy",
 ]
 
 TT_SLOT = np.dtype([("key", "<u8"), ("node", "<i4"), ("depth", "<i4")])
@@ -187,6 +187,9 @@ class Forest:
         assert arr.flags["C_CONTIGUOUS"]
         _check(self._lib.omk_dev_d2h(self._h, arr.ctypes.data_as(C.c_void_p), C.c_void_p(dptr), arr.nbytes))
 
+    def dev_copy(self, dst, src, nbytes):
+        _check(self._lib.omk_dev_copy(self._h, C.c_void_p(dst), C.c_void_p(src), int(nbytes)))
+
     # the three node operations over caller-supplied device paths (level-major)
     def apply_vl_paths(self, d_paths, d_len, n, stride, max_len, vl):
         _check(self._lib.omk_apply_vl_paths(self._h, C.c_void_p(d_paths), C.c_void_p(d_len), int(n), int(stride),
@@ -262,7 +265,7 @@ class Batch:
         out = np.zeros(16, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
-                "replayed_nodes", "threshold_probes", "single_visitor_steps", "unused7", "cyc_threshold",
+                "replayed_nodes", "threshold_probes", "single_visitor_steps", "fail_code", "cyc_threshold",
                 "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "unused15")
         return dict(zip(keys, map(int, out)))
 

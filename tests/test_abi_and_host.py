@@ -1,0 +1,165 @@
+"""CPU-side checks of the shipped pieces: the C ABI library loads and exports exactly what
+include/omk_forest.h declares, errors come back as status codes, the synthetic forest
+generator produces well-formed forests with the documented statistics, and the benchmark's
+byte model is what it says.  No GPU compute here."""
+import json
+import math
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "omk_forest.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(omk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import ctypes
+    import omoknuni_small_amd as omk
+    from omoknuni_small_amd import forest
+    lib = omk.load_library()
+    names = declared_functions()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), "libomk_forest.so does not export " + n
+    assert sorted(forest.EXPORTS) == names, "the Python mirror and the header disagree"
+    assert lib.omk_version() >= 1
+    assert isinstance(ctypes.c_char_p(lib.omk_last_error()).value, bytes)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from omoknuni_small_amd import forest
+    monkeypatch.setattr(forest, "_LIB", None)
+    monkeypatch.setattr(forest, "_HERE", str(tmp_path))
+    with pytest.raises(OSError, match="no host fallback"):
+        forest.load_library()
+
+
+def test_errors_are_status_codes_not_crashes():
+    import omoknuni_small_amd as omk
+    with pytest.raises(omk.OmkError) as e:
+        omk.Forest(0)
+    assert e.value.code == -1 and "capacity" in str(e.value)
+    try:
+        f = omk.Forest(16)
+    except omk.OmkError as err:
+        # no GPU in this process: creation reports the HIP failure and nothing leaks
+        assert err.code == -2
+        return
+    f.close()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
+
+
+def check_forest(soa, roots, meta):
+    n = len(soa["N"])
+    cb, cc = soa["child_begin"].astype(np.int64), soa["child_count"].astype(np.int64)
+    exp = np.nonzero(cc > 0)[0]
+    assert (cb[exp] >= 0).all() and (cb[exp] + cc[exp] <= n).all()
+    owner = np.zeros(n, np.int32)
+    for v in exp:
+        owner[cb[v]:cb[v] + cc[v]] += 1
+    assert owner.max() == 1, "a node has two parents"
+    assert (owner[roots] == 0).all()
+    legal = np.ones(n, bool)
+    if soa.get("legal") is not None:
+        legal = np.unpackbits(soa["legal"].view(np.uint8), bitorder="little")[:n].astype(bool)
+    kids = owner == 1
+    assert (soa["N"][kids & legal] >= 1).all() and (soa["N"] <= max(meta["n_cap"], soa["N"][exp].max())).all()
+    assert (np.abs(soa["W"]) <= soa["N"] + 1e-3).all()
+    assert (soa["VL"] == 0).all()
+    for v in exp[:200]:
+        sl = slice(cb[v], cb[v] + cc[v])
+        lg = legal[sl]
+        assert lg.any()
+        assert abs(float(soa["P"][sl][lg].sum()) - 1.0) < 1e-4
+        assert (soa["P"][sl][~lg] == 0).all()
+        if (cc[sl] == 0).all():  # N of an expanded node was set from its children as drawn at that time
+            assert soa["N"][v] == 1 + int(soa["N"][sl][lg].sum())
+        assert sorted(soa["action"][sl]) == list(range(cc[v]))
+    d = meta["depth"]
+    assert d.max() <= meta["max_depth"] and (cc[d == meta["max_depth"]] == 0).all()
+    return exp, legal
+
+
+def test_synthetic_forests_are_well_formed():
+    from omoknuni_small_amd import synth
+    soa, roots, meta = synth.generate("c0", nodes_per_tree=30000, seed=5)
+    exp, legal = check_forest(soa, roots, meta)
+    assert (soa["child_count"][exp] == 225).all()
+    frac = legal[soa["child_begin"][exp[0]]:][: 225 * 20].mean()
+    assert 0.4 < frac < 0.6
+    # same seed, same forest; another seed, another forest
+    again, _, _ = synth.generate("c0", nodes_per_tree=30000, seed=5)
+    assert all((soa[k] == again[k]).all() for k in soa)
+    other, _, _ = synth.generate("c0", nodes_per_tree=30000, seed=6)
+    assert (other["N"] != soa["N"]).any()
+
+    soa, roots, meta = synth.generate("c2", n_trees=3, nodes_per_tree=40000, seed=5)
+    exp, legal = check_forest(soa, roots, meta)
+    assert list(roots) == [0, 40000, 80000]
+    last = soa["child_begin"][exp] + 361
+    assert legal[last].all(), "the pass move always has a child"
+
+    soa, roots, meta = synth.generate("c3", nodes_per_tree=60000, seed=5)
+    exp, _ = check_forest(soa, roots, meta)
+    assert soa.get("legal") is None
+    fo = soa["child_count"][exp]
+    assert fo.min() >= 1 and fo.max() <= 218 and 30 < fo.mean() < 40
+    for v in exp[:300]:
+        p = soa["P"][soa["child_begin"][v]: soa["child_begin"][v] + soa["child_count"][v]]
+        assert (np.diff(p) <= 0).all(), "children are stored by descending prior"
+
+    soa, roots, meta = synth.generate("c4", nodes_per_tree=50000, seed=5)
+    check_forest(soa, roots, meta)
+    assert soa["rN"].max() <= 10000 and (np.abs(soa["rW"]) <= soa["rN"] + 1e-3).all()
+    assert len(np.unique(soa["hash"])) == len(soa["hash"])
+
+
+def test_zipf_statistics():
+    from omoknuni_small_amd import synth
+    soa, _, meta = synth.generate("c0", nodes_per_tree=120000, seed=9)
+    legal = np.unpackbits(soa["legal"].view(np.uint8), bitorder="little")[: len(soa["N"])].astype(bool)
+    leaves = legal & (soa["child_count"] == 0)
+    leaves[0] = False
+    n = soa["N"][leaves]
+    # P(N = 1) = 1 / zeta(1.2), P(N >= cap) = tail mass of Zipf(1.2) beyond 10^4
+    assert abs((n == 1).mean() - 1 / 5.5916) < 0.01
+    assert abs((n == 2).mean() - 2 ** -1.2 / 5.5916) < 0.01
+    assert abs((n == 10000).mean() - 0.142) < 0.02
+    q = soa["W"][leaves] / n
+    assert abs(q.mean()) < 0.02 and abs(q.std() - 1 / math.sqrt(3)) < 0.02  # uniform in [-1, 1]
+
+
+def test_bench_byte_model_on_a_known_tree():
+    sys.path.insert(0, ROOT)
+    import bench
+    # root with 3 slots (2 legal) -> child 1 expanded with 2 slots (both legal)
+    soa = dict(child_begin=np.array([1, 4, 0, 0, 0, 0], np.int32), child_count=np.array([3, 2, 0, 0, 0, 0], np.int32),
+               legal=np.array([0b110111], np.uint32))
+    L = bench.legal_children_per_node(soa)
+    assert list(L[:2]) == [2, 2]
+    paths = np.array([[0, 1, 4], [0, 1, 5], [0, 3, -1]], np.int32)
+    plen = np.array([3, 3, 2], np.int32)
+    sel, bak, steps = bench.algorithmic_bytes(soa, {}, paths, plen, np.zeros(6, np.int32))
+    assert steps == 5
+    # per selection step: L*16 + ceil(F/8) + 24; per path entry written: 4
+    assert sel == 3 * (2 * 16 + 1 + 24) + 2 * (2 * 16 + 1 + 24) + 4 * 8
+    assert bak == 24 * 8 + 4 * 3 + 4 * 8
+
+
+def test_golden_fixture_is_data_only():
+    with open(os.path.join(ROOT, "tests", "golden", "kat_reference.json")) as f:
+        g = json.load(f)
+    assert {"select", "score_bits", "backup", "virtual_loss_probe"} <= set(g)
