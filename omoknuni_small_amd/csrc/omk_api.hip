@@ -80,7 +80,14 @@ struct omk_batch {
     int32_t n_singles0 = 0;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
-    int32_t *counters = nullptr;  // [max_depth + 2] level counters, 1 truncated counter, 8 work statistics
+    // [0] simulations cut by max_depth, [1..16] work statistics, [17] single-visitor queue length,
+    // [18..21] scheduler state of the multi-visitor kernel
+    int32_t *counters = nullptr;
+    int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
+    int32_t q_cap = 0;
+    int32_t epoch = 0;           // select calls so far
+    int32_t spin_limit = 1 << 22;
+    int32_t n_cus = 0;
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
 };
@@ -319,7 +326,11 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->leaf, B);
     if (e == hipSuccess) e = dalloc(&b->values, B);
     if (e == hipSuccess) e = dalloc(&b->items0, B);
-    if (e == hipSuccess) e = dalloc(&b->items_q, B * (max_depth + 1));
+    // a multi-visitor item has at least two visitors, and a level holds each visitor once
+    b->q_cap = (int32_t)((B / 2) * (max_depth + 1));
+    if (e == hipSuccess) e = dalloc(&b->items_q, b->q_cap);
+    if (e == hipSuccess) e = dalloc(&b->q_ready, b->q_cap);
+    if (e == hipSuccess) e = hipMemset(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4);
     if (e == hipSuccess) e = dalloc(&b->singles0, B);
     if (e == hipSuccess) e = dalloc(&b->singles_q, B);
     if (e == hipSuccess) e = dalloc(&b->seg0, B);
@@ -327,7 +338,9 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, B);
     if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
-    if (e == hipSuccess) e = dalloc(&b->counters, (int64_t)max_depth + 3 + 16 + 1);
+    if (e == hipSuccess) e = dalloc(&b->counters, 32);
+    if (e == hipSuccess) e = hipMemset(b->counters, 0, 32 * 4);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&b->n_cus, hipDeviceAttributeMultiprocessorCount, f->device);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
     if (e == hipSuccess) e = hipMemset(b->values, 0, (size_t)B * 4);
@@ -346,7 +359,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q};
+                    b->singles0, b->singles_q, b->q_ready};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -374,19 +387,21 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
         int32_t j = i;
         while (j < n && h_roots[order[(size_t)j]] == h_roots[order[(size_t)i]]) j++;
         Item it;
+        memset(&it, 0, sizeof(it));
         it.node = h_roots[order[(size_t)i]];
-        it.np = 0;
         if (j - i > 1) {
             it.off = i;
             it.m = j - i;
             items.push_back(it);
         } else {
             it.off = order[(size_t)i];  // the traversal itself
-            it.m = 0;                   // depth
+            it.m = 1;
             singles.push_back(it);
         }
         i = j;
     }
+    // the most crowded roots head the longest chains of work: start them first
+    std::stable_sort(items.begin(), items.end(), [](const Item &x, const Item &y) { return x.m > y.m; });
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     HIP_TRY(hipMemcpy(b->seg0, order.data(), (size_t)n * 4, hipMemcpyHostToDevice));
@@ -440,10 +455,19 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.items_q = b->items_q;
     a.seg[0] = b->seg[0];
     a.seg[1] = b->seg[1];
-    a.counters = b->counters;
-    a.truncated = b->counters + b->max_depth + 2;
-    a.stats = b->counters + b->max_depth + 3;
-    a.n_singles = b->counters + b->max_depth + 19;
+    if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
+        HIP_TRY(hipMemsetAsync(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4, f->stream));
+        b->epoch = 0;
+    }
+    b->epoch++;
+    a.q_ready = b->q_ready;
+    a.q_cap = b->q_cap;
+    a.epoch = b->epoch;
+    a.spin_limit = b->spin_limit;
+    a.truncated = b->counters + 0;
+    a.stats = b->counters + 1;
+    a.n_singles = b->counters + 17;
+    a.sched = b->counters + 18;
     a.singles0 = b->singles0;
     a.singles_q = b->singles_q;
     a.sc_child = b->sc_child;
@@ -457,7 +481,8 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.pw = p->pw;
     a.c_puct = p->c_puct;
     a.rave_k = p->rave_k;
-    HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n_singles0, b->n, f->max_fanout, p->use_rave != 0, f->stream));
+    HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n_singles0, b->n, f->max_fanout, p->use_rave != 0, b->n_cus,
+                          f->stream));
     b->selected = true;
     return OMK_OK;
 }
@@ -525,7 +550,14 @@ int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t 
     if (h_actions) HIP_TRY(hipMemcpyAsync(h_actions, b->out_actions, (size_t)n * D * 4, hipMemcpyDeviceToHost, s));
     if (h_path_len) HIP_TRY(hipMemcpyAsync(h_path_len, b->path_len, (size_t)n * 4, hipMemcpyDeviceToHost, s));
     if (h_leaf) HIP_TRY(hipMemcpyAsync(h_leaf, b->leaf, (size_t)n * 4, hipMemcpyDeviceToHost, s));
+    int32_t aborted = 0;
+    HIP_TRY(hipMemcpyAsync(&aborted, b->counters + 21, 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
+    if (aborted)
+        return fail(OMK_ERR_STATE,
+                    "omk_batch_read: the selection gave up (%s); its paths are incomplete, revert the virtual "
+                    "losses with omk_forest_upload or omk_revert_vl_paths over known paths",
+                    aborted == 1 ? "a wavefront waited longer than the spin limit" : "work queue overflow");
     return OMK_OK;
 }
 
@@ -533,7 +565,7 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     if (!b || !h_count) return fail(OMK_ERR_INVALID, "omk_batch_truncated: null argument");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_truncated: no selected paths");
     if (int rc = use_device(b->f)) return rc;
-    HIP_TRY(hipMemcpyAsync(h_count, b->counters + b->max_depth + 2, 4, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipMemcpyAsync(h_count, b->counters + 0, 4, hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }
@@ -543,7 +575,7 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     if (!b || !h_stats8) return fail(OMK_ERR_INVALID, "omk_batch_stats: null argument");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_stats: no selected paths");
     if (int rc = use_device(b->f)) return rc;
-    HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + b->max_depth + 3, 64, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + 1, 64, hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }

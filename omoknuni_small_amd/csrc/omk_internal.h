@@ -27,9 +27,11 @@ struct ForestDev {
 // indices in ascending order.  np is the node's visit count as read by the parent's wave.
 struct Item {
     int32_t node;
-    int32_t off;
-    int32_t m;
-    int32_t np;
+    int32_t off;    // first entry of its visitor list (single-visitor queue: the traversal itself)
+    int32_t m;      // visitors
+    int32_t np;     // N(node) as read by the parent's wavefront
+    int32_t depth;  // depth of the node on the visitors' paths
+    int32_t pad[3];
 };
 
 struct SelectArgs {
@@ -38,8 +40,13 @@ struct SelectArgs {
     const Item *singles0;  // traversals alone at their root: (node, traversal, depth 0, -)
     Item *singles_q;       // single visitors: (node, traversal, depth, N of the node)
     int32_t *n_singles;
-    Item *items_q;         // queue of level L >= 1 at items_q + (L-1)*stride
-    int32_t *counters;     // counters[L] = number of items of level L
+    Item *items_q;         // multi-visitor work queue, q_cap slots, filled front to back
+    int32_t *q_ready;      // per slot: == epoch once the item and everything it refers to is written
+    int32_t *sched;        // [0] next ticket, [1] slots handed out, [2] visitors still in multi-visitor
+                           // items, [3] abort flag (a waiting wavefront gave up)
+    int32_t q_cap;
+    int32_t epoch;         // number of this select call on the batch, > 0
+    int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
     int32_t *sc_child;     // per visitor: chosen child index
     int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child
@@ -57,7 +64,7 @@ struct SelectArgs {
 };
 
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
-                         int max_fanout, bool rave, hipStream_t s);
+                         int max_fanout, bool rave, int n_cus, hipStream_t s);
 
 hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                            int max_len, int vl, hipStream_t s);

@@ -48,7 +48,6 @@ constexpr int kBatchCap = 2048;           // entries put in winner order at a ti
 constexpr int kDigitBits = 10;            // radix digit of that sort
 constexpr int kBins = 1 << kDigitBits;
 constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
-constexpr int kWalkOnSmall = 32;          // groups up to this size walk on with their dominant part
 
 // Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
 // multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
@@ -941,15 +940,15 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
 #pragma unroll
     for (int r = R - 1; r >= 0; r--)
         if ((uint32_t)cnt[r] == gmax) lidx = (uint32_t)(r * kWave + lane);
-    // Walk on when the group stays together, or when it is small and most of it does (the rest
-    // goes to the queues); a large group that splits is handed to the next level's launch
-    // whole, so that its parts are played side by side.
-    const bool walk_on = gmax == (uint32_t)m || (m <= kWalkOnSmall && gmax * 4u >= (uint32_t)m * 3u);
-    const int keep = walk_on ? (int)wave_min_u32(lidx) : -1;
+    // This wavefront walks on with the largest part; the other parts go to the work queue,
+    // where idle wavefronts pick them up at once.
+    const int keep = gmax >= 2u ? (int)wave_min_u32(lidx) : -1;
 
     // exclusive prefix of the visit counts in child order -> segment of every child
     int carry = 0;
     int keep_np = 0;
+    int myslot[R];
+    int n_lone = 0, n_pushed = 0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         int inc = wave_inclusive_sum(cnt[r], lane);
@@ -959,20 +958,30 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         lds.st_j0[i] = cnt[r];
         lds.st_n[i] = k.n[r];
         if (i == keep) keep_np = k.n[r];
+        myslot[r] = -1;
+        n_lone += __popcll(__ballot(cnt[r] == 1));
         uint64_t has = __ballot(cnt[r] > 1 && i != keep);
         int nnew = __popcll(has);
+        n_pushed += nnew;
         if (nnew > 0) {
             int slot0 = 0;
-            if (lane == 0) slot0 = atomicAdd(a.counters + depth + 1, nnew);
+            if (lane == 0) slot0 = atomicAdd(a.sched + 1, nnew);
             slot0 = __builtin_amdgcn_readfirstlane(slot0);
             if (cnt[r] > 1 && i != keep) {
                 int slot = slot0 + __popcll(has & ((1ull << lane) - 1ull));
-                Item it;
-                it.node = c.cb + i;
-                it.off = off + excl;
-                it.m = cnt[r];
-                it.np = k.n[r];
-                a.items_q[(size_t)depth * a.stride + slot] = it;
+                if (slot < a.q_cap) {
+                    Item it;
+                    it.node = c.cb + i;
+                    it.off = off + excl;
+                    it.m = cnt[r];
+                    it.np = k.n[r];
+                    it.depth = depth + 1;
+                    it.pad[0] = it.pad[1] = it.pad[2] = 0;
+                    a.items_q[slot] = it;
+                    myslot[r] = slot;
+                } else {
+                    atomicExch(a.sched + 3, 2);  // queue overflow: cannot happen on a tree
+                }
             }
         }
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
@@ -1002,12 +1011,24 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                 Item it;
                 it.node = c.cb + i;
                 it.off = t;
-                it.m = depth + 1;
+                it.m = 1;
                 it.np = lds.st_n[i];
+                it.depth = depth + 1;
+                it.pad[0] = it.pad[1] = it.pad[2] = 0;
                 a.singles_q[s0 + __popcll(lm & ((1ull << lane) - 1ull))] = it;
             }
         }
     }
+    // publish the new items: everything they refer to is written, make it visible to the
+    // whole device first
+    if (n_pushed > 0) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (myslot[r] >= 0)
+                __hip_atomic_store(a.q_ready + myslot[r], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (n_lone > 0 && lane == 0) atomicSub(a.sched + 2, n_lone);  // lone visitors leave the multi-visitor items
     next.node = -1;
     if (keep >= 0) {
         next.node = c.cb + keep;
@@ -1021,52 +1042,93 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     return true;
 }
 
-// Multi-visitor items of one tree level; a group that stays together is walked on.
+// Multi-visitor items: a persistent kernel over a device-side work queue.  A wavefront takes
+// a ticket, waits until the item with that number is published (or until no visitor is
+// left in any multi-visitor item), processes the node, keeps the largest part of the group
+// and publishes the other parts.  Items depend only on their ancestors, so there is no
+// level barrier: the critical path is the longest chain of crowded nodes.  Every wait is
+// bounded: a wavefront that polls spin_limit times raises the abort flag and all leave.
 template <int RMAX, bool RAVE>
-__global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev f, SelectArgs a, int level) {
+__global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev f, SelectArgs a) {
     __shared__ WaveLds<RMAX> s_lds[kGroupWaves];
     const int lane = threadIdx.x & 63;
     const int wib = threadIdx.x >> 6;
-    const int wave = blockIdx.x * kGroupWaves + wib;
-    if (wave >= a.counters[level]) return;
-    const Item it = level == 0 ? a.items0[wave] : a.items_q[(size_t)(level - 1) * a.stride + wave];
-    int node = it.node;
-    int np = level == 0 ? f.N[node] : it.np;
-    int off = it.off;
-    int m = it.m;
-    int depth = level;
-    if (level == 0) {
-        for (int j = lane; j < m; j += kWave) a.paths[a.seg0[off + j]] = node;
-    }
     for (;;) {
-        const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
-        int32_t *seg_out = a.seg[depth & 1];
-        NodeCtx c = node_ctx(f, a, node, np);
-        bool descended = false;
-        Continuation next;
-        next.node = -1;
-        if (c.cc > 0 && depth < a.max_depth) {
-            if (c.cc <= kWave)
-                descended = select_group<1, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth,
-                                                  reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
-            else
-                descended = select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_lds[wib], next);
-        }
-        if (!descended) {
-            for (int j = lane; j < m; j += kWave) {
-                int t = seg_in[off + j];
-                a.leaf[t] = node;
-                a.path_len[t] = depth + 1;
+        int ticket = 0;
+        if (lane == 0) ticket = atomicAdd(a.sched + 0, 1);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        if (ticket >= a.q_cap) return;
+        bool got = false;
+        for (int spins = 0;; spins++) {
+            int rdy = 0, open = 1, ab = 0;
+            if (lane == 0) {
+                rdy = __hip_atomic_load(a.q_ready + ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
+                if (!rdy && (spins & 3) == 3) {
+                    open = __hip_atomic_load(a.sched + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ab = __hip_atomic_load(a.sched + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
-            if (c.cc > 0 && depth >= a.max_depth && lane == 0) atomicAdd(a.truncated, m);
-            return;
+            rdy = __builtin_amdgcn_readfirstlane(rdy);
+            open = __builtin_amdgcn_readfirstlane(open);
+            ab = __builtin_amdgcn_readfirstlane(ab);
+            if (rdy) {
+                got = true;
+                break;
+            }
+            if (open <= 0 || ab) break;
+            if (spins >= a.spin_limit) {
+                if (lane == 0) atomicExch(a.sched + 3, 1);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(32);
         }
-        if (next.node < 0) return;
-        node = next.node;
-        off = next.off;
-        m = next.m;
-        np = next.np;
-        depth++;
+        if (!got) return;
+        // polling is relaxed (an acquire per poll would drop cached lines for the whole
+        // compute unit every time); one acquire once the item is there
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const Item it = a.items_q[ticket];
+        int node = it.node;
+        int depth = it.depth;
+        int np = depth == 0 ? f.N[node] : it.np;
+        int off = it.off;
+        int m = it.m;
+        if (depth == 0) {
+            for (int j = lane; j < m; j += kWave) a.paths[a.seg0[off + j]] = node;
+        }
+        for (;;) {
+            const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
+            int32_t *seg_out = a.seg[depth & 1];
+            NodeCtx c = node_ctx(f, a, node, np);
+            bool descended = false;
+            Continuation next;
+            next.node = -1;
+            if (c.cc > 0 && depth < a.max_depth) {
+                if (c.cc <= kWave)
+                    descended = select_group<1, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth,
+                                                      reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
+                else
+                    descended =
+                        select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_lds[wib], next);
+            }
+            if (!descended) {
+                for (int j = lane; j < m; j += kWave) {
+                    int t = seg_in[off + j];
+                    a.leaf[t] = node;
+                    a.path_len[t] = depth + 1;
+                }
+                if (lane == 0) {
+                    if (c.cc > 0 && depth >= a.max_depth) atomicAdd(a.truncated, m);
+                    atomicSub(a.sched + 2, m);  // these visitors are done
+                }
+                break;
+            }
+            if (next.node < 0) break;
+            node = next.node;
+            off = next.off;
+            m = next.m;
+            np = next.np;
+            depth++;
+        }
     }
 }
 
@@ -1079,7 +1141,7 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
     const Item it = a.singles_q[wave];
     int node = it.node;
     const int t = it.off;
-    int d = it.m;
+    int d = it.depth;
     int np = it.np;
     if (d == 0) {
         np = f.N[node];
@@ -1113,40 +1175,56 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
     }
 }
 
-// Level counters, statistics, and the single-visitor queue seeded with the traversals
-// that are alone at their root.
-__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0) {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < a.max_depth + 2) a.counters[i] = (i == 0) ? n_items0 : 0;
-    if (i == 0) {
+// Scheduler state, statistics, the work queue seeded with the items of the roots, and the
+// single-visitor queue seeded with the traversals that are alone at their root.
+__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0) {
+    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const int step = gridDim.x * blockDim.x;
+    if (gid == 0) {
         *a.truncated = 0;
         *a.n_singles = n_singles0;
+        a.sched[0] = 0;
+        a.sched[1] = n_items0;
+        a.sched[2] = open0;
+        a.sched[3] = 0;
     }
-    if (a.stats && i < 16) a.stats[i] = 0;
-    if (i < n_singles0) a.singles_q[i] = a.singles0[i];
+    if (a.stats && gid < 16) a.stats[gid] = 0;
+    for (int i = gid; i < n_items0; i += step) {
+        a.items_q[i] = a.items0[i];
+        a.q_ready[i] = a.epoch;
+    }
+    for (int i = gid; i < n_singles0; i += step) a.singles_q[i] = a.singles0[i];
 }
 
 template <int RMAX, bool RAVE>
 static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals,
-                                 hipStream_t s) {
+                                 int n_cus, hipStream_t s) {
     if (n_items0 > 0) {
-        // an item has at least two visitors
-        const int grid = (n_traversals / 2 + kGroupWaves - 1) / kGroupWaves;
-        for (int level = 0; level <= a.max_depth; level++)
-            hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid > 0 ? grid : 1), dim3(kGroupWaves * kWave), 0,
-                               s, f, a, level);
+        // as many wavefronts as can be resident, but no more than there can be items at once
+        // (an item has at least two visitors)
+        int per_cu = 1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_select_groups<RMAX, RAVE>, kGroupWaves * kWave, 0) !=
+                hipSuccess ||
+            per_cu < 1)
+            per_cu = 1;
+        int grid = n_cus * per_cu;
+        const int most = (n_traversals / 2 + kGroupWaves - 1) / kGroupWaves;
+        if (grid > most) grid = most;
+        if (grid < 1) grid = 1;
+        hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kGroupWaves * kWave), 0, s, f, a);
     }
     hipLaunchKernelGGL((k_select_singles<RMAX, RAVE>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
     return hipGetLastError();
 }
 
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
-                         int max_fanout, bool rave, hipStream_t s) {
-    const int n_reset = std::max(std::max(a.max_depth + 2, 8), n_singles0);
-    hipLaunchKernelGGL(k_select_reset, dim3((n_reset + 255) / 256), dim3(256), 0, s, a, n_items0, n_singles0);
-#define OMK_DISPATCH(RM)                                                           \
-    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, s)        \
-                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, s)
+                         int max_fanout, bool rave, int n_cus, hipStream_t s) {
+    int reset_blocks = (n_traversals + 255) / 256;
+    hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
+                       n_traversals - n_singles0);
+#define OMK_DISPATCH(RM)                                                                  \
+    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, s)        \
+                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, s)
     if (max_fanout <= 64) { OMK_DISPATCH(1); }
     if (max_fanout <= 256) { OMK_DISPATCH(4); }
     if (max_fanout <= 384) { OMK_DISPATCH(6); }
