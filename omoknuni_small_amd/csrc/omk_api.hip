@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -67,6 +68,8 @@ struct omk_forest {
     }
 };
 
+constexpr int kSchedStep = 1024;  // int32 words between two scheduler words: 4 KiB
+
 struct omk_batch {
     omk_forest *f = nullptr;
     int32_t max_traversals = 0;
@@ -80,9 +83,11 @@ struct omk_batch {
     int32_t n_singles0 = 0;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
-    // [0] simulations cut by max_depth, [1..16] work statistics, [17] single-visitor queue length,
-    // [18..21] scheduler state of the multi-visitor kernel
+    // [0] simulations cut by max_depth, [1..16] work statistics, [17] single-visitor queue length;
+    // the scheduler words of the multi-visitor kernel follow at 4 KiB steps (kSchedStep), so
+    // that each lies in a memory channel of its own
     int32_t *counters = nullptr;
+    int32_t poll_sleep = 1;
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
     int32_t q_cap = 0;
     int32_t epoch = 0;           // select calls so far
@@ -338,8 +343,8 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, B);
     if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
-    if (e == hipSuccess) e = dalloc(&b->counters, 32);
-    if (e == hipSuccess) e = hipMemset(b->counters, 0, 32 * 4);
+    if (e == hipSuccess) e = dalloc(&b->counters, 4 * kSchedStep);
+    if (e == hipSuccess) e = hipMemset(b->counters, 0, 4 * kSchedStep * 4);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&b->n_cus, hipDeviceAttributeMultiprocessorCount, f->device);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
@@ -467,7 +472,16 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.truncated = b->counters + 0;
     a.stats = b->counters + 1;
     a.n_singles = b->counters + 17;
-    a.sched = b->counters + 18;
+    a.sched_head = b->counters + 1 * kSchedStep;
+    a.sched_tail = b->counters + 2 * kSchedStep;
+    a.sched_wait = b->counters + 3 * kSchedStep;
+    a.poll_sleep = b->poll_sleep;
+#ifdef OMK_PHASE_TIMERS
+    a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
+    a.trace_n = b->counters + 24;
+    a.trace_cap = (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 8);
+    a.dbg_grid = getenv("OMK_DBG_GRID") ? atoi(getenv("OMK_DBG_GRID")) : 0;
+#endif
     a.singles0 = b->singles0;
     a.singles_q = b->singles_q;
     a.sc_child = b->sc_child;
@@ -551,7 +565,7 @@ int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t 
     if (h_path_len) HIP_TRY(hipMemcpyAsync(h_path_len, b->path_len, (size_t)n * 4, hipMemcpyDeviceToHost, s));
     if (h_leaf) HIP_TRY(hipMemcpyAsync(h_leaf, b->leaf, (size_t)n * 4, hipMemcpyDeviceToHost, s));
     int32_t aborted = 0;
-    HIP_TRY(hipMemcpyAsync(&aborted, b->counters + 21, 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipMemcpyAsync(&aborted, b->counters + 3 * kSchedStep + 1, 4, hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     if (aborted)
         return fail(OMK_ERR_STATE,
@@ -579,6 +593,19 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }
+
+#ifdef OMK_PHASE_TIMERS
+// measurement builds only: the per-node timeline of the last selection (4 x int64 per node)
+int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(hipStreamSynchronize(b->f->stream));
+    HIP_TRY(hipMemcpy(h_n, b->counters + 24, 4, hipMemcpyDeviceToHost));
+    int32_t n = std::min(std::min(*h_n, max_entries), (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 8));
+    if (n > 0) HIP_TRY(hipMemcpy(h_trace, b->out_paths, (size_t)n * 32, hipMemcpyDeviceToHost));
+    *h_n = n;
+    return OMK_OK;
+}
+#endif
 
 // ---------------------------------------------------------------- transposition table
 

@@ -42,10 +42,21 @@ struct SelectArgs {
     int32_t *n_singles;
     Item *items_q;         // multi-visitor work queue, q_cap slots, filled front to back
     int32_t *q_ready;      // per slot: == epoch once the item and everything it refers to is written
-    int32_t *sched;        // [0] next ticket, [1] slots handed out, [2] visitors still in multi-visitor
-                           // items, [3] abort flag (a waiting wavefront gave up)
+    // Scheduler words, each on a memory line (and channel) of its own: waiting wavefronts
+    // poll sched_wait, working wavefronts bump the others, and neither queues behind the other.
+    int32_t *sched_head;   // next ticket
+    int32_t *sched_tail;   // slots handed out
+    int32_t *sched_wait;   // [0] visitors still in multi-visitor items, [1] abort flag (a waiting
+                           // wavefront gave up, or the queue overflowed)
+    int32_t poll_sleep;    // s_sleep(32) units between two polls of a waiting wavefront
     int32_t q_cap;
     int32_t epoch;         // number of this select call on the batch, > 0
+#ifdef OMK_PHASE_TIMERS
+    long long *trace;      // per processed node: start, end (100 MHz clock), visitors | depth << 32, node
+    int32_t *trace_n;
+    int32_t trace_cap;
+    int32_t dbg_grid;      // cap on the blocks of the multi-visitor kernel (0 = none)
+#endif
     int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
     int32_t *sc_child;     // per visitor: chosen child index

@@ -965,7 +965,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         n_pushed += nnew;
         if (nnew > 0) {
             int slot0 = 0;
-            if (lane == 0) slot0 = atomicAdd(a.sched + 1, nnew);
+            if (lane == 0) slot0 = atomicAdd(a.sched_tail, nnew);
             slot0 = __builtin_amdgcn_readfirstlane(slot0);
             if (cnt[r] > 1 && i != keep) {
                 int slot = slot0 + __popcll(has & ((1ull << lane) - 1ull));
@@ -980,7 +980,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                     a.items_q[slot] = it;
                     myslot[r] = slot;
                 } else {
-                    atomicExch(a.sched + 3, 2);  // queue overflow: cannot happen on a tree
+                    atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
                 }
             }
         }
@@ -1028,7 +1028,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             if (myslot[r] >= 0)
                 __hip_atomic_store(a.q_ready + myslot[r], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (n_lone > 0 && lane == 0) atomicSub(a.sched + 2, n_lone);  // lone visitors leave the multi-visitor items
+    if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);  // lone visitors leave the multi-visitor items
     next.node = -1;
     if (keep >= 0) {
         next.node = c.cb + keep;
@@ -1055,7 +1055,7 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
     const int wib = threadIdx.x >> 6;
     for (;;) {
         int ticket = 0;
-        if (lane == 0) ticket = atomicAdd(a.sched + 0, 1);
+        if (lane == 0) ticket = atomicAdd(a.sched_head, 1);
         ticket = __builtin_amdgcn_readfirstlane(ticket);
         if (ticket >= a.q_cap) return;
         bool got = false;
@@ -1064,8 +1064,8 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
             if (lane == 0) {
                 rdy = __hip_atomic_load(a.q_ready + ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
                 if (!rdy && (spins & 3) == 3) {
-                    open = __hip_atomic_load(a.sched + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ab = __hip_atomic_load(a.sched + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    open = __hip_atomic_load(a.sched_wait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
             rdy = __builtin_amdgcn_readfirstlane(rdy);
@@ -1077,10 +1077,10 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
             }
             if (open <= 0 || ab) break;
             if (spins >= a.spin_limit) {
-                if (lane == 0) atomicExch(a.sched + 3, 1);
+                if (lane == 0) atomicExch(a.sched_wait + 1, 1);
                 break;
             }
-            __builtin_amdgcn_s_sleep(32);
+            for (int z = 0; z < a.poll_sleep; z++) __builtin_amdgcn_s_sleep(32);
         }
         if (!got) return;
         // polling is relaxed (an acquire per poll would drop cached lines for the whole
@@ -1098,6 +1098,10 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
         for (;;) {
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
             int32_t *seg_out = a.seg[depth & 1];
+#ifdef OMK_PHASE_TIMERS
+            const long long tr0 = wall_clock64();
+            const int tr_m = m, tr_node = node;
+#endif
             NodeCtx c = node_ctx(f, a, node, np);
             bool descended = false;
             Continuation next;
@@ -1110,6 +1114,17 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
                     descended =
                         select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_lds[wib], next);
             }
+#ifdef OMK_PHASE_TIMERS
+            if (lane == 0) {
+                int ti = atomicAdd(a.trace_n, 1);
+                if (ti < a.trace_cap) {
+                    a.trace[4 * ti + 0] = tr0;
+                    a.trace[4 * ti + 1] = wall_clock64();
+                    a.trace[4 * ti + 2] = (long long)tr_m | ((long long)depth << 32);
+                    a.trace[4 * ti + 3] = tr_node;
+                }
+            }
+#endif
             if (!descended) {
                 for (int j = lane; j < m; j += kWave) {
                     int t = seg_in[off + j];
@@ -1118,7 +1133,7 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
                 }
                 if (lane == 0) {
                     if (c.cc > 0 && depth >= a.max_depth) atomicAdd(a.truncated, m);
-                    atomicSub(a.sched + 2, m);  // these visitors are done
+                    atomicSub(a.sched_wait, m);  // these visitors are done
                 }
                 break;
             }
@@ -1183,10 +1198,13 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
     if (gid == 0) {
         *a.truncated = 0;
         *a.n_singles = n_singles0;
-        a.sched[0] = 0;
-        a.sched[1] = n_items0;
-        a.sched[2] = open0;
-        a.sched[3] = 0;
+        *a.sched_head = 0;
+        *a.sched_tail = n_items0;
+        a.sched_wait[0] = open0;
+        a.sched_wait[1] = 0;
+#ifdef OMK_PHASE_TIMERS
+        *a.trace_n = 0;
+#endif
     }
     if (a.stats && gid < 16) a.stats[gid] = 0;
     for (int i = gid; i < n_items0; i += step) {
@@ -1211,6 +1229,9 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
         const int most = (n_traversals / 2 + kGroupWaves - 1) / kGroupWaves;
         if (grid > most) grid = most;
         if (grid < 1) grid = 1;
+#ifdef OMK_PHASE_TIMERS
+        if (a.dbg_grid > 0 && grid > a.dbg_grid) grid = a.dbg_grid;
+#endif
         hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kGroupWaves * kWave), 0, s, f, a);
     }
     hipLaunchKernelGGL((k_select_singles<RMAX, RAVE>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
