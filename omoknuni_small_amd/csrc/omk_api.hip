@@ -89,6 +89,8 @@ struct omk_batch {
     int32_t *counters = nullptr;
     int32_t poll_sleep = 1;
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
+    int32_t *hctx = nullptr;     // contexts of heavy nodes
+    int32_t hctx_cap = 0;
     int32_t q_cap = 0;
     int32_t epoch = 0;           // select calls so far
     int32_t spin_limit = 1 << 22;
@@ -331,8 +333,11 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->leaf, B);
     if (e == hipSuccess) e = dalloc(&b->values, B);
     if (e == hipSuccess) e = dalloc(&b->items0, B);
-    // a multi-visitor item has at least two visitors, and a level holds each visitor once
-    b->q_cap = (int32_t)((B / 2) * (max_depth + 1));
+    // a multi-visitor item has at least two visitors, and a level holds each visitor once; a heavy
+    // node (kHeavyMin visitors or more) adds at most 63 slice items
+    b->q_cap = (int32_t)((B / 2 + B / 16 + 64) * (max_depth + 1));
+    b->hctx_cap = (int32_t)std::min<int64_t>(4096, (B / kHeavyMin) * (max_depth + 1));
+    if (e == hipSuccess) e = dalloc(&b->hctx, (int64_t)b->hctx_cap * kHeavyCtxInts);
     if (e == hipSuccess) e = dalloc(&b->items_q, b->q_cap);
     if (e == hipSuccess) e = dalloc(&b->q_ready, b->q_cap);
     if (e == hipSuccess) e = hipMemset(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4);
@@ -364,7 +369,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q, b->q_ready};
+                    b->singles0, b->singles_q, b->q_ready, b->hctx};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -476,6 +481,10 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.sched_tail = b->counters + 2 * kSchedStep;
     a.sched_wait = b->counters + 3 * kSchedStep;
     a.poll_sleep = b->poll_sleep;
+    a.hctx = b->hctx;
+    a.hctx_n = b->counters + 2 * kSchedStep + 64;
+    a.hctx_cap = b->hctx_cap;
+    static_assert(kHeavyCtxInts >= 16 + OMK_MAX_FANOUT, "context too small");
 #ifdef OMK_PHASE_TIMERS
     a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
     a.trace_n = b->counters + 24;

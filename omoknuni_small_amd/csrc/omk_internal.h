@@ -31,8 +31,11 @@ struct Item {
     int32_t m;      // visitors
     int32_t np;     // N(node) as read by the parent's wavefront
     int32_t depth;  // depth of the node on the visitors' paths
-    int32_t pad[3];
+    int32_t pad[3]; // [0] 0 = node, 1 = slice of a heavy node; [1] context; [2] slice | slices << 16
 };
+
+constexpr int kHeavyCtxInts = 16 + 1024;  // 16 + the widest fan-out
+constexpr int kHeavyMin = 1024;          // visitors from which a node is settled by several wavefronts
 
 struct SelectArgs {
     const Item *items0;    // level-0 items with several visitors, built when the roots are set
@@ -48,6 +51,10 @@ struct SelectArgs {
     int32_t *sched_tail;   // slots handed out
     int32_t *sched_wait;   // [0] visitors still in multi-visitor items, [1] abort flag (a waiting
                            // wavefront gave up, or the queue overflowed)
+    int32_t *hctx;         // contexts of heavy nodes, kHeavyCtxInts each: [0] slices still running,
+                           // [1] a slice failed a check, [16 + i] visits of child i
+    int32_t *hctx_n;       // contexts handed out
+    int32_t hctx_cap;
     int32_t poll_sleep;    // s_sleep(32) units between two polls of a waiting wavefront
     int32_t q_cap;
     int32_t epoch;         // number of this select call on the batch, > 0

@@ -48,6 +48,14 @@ constexpr int kBatchCap = 2048;           // entries put in winner order at a ti
 constexpr int kDigitBits = 10;            // radix digit of that sort
 constexpr int kBins = 1 << kDigitBits;
 constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
+constexpr int kSliceEntries = 512;        // visitors per slice of such a node, about
+constexpr int kMaxSlices = 64;
+constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
+constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
+constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
+constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
+
+enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
 
 // Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
 // multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
@@ -56,6 +64,10 @@ constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-v
     do {                                                                    \
         if (a.stats && lane == 0) atomicExch(a.stats + 7, (code));          \
         return false;                                                       \
+    } while (0)
+#define OMK_NOTE(code)                                             \
+    do {                                                           \
+        if (a.stats && lane == 0) atomicExch(a.stats + 7, (code)); \
     } while (0)
 #define OMK_T0() long long t_phase_ = clock64()
 #define OMK_TICK(slot)                                                              \
@@ -66,6 +78,9 @@ constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-v
     } while (0)
 #else
 #define OMK_FAIL(code) return false
+#define OMK_NOTE(code) \
+    do {               \
+    } while (0)
 #define OMK_T0() \
     do {         \
     } while (0)
@@ -314,20 +329,28 @@ __device__ __forceinline__ int predict_count(int n, float w, float p, int vl, fl
 // LDS, sort them, and keep the first `remaining` of them when this is the last batch.
 // The threshold does not have to be anything in particular: whatever it is, the entries at
 // or above it are played before every entry below it, provided the checks hold.
+//
+// The visitors settled are those with ranks [rank0, rank0 + todo) of the node's winner
+// order, starting from the state in which child i has had tk0[i] visits already (all zero
+// and rank0 = 0 for a whole node; a slice of a heavy node otherwise).
 template <int R, bool RAVE>
 __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
-                                            int off, int m, WaveLds<R> &lds, int (&cnt)[R]) {
+                                            int off, int rank0, int todo, const int (&tk0)[R], WaveLds<R> &lds,
+                                            int (&cnt)[R]) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
-    if (m > kWaterLevelMaxJ) OMK_FAIL(1);
+    const int m = todo;
+    off += rank0;
 
     int tk[R];                    // visits settled so far, per child
     uint32_t headk[R], headp[R];  // the entry each child shows next
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int i = r * kWave + lane;
-        tk[r] = 0;
-        if (k.k2[r] > k.k1[r]) {
+        tk[r] = tk0[r];
+        if (tk0[r] > 0 && k.part[r]) {
+            entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk0[r], i, headk[r], headp[r]);
+        } else if (k.k2[r] > k.k1[r]) {
             headk[r] = k.k2[r];
             headp[r] = (uint32_t)(F + i);
         } else {
@@ -356,6 +379,96 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         wave_best(lbk, lbp, hi_key, hi_pos);
         if (hi_key == 0u) OMK_FAIL(2);
         const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
+
+        // ---- 0. a long run of the best child ----
+        // When the best child's next entries stay ahead of every other child's next entry (its
+        // score hardly moves with virtual loss, e.g. a RAVE blend that dominates), they are the
+        // next winners one after another: count them, check them, emit them without sorting.
+        if (remaining >= kRunShortcutMin) {
+            uint32_t ok2 = 0u, opos2 = 0xFFFFFFFFu;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (r * kWave + lane != best && headk[r] != 0u && comes_before(headk[r], headp[r], ok2, opos2)) {
+                    ok2 = headk[r];
+                    opos2 = headp[r];
+                }
+            uint32_t sk, spos;
+            wave_best(ok2, opos2, sk, spos);
+            int tn = 0, tvl = 0, ttk = 0;
+            float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (r == (best >> 6)) {
+                    tn = k.n[r];
+                    tw = k.w[r];
+                    tp = k.p[r];
+                    tvl = k.vl[r];
+                    tq2 = k.q2[r];
+                    ttk = tk[r];
+                }
+            }
+            const int bl = best & 63;
+            const int bn = __builtin_amdgcn_readlane(tn, bl);
+            const float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), bl));
+            const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), bl));
+            const int bvl = __builtin_amdgcn_readlane(tvl, bl);
+            const float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), bl));
+            const int btk = __builtin_amdgcn_readlane(ttk, bl);
+            // probe: does the run reach kRunShortcutMin entries at all?
+            uint32_t pk_, pp_;
+            entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + kRunShortcutMin - 1, best, pk_, pp_);
+            if (pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos))) {
+                // largest L <= remaining whose last entry still comes before the others' best
+                int lo_l = kRunShortcutMin, hi_l = remaining;
+                while (lo_l < hi_l) {
+                    const int mid_l = (lo_l + hi_l + 1) >> 1;
+                    entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + mid_l - 1, best, pk_, pp_);
+                    if (pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos))) lo_l = mid_l;
+                    else hi_l = mid_l - 1;
+                }
+                const int L = lo_l;
+                // every entry of the run: a real key, never before its predecessor
+                bool bad_run = false;
+                uint32_t carry_k = hi_key, carry_p = hi_pos;
+                for (int base = 0; base < L; base += kWave) {
+                    const int j = base + lane;
+                    uint32_t kk = 0u, pp = 0xFFFFFFFFu;
+                    if (j < L) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + j, best, kk, pp);
+                    uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+                    uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+                    if (lane == 0) {
+                        pk = carry_k;
+                        ppos = carry_p;
+                    }
+                    if (j < L && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad_run = true;
+                    if (j < L && j == L - 1 && sk != 0u && !comes_before(kk, pp, sk, spos)) bad_run = true;
+                    carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+                    carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+                }
+                // the entry after the run must not come before the run's last one either
+                uint32_t nk, np2, lk_, lp_;
+                entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L, best, nk, np2);
+                entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L - 1, best, lk_, lp_);
+                if (nk != 0u && comes_before(nk, np2, lk_, lp_)) bad_run = true;
+                if (__ballot(bad_run) == 0ull) {
+                    for (int j = lane; j < L; j += kWave) {
+                        a.sc_child[off + done + j] = best;
+                        a.sc_occ[off + done + j] = btk + j;
+                    }
+                    if (lane == bl) {
+#pragma unroll
+                        for (int r = 0; r < R; r++)
+                            if (r == (best >> 6)) {
+                                tk[r] = btk + L;
+                                headk[r] = nk;
+                                headp[r] = np2;
+                            }
+                    }
+                    done += L;
+                    continue;
+                }
+            }
+        }
         const int want = remaining < kBatchCap ? remaining : kBatchCap;
         // lower bound of any useful threshold: the best child alone has `want` entries at or
         // above the key of its want-th next visit
@@ -772,6 +885,104 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
     return true;
 }
 
+// For a heavy node: a score threshold at or above which about `target` of the node's
+// entries lie (estimated), and EXACTLY how many entries of every own child lie at or above
+// it (ct, at most m each).  Every wavefront that asks for the same target gets the same
+// threshold: the computation is deterministic and depends on the node's state only.
+template <int R, bool RAVE>
+__device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const NodeCtx &c, int lane,
+                                                 const Kids<R, RAVE> &k, int m, int target, int (&ct)[R],
+                                                 uint32_t &T_out) {
+    constexpr int F = R * kWave;
+    const uint32_t uvl = (uint32_t)a.vl;
+    uint32_t headk[R];
+    uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        uint32_t hp;
+        if (k.k2[r] > k.k1[r]) {
+            headk[r] = k.k2[r];
+            hp = (uint32_t)(F + i);
+        } else {
+            headk[r] = k.k1[r];
+            hp = (uint32_t)i;
+        }
+        if (headk[r] != 0u && comes_before(headk[r], hp, lbk, lbp)) {
+            lbk = headk[r];
+            lbp = hp;
+        }
+    }
+    uint32_t hi_key, hi_pos;
+    wave_best(lbk, lbp, hi_key, hi_pos);
+    if (hi_key == 0u) return false;
+    const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
+    // The best child alone has m entries at or above the key of its m-th visit: a lower bound
+    // for every threshold of the node.  All targets bisect the SAME interval, so that their
+    // thresholds come out ordered like the targets (two searches see the same midpoints until
+    // they part, and from then on one interval lies above the other).
+    uint32_t lo_key = 0u;
+    {
+        uint32_t kk = 0u, pp = 0u;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (r == (best >> 6))
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, m - 1, best, kk, pp);
+        }
+        lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
+    }
+    if (lo_key == 0u) lo_key = 1u;
+    if (lo_key > hi_key) return false;
+    // bisection on the key itself, down to neighbouring binary32 values: where thousands of
+    // entries crowd into a sliver of the score range (a child whose score hardly moves with
+    // virtual loss) the thresholds of different targets still come apart
+    uint32_t klo = lo_key, khi = hi_key;  // est(klo) >= target is taken for granted, est(khi) < target
+    while (khi - klo > 1u) {
+        const uint32_t kmid = klo + ((khi - klo) >> 1);
+        const float mid = key_score(kmid);
+        int est = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (k.part[r] && headk[r] >= lo_key)
+                est += predict_count<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, mid, m);
+        if (wave_sum_i32(est) >= target) klo = kmid;
+        else khi = kmid;
+    }
+    const uint32_t T = klo;
+    const float tau = key_score(T);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        ct[r] = 0;
+        if (k.part[r] && headk[r] >= T) {
+            const int i = r * kWave + lane;
+            int lo_c = 1, hi_c = m;  // the first entry itself is at or above T
+            int g = predict_count<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tau, m);
+            g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
+            uint32_t kk, pp;
+            if (g > lo_c) {
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, g - 1, i, kk, pp);
+                if (kk >= T) lo_c = g;
+                else hi_c = g - 1;
+            }
+            if (lo_c == g && g < hi_c) {
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, g, i, kk, pp);
+                if (kk >= T) lo_c = g + 1;
+                else hi_c = g;
+            }
+            while (lo_c < hi_c) {
+                int t = (lo_c + hi_c + 1) >> 1;
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, t - 1, i, kk, pp);
+                if (kk >= T) lo_c = t;
+                else hi_c = t - 1;
+            }
+            ct[r] = lo_c;
+        }
+    }
+    if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
+    T_out = T;
+    return true;
+}
+
 // The commonest crowded node: one child wins every time.  That is the case exactly when
 // the score it shows to the last visitor still comes before the first score of every
 // other child and its own scores never increase on the way; both are checked on the exact
@@ -859,15 +1070,27 @@ struct Continuation {
 
 // All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
 // virtual loss, partitions the visitors by child into seg_out, writes the next path
-// entry; children with several visitors become items of the next level's queue, children
-// with one visitor go to the single-visitor queue (none when all visitors chose the same
-// child: then the caller walks on with them).  Returns false when no child takes part in
-// the selection.
+// entry; the largest part stays with this wavefront (next), the other parts with several
+// visitors become items of the work queue, children with one visitor go to the
+// single-visitor queue.  Returns kStepLeaf when no child takes part in the selection.
+//
+// A heavy node (kHeavyMin visitors or more) is cut into slices of its winner order, one
+// queue item each, that wavefronts settle side by side: slice s covers the ranks between
+// the exact entry counts at two score thresholds, T_s and T_s+1, which every slice derives
+// for itself (threshold_counts: same input, same result).  A slice starts the batch loop
+// from the state "child i has had count_i(T_s) visits" and must arrive exactly at
+// count_i(T_s+1); with that check, T_s >= T_s+1, and the batch loop's own checks, slice
+// after slice starts from the true serial state, so the slices together are the serial
+// order.  The slice that reaches the last visitor writes the visits per child; the
+// wavefront that finishes last (a counter in the node's context) partitions the visitors
+// and walks on, every other returns kStepParked.  Any failed check sends the whole node
+// back to the one-wavefront path.
 template <int R, bool RAVE>
-__device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
-                                             const int32_t *seg_in, int32_t *seg_out, int off, int m, int depth,
-                                             WaveLds<R> &lds, Continuation &next) {
+__device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
+                                            const Item &item, const int32_t *seg_in, int32_t *seg_out,
+                                            WaveLds<R> &lds, Continuation &next) {
     OMK_T0();
+    const int off = item.off, m = item.m, depth = item.depth;
     Kids<R, RAVE> k;
     int cnt[R];
     load_kids<R, RAVE>(f, c.cb, c.nelig, lane, a.rave_k, k);
@@ -883,16 +1106,144 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
 
     bool settled = false;
     int st_replay = 0;
-    if (m >= kRunMin && a.vl > 0) settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, cnt);
-    if (!settled && m >= kWaterLevelMin && a.vl > 0) {
-        settled = water_level<R, RAVE>(a, c, lane, k, off, m, lds, cnt);
+    bool as_slice = item.pad[0] == 1;
+    const bool as_scatter = item.pad[0] == 2;
+    int hid = item.pad[0] != 0 ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF, n_slices = item.pad[2] >> 16;
+    if (as_scatter) {
+        // a part of the partition of a heavy node: the visits per child are in its context
+        const int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
+#pragma unroll
+        for (int r = 0; r < R; r++) cnt[r] = ctx[16 + r * kWave + lane];
+        settled = true;
+    }
+    if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
+        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, cnt);
+    if (R * kWave <= kHeavyFanout) {
+        if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
+            // cut the node into slices: the others go to the queue, this wavefront takes the first
+            const int K = (m + kSliceEntries - 1) / kSliceEntries < kMaxSlices ? (m + kSliceEntries - 1) / kSliceEntries
+                                                                               : kMaxSlices;
+            int id = a.hctx_cap;
+            if (lane == 0) id = atomicAdd(a.hctx_n, 1);
+            id = __builtin_amdgcn_readfirstlane(id);
+            if (id < a.hctx_cap) {
+                int slot0 = 0;
+                if (lane == 0) slot0 = atomicAdd(a.sched_tail, K - 1);
+                slot0 = __builtin_amdgcn_readfirstlane(slot0);
+                if (slot0 + K - 1 <= a.q_cap) {
+                    int *ctx = a.hctx + (size_t)id * kHeavyCtxInts;
+                    if (lane == 0) {
+                        ctx[0] = K;
+                        ctx[1] = 0;
+                    }
+                    if (lane < K - 1) {
+                        Item it = item;
+                        it.pad[0] = 1;
+                        it.pad[1] = id;
+                        it.pad[2] = (lane + 1) | (K << 16);
+                        a.items_q[slot0 + lane] = it;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                    if (lane < K - 1)
+                        __hip_atomic_store(a.q_ready + slot0 + lane, a.epoch, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    as_slice = true;
+                    hid = id;
+                    slice = 0;
+                    n_slices = K;
+                    if (a.stats && lane == 0) atomicAdd(a.stats + 15, 1);
+                } else if (lane == 0) {
+                    atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
+                }
+            }
+        }
+        if (as_slice) {
+            int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
+            const int S = (m + n_slices - 1) / n_slices;
+            const bool last = slice == n_slices - 1;
+            int ct_hi[R], ct_lo[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) ct_hi[r] = ct_lo[r] = 0;
+            bool ok = true;
+            int rank_hi = 0, rank_lo = m;
+            uint32_t T_hi = 0xFFFFFFFFu, T_lo = 0u;
+            if (slice > 0) {
+                ok = threshold_counts<R, RAVE>(a, c, lane, k, m, slice * S, ct_hi, T_hi);
+                if (!ok) OMK_NOTE(20);
+                int sum = 0;
+#pragma unroll
+                for (int r = 0; r < R; r++) sum += ct_hi[r];
+                rank_hi = wave_sum_i32(sum);
+            }
+            if (ok && !last) {
+                ok = threshold_counts<R, RAVE>(a, c, lane, k, m, (slice + 1) * S, ct_lo, T_lo);
+                int sum = 0;
+                bool bad = false;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    sum += ct_lo[r];
+                    if (ct_lo[r] < ct_hi[r]) bad = true;
+                }
+                rank_lo = wave_sum_i32(sum);
+                if (!ok) OMK_NOTE(21);
+                if (T_lo > T_hi || __ballot(bad) != 0ull) {
+                    ok = false;
+                    OMK_NOTE(22);
+                }
+            }
+            if (ok && rank_hi < m) {
+                const bool closing = last || rank_lo >= m;
+                const int todo = (closing ? m : rank_lo) - rank_hi;
+                if (todo > 0) {
+                    ok = water_level<R, RAVE>(a, c, lane, k, off, rank_hi, todo, ct_hi, lds, cnt);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < R; r++) cnt[r] = ct_hi[r];
+                }
+                if (ok && closing) {
+#pragma unroll
+                    for (int r = 0; r < R; r++) ctx[16 + r * kWave + lane] = cnt[r];
+                } else if (ok) {
+                    bool bad = false;
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                        if (cnt[r] != ct_lo[r]) bad = true;
+                    if (__ballot(bad) != 0ull) {
+                        ok = false;
+                        OMK_NOTE(23);
+                    }
+                }
+            }
+            if (!ok && lane == 0) atomicExch(ctx + 1, 1);
+            // join: the wavefront that finishes last goes on with the node
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            int before = 0;
+            if (lane == 0) before = atomicSub(ctx + 0, 1);
+            before = __builtin_amdgcn_readfirstlane(before);
+            if (before != 1) return kStepParked;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            const int failed = __hip_atomic_load(ctx + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                cnt[r] = failed ? 0
+                                : __hip_atomic_load(ctx + 16 + r * kWave + lane, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+            settled = !failed;
+            if (failed) st_replay = 1;
+        }
+    }
+    if (!settled && m >= kWaterLevelMin && m <= kWaterLevelMaxJ && a.vl > 0) {
+        int zero[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) zero[r] = 0;
+        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt);
         if (!settled) st_replay = 1;
     }
     if (!settled) {
         // one visitor after the other
         for (int done = 0; done < m; done++) {
             int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
-            if (i < 0) return false;  // no child takes part: uniform, and then for every visitor
+            if (i < 0) return kStepLeaf;  // no child takes part: uniform, and then for every visitor
             if (a.vl <= 0) {
                 // no virtual loss: nothing changes between visitors, they all follow the first
                 for (int j = lane; j < m; j += kWave) {
@@ -924,7 +1275,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         }
     }
     OMK_TICK(13);
-    if (a.stats && lane == 0) {
+    if (a.stats && lane == 0 && !as_scatter) {
         atomicAdd(a.stats + 0, 1);
         atomicAdd(a.stats + 1, settled ? 1 : 0);
         atomicAdd(a.stats + 2, settled ? m : 0);
@@ -932,6 +1283,8 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
         atomicAdd(a.stats + 4, st_replay);
     }
 
+    // ---- partition of the visitors by chosen child ----
+    // (1) from the visits per child: the segment of every child, in LDS for all lanes
     uint32_t lmax = 0u;
 #pragma unroll
     for (int r = 0; r < R; r++) lmax = umax32(lmax, (uint32_t)cnt[r]);
@@ -943,23 +1296,138 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     // This wavefront walks on with the largest part; the other parts go to the work queue,
     // where idle wavefronts pick them up at once.
     const int keep = gmax >= 2u ? (int)wave_min_u32(lidx) : -1;
-
-    // exclusive prefix of the visit counts in child order -> segment of every child
     int carry = 0;
     int keep_np = 0;
-    int myslot[R];
-    int n_lone = 0, n_pushed = 0;
+    int excl[R];
+    int n_lone = 0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         int inc = wave_inclusive_sum(cnt[r], lane);
-        int excl = carry + inc - cnt[r];
+        excl[r] = carry + inc - cnt[r];
         int i = r * kWave + lane;
-        lds.offs[i] = excl;
+        lds.offs[i] = excl[r];
         lds.st_j0[i] = cnt[r];
         lds.st_n[i] = k.n[r];
         if (i == keep) keep_np = k.n[r];
-        myslot[r] = -1;
         n_lone += __popcll(__ballot(cnt[r] == 1));
+        carry += __builtin_amdgcn_readlane(inc, 63);
+    }
+    wave_sync_memory();
+
+    // (2) the scatter; for a heavy node it is shared out in parts of the visitor list, again
+    // through the queue, and the wavefront that finishes last goes on
+    int r0 = 0, r1 = m;
+    bool shared = false;
+    if (R * kWave <= kHeavyFanout) {
+        int part = 0, n_parts = 1;
+        if (as_scatter) {
+            part = slice;
+            n_parts = n_slices;
+            shared = true;
+        } else if (m >= kHeavyMin) {
+            if (hid < 0) {
+                int id = a.hctx_cap;
+                if (lane == 0) id = atomicAdd(a.hctx_n, 1);
+                id = __builtin_amdgcn_readfirstlane(id);
+                if (id < a.hctx_cap) hid = id;
+            }
+            const int K2 = (m + kScatterPart - 1) / kScatterPart < kMaxSlices ? (m + kScatterPart - 1) / kScatterPart
+                                                                             : kMaxSlices;
+            if (hid >= 0) {
+                int slot0 = 0;
+                if (lane == 0) slot0 = atomicAdd(a.sched_tail, K2 - 1);
+                slot0 = __builtin_amdgcn_readfirstlane(slot0);
+                if (slot0 + K2 - 1 <= a.q_cap) {
+                    int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
+#pragma unroll
+                    for (int r = 0; r < R; r++) ctx[16 + r * kWave + lane] = cnt[r];
+                    if (lane == 0) ctx[2] = K2;
+                    if (lane < K2 - 1) {
+                        Item it = item;
+                        it.pad[0] = 2;
+                        it.pad[1] = hid;
+                        it.pad[2] = (lane + 1) | (K2 << 16);
+                        a.items_q[slot0 + lane] = it;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                    if (lane < K2 - 1)
+                        __hip_atomic_store(a.q_ready + slot0 + lane, a.epoch, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                    n_parts = K2;
+                    shared = true;
+                } else if (lane == 0) {
+                    atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
+                }
+            }
+        }
+        if (shared) {
+            const int per = (((m + n_parts - 1) / n_parts) + kWave - 1) & ~(kWave - 1);
+            r0 = part * per < m ? part * per : m;
+            r1 = r0 + per < m ? r0 + per : m;
+        }
+    }
+    int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
+    // kScatterUnroll chunks of 64 visitors at a time: their loads are issued together, so the
+    // loop pays the memory latency once per group of chunks instead of once per chunk
+    for (int base = r0; base < r1; base += kScatterUnroll * kWave) {
+        int tt[kScatterUnroll], ii[kScatterUnroll], oo[kScatterUnroll];
+#pragma unroll
+        for (int u = 0; u < kScatterUnroll; u++) {
+            const int j = base + u * kWave + lane;
+            const bool in = j < r1;
+            tt[u] = in ? seg_in[off + j] : 0;
+            ii[u] = in ? a.sc_child[off + j] : 0;
+            oo[u] = in ? a.sc_occ[off + j] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kScatterUnroll; u++) {
+            if (base + u * kWave >= r1) break;
+            const bool in = base + u * kWave + lane < r1;
+            const int t = tt[u], i = ii[u];
+            bool lone = false;
+            if (in) {
+                path_next[t] = c.cb + i;
+                seg_out[off + lds.offs[i] + oo[u]] = t;
+                lone = lds.st_j0[i] == 1;
+            }
+            // a visitor that is now alone goes to the single-visitor walk
+            uint64_t lm = __ballot(lone);
+            if (lm != 0ull) {
+                int s0 = 0;
+                if (lane == 0) s0 = atomicAdd(a.n_singles, __popcll(lm));
+                s0 = __builtin_amdgcn_readfirstlane(s0);
+                if (lone) {
+                    Item it;
+                    it.node = c.cb + i;
+                    it.off = t;
+                    it.m = 1;
+                    it.np = lds.st_n[i];
+                    it.depth = depth + 1;
+                    it.pad[0] = it.pad[1] = it.pad[2] = 0;
+                    a.singles_q[s0 + __popcll(lm & ((1ull << lane) - 1ull))] = it;
+                }
+            }
+        }
+    }
+    if (shared) {
+        int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        int before = 0;
+        if (lane == 0) before = atomicSub(ctx + 2, 1);
+        before = __builtin_amdgcn_readfirstlane(before);
+        if (before != 1) return kStepParked;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+
+    // (3) virtual loss of the chosen children, and the parts with several visitors that this
+    // wavefront does not keep become items of the queue: everything they refer to is written,
+    // make it visible to the whole device, then mark them ready
+    int myslot[R];
+    int n_pushed = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        myslot[r] = -1;
         uint64_t has = __ballot(cnt[r] > 1 && i != keep);
         int nnew = __popcll(has);
         n_pushed += nnew;
@@ -972,7 +1440,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
                 if (slot < a.q_cap) {
                     Item it;
                     it.node = c.cb + i;
-                    it.off = off + excl;
+                    it.off = off + excl[r];
                     it.m = cnt[r];
                     it.np = k.n[r];
                     it.depth = depth + 1;
@@ -985,42 +1453,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
             }
         }
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
-        carry += __builtin_amdgcn_readlane(inc, 63);
     }
-    wave_sync_memory();
-    int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
-    for (int base = 0; base < m; base += kWave) {
-        const int j = base + lane;
-        const bool in = j < m;
-        int t = 0, i = 0;
-        bool lone = false;
-        if (in) {
-            t = seg_in[off + j];
-            i = a.sc_child[off + j];
-            path_next[t] = c.cb + i;
-            seg_out[off + lds.offs[i] + a.sc_occ[off + j]] = t;
-            lone = lds.st_j0[i] == 1;
-        }
-        // a visitor that is now alone goes to the single-visitor walk
-        uint64_t lm = __ballot(lone);
-        if (lm != 0ull) {
-            int s0 = 0;
-            if (lane == 0) s0 = atomicAdd(a.n_singles, __popcll(lm));
-            s0 = __builtin_amdgcn_readfirstlane(s0);
-            if (lone) {
-                Item it;
-                it.node = c.cb + i;
-                it.off = t;
-                it.m = 1;
-                it.np = lds.st_n[i];
-                it.depth = depth + 1;
-                it.pad[0] = it.pad[1] = it.pad[2] = 0;
-                a.singles_q[s0 + __popcll(lm & ((1ull << lane) - 1ull))] = it;
-            }
-        }
-    }
-    // publish the new items: everything they refer to is written, make it visible to the
-    // whole device first
     if (n_pushed > 0) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
 #pragma unroll
@@ -1039,7 +1472,7 @@ __device__ __forceinline__ bool select_group(const ForestDev &f, const SelectArg
     // the next step of the walk reads seg_out and reuses the LDS scratch
     wave_sync_memory();
     OMK_TICK(14);
-    return true;
+    return kStepDescended;
 }
 
 // Multi-visitor items: a persistent kernel over a device-side work queue.  A wavefront takes
@@ -1086,33 +1519,28 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
         // polling is relaxed (an acquire per poll would drop cached lines for the whole
         // compute unit every time); one acquire once the item is there
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const Item it = a.items_q[ticket];
-        int node = it.node;
-        int depth = it.depth;
-        int np = depth == 0 ? f.N[node] : it.np;
-        int off = it.off;
-        int m = it.m;
-        if (depth == 0) {
-            for (int j = lane; j < m; j += kWave) a.paths[a.seg0[off + j]] = node;
+        Item it = a.items_q[ticket];
+        if (it.depth == 0 && it.pad[0] == 0) {
+            it.np = f.N[it.node];
+            for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
         for (;;) {
+            const int depth = it.depth;
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
             int32_t *seg_out = a.seg[depth & 1];
 #ifdef OMK_PHASE_TIMERS
             const long long tr0 = wall_clock64();
-            const int tr_m = m, tr_node = node;
 #endif
-            NodeCtx c = node_ctx(f, a, node, np);
-            bool descended = false;
+            NodeCtx c = node_ctx(f, a, it.node, it.np);
+            int status = kStepLeaf;
             Continuation next;
             next.node = -1;
             if (c.cc > 0 && depth < a.max_depth) {
                 if (c.cc <= kWave)
-                    descended = select_group<1, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth,
-                                                      reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
+                    status = select_group<1, RAVE>(f, a, c, lane, it, seg_in, seg_out,
+                                                   reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
                 else
-                    descended =
-                        select_group<RMAX, RAVE>(f, a, c, lane, seg_in, seg_out, off, m, depth, s_lds[wib], next);
+                    status = select_group<RMAX, RAVE>(f, a, c, lane, it, seg_in, seg_out, s_lds[wib], next);
             }
 #ifdef OMK_PHASE_TIMERS
             if (lane == 0) {
@@ -1120,29 +1548,31 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
                 if (ti < a.trace_cap) {
                     a.trace[4 * ti + 0] = tr0;
                     a.trace[4 * ti + 1] = wall_clock64();
-                    a.trace[4 * ti + 2] = (long long)tr_m | ((long long)depth << 32);
-                    a.trace[4 * ti + 3] = tr_node;
+                    a.trace[4 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
+                    a.trace[4 * ti + 3] = it.node;
                 }
             }
 #endif
-            if (!descended) {
-                for (int j = lane; j < m; j += kWave) {
-                    int t = seg_in[off + j];
-                    a.leaf[t] = node;
+            if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
+            if (status == kStepLeaf) {
+                for (int j = lane; j < it.m; j += kWave) {
+                    int t = seg_in[it.off + j];
+                    a.leaf[t] = it.node;
                     a.path_len[t] = depth + 1;
                 }
                 if (lane == 0) {
-                    if (c.cc > 0 && depth >= a.max_depth) atomicAdd(a.truncated, m);
-                    atomicSub(a.sched_wait, m);  // these visitors are done
+                    if (c.cc > 0 && depth >= a.max_depth) atomicAdd(a.truncated, it.m);
+                    atomicSub(a.sched_wait, it.m);  // these visitors are done
                 }
                 break;
             }
             if (next.node < 0) break;
-            node = next.node;
-            off = next.off;
-            m = next.m;
-            np = next.np;
-            depth++;
+            it.node = next.node;
+            it.off = next.off;
+            it.m = next.m;
+            it.np = next.np;
+            it.depth = depth + 1;
+            it.pad[0] = it.pad[1] = it.pad[2] = 0;
         }
     }
 }
@@ -1202,6 +1632,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         *a.sched_tail = n_items0;
         a.sched_wait[0] = open0;
         a.sched_wait[1] = 0;
+        *a.hctx_n = 0;
 #ifdef OMK_PHASE_TIMERS
         *a.trace_n = 0;
 #endif
