@@ -205,12 +205,13 @@ def main():
     batch.backup(vl)
     forest.sync()
     sel_bytes, bak_bytes, n_sel_steps = algorithmic_bytes(soa, meta, paths, plen, N_now)
-    # selection = 1 reset + (D+1) launches of the multi-visitor kernel (when any traversals share a
-    # root) + 1 launch of the single-visitor kernel; the roofline is quoted per launch of the kernel
-    # that carries the work, with the whole selection phase as its time
+    # selection = 1 reset + 1 launch of the multi-visitor kernel (a persistent kernel over a work
+    # queue; only when any traversals share a root) + 1 launch of the single-visitor kernel; the
+    # roofline is quoted for the kernel that carries the work, with the whole selection phase
+    # (HIP events around it on the forest's stream) as its launch duration
     has_groups = len(np.unique(troots)) < B
     dominant = "k_select_groups" if has_groups else "k_select_singles"
-    launches_per_select = (D + 1) if has_groups else 1
+    launches_per_select = 1
     sel_ms_step = sel_ms / K
     bak_ms_step = bak_ms / K
     achieved = sel_bytes / (sel_ms_step * 1e-3) / 1e9

@@ -531,6 +531,10 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const bool can_finish = remaining + 2 * margin <= kBatchCap;
         int target = can_finish ? remaining + margin : kBatchCap - margin;
         if (target < 1) OMK_FAIL(4);
+        // No child can win more than the visits that are left: its entries beyond that are
+        // never looked at (the batch is cut at `remaining` entries anyway, and such a child's
+        // last counted entry lies at or after that cut).
+        const int child_cap = remaining < kBatchCap + 1 ? remaining : kBatchCap + 1;
         int ct[R];
         int total = 0;
         int tries = 0;
@@ -545,7 +549,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
 #pragma unroll
                 for (int r = 0; r < R; r++)
                     if (r < rounds && ac[r] >= 0)
-                        est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, kBatchCap);
+                        est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, child_cap);
                 if (wave_sum_i32(est) >= target) flo = mid;
                 else fhi = mid;
             }
@@ -559,8 +563,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             for (int r = 0; r < R; r++) {
                 ct[r] = 0;
                 if (r < rounds && ac[r] >= 0 && ahead[r] >= T) {
-                    int lo_c = 1, hi_c = kBatchCap + 1;  // the next entry itself is at or above T
-                    int g = predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, tau, kBatchCap);
+                    int lo_c = 1, hi_c = child_cap;  // the next entry itself is at or above T
+                    int g = predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, tau, child_cap);
                     g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
                     uint32_t kk, pp;
                     if (g > lo_c) {
