@@ -45,8 +45,8 @@ constexpr int kRunMin = 4;                // visitors from which the one-winner 
 constexpr int kWaterLevelMin = 24;        // visitors from which the parallel path is tried
 constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in the sort payload
 constexpr int kBatchCap = 2048;           // entries put in winner order at a time (LDS resident)
-constexpr int kDigitBits = 10;            // radix digit of that sort
-constexpr int kBins = 1 << kDigitBits;
+constexpr int kSortBits = 4;              // radix digit of that sort
+constexpr int kSortBins = 1 << kSortBits;
 constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
 constexpr int kSliceEntries = 512;        // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
@@ -113,11 +113,10 @@ struct WaveLds {
     int st_vl[R * kWave];
     float st_q2[R * kWave];
     int st_j0[R * kWave];  // visits already settled / visit count, by phase
-    int hist[kBins];
-    uint32_t key[kBatchCap];  // entries of the batch being ordered
-    uint32_t pay[kBatchCap];   // per child: entries of the batch
-    uint32_t pay2[kBatchCap];  // per entry: pass flag, child, visit number
-    uint16_t idx[2][kBatchCap];
+    int hist[kSortBins * kWave + kSortBins * kWave / 16];  // sort: one counter per (digit value, lane), padded
+    uint32_t pay[R * kWave];         // per child: entries of the batch
+    uint32_t key[2][kBatchCap];      // entries of the batch being ordered: inverted score key ...
+    uint32_t pay2[2][kBatchCap];     // ... and pass flag, child, visit number; two buffers, ping-pong
 };
 
 template <int R, bool RAVE>
@@ -495,9 +494,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             const int i = r * kWave + lane;
             const bool act = headk[r] != 0u && headk[r] >= lo_key;
             const uint64_t am = __ballot(act);
-            if (act) lds.idx[1][n_act + __popcll(am & ((1ull << lane) - 1ull))] = (uint16_t)i;
+            if (act) lds.pay2[1][n_act + __popcll(am & ((1ull << lane) - 1ull))] = (uint32_t)i;
             n_act += __popcll(am);
-            lds.key[i] = headk[r];  // key of the child's next entry
+            lds.key[1][i] = headk[r];  // key of the child's next entry
             lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
             lds.st_j0[i] = tk[r];
             lds.pay[i] = 0u;  // result: entries of the batch
@@ -515,14 +514,14 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             aw[r] = ap[r] = aq2[r] = 0.0f;
             ahead[r] = 0u;
             if (r < rounds && r * kWave + lane < n_act) {
-                const int ci = (int)lds.idx[1][r * kWave + lane];
+                const int ci = (int)lds.pay2[1][r * kWave + lane];
                 ac[r] = ci;
                 an[r] = lds.st_n[ci];
                 aw[r] = lds.st_w[ci];
                 ap[r] = lds.st_p[ci];
                 avl[r] = lds.st_vl[ci];
                 aq2[r] = lds.st_q2[ci];
-                ahead[r] = lds.key[ci];
+                ahead[r] = lds.key[1][ci];
             }
         }
         // the estimate is off by about one entry per active child: aim a margin above what is
@@ -550,8 +549,18 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 for (int r = 0; r < R; r++)
                     if (r < rounds && ac[r] >= 0)
                         est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, child_cap);
-                if (wave_sum_i32(est) >= target) flo = mid;
-                else fhi = mid;
+                const int e = wave_sum_i32(est);
+                if (e >= target) {
+                    flo = mid;
+                    // close enough: a quarter more entries than aimed at cost less than more steps
+                    if (e <= target + (target >> 2) && e <= kBatchCap - margin) break;
+                } else {
+                    fhi = mid;
+                    if (!can_finish && e >= target - (target >> 2)) {
+                        flo = mid;  // a batch that cannot finish anyway may as well be a little smaller
+                        break;
+                    }
+                }
             }
             uint32_t T = score_key(flo);
             if (T < lo_key) T = lo_key;
@@ -692,8 +701,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 const int jl = q - lds.offs[child];
                 uint32_t kk, pp;
                 entry_key<R, RAVE>(sn, sw, sp, svl, sq2, c.ep, uvl, jl, child, kk, pp);
-                lds.key[q] = ~kk;
-                lds.pay2[q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)(sj0 + jl);
+                lds.key[0][q] = ~kk;
+                lds.pay2[0][q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)(sj0 + jl);
                 kmin = umin32(kmin, ~kk);
                 kmax = umax32(kmax, ~kk);
                 if (pp >= (uint32_t)F) any_second = true;
@@ -724,67 +733,134 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
 
         // ---- 3. stable radix sort of the batch, in LDS ----
         // Order wanted: key descending, then candidate position ascending, then visit number.
-        // The entries start in (child, visit) order; least significant digit first, a 1-bit
-        // pass on the scan kind (only when both kinds occur: candidates of the first scan sit
-        // before those of the second) and then the key digits, over the bits that differ.
-        const uint32_t diff = kmin ^ kmax;
-        const int nbits = diff == 0u ? 0 : 32 - __clz((int)diff);
+        // The entries start in (child, visit) order; least significant digit first, a pass on
+        // the scan kind (only when both kinds occur: candidates of the first scan sit before
+        // those of the second) and then the key digits, over the bits that differ.
+        // One pass: every lane owns a contiguous block of the current order, counts its digits
+        // in registers (sixteen 8-bit counters), a scan over (digit value, lane) turns the
+        // counts into start positions, kept in LDS per (digit value, lane), and every lane moves
+        // its block in order.  No two lanes share a counter, so the order inside a digit value
+        // is (lane, position in block): stable.
+        // A small batch (two entries per lane at most) is ranked by comparing every entry with
+        // every other one instead, through lane reads.
+        const uint32_t range = kmax - kmin;
+        const int nbits = range == 0u ? 0 : 32 - __clz((int)range);
         const bool mixed = __ballot(any_first) != 0ull && __ballot(any_second) != 0ull;
-        int cur = -1;  // -1: identity order, else lds.idx[cur]
-        for (int sh = mixed ? -kDigitBits : 0; sh < nbits; sh += kDigitBits) {
-            wave_sync_memory();
-#pragma unroll
-            for (int t = 0; t < kBins / kWave; t++) lds.hist[t * kWave + lane] = 0;
-            wave_sync_memory();
-            for (int q = lane; q < total; q += kWave) {
-                const int i = cur < 0 ? q : (int)lds.idx[cur][q];
-                const uint32_t d = sh < 0 ? lds.pay2[i] >> 31 : (lds.key[i] >> sh) & (uint32_t)(kBins - 1);
-                atomicAdd(&lds.hist[d], 1);
+        int cur = 0;
+        if (total <= 2 * kWave) {
+            // entry q of the batch: (key, kind bit | q) compared as a pair; entries lane and 64 + lane
+            const bool in0 = lane < total, in1 = kWave + lane < total;
+            const uint32_t k0 = in0 ? lds.key[0][lane] : 0xFFFFFFFFu, k1 = in1 ? lds.key[0][kWave + lane] : 0xFFFFFFFFu;
+            const uint32_t p0 = in0 ? lds.pay2[0][lane] : 0u, p1 = in1 ? lds.pay2[0][kWave + lane] : 0u;
+            const uint32_t t0 = in0 ? (p0 & 0x80000000u) | (uint32_t)lane : 0xFFFFFFFFu;
+            const uint32_t t1 = in1 ? (p1 & 0x80000000u) | (uint32_t)(kWave + lane) : 0xFFFFFFFFu;
+            int rank0 = 0, rank1 = 0;
+            const int n0 = total < kWave ? total : kWave;
+            for (int s = 0; s < n0; s++) {
+                const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k0, s);
+                const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t0, s);
+                rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
+                rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
+            }
+            for (int s = 0; s < total - kWave; s++) {
+                const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k1, s);
+                const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t1, s);
+                rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
+                rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
+            }
+            if (in0) {
+                lds.key[1][rank0] = k0;
+                lds.pay2[1][rank0] = p0;
+            }
+            if (in1) {
+                lds.key[1][rank1] = k1;
+                lds.pay2[1][rank1] = p1;
             }
             wave_sync_memory();
-            {
-                // exclusive scan of the bins: lane owns bins [16*lane, 16*lane+16)
-                int h[kBins / kWave];
-                int lsum = 0;
+            cur = 1;
+        } else {
+            const int per = ((total + kWave - 1) / kWave) | 1;  // odd: conflict-free block starts
+            const int q0 = lane * per < total ? lane * per : total;
+            const int q1 = q0 + per < total ? q0 + per : total;
+            for (int sh = mixed ? -kSortBits : 0; sh < nbits; sh += kSortBits) {
+                const uint32_t *src_k = lds.key[cur], *src_p = lds.pay2[cur];
+                uint32_t *dst_k = lds.key[cur ^ 1], *dst_p = lds.pay2[cur ^ 1];
+                uint64_t c_lo = 0ull, c_hi = 0ull;  // counters of digit values 0..7 and 8..15
+                for (int q = q0; q < q1; q += 4) {
+                    uint32_t v[4];
 #pragma unroll
-                for (int t = 0; t < kBins / kWave; t++) {
-                    h[t] = lds.hist[lane * (kBins / kWave) + t];
-                    lsum += h[t];
+                    for (int u = 0; u < 4; u++) v[u] = q + u < q1 ? (sh < 0 ? src_p[q + u] : src_k[q + u]) : 0u;
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        if (q + u < q1) {
+                            const uint32_t d = sh < 0 ? v[u] >> 31 : ((v[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
+                            const uint64_t one = 1ull << ((d & 7u) * 8u);
+                            if (d & 8u) c_hi += one;
+                            else c_lo += one;
+                        }
+                    }
                 }
-                int run = wave_inclusive_sum(lsum, lane) - lsum;
+                // Start positions: exclusive prefix of the counts in (digit value, lane) order.
+                // The counts go to LDS in that order with one pad word per sixteen, every lane
+                // then owns sixteen consecutive ones (stride 17: conflict-free), sums them, one
+                // wave scan over the sums, and the prefixes go back to the same places.
+#pragma unroll
+                for (int b = 0; b < kSortBins; b++) {
+                    const int e = b * kWave + lane;
+                    lds.hist[e + (e >> 4)] = (int)(((b < 8 ? c_lo : c_hi) >> ((b & 7) * 8)) & 0xFFull);
+                }
                 wave_sync_memory();
+                {
+                    int h[16];
+                    int lsum = 0;
 #pragma unroll
-                for (int t = 0; t < kBins / kWave; t++) {
-                    lds.hist[lane * (kBins / kWave) + t] = run;
-                    run += h[t];
+                    for (int t = 0; t < 16; t++) {
+                        h[t] = lds.hist[lane * 17 + t];
+                        lsum += h[t];
+                    }
+                    int run = wave_inclusive_sum(lsum, lane) - lsum;
+#pragma unroll
+                    for (int t = 0; t < 16; t++) {
+                        lds.hist[lane * 17 + t] = run;
+                        run += h[t];
+                    }
                 }
+                wave_sync_memory();
+                // the counters are private to their lane from here on
+                for (int q = q0; q < q1; q += 4) {
+                    uint32_t kk[4], pp[4];
+                    int pos[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        kk[u] = q + u < q1 ? src_k[q + u] : 0u;
+                        pp[u] = q + u < q1 ? src_p[q + u] : 0u;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        pos[u] = 0;
+                        if (q + u < q1) {
+                            const uint32_t d = sh < 0 ? pp[u] >> 31 : ((kk[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
+                            const int e = (int)d * kWave + lane;
+                            pos[u] = __hip_atomic_fetch_add(&lds.hist[e + (e >> 4)], 1, __ATOMIC_RELAXED,
+                                                            __HIP_MEMORY_SCOPE_WAVEFRONT);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        if (q + u < q1) {
+                            dst_k[pos[u]] = kk[u];
+                            dst_p[pos[u]] = pp[u];
+                        }
+                    }
+                }
+                wave_sync_memory();
+                cur ^= 1;
+#ifdef OMK_PHASE_TIMERS
+                if (a.stats && lane == 0) atomicAdd(a.stats + 15, 1);
+#endif
             }
-            wave_sync_memory();
-            const int nxt = cur == 0 ? 1 : 0;
-            for (int base = 0; base < total; base += kWave) {
-                const int q = base + lane;
-                const bool in = q < total;
-                const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
-                const uint32_t d =
-                    !in ? 0u : (sh < 0 ? lds.pay2[i] >> 31 : (lds.key[i] >> sh) & (uint32_t)(kBins - 1));
-                // lanes of this chunk with the same digit
-                uint64_t same = __ballot(in);
-#pragma unroll
-                for (int b = 0; b < kDigitBits; b++) {
-                    uint64_t bal = __ballot(in && ((d >> b) & 1u));
-                    same &= ((d >> b) & 1u) ? bal : ~bal;
-                }
-                const int rank = __popcll(same & ((1ull << lane) - 1ull));
-                const int count = __popcll(same);
-                const int basepos = in ? lds.hist[d] : 0;
-                if (in) lds.idx[nxt][basepos + rank] = (uint16_t)i;
-                wave_sync_memory();
-                if (in && rank == 0) lds.hist[d] = basepos + count;
-                wave_sync_memory();
-            }
-            cur = nxt;
         }
-        wave_sync_memory();
+        const uint32_t *skey = lds.key[cur], *spay = lds.pay2[cur];
         OMK_TICK(10);
 
         // ---- 4. winner order: keep what is needed, check ties across children, emit ----
@@ -794,24 +870,22 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             uint32_t qcut = 0xFFFFFFFFu;
             const uint32_t want_pay = ((uint32_t)capped_child << 21) | (uint32_t)capped_last;
             for (int q = lane; q < total; q += kWave) {
-                const int i = cur < 0 ? q : (int)lds.idx[cur][q];
-                if ((lds.pay2[i] & 0x7FFFFFFFu) == want_pay) qcut = umin32(qcut, (uint32_t)q);
+                if ((spay[q] & 0x7FFFFFFFu) == want_pay) qcut = umin32(qcut, (uint32_t)q);
             }
             qcut = wave_min_u32(qcut);
             if (qcut == 0xFFFFFFFFu) OMK_FAIL(10);
             if ((int)qcut + 1 < keep) keep = (int)qcut + 1;
         }
 #pragma unroll
-        for (int t = 0; t < kBins / kWave; t++) lds.hist[t * kWave + lane] = 0;  // visits per child after this batch
+        for (int t = 0; t < kSortBins; t++) lds.hist[t * kWave + lane] = 0;  // visits per child after this batch
         wave_sync_memory();
         uint32_t pk63 = 0u, ppay63 = 0u;
         bool have_prev = false;
         for (int base = 0; base < total; base += kWave) {
             const int q = base + lane;
             const bool in = q < total;
-            const int i = in ? (cur < 0 ? q : (int)lds.idx[cur][q]) : 0;
-            uint32_t kk = in ? lds.key[i] : 0u;
-            uint32_t pay = in ? lds.pay2[i] : 0u;
+            uint32_t kk = in ? skey[q] : 0u;
+            uint32_t pay = in ? spay[q] : 0u;
             uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
             uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
             bool hp = lane > 0 || have_prev;
@@ -848,9 +922,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             // The last kept entry must come before every child's first unevaluated entry (a
             // child with dropped entries is covered by the order check above), and that entry
             // must not come before the child's own last evaluated one.
-            const int il = cur < 0 ? keep - 1 : (int)lds.idx[cur][keep - 1];
-            const uint32_t lk = ~lds.key[il];
-            const uint32_t lpay = lds.pay2[il];
+            const uint32_t lk = ~skey[keep - 1];
+            const uint32_t lpay = spay[keep - 1];
             const uint32_t lchild = (lpay >> 21) & 1023u;
             const uint32_t lpos = lchild + ((lpay >> 31) ? (uint32_t)F : 0u);
 #pragma unroll
@@ -949,8 +1022,16 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
         for (int r = 0; r < R; r++)
             if (k.part[r] && headk[r] >= lo_key)
                 est += predict_count<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, mid, m);
-        if (wave_sum_i32(est) >= target) klo = kmid;
-        else khi = kmid;
+        const int e = wave_sum_i32(est);
+        if (e >= target) {
+            klo = kmid;
+            // Close enough.  The window is narrower than the distance between the targets of
+            // two slices, so the order of the thresholds is kept: a search for a later target
+            // that reaches this midpoint goes below it.
+            if (e <= target + (kSliceEntries >> 3)) break;
+        } else {
+            khi = kmid;
+        }
     }
     const uint32_t T = klo;
     const float tau = key_score(T);
@@ -1155,7 +1236,9 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     hid = id;
                     slice = 0;
                     n_slices = K;
+#ifndef OMK_PHASE_TIMERS
                     if (a.stats && lane == 0) atomicAdd(a.stats + 15, 1);
+#endif
                 } else if (lane == 0) {
                     atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
                 }
