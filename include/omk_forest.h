@@ -154,8 +154,16 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * [1] of these settled by the parallel paths, [2] visitors settled by them, [3] visitors
  * settled one at a time, [4] nodes replayed one visitor at a time because the parallel
  * path's exactness checks did not hold, [5] threshold probes, [6] single-visitor selection
- * steps, [7] unused, [8..15] per-phase cycle counts in measurement builds (else 0). */
+ * steps, [7] unused, [8..14] per-phase cycle counts in measurement builds (else 0),
+ * [15] nodes cut into slices for several wavefronts. */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
+/* The multi-visitor selection kernel is persistent: its wavefronts wait for work items that
+ * other wavefronts publish.  Every wait is bounded; a wavefront that polls `polls` times in
+ * vain raises an abort flag, all wavefronts leave, and omk_batch_read reports OMK_ERR_STATE
+ * for that selection (its paths are incomplete; upload the statistics again before the next
+ * one).  The default (about four million polls, seconds) is never reached in normal
+ * operation; tests of the error path set a tiny limit.  No counterpart in the reference. */
+int omk_batch_set_spin_limit(omk_batch *b, int32_t polls);
 
 /* ---- transposition table: the lookup/store call sites of
  *      mcts_engine_batch_tree_simple.cpp:126,141 (PHMapTranspositionTable::store / lookup,

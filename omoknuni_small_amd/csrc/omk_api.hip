@@ -593,6 +593,13 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     return OMK_OK;
 }
 
+int omk_batch_set_spin_limit(omk_batch *b, int32_t polls) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_batch_set_spin_limit: null batch");
+    if (polls < 0) return fail(OMK_ERR_INVALID, "omk_batch_set_spin_limit: polls %d", polls);
+    b->spin_limit = polls;
+    return OMK_OK;
+}
+
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     int32_t *h_stats8 = h_stats16;
     if (!b || !h_stats8) return fail(OMK_ERR_INVALID, "omk_batch_stats: null argument");

@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void k_export(ForestDev f, const int32_t *path
     int d = (int)(g - (int64_t)t * row);
     int len = path_len[t];
     int node = d < len ? paths[(size_t)d * stride + t] : -1;
+    if (node >= f.n_nodes) node = -1;  // never index the forest with an id it does not have
     if (out_paths) out_paths[g] = node;
     if (out_actions && d >= 1) {
         int act = -1;
@@ -214,7 +215,9 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
                                                   int min_depth, int32_t *out) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    unsigned long long key = keys ? keys[i] : node_hash[leaf[i]];
+    unsigned long long key = kTTEmpty;
+    if (keys) key = keys[i];
+    else if (leaf[i] >= 0) key = node_hash[leaf[i]];  // a traversal without a leaf finds nothing
     int found = -1;
     if (key != kTTEmpty) {
         uint64_t mask = (1ull << log2_slots) - 1ull;

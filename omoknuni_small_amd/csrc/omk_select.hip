@@ -1709,7 +1709,7 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
 
 // Scheduler state, statistics, the work queue seeded with the items of the roots, and the
 // single-visitor queue seeded with the traversals that are alone at their root.
-__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0) {
+__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0, int n_traversals) {
     const int gid = blockIdx.x * blockDim.x + threadIdx.x;
     const int step = gridDim.x * blockDim.x;
     if (gid == 0) {
@@ -1730,6 +1730,11 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         a.q_ready[i] = a.epoch;
     }
     for (int i = gid; i < n_singles0; i += step) a.singles_q[i] = a.singles0[i];
+    // a traversal that the selection does not finish (the kernel gave up) has an empty path
+    for (int i = gid; i < n_traversals; i += step) {
+        a.path_len[i] = 0;
+        a.leaf[i] = -1;
+    }
 }
 
 template <int RMAX, bool RAVE>
@@ -1760,7 +1765,7 @@ hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, 
                          int max_fanout, bool rave, int n_cus, hipStream_t s) {
     int reset_blocks = (n_traversals + 255) / 256;
     hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
-                       n_traversals - n_singles0);
+                       n_traversals - n_singles0, n_traversals);
 #define OMK_DISPATCH(RM)                                                                  \
     return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, s)        \
                 : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, s)

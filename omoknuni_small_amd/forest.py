@@ -25,7 +25,7 @@ EXPORTS = [
     "omk_forest_upload", "omk_forest_download", "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_truncated", "omk_batch_stats", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
 ]
@@ -261,12 +261,16 @@ class Batch:
         _check(self._lib.omk_batch_truncated(self._h, C.byref(c)))
         return c.value
 
+    def set_spin_limit(self, polls):
+        """Bound of the waits inside the persistent selection kernel (error-path tests)."""
+        _check(self._lib.omk_batch_set_spin_limit(self._h, C.c_int32(int(polls))))
+
     def stats(self):
         out = np.zeros(16, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
                 "replayed_nodes", "threshold_probes", "single_visitor_steps", "fail_code", "cyc_threshold",
-                "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "unused15")
+                "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "sliced_nodes")
         return dict(zip(keys, map(int, out)))
 
     def device(self):

@@ -1,0 +1,143 @@
+"""GPU parity for the parts of the selection kernel that only crowded trees reach: nodes with
+a thousand visitors or more, which several wavefronts settle together (slices of the winner
+order, shared partition), several such nodes at once, fan-outs beyond the widest node that
+is settled that way, children whose score hardly moves with virtual loss (long runs of one
+winner), and the bounded wait of the persistent kernel."""
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+
+pytestmark = pytest.mark.gpu
+
+
+def layered_forest(seed, fans, n_trees=1, rave=False, plateau=False):
+    """n_trees complete trees, level l has fan-out fans[l]; benchmark-like statistics."""
+    rng = np.random.default_rng(seed)
+    N, W, P, cb, cc, act, rN, rW = ([] for _ in range(8))
+    roots = []
+
+    def stats(k, parent_sorted=False):
+        n = np.minimum(rng.zipf(1.2, k), 10_000).astype(np.int64)
+        n[rng.random(k) < 0.2] = 0
+        w = rng.uniform(-1, 1, k) * n
+        logits = rng.normal(0, 1.5, k)
+        p = np.exp(logits - logits.max())
+        p /= p.sum()
+        return n, w, p
+
+    for _ in range(n_trees):
+        roots.append(len(N))
+        N.append(200_000); W.append(0.0); P.append(0.0); cb.append(0); cc.append(0); act.append(-1)
+        rN.append(0); rW.append(0.0)
+        level = [roots[-1]]
+        for f in fans:
+            nxt = []
+            for node in level:
+                n, w, p = stats(f)
+                cb[node] = len(N)
+                cc[node] = f
+                for i in range(f):
+                    nxt.append(len(N))
+                    N.append(int(n[i])); W.append(float(w[i])); P.append(float(p[i]))
+                    cb.append(0); cc.append(0); act.append(i)
+                    r = int(min(rng.zipf(1.3), 5000))
+                    rN.append(r); rW.append(float(rng.uniform(-1, 1) * r))
+                if plateau:
+                    # a few heavily visited children with a high blended value and a tiny prior:
+                    # their score hardly moves with virtual loss
+                    for i in rng.choice(f, 3, replace=False):
+                        c = cb[node] + int(i)
+                        N[c] = 9000; W[c] = 0.93 * 9000; P[c] = 1e-4; rN[c] = 4000; rW[c] = 0.95 * 4000
+                N[node] = max(N[node], 1 + int(sum(N[cb[node] + i] for i in range(f))))
+            level = nxt
+    soa = dict(N=np.array(N, np.int32), W=np.array(W, np.float32), P=np.array(P, np.float32),
+               VL=np.zeros(len(N), np.int32), child_begin=np.array(cb, np.int32), child_count=np.array(cc, np.int32),
+               action=np.array(act, np.int32))
+    if rave:
+        soa["rN"] = np.array(rN, np.int32)
+        soa["rW"] = np.array(rW, np.float32)
+    return soa, np.array(roots, np.int32)
+
+
+def select_both(soa, troots, D, vl=3, rave=False, rave_k=1000.0, steps=2):
+    import omoknuni_small_amd as omk
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=rave_k, max_depth=D)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, len(troots), D)
+    b.set_roots(troots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=rave_k)
+    rng = np.random.default_rng(1)
+    stats = None
+    for step in range(steps):
+        rpaths, rlen, rleaf, near = ref.select_batch(troots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        bad = np.nonzero((gpaths != rpaths).any(axis=1) | (glen != rlen) | (gleaf != rleaf))[0]
+        assert len(bad) == 0, "step %d: %d paths differ, first traversal %d (near ties flagged: %d)" % (
+            step, len(bad), bad[0], int((near >= 0).sum()))
+        assert (f.download()["VL"] == ref.VL).all()
+        stats = b.stats()
+        values = rng.uniform(-1, 1, len(troots)).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, values, vl)
+        b.set_values(values)
+        b.backup(vl)
+        st = f.download()
+        assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all()
+        ref.W[:] = st["W"]
+    return stats
+
+
+@pytest.mark.parametrize("fan,rave,plateau", [(300, False, False), (300, True, False), (300, True, True),
+                                              (48, False, False), (362, True, True)])
+def test_heavy_nodes_are_sliced(fan, rave, plateau):
+    soa, roots = layered_forest(7, [fan, 40], rave=rave, plateau=plateau)
+    st = select_both(soa, np.zeros(20_000, np.int32), 3, rave=rave)
+    assert st["sliced_nodes"] >= 1, st
+    assert st["replayed_nodes"] == 0, st
+
+
+def test_fanout_beyond_the_sliced_path():
+    # the root is wider than the widest node that several wavefronts share: one wavefront
+    # settles its 6000 visitors batch after batch (its children may still be sliced)
+    soa, roots = layered_forest(8, [700, 20])
+    st = select_both(soa, np.zeros(6000, np.int32), 3)
+    assert st["replayed_nodes"] == 0, st
+
+
+def test_several_heavy_roots_at_once():
+    soa, roots = layered_forest(9, [120, 30], n_trees=5, rave=True, plateau=True)
+    troots = roots[np.arange(5 * 2500) % 5]
+    st = select_both(soa, troots, 3, rave=True)
+    assert st["sliced_nodes"] >= 5, st
+
+
+def test_tiny_virtual_loss_many_visitors():
+    soa, roots = layered_forest(10, [200, 25])
+    select_both(soa, np.zeros(9000, np.int32), 3, vl=1)
+
+
+def test_bounded_wait_reports_and_recovers():
+    """A spin limit of zero makes every waiting wavefront give up at once: the kernel still
+    ends normally, the selection is reported as incomplete, and the batch works again."""
+    import omoknuni_small_amd as omk
+    soa, roots = layered_forest(11, [60, 30, 10])
+    troots = np.zeros(3000, np.int32)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, len(troots), 4)
+    b.set_roots(troots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3)
+    b.set_spin_limit(0)
+    b.select(sp)
+    with pytest.raises(omk.OmkError) as e:
+        b.read()
+    assert e.value.code == -6, e.value  # OMK_ERR_STATE
+    b.set_spin_limit(1 << 22)
+    f.upload(soa)
+    ref = R.RefTree.from_soa(soa)
+    rpaths, rlen, rleaf, _ = ref.select_batch(troots, R.make_params(c_puct=1.4, virtual_loss=3, max_depth=4))
+    b.select(sp)
+    gpaths, glen, gleaf, _ = b.read()
+    assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
+    assert (f.download()["VL"] == ref.VL).all()
