@@ -586,6 +586,19 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                         if (kk >= T) lo_c = g + 1;
                         else hi_c = g;
                     }
+                    // estimate off by more than one: gallop away from it, then bisect what is left
+                    if (lo_c < hi_c) {
+                        const bool up = lo_c > g;
+                        for (int step = 2; lo_c < hi_c; step <<= 1) {
+                            int t = up ? lo_c + step : hi_c - step + 1;
+                            t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+                            entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, t - 1, ac[r], kk, pp);
+                            const bool ge = kk >= T;
+                            if (ge) lo_c = t;
+                            else hi_c = t - 1;
+                            if (ge != up) break;
+                        }
+                    }
                     while (lo_c < hi_c) {
                         int t = (lo_c + hi_c + 1) >> 1;
                         entry_key<R, RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, t - 1, ac[r], kk, pp);
@@ -1053,6 +1066,18 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
                 entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, g, i, kk, pp);
                 if (kk >= T) lo_c = g + 1;
                 else hi_c = g;
+            }
+            if (lo_c < hi_c) {
+                const bool up = lo_c > g;
+                for (int step = 2; lo_c < hi_c; step <<= 1) {
+                    int t = up ? lo_c + step : hi_c - step + 1;
+                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, t - 1, i, kk, pp);
+                    const bool ge = kk >= T;
+                    if (ge) lo_c = t;
+                    else hi_c = t - 1;
+                    if (ge != up) break;
+                }
             }
             while (lo_c < hi_c) {
                 int t = (lo_c + hi_c + 1) >> 1;
