@@ -47,7 +47,10 @@ constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in 
 constexpr int kBatchCap = 2048;           // entries put in winner order at a time (LDS resident)
 constexpr int kSortBits = 4;              // radix digit of that sort
 constexpr int kSortBins = 1 << kSortBits;
-constexpr int kGroupWaves = 2;            // wavefronts per block of the multi-visitor kernel
+constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-visitor kernel: one owner that
+                                          // takes the items, three helpers for the batch work of its node
+constexpr int kTeam = kTeamWaves * 64;
+constexpr int kTeamMin = 192;             // batch entries from which the helpers are called in
 constexpr int kSliceEntries = 512;        // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
@@ -103,20 +106,37 @@ struct Kids {
     bool part[R];
 };
 
-// Per-wavefront scratch in LDS of the multi-visitor kernel.
+// What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
+// so that it sits at the same place for every fan-out class.
+enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2 };
+struct TeamCmd {
+    int op;
+    int rounds;  // R of the node's fan-out class: 1, or the kernel's RMAX
+    int total;   // entries of the batch
+    int keep;    // of which the first `keep` are winners
+    int goff;    // where the batch's winners go in sc_child / sc_occ
+    int cur;     // which of the two buffers holds the ordered batch
+    float ep;
+    uint32_t uvl;
+};
+
+// Scratch in LDS of one block of the multi-visitor kernel (one node at a time).
 template <int R>
 struct WaveLds {
-    int offs[R * kWave];  // exclusive prefix of the visit counts in child order
-    int st_n[R * kWave];  // statistics of every child, readable by any lane
+    TeamCmd cmd;
+    uint32_t red[4];       // team reductions: smallest / largest inverted key, flags
+    int wsum[kTeamWaves];  // team prefix scan: totals of the wavefronts
+    int offs[R * kWave];   // exclusive prefix of the visit counts in child order
+    int st_n[R * kWave];   // statistics of every child, readable by any lane
     float st_w[R * kWave];
     float st_p[R * kWave];
     int st_vl[R * kWave];
     float st_q2[R * kWave];
     int st_j0[R * kWave];  // visits already settled / visit count, by phase
-    int hist[kSortBins * kWave + kSortBins * kWave / 16];  // sort: one counter per (digit value, lane), padded
-    uint32_t pay[R * kWave];         // per child: entries of the batch
-    uint32_t key[2][kBatchCap];      // entries of the batch being ordered: inverted score key ...
-    uint32_t pay2[2][kBatchCap];     // ... and pass flag, child, visit number; two buffers, ping-pong
+    int hist[kSortBins * kTeam + kSortBins * kTeam / 16];  // sort: one counter per (digit value, thread), padded
+    uint32_t pay[R * kWave];      // per child: entries of the batch
+    uint32_t key[2][kBatchCap];   // entries of the batch being ordered: inverted score key ...
+    uint32_t pay2[2][kBatchCap];  // ... and pass flag, child, visit number; two buffers, ping-pong
 };
 
 template <int R, bool RAVE>
@@ -315,6 +335,288 @@ __device__ __forceinline__ int predict_count(int n, float w, float p, int vl, fl
     float cnt = floorf((xs - x0) * inv_step) + 1.0f;
     if (!(cnt > 0.0f)) return 0;
     return cnt >= (float)cap ? cap : (int)cnt;
+}
+
+template <int NT>
+__device__ __forceinline__ void team_sync() {
+    if (NT == kWave) wave_sync_memory();
+    else __syncthreads();
+}
+
+// One batch of a crowded node, steps 2 and 3: evaluate its entries in (child, visit) order
+// into LDS (child i contributes pay[i] entries starting at offs[i], from visit st_j0[i] on),
+// then put them in winner order.  Run by NT threads with the same arguments: one wavefront,
+// or the whole block (the owner wavefront and its helpers).  Returns which buffer holds the
+// ordered batch; red[2] bit 2 is set when an entry has no real key or a child's entries
+// increase.
+template <int R, bool RAVE, int NT>
+__device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, float ep, uint32_t uvl) {
+    constexpr int F = R * kWave;
+    const int lane = tid & 63;
+    if (tid == 0) {
+        lds.red[0] = 0xFFFFFFFFu;
+        lds.red[1] = 0u;
+        lds.red[2] = 0u;
+    }
+    team_sync<NT>();
+    // every thread evaluates a contiguous run of `per` entries (odd, so that the LDS writes of
+    // the threads fall into different banks)
+    const int per = ((total + NT - 1) / NT) | 1;
+    const int q0 = tid * per < total ? tid * per : total;
+    const int q1 = q0 + per < total ? q0 + per : total;
+    {
+        bool bad_entry = false;
+        bool kind1 = false, kind2 = false;  // candidates of the first / second scan present
+        uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
+        int q = q0;
+        int child = 0, seg_end = 0;
+        int sn = 0, svl = 0, sj0 = 0;
+        float sw = 0.0f, sp = 0.0f, sq2 = 0.0f;
+        uint32_t pk = 0u, ppos = 0u;
+        bool have = false;
+        if (q < q1) {
+            // last child whose segment starts at or before q
+            int lo_i = 0, hi_i = F;
+            while (hi_i - lo_i > 1) {
+                int mid = (lo_i + hi_i) >> 1;
+                if (lds.offs[mid] <= q) lo_i = mid;
+                else hi_i = mid;
+            }
+            child = lo_i;
+            seg_end = lds.offs[child] + (int)lds.pay[child];
+        }
+        bool fresh = true;
+        uint32_t firstk = 0u, firstp = 0u;
+        int firstj = 0;
+        for (; q < q1; q++) {
+            while (q >= seg_end) {  // next child with entries
+                child++;
+                seg_end = lds.offs[child] + (int)lds.pay[child];
+                fresh = true;
+            }
+            if (fresh) {
+                sn = lds.st_n[child];
+                sw = lds.st_w[child];
+                sp = lds.st_p[child];
+                svl = lds.st_vl[child];
+                sq2 = lds.st_q2[child];
+                sj0 = lds.st_j0[child];
+                fresh = false;
+                have = false;
+            }
+            const int jl = q - lds.offs[child];
+            uint32_t kk, pp;
+            entry_key<R, RAVE>(sn, sw, sp, svl, sq2, ep, uvl, jl, child, kk, pp);
+            lds.key[0][q] = ~kk;
+            lds.pay2[0][q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)(sj0 + jl);
+            kmin = umin32(kmin, ~kk);
+            kmax = umax32(kmax, ~kk);
+            if (pp >= (uint32_t)F) kind2 = true;
+            else kind1 = true;
+            if (kk == 0u) bad_entry = true;
+            // within a child the entries must not increase
+            if (have && comes_before(kk, pp, pk, ppos)) bad_entry = true;
+            if (q == q0) {
+                firstk = kk;
+                firstp = pp;
+                firstj = jl;
+            }
+            pk = kk;
+            ppos = pp;
+            have = true;
+        }
+        kmin = wave_min_u32(kmin);
+        kmax = wave_max_u32(kmax);
+        const uint32_t flags = (__ballot(kind1) != 0ull ? 1u : 0u) | (__ballot(kind2) != 0ull ? 2u : 0u) |
+                               (__ballot(bad_entry) != 0ull ? 4u : 0u);
+        if (lane == 0) {
+            atomicMin(&lds.red[0], kmin);
+            atomicMax(&lds.red[1], kmax);
+            atomicOr(&lds.red[2], flags);
+        }
+        team_sync<NT>();
+        // the run of the previous thread may end inside the same child: check the seam
+        bool bad_seam = false;
+        if (q0 < q1 && firstj > 0) {
+            const uint32_t lk = ~lds.key[0][q0 - 1];
+            const uint32_t lpay = lds.pay2[0][q0 - 1];
+            const uint32_t lp = ((lpay >> 21) & 1023u) + ((lpay >> 31) ? (uint32_t)F : 0u);
+            if (comes_before(firstk, firstp, lk, lp)) bad_seam = true;
+        }
+        if (__ballot(bad_seam) != 0ull && lane == 0) atomicOr(&lds.red[2], 4u);
+    }
+    // the same for every thread: keep them on the scalar unit, the loops below hold barriers
+    const uint32_t kmin = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[0]);
+    const uint32_t kmax = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[1]);
+    const bool mixed = ((uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[2]) & 3u) == 3u;
+
+    // Stable radix sort, in LDS.  Order wanted: key descending, then candidate position
+    // ascending, then visit number.  The entries start in (child, visit) order; least
+    // significant digit first, a pass on the scan kind (only when both kinds occur:
+    // candidates of the first scan sit before those of the second) and then the key digits,
+    // over the bits of the key range.  One pass: every thread owns a contiguous block of the
+    // current order, counts its digits in registers (sixteen 8-bit counters), a scan over
+    // (digit value, thread) turns the counts into start positions, kept in LDS per (digit
+    // value, thread), and every thread moves its block in order.  No two threads share a
+    // counter, so the order inside a digit value is (thread, position in block): stable.
+    // A small batch (two entries per lane at most) is ranked by comparing every entry with
+    // every other one instead, through lane reads.
+    const uint32_t range = kmax - kmin;
+    const int nbits = range == 0u ? 0 : 32 - __clz((int)range);
+    int cur = 0;
+    if (NT == kWave && total <= 2 * kWave) {
+        // entry q of the batch: (key, kind bit | q) compared as a pair; entries lane and 64 + lane
+        const bool in0 = lane < total, in1 = kWave + lane < total;
+        const uint32_t k0 = in0 ? lds.key[0][lane] : 0xFFFFFFFFu, k1 = in1 ? lds.key[0][kWave + lane] : 0xFFFFFFFFu;
+        const uint32_t p0 = in0 ? lds.pay2[0][lane] : 0u, p1 = in1 ? lds.pay2[0][kWave + lane] : 0u;
+        const uint32_t t0 = in0 ? (p0 & 0x80000000u) | (uint32_t)lane : 0xFFFFFFFFu;
+        const uint32_t t1 = in1 ? (p1 & 0x80000000u) | (uint32_t)(kWave + lane) : 0xFFFFFFFFu;
+        int rank0 = 0, rank1 = 0;
+        const int n0 = total < kWave ? total : kWave;
+        for (int s = 0; s < n0; s++) {
+            const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k0, s);
+            const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t0, s);
+            rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
+            rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
+        }
+        for (int s = 0; s < total - kWave; s++) {
+            const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k1, s);
+            const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t1, s);
+            rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
+            rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
+        }
+        if (in0) {
+            lds.key[1][rank0] = k0;
+            lds.pay2[1][rank0] = p0;
+        }
+        if (in1) {
+            lds.key[1][rank1] = k1;
+            lds.pay2[1][rank1] = p1;
+        }
+        cur = 1;
+    } else {
+        const int wave = tid >> 6;
+        for (int sh = mixed ? -kSortBits : 0; sh < nbits; sh += kSortBits) {
+            const uint32_t *src_k = lds.key[cur], *src_p = lds.pay2[cur];
+            uint32_t *dst_k = lds.key[cur ^ 1], *dst_p = lds.pay2[cur ^ 1];
+            uint64_t c_lo = 0ull, c_hi = 0ull;  // counters of digit values 0..7 and 8..15
+            for (int q = q0; q < q1; q += 4) {
+                uint32_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) v[u] = q + u < q1 ? (sh < 0 ? src_p[q + u] : src_k[q + u]) : 0u;
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    if (q + u < q1) {
+                        const uint32_t d = sh < 0 ? v[u] >> 31 : ((v[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
+                        const uint64_t one = 1ull << ((d & 7u) * 8u);
+                        if (d & 8u) c_hi += one;
+                        else c_lo += one;
+                    }
+                }
+            }
+            // Start positions: exclusive prefix of the counts in (digit value, thread) order.
+            // The counts go to LDS in that order with one pad word per sixteen, every thread
+            // then owns sixteen consecutive ones (stride 17: conflict-free), sums them, one
+            // scan over the sums of the team, and the prefixes go back to the same places.
+#pragma unroll
+            for (int b = 0; b < kSortBins; b++) {
+                const int e = b * NT + tid;
+                lds.hist[e + (e >> 4)] = (int)(((b < 8 ? c_lo : c_hi) >> ((b & 7) * 8)) & 0xFFull);
+            }
+            team_sync<NT>();
+            {
+                int h[16];
+                int lsum = 0;
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    h[t] = lds.hist[tid * 17 + t];
+                    lsum += h[t];
+                }
+                const int inc = wave_inclusive_sum(lsum, lane);
+                int run = inc - lsum;
+                if (NT > kWave) {
+                    if (lane == kWave - 1) lds.wsum[wave] = inc;
+                    team_sync<NT>();
+                    for (int w = 0; w < wave; w++) run += lds.wsum[w];
+                }
+#pragma unroll
+                for (int t = 0; t < 16; t++) {
+                    lds.hist[tid * 17 + t] = run;
+                    run += h[t];
+                }
+            }
+            team_sync<NT>();
+            // the counters are private to their thread from here on
+            for (int q = q0; q < q1; q += 4) {
+                uint32_t kk[4], pp[4];
+                int pos[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    kk[u] = q + u < q1 ? src_k[q + u] : 0u;
+                    pp[u] = q + u < q1 ? src_p[q + u] : 0u;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    pos[u] = 0;
+                    if (q + u < q1) {
+                        const uint32_t d = sh < 0 ? pp[u] >> 31 : ((kk[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
+                        const int e = (int)d * NT + tid;
+                        pos[u] = __hip_atomic_fetch_add(&lds.hist[e + (e >> 4)], 1, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    if (q + u < q1) {
+                        dst_k[pos[u]] = kk[u];
+                        dst_p[pos[u]] = pp[u];
+                    }
+                }
+            }
+            team_sync<NT>();
+            cur ^= 1;
+        }
+    }
+    team_sync<NT>();
+    return cur;
+}
+
+// Step 4 of a batch: the first `keep` entries of the ordered batch are the next winners;
+// records (child, visit number) of each at its rank, leaves in hist[i] the visits child i
+// has after them, and checks the order of the whole batch, kept or not (what is dropped
+// must come after what is kept): red[2] bit 2 on failure.
+template <int R, int NT>
+__device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds, int tid, int total, int keep,
+                                           int goff, int cur) {
+    constexpr int F = R * kWave;
+    const uint32_t *skey = lds.key[cur], *spay = lds.pay2[cur];
+    for (int i = tid; i < F; i += NT) lds.hist[i] = 0;
+    team_sync<NT>();
+    bool bad_order = false;
+    for (int q = tid; q < total; q += NT) {
+        const uint32_t kk = skey[q];
+        const uint32_t pay = spay[q];
+        const int child = (int)((pay >> 21) & 1023u);
+        const int j = (int)(pay & 0x1FFFFFu);
+        if (q < keep) {
+            a.sc_child[goff + q] = child;
+            a.sc_occ[goff + q] = j;
+            atomicMax(&lds.hist[child], j + 1);
+        }
+        if (q > 0) {
+            const uint32_t pk = skey[q - 1];
+            const uint32_t ppay = spay[q - 1];
+            if (pk > kk) bad_order = true;  // not sorted
+            if (pk == kk) {
+                const uint32_t pchild = (ppay >> 21) & 1023u;
+                const uint32_t ppos_ = pchild + ((ppay >> 31) ? (uint32_t)F : 0u);
+                const uint32_t pos_ = (uint32_t)child + ((pay >> 31) ? (uint32_t)F : 0u);
+                if (pchild != (uint32_t)child && ppos_ > pos_) bad_order = true;
+            }
+        }
+    }
+    if (__ballot(bad_order) != 0ull && (tid & 63) == 0) atomicOr(&lds.red[2], 4u);
+    team_sync<NT>();
 }
 
 // The visitors of a crowded node in batches (see the file header).  On success cnt[r]
@@ -667,212 +969,25 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             carry += __builtin_amdgcn_readlane(inc, 63);
         }
         wave_sync_memory();
-        bool bad = false;
-        bool any_first = false, any_second = false;  // candidates of the first / second scan present
-        uint32_t kmin = 0xFFFFFFFFu, kmax = 0u;
-        {
-            // every lane evaluates a contiguous run of `per` entries (odd, so that the LDS
-            // writes of the lanes fall into different banks)
-            const int per = ((total + kWave - 1) / kWave) | 1;
-            int q = lane * per;
-            const int q_end = q + per < total ? q + per : total;
-            int child = 0, seg_end = 0;
-            int sn = 0, svl = 0, sj0 = 0;
-            float sw = 0.0f, sp = 0.0f, sq2 = 0.0f;
-            uint32_t pk = 0u, ppos = 0u;
-            bool have = false;
-            if (q < q_end) {
-                // last child whose segment starts at or before q
-                int lo_i = 0, hi_i = F;
-                while (hi_i - lo_i > 1) {
-                    int mid = (lo_i + hi_i) >> 1;
-                    if (lds.offs[mid] <= q) lo_i = mid;
-                    else hi_i = mid;
-                }
-                child = lo_i;
-                seg_end = lds.offs[child] + (int)lds.pay[child];
+        // ---- 2./3. evaluate the batch and put it in winner order; a batch that is worth it
+        // is shared with the helper wavefronts of the block ----
+        const bool team = total >= kTeamMin;
+        int cur;
+        if (team) {
+            if (lane == 0) {
+                lds.cmd.op = kOpOrder;
+                lds.cmd.rounds = R;
+                lds.cmd.total = total;
+                lds.cmd.ep = c.ep;
+                lds.cmd.uvl = uvl;
             }
-            bool fresh = true;
-            uint32_t firstk = 0u, firstp = 0u;
-            int firstchild = -1, firstj = 0;
-            for (; q < q_end; q++) {
-                while (q >= seg_end) {  // next child with entries
-                    child++;
-                    seg_end = lds.offs[child] + (int)lds.pay[child];
-                    fresh = true;
-                }
-                if (fresh) {
-                    sn = lds.st_n[child];
-                    sw = lds.st_w[child];
-                    sp = lds.st_p[child];
-                    svl = lds.st_vl[child];
-                    sq2 = lds.st_q2[child];
-                    sj0 = lds.st_j0[child];
-                    fresh = false;
-                    have = false;
-                }
-                const int jl = q - lds.offs[child];
-                uint32_t kk, pp;
-                entry_key<R, RAVE>(sn, sw, sp, svl, sq2, c.ep, uvl, jl, child, kk, pp);
-                lds.key[0][q] = ~kk;
-                lds.pay2[0][q] = (pp >= (uint32_t)F ? 0x80000000u : 0u) | ((uint32_t)child << 21) | (uint32_t)(sj0 + jl);
-                kmin = umin32(kmin, ~kk);
-                kmax = umax32(kmax, ~kk);
-                if (pp >= (uint32_t)F) any_second = true;
-                else any_first = true;
-                if (kk == 0u) bad = true;
-                // within a child the entries must not increase
-                if (have && comes_before(kk, pp, pk, ppos)) bad = true;
-                if (firstchild < 0) {
-                    firstk = kk;
-                    firstp = pp;
-                    firstchild = child;
-                    firstj = jl;
-                }
-                pk = kk;
-                ppos = pp;
-                have = true;
-            }
-            // the run of the previous lane may end inside the same child: check the seam
-            uint32_t lk = (uint32_t)__shfl_up((int)pk, 1, kWave);
-            uint32_t lp = (uint32_t)__shfl_up((int)ppos, 1, kWave);
-            if (lane > 0 && firstchild >= 0 && firstj > 0 && comes_before(firstk, firstp, lk, lp)) bad = true;
-        }
-        if (__ballot(bad) != 0ull) OMK_FAIL(8);
-        kmin = wave_min_u32(kmin);
-        kmax = wave_max_u32(kmax);
-        wave_sync_memory();
-        OMK_TICK(9);
-
-        // ---- 3. stable radix sort of the batch, in LDS ----
-        // Order wanted: key descending, then candidate position ascending, then visit number.
-        // The entries start in (child, visit) order; least significant digit first, a pass on
-        // the scan kind (only when both kinds occur: candidates of the first scan sit before
-        // those of the second) and then the key digits, over the bits that differ.
-        // One pass: every lane owns a contiguous block of the current order, counts its digits
-        // in registers (sixteen 8-bit counters), a scan over (digit value, lane) turns the
-        // counts into start positions, kept in LDS per (digit value, lane), and every lane moves
-        // its block in order.  No two lanes share a counter, so the order inside a digit value
-        // is (lane, position in block): stable.
-        // A small batch (two entries per lane at most) is ranked by comparing every entry with
-        // every other one instead, through lane reads.
-        const uint32_t range = kmax - kmin;
-        const int nbits = range == 0u ? 0 : 32 - __clz((int)range);
-        const bool mixed = __ballot(any_first) != 0ull && __ballot(any_second) != 0ull;
-        int cur = 0;
-        if (total <= 2 * kWave) {
-            // entry q of the batch: (key, kind bit | q) compared as a pair; entries lane and 64 + lane
-            const bool in0 = lane < total, in1 = kWave + lane < total;
-            const uint32_t k0 = in0 ? lds.key[0][lane] : 0xFFFFFFFFu, k1 = in1 ? lds.key[0][kWave + lane] : 0xFFFFFFFFu;
-            const uint32_t p0 = in0 ? lds.pay2[0][lane] : 0u, p1 = in1 ? lds.pay2[0][kWave + lane] : 0u;
-            const uint32_t t0 = in0 ? (p0 & 0x80000000u) | (uint32_t)lane : 0xFFFFFFFFu;
-            const uint32_t t1 = in1 ? (p1 & 0x80000000u) | (uint32_t)(kWave + lane) : 0xFFFFFFFFu;
-            int rank0 = 0, rank1 = 0;
-            const int n0 = total < kWave ? total : kWave;
-            for (int s = 0; s < n0; s++) {
-                const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k0, s);
-                const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t0, s);
-                rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
-                rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
-            }
-            for (int s = 0; s < total - kWave; s++) {
-                const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k1, s);
-                const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t1, s);
-                rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
-                rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
-            }
-            if (in0) {
-                lds.key[1][rank0] = k0;
-                lds.pay2[1][rank0] = p0;
-            }
-            if (in1) {
-                lds.key[1][rank1] = k1;
-                lds.pay2[1][rank1] = p1;
-            }
-            wave_sync_memory();
-            cur = 1;
+            __syncthreads();
+            cur = batch_order<R, RAVE, kTeam>(lds, lane, total, c.ep, uvl);
+            __syncthreads();
         } else {
-            const int per = ((total + kWave - 1) / kWave) | 1;  // odd: conflict-free block starts
-            const int q0 = lane * per < total ? lane * per : total;
-            const int q1 = q0 + per < total ? q0 + per : total;
-            for (int sh = mixed ? -kSortBits : 0; sh < nbits; sh += kSortBits) {
-                const uint32_t *src_k = lds.key[cur], *src_p = lds.pay2[cur];
-                uint32_t *dst_k = lds.key[cur ^ 1], *dst_p = lds.pay2[cur ^ 1];
-                uint64_t c_lo = 0ull, c_hi = 0ull;  // counters of digit values 0..7 and 8..15
-                for (int q = q0; q < q1; q += 4) {
-                    uint32_t v[4];
-#pragma unroll
-                    for (int u = 0; u < 4; u++) v[u] = q + u < q1 ? (sh < 0 ? src_p[q + u] : src_k[q + u]) : 0u;
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        if (q + u < q1) {
-                            const uint32_t d = sh < 0 ? v[u] >> 31 : ((v[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
-                            const uint64_t one = 1ull << ((d & 7u) * 8u);
-                            if (d & 8u) c_hi += one;
-                            else c_lo += one;
-                        }
-                    }
-                }
-                // Start positions: exclusive prefix of the counts in (digit value, lane) order.
-                // The counts go to LDS in that order with one pad word per sixteen, every lane
-                // then owns sixteen consecutive ones (stride 17: conflict-free), sums them, one
-                // wave scan over the sums, and the prefixes go back to the same places.
-#pragma unroll
-                for (int b = 0; b < kSortBins; b++) {
-                    const int e = b * kWave + lane;
-                    lds.hist[e + (e >> 4)] = (int)(((b < 8 ? c_lo : c_hi) >> ((b & 7) * 8)) & 0xFFull);
-                }
-                wave_sync_memory();
-                {
-                    int h[16];
-                    int lsum = 0;
-#pragma unroll
-                    for (int t = 0; t < 16; t++) {
-                        h[t] = lds.hist[lane * 17 + t];
-                        lsum += h[t];
-                    }
-                    int run = wave_inclusive_sum(lsum, lane) - lsum;
-#pragma unroll
-                    for (int t = 0; t < 16; t++) {
-                        lds.hist[lane * 17 + t] = run;
-                        run += h[t];
-                    }
-                }
-                wave_sync_memory();
-                // the counters are private to their lane from here on
-                for (int q = q0; q < q1; q += 4) {
-                    uint32_t kk[4], pp[4];
-                    int pos[4];
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        kk[u] = q + u < q1 ? src_k[q + u] : 0u;
-                        pp[u] = q + u < q1 ? src_p[q + u] : 0u;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        pos[u] = 0;
-                        if (q + u < q1) {
-                            const uint32_t d = sh < 0 ? pp[u] >> 31 : ((kk[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
-                            const int e = (int)d * kWave + lane;
-                            pos[u] = __hip_atomic_fetch_add(&lds.hist[e + (e >> 4)], 1, __ATOMIC_RELAXED,
-                                                            __HIP_MEMORY_SCOPE_WAVEFRONT);
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        if (q + u < q1) {
-                            dst_k[pos[u]] = kk[u];
-                            dst_p[pos[u]] = pp[u];
-                        }
-                    }
-                }
-                wave_sync_memory();
-                cur ^= 1;
-#ifdef OMK_PHASE_TIMERS
-                if (a.stats && lane == 0) atomicAdd(a.stats + 15, 1);
-#endif
-            }
+            cur = batch_order<R, RAVE, kWave>(lds, lane, total, c.ep, uvl);
         }
+        if ((lds.red[2] & 4u) != 0u) OMK_FAIL(8);
         const uint32_t *skey = lds.key[cur], *spay = lds.pay2[cur];
         OMK_TICK(10);
 
@@ -889,47 +1004,22 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (qcut == 0xFFFFFFFFu) OMK_FAIL(10);
             if ((int)qcut + 1 < keep) keep = (int)qcut + 1;
         }
-#pragma unroll
-        for (int t = 0; t < kSortBins; t++) lds.hist[t * kWave + lane] = 0;  // visits per child after this batch
-        wave_sync_memory();
-        uint32_t pk63 = 0u, ppay63 = 0u;
-        bool have_prev = false;
-        for (int base = 0; base < total; base += kWave) {
-            const int q = base + lane;
-            const bool in = q < total;
-            uint32_t kk = in ? skey[q] : 0u;
-            uint32_t pay = in ? spay[q] : 0u;
-            uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-            uint32_t ppay = (uint32_t)__shfl_up((int)pay, 1, kWave);
-            bool hp = lane > 0 || have_prev;
+        if (team) {
             if (lane == 0) {
-                pk = pk63;
-                ppay = ppay63;
+                lds.cmd.op = kOpEmit;
+                lds.cmd.rounds = R;
+                lds.cmd.total = total;
+                lds.cmd.keep = keep;
+                lds.cmd.goff = off + done;
+                lds.cmd.cur = cur;
             }
-            if (in) {
-                const int child = (int)((pay >> 21) & 1023u);
-                const int j = (int)(pay & 0x1FFFFFu);
-                if (q < keep) {
-                    a.sc_child[off + done + q] = child;
-                    a.sc_occ[off + done + q] = j;
-                    atomicMax(&lds.hist[child], j + 1);
-                }
-                // the order of the whole batch is checked, kept or not: what is dropped must
-                // come after what is kept
-                if (hp) {
-                    if (pk > kk) bad = true;  // not sorted
-                    if (pk == kk) {
-                        const uint32_t pchild = (ppay >> 21) & 1023u;
-                        const uint32_t ppos_ = pchild + ((ppay >> 31) ? (uint32_t)F : 0u);
-                        const uint32_t pos_ = (uint32_t)child + ((pay >> 31) ? (uint32_t)F : 0u);
-                        if (pchild != (uint32_t)child && ppos_ > pos_) bad = true;
-                    }
-                }
-            }
-            pk63 = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-            ppay63 = (uint32_t)__builtin_amdgcn_readlane((int)pay, 63);
-            have_prev = true;
+            __syncthreads();
+            batch_emit<R, kTeam>(a, lds, lane, total, keep, off + done, cur);
+            __syncthreads();
+        } else {
+            batch_emit<R, kWave>(a, lds, lane, total, keep, off + done, cur);
         }
+        bool bad = (lds.red[2] & 4u) != 0u;
         wave_sync_memory();
         {
             // The last kept entry must come before every child's first unevaluated entry (a
@@ -1593,11 +1683,11 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 // and publishes the other parts.  Items depend only on their ancestors, so there is no
 // level barrier: the critical path is the longest chain of crowded nodes.  Every wait is
 // bounded: a wavefront that polls spin_limit times raises the abort flag and all leave.
+//
+// A block is a team: its first wavefront (the owner) runs this loop, the other wavefronts
+// wait at a block barrier until the owner shares out the batch work of a node (team_help).
 template <int RMAX, bool RAVE>
-__global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev f, SelectArgs a) {
-    __shared__ WaveLds<RMAX> s_lds[kGroupWaves];
-    const int lane = threadIdx.x & 63;
-    const int wib = threadIdx.x >> 6;
+__device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs &a, WaveLds<RMAX> &s_lds, int lane) {
     for (;;) {
         int ticket = 0;
         if (lane == 0) ticket = atomicAdd(a.sched_head, 1);
@@ -1650,9 +1740,9 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
             if (c.cc > 0 && depth < a.max_depth) {
                 if (c.cc <= kWave)
                     status = select_group<1, RAVE>(f, a, c, lane, it, seg_in, seg_out,
-                                                   reinterpret_cast<WaveLds<1> &>(s_lds[wib]), next);
+                                                   reinterpret_cast<WaveLds<1> &>(s_lds), next);
                 else
-                    status = select_group<RMAX, RAVE>(f, a, c, lane, it, seg_in, seg_out, s_lds[wib], next);
+                    status = select_group<RMAX, RAVE>(f, a, c, lane, it, seg_in, seg_out, s_lds, next);
             }
 #ifdef OMK_PHASE_TIMERS
             if (lane == 0) {
@@ -1686,6 +1776,44 @@ __global__ __launch_bounds__(kGroupWaves *kWave) void k_select_groups(ForestDev 
             it.depth = depth + 1;
             it.pad[0] = it.pad[1] = it.pad[2] = 0;
         }
+    }
+}
+
+// What a helper wavefront does with one request of its owner.
+template <int R, bool RAVE>
+__device__ __forceinline__ void team_help(const SelectArgs &a, WaveLds<R> &lds, int tid, int op, int total, int keep,
+                                          int goff, int cur, float ep, uint32_t uvl) {
+    if (op == kOpOrder) batch_order<R, RAVE, kTeam>(lds, tid, total, ep, uvl);
+    else if (op == kOpEmit) batch_emit<R, kTeam>(a, lds, tid, total, keep, goff, cur);
+}
+
+template <int RMAX, bool RAVE>
+__global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs a) {
+    __shared__ WaveLds<RMAX> s_lds;
+    const int tid = threadIdx.x;
+    if (tid < kWave) {
+        // every path out of the owner's loop comes back here: the helpers are always released
+        owner_loop<RMAX, RAVE>(f, a, s_lds, tid);
+        if (tid == 0) s_lds.cmd.op = kOpExit;
+        __syncthreads();
+        return;
+    }
+    for (;;) {
+        __syncthreads();  // the owner has written a request
+        const int op = __builtin_amdgcn_readfirstlane(s_lds.cmd.op);
+        if (op == kOpExit) return;
+        const int rounds = __builtin_amdgcn_readfirstlane(s_lds.cmd.rounds);
+        const int total = __builtin_amdgcn_readfirstlane(s_lds.cmd.total);
+        const int keep = __builtin_amdgcn_readfirstlane(s_lds.cmd.keep);
+        const int goff = __builtin_amdgcn_readfirstlane(s_lds.cmd.goff);
+        const int cur = __builtin_amdgcn_readfirstlane(s_lds.cmd.cur);
+        const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
+        const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
+        if (rounds == 1)
+            team_help<1, RAVE>(a, reinterpret_cast<WaveLds<1> &>(s_lds), tid, op, total, keep, goff, cur, ep, uvl);
+        else
+            team_help<RMAX, RAVE>(a, s_lds, tid, op, total, keep, goff, cur, ep, uvl);
+        __syncthreads();  // the request is done
     }
 }
 
@@ -1769,18 +1897,18 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
         // as many wavefronts as can be resident, but no more than there can be items at once
         // (an item has at least two visitors)
         int per_cu = 1;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_select_groups<RMAX, RAVE>, kGroupWaves * kWave, 0) !=
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_select_groups<RMAX, RAVE>, kTeam, 0) !=
                 hipSuccess ||
             per_cu < 1)
             per_cu = 1;
         int grid = n_cus * per_cu;
-        const int most = (n_traversals / 2 + kGroupWaves - 1) / kGroupWaves;
+        const int most = n_traversals / 2;
         if (grid > most) grid = most;
         if (grid < 1) grid = 1;
 #ifdef OMK_PHASE_TIMERS
         if (a.dbg_grid > 0 && grid > a.dbg_grid) grid = a.dbg_grid;
 #endif
-        hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kGroupWaves * kWave), 0, s, f, a);
+        hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kTeam), 0, s, f, a);
     }
     hipLaunchKernelGGL((k_select_singles<RMAX, RAVE>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
     return hipGetLastError();
