@@ -235,9 +235,10 @@ struct NodeCtx {
     float ep;
 };
 
-__device__ __forceinline__ NodeCtx node_ctx(const ForestDev &f, const SelectArgs &a, int node, int np) {
+__device__ __forceinline__ NodeCtx node_ctx(const ForestDev &f, const SelectArgs &a, int node, int np,
+                                            bool have_span = false, int2 span = int2{0, 0}) {
     NodeCtx c;
-    int2 sp = f.span[node];
+    int2 sp = have_span ? span : f.span[node];
     c.cb = sp.x;
     c.cc = sp.y;
     c.nelig = c.cc;
@@ -599,8 +600,10 @@ __device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds,
         const int child = (int)((pay >> 21) & 1023u);
         const int j = (int)(pay & 0x1FFFFFu);
         if (q < keep) {
-            a.sc_child[goff + q] = child;
-            a.sc_occ[goff + q] = j;
+            if (goff >= 0) {  // else the caller reads the order from LDS
+                a.sc_child[goff + q] = child;
+                a.sc_occ[goff + q] = j;
+            }
             atomicMax(&lds.hist[child], j + 1);
         }
         if (q > 0) {
@@ -637,7 +640,9 @@ __device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds,
 template <int R, bool RAVE>
 __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
                                             int off, int rank0, int todo, const int (&tk0)[R], WaveLds<R> &lds,
-                                            int (&cnt)[R]) {
+                                            int (&cnt)[R], bool allow_lds, int &lds_cur, bool use_preset,
+                                            const int (&preset)[R]) {
+    lds_cur = -1;
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     const int m = todo;
@@ -681,6 +686,29 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         if (hi_key == 0u) OMK_FAIL(2);
         const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
 
+        // A slice of a heavy node knows exactly how many entries every child contributes to its
+        // (first) batch: the entries between its two thresholds.  Nothing to search then.
+        int total = 0;
+        int capped_child = -1, capped_last = 0;
+        bool preset_done = false;
+        if (use_preset && done == 0) {
+            int sum = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) sum += preset[r];
+            total = wave_sum_i32(sum);
+            if (total >= 1 && total <= kBatchCap) {
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int i = r * kWave + lane;
+                    lds.st_vl[i] = (int)((uint32_t)k.vl[r] + (uint32_t)tk[r] * uvl);
+                    lds.st_j0[i] = tk[r];
+                    lds.pay[i] = (uint32_t)preset[r];
+                }
+                wave_sync_memory();
+                preset_done = true;
+            }
+        }
+        if (!preset_done) {
         // ---- 0. a long run of the best child ----
         // When the best child's next entries stay ahead of every other child's next entry (its
         // score hardly moves with virtual loss, e.g. a RAVE blend that dominates), they are the
@@ -837,9 +865,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         // last counted entry lies at or after that cut).
         const int child_cap = remaining < kBatchCap + 1 ? remaining : kBatchCap + 1;
         int ct[R];
-        int total = 0;
+        total = 0;
         int tries = 0;
-        int capped_child = -1, capped_last = 0;
         for (;;) {
             if (++tries > 6) OMK_FAIL(5);
             // bisection on the score with the estimated counts only (no exact evaluation)
@@ -953,6 +980,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         for (int r = 0; r < R; r++)
             if (ac[r] >= 0) lds.pay[ac[r]] = (uint32_t)ct[r];
         wave_sync_memory();
+        }  // !preset_done
         int nb[R];  // entries of every own child in this batch
 #pragma unroll
         for (int r = 0; r < R; r++) nb[r] = (int)lds.pay[r * kWave + lane];
@@ -1004,21 +1032,24 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (qcut == 0xFFFFFFFFu) OMK_FAIL(10);
             if ((int)qcut + 1 < keep) keep = (int)qcut + 1;
         }
+        // a node that this one batch settles keeps its winner order in LDS for the partition
+        const bool only_batch = allow_lds && done == 0 && keep == m;
         if (team) {
             if (lane == 0) {
                 lds.cmd.op = kOpEmit;
                 lds.cmd.rounds = R;
                 lds.cmd.total = total;
                 lds.cmd.keep = keep;
-                lds.cmd.goff = off + done;
+                lds.cmd.goff = only_batch ? -1 : off + done;
                 lds.cmd.cur = cur;
             }
             __syncthreads();
-            batch_emit<R, kTeam>(a, lds, lane, total, keep, off + done, cur);
+            batch_emit<R, kTeam>(a, lds, lane, total, keep, only_batch ? -1 : off + done, cur);
             __syncthreads();
         } else {
-            batch_emit<R, kWave>(a, lds, lane, total, keep, off + done, cur);
+            batch_emit<R, kWave>(a, lds, lane, total, keep, only_batch ? -1 : off + done, cur);
         }
+        if (only_batch) lds_cur = cur;
         bool bad = (lds.red[2] & 4u) != 0u;
         wave_sync_memory();
         {
@@ -1189,7 +1220,8 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
 // values (m evaluations spread over the lanes).  Returns false when it is not that case.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
-                                           uint32_t bk, uint32_t bpos, int off, int m, int (&cnt)[R]) {
+                                           uint32_t bk, uint32_t bpos, int off, int m, bool to_global, int (&cnt)[R],
+                                           int &run_child) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     uint32_t hi_key, hi_pos;
@@ -1248,15 +1280,18 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
         carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
     }
     if (__ballot(bad) != 0ull) return false;
-    for (int j = lane; j < m; j += kWave) {
-        a.sc_child[off + j] = best;
-        a.sc_occ[off + j] = j;
+    if (to_global) {
+        for (int j = lane; j < m; j += kWave) {
+            a.sc_child[off + j] = best;
+            a.sc_occ[off + j] = j;
+        }
     }
     if (lane == bl) {
 #pragma unroll
         for (int r = 0; r < R; r++)
             if (r == (best >> 6)) cnt[r] = m;
     }
+    run_child = best;
     return true;
 }
 
@@ -1266,6 +1301,7 @@ struct Continuation {
     int off;
     int m;
     int np;
+    int2 span;  // (child_begin, child_count) of that node, loaded ahead of time
 };
 
 // All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
@@ -1306,6 +1342,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 
     bool settled = false;
     int st_replay = 0;
+    // where the partition finds (child, visit number) of every visitor: all visitors chose
+    // run_child, or the winner order is still in LDS buffer lds_cur, or (both -1) it is in the
+    // sc_child / sc_occ arrays in device memory
+    int run_child = -1, lds_cur = -1;
     bool as_slice = item.pad[0] == 1;
     const bool as_scatter = item.pad[0] == 2;
     int hid = item.pad[0] != 0 ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF, n_slices = item.pad[2] >> 16;
@@ -1317,7 +1357,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         settled = true;
     }
     if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
-        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, cnt);
+        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, m >= kHeavyMin, cnt, run_child);
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
@@ -1397,7 +1437,14 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 const bool closing = last || rank_lo >= m;
                 const int todo = (closing ? m : rank_lo) - rank_hi;
                 if (todo > 0) {
-                    ok = water_level<R, RAVE>(a, c, lane, k, off, rank_hi, todo, ct_hi, lds, cnt);
+                    {
+                        int unused_cur;
+                        int between[R];  // entries of every child between the two thresholds
+#pragma unroll
+                        for (int r = 0; r < R; r++) between[r] = ct_lo[r] - ct_hi[r];
+                        ok = water_level<R, RAVE>(a, c, lane, k, off, rank_hi, todo, ct_hi, lds, cnt, false, unused_cur,
+                                                  !last, between);
+                    }
                 } else {
 #pragma unroll
                     for (int r = 0; r < R; r++) cnt[r] = ct_hi[r];
@@ -1438,25 +1485,31 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         int zero[R];
 #pragma unroll
         for (int r = 0; r < R; r++) zero[r] = 0;
-        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt);
+        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt, m < kHeavyMin, lds_cur, false, zero);
         if (!settled) st_replay = 1;
     }
     if (!settled) {
         // one visitor after the other
+        run_child = -1;
+        lds_cur = -1;
+        const bool seq_lds = m < kHeavyMin;  // few enough visitors to keep their order in LDS
         for (int done = 0; done < m; done++) {
             int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
             if (i < 0) return kStepLeaf;  // no child takes part: uniform, and then for every visitor
             if (a.vl <= 0) {
                 // no virtual loss: nothing changes between visitors, they all follow the first
-                for (int j = lane; j < m; j += kWave) {
-                    a.sc_child[off + j] = i;
-                    a.sc_occ[off + j] = j;
+                if (!seq_lds) {
+                    for (int j = lane; j < m; j += kWave) {
+                        a.sc_child[off + j] = i;
+                        a.sc_occ[off + j] = j;
+                    }
                 }
                 if (lane == (i & 63)) {
 #pragma unroll
                     for (int r = 0; r < R; r++)
                         if (r == (i >> 6)) cnt[r] = m;
                 }
+                run_child = i;
                 break;
             }
             if (lane == (i & 63)) {
@@ -1471,10 +1524,16 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     }
                 }
                 lane_best<R, RAVE>(k, lane, bk, bpos);
-                a.sc_child[off + done] = i;
-                a.sc_occ[off + done] = occ;
+                if (seq_lds) {
+                    lds.pay2[0][done] = ((uint32_t)i << 21) | (uint32_t)occ;
+                } else {
+                    a.sc_child[off + done] = i;
+                    a.sc_occ[off + done] = occ;
+                }
             }
         }
+        if (run_child < 0 && seq_lds) lds_cur = 0;
+        wave_sync_memory();
     }
     OMK_TICK(13);
     if (a.stats && lane == 0 && !as_scatter) {
@@ -1498,6 +1557,9 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // This wavefront walks on with the largest part; the other parts go to the work queue,
     // where idle wavefronts pick them up at once.
     const int keep = gmax >= 2u ? (int)wave_min_u32(lidx) : -1;
+    // where the walk goes on: ask for that node's child range now, it arrives during the scatter
+    int2 keep_span = int2{0, 0};
+    if (keep >= 0) keep_span = f.span[c.cb + keep];
     int carry = 0;
     int keep_np = 0;
     int excl[R];
@@ -1578,8 +1640,17 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             const int j = base + u * kWave + lane;
             const bool in = j < r1;
             tt[u] = in ? seg_in[off + j] : 0;
-            ii[u] = in ? a.sc_child[off + j] : 0;
-            oo[u] = in ? a.sc_occ[off + j] : 0;
+            if (run_child >= 0) {
+                ii[u] = run_child;
+                oo[u] = j;
+            } else if (lds_cur >= 0) {
+                const uint32_t pay = in ? lds.pay2[lds_cur][j] : 0u;
+                ii[u] = (int)((pay >> 21) & 1023u);
+                oo[u] = (int)(pay & 0x1FFFFFu);
+            } else {
+                ii[u] = in ? a.sc_child[off + j] : 0;
+                oo[u] = in ? a.sc_occ[off + j] : 0;
+            }
         }
 #pragma unroll
         for (int u = 0; u < kScatterUnroll; u++) {
@@ -1670,6 +1741,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         next.off = off + lds.offs[keep];
         next.m = (int)gmax;
         next.np = __builtin_amdgcn_readlane(keep_np, keep & 63);
+        next.span = keep_span;
     }
     // the next step of the walk reads seg_out and reuses the LDS scratch
     wave_sync_memory();
@@ -1726,6 +1798,8 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = f.N[it.node];
             for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
+        bool have_span = false;
+        int2 pre_span = int2{0, 0};
         for (;;) {
             const int depth = it.depth;
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
@@ -1733,7 +1807,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
 #ifdef OMK_PHASE_TIMERS
             const long long tr0 = wall_clock64();
 #endif
-            NodeCtx c = node_ctx(f, a, it.node, it.np);
+            NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
             int status = kStepLeaf;
             Continuation next;
             next.node = -1;
@@ -1775,6 +1849,8 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = next.np;
             it.depth = depth + 1;
             it.pad[0] = it.pad[1] = it.pad[2] = 0;
+            have_span = true;
+            pre_span = next.span;
         }
     }
 }
