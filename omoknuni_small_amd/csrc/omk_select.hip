@@ -748,12 +748,23 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + kRunShortcutMin - 1, best, pk_, pp_);
             if (pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos))) {
                 // largest L <= remaining whose last entry still comes before the others' best
+                // (64 candidate lengths at a time, one per lane; the entries are checked one by
+                // one below, so this search only has to propose)
                 int lo_l = kRunShortcutMin, hi_l = remaining;
                 while (lo_l < hi_l) {
-                    const int mid_l = (lo_l + hi_l + 1) >> 1;
-                    entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + mid_l - 1, best, pk_, pp_);
-                    if (pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos))) lo_l = mid_l;
-                    else hi_l = mid_l - 1;
+                    const int step = (hi_l - lo_l + kWave - 1) / kWave;
+                    const int cand = lo_l + (lane + 1) * step;
+                    bool okc = false;
+                    if (cand <= hi_l) {
+                        entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + cand - 1, best, pk_, pp_);
+                        okc = pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos));
+                    }
+                    const uint64_t okm = __ballot(okc);
+                    const int n_ok = okm == ~0ull ? kWave : __builtin_ctzll(~okm);  // leading run of successes
+                    const int new_lo = lo_l + n_ok * step;
+                    const int new_hi = lo_l + (n_ok + 1) * step - 1;
+                    lo_l = new_lo < hi_l ? new_lo : hi_l;
+                    hi_l = new_hi < hi_l ? new_hi : hi_l;
                 }
                 const int L = lo_l;
                 // every entry of the run: a real key, never before its predecessor
