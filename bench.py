@@ -7,7 +7,7 @@ backup of one value per leaf (update + revert virtual loss, sign flipped per ply
 the leaf-key table probes on the workload that has them.  Everything a step touches is
 resident in HBM before the timed region starts; nothing returns to the host inside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0..c4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0..c4|wide]
 
 Prints ONE JSON line.  `value` is traversals per second over whole steps (every
 traversal is selected AND backed up inside the timed region).  `roofline` prices the
@@ -100,7 +100,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c0", "c1", "c2", "c3", "c4"])
+    ap.add_argument("--workload", default="c3", choices=["c0", "c1", "c2", "c3", "c4", "wide"])
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--scale", type=float, default=1.0, help="scale nodes_per_tree (debugging only)")

@@ -157,6 +157,10 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * steps, [7] unused, [8..14] per-phase cycle counts in measurement builds (else 0),
  * [15] nodes cut into slices for several wavefronts. */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
+/* The counters above cost one atomic per processed node (and per single-visitor step), all on
+ * the same few addresses, so they are off unless switched on here (enabled != 0); with
+ * them off omk_batch_stats returns zeros.  Diagnostics only; no counterpart in the reference. */
+int omk_batch_set_stats(omk_batch *b, int32_t enabled);
 /* The multi-visitor selection kernel is persistent: its wavefronts wait for work items that
  * other wavefronts publish.  Every wait is bounded; a wavefront that polls `polls` times in
  * vain raises an abort flag, all wavefronts leave, and omk_batch_read reports OMK_ERR_STATE

@@ -88,6 +88,7 @@ struct omk_batch {
     // that each lies in a memory channel of its own
     int32_t *counters = nullptr;
     int32_t poll_sleep = 1;
+    bool stats_on = false;
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
     int32_t *hctx = nullptr;     // contexts of heavy nodes
     int32_t hctx_cap = 0;
@@ -475,7 +476,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.epoch = b->epoch;
     a.spin_limit = b->spin_limit;
     a.truncated = b->counters + 0;
-    a.stats = b->counters + 1;
+    a.stats = b->stats_on ? b->counters + 1 : nullptr;
     a.n_singles = b->counters + 17;
     a.sched_head = b->counters + 1 * kSchedStep;
     a.sched_tail = b->counters + 2 * kSchedStep;
@@ -590,6 +591,12 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipMemcpyAsync(h_count, b->counters + 0, 4, hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
+    return OMK_OK;
+}
+
+int omk_batch_set_stats(omk_batch *b, int32_t enabled) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_batch_set_stats: null batch");
+    b->stats_on = enabled != 0;
     return OMK_OK;
 }
 

@@ -25,7 +25,7 @@ EXPORTS = [
     "omk_forest_upload", "omk_forest_download", "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
 ]
@@ -260,6 +260,10 @@ class Batch:
         c = C.c_int32()
         _check(self._lib.omk_batch_truncated(self._h, C.byref(c)))
         return c.value
+
+    def enable_stats(self, on=True):
+        """Work statistics of select() (see stats()); off by default, they cost atomics."""
+        _check(self._lib.omk_batch_set_stats(self._h, C.c_int32(1 if on else 0)))
 
     def set_spin_limit(self, polls):
         """Bound of the waits inside the persistent selection kernel (error-path tests)."""

@@ -49,6 +49,12 @@ CONFIGS = {
     "c4": dict(n_trees=1, nodes_per_tree=16_000_000, dense=1, fanout=362, legal_frac=0.6, last_legal=1, zipf_s=1.1,
                n_cap=10_000, logit_sigma=1.5, max_depth=30, growth_width=2048, has_rave=1, with_hash=1,
                n_traversals=16384, c_puct=1.4, virtual_loss=3, rave_k=1000.0, tt_log2=24),
+    # Not one of the benchmark configurations: a wide forest in which every descent is alone in
+    # its tree, the regime where selection is bound by HBM bandwidth rather than by the chain of
+    # crowded nodes (used to place the single-visitor kernel on the roofline).
+    "wide": dict(n_trees=32768, nodes_per_tree=1000, dense=1, fanout=225, legal_frac=0.5, last_legal=0, zipf_s=1.2,
+                 n_cap=10_000, logit_sigma=1.0, max_depth=12, growth_width=8, n_traversals=32768, c_puct=1.4,
+                 virtual_loss=3),
 }
 
 

@@ -67,6 +67,7 @@ def select_both(soa, troots, D, vl=3, rave=False, rave_k=1000.0, steps=2):
     f = omk.Forest.from_soa(soa)
     b = omk.Batch(f, len(troots), D)
     b.set_roots(troots)
+    b.enable_stats()
     sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=rave_k)
     rng = np.random.default_rng(1)
     stats = None
