@@ -63,39 +63,51 @@ __global__ __launch_bounds__(256) void k_revert_vl(ForestDev f, const int32_t *p
     if (act) vl_sub_clamp(f.VL + node, vl);
 }
 
+// One thread per (traversal, depth).  Many traversals of a block meet on the same nodes near
+// the root (thousands of visitors on a handful of nodes), and atomics on one address are
+// served one after another: the block first combines its visits per node in a small LDS
+// table (count, value sum) and then issues one set of global atomics per distinct node.
+constexpr int kBackupSlots = 512;  // two per thread: the table never fills
+
 __global__ __launch_bounds__(256) void k_backup(ForestDev f, const int32_t *paths, const int32_t *path_len,
                                                 const float *values, int n, int stride, int vl) {
-    int t = blockIdx.x * 256 + threadIdx.x;
+    __shared__ int s_key[kBackupSlots];
+    __shared__ int s_cnt[kBackupSlots];
+    __shared__ float s_w[kBackupSlots];
+    const int tid = threadIdx.x;
+    int t = blockIdx.x * 256 + tid;
     int d = blockIdx.y;
     int len = t < n ? path_len[t] : 0;
     bool act = d < len;
-    int node = act ? paths[(size_t)d * stride + t] : -1;
-    float v = 0.0f;
+    if (__syncthreads_or(act ? 1 : 0) == 0) return;  // nothing this deep in this block
+    for (int i = tid; i < kBackupSlots; i += 256) {
+        s_key[i] = -1;
+        s_cnt[i] = 0;
+        s_w[i] = 0.0f;
+    }
+    __syncthreads();
     if (act) {
-        v = values[t];
+        int node = paths[(size_t)d * stride + t];
+        float v = values[t];
         if ((len - 1 - d) & 1) v = -v;  // the leaf receives +value, every ply up flips it
-    }
-    uint64_t mask = __ballot(act);
-    if (mask == 0ull) return;
-    int leader = __ffsll((long long)mask) - 1;
-    int node0 = __builtin_amdgcn_readlane(node, leader);
-    bool same = __ballot(act && node != node0) == 0ull;
-    if (same) {
-        float sum = wave_sum_f32(v);
-        if ((int)(threadIdx.x & 63) == leader) {
-            int cnt = __popcll(mask);
-            atomicAdd(f.N + node0, cnt);
-            unsafeAtomicAdd(f.W + node0, sum);
-            if (vl > 0) vl_sub_clamp(f.VL + node0, (vl + 1) * cnt);
-            else vl_dec_if_positive(f.VL + node0, cnt);
+        uint32_t h = ((uint32_t)node * 2654435761u) >> 23;
+        for (;;) {
+            int prev = atomicCAS(&s_key[h], -1, node);
+            if (prev == -1 || prev == node) break;
+            h = (h + 1u) & (uint32_t)(kBackupSlots - 1);
         }
-        return;
+        atomicAdd(&s_cnt[h], 1);
+        atomicAdd(&s_w[h], v);
     }
-    if (act) {
-        atomicAdd(f.N + node, 1);
-        unsafeAtomicAdd(f.W + node, v);
-        if (vl > 0) vl_sub_clamp(f.VL + node, vl + 1);
-        else vl_dec_if_positive(f.VL + node, 1);
+    __syncthreads();
+    for (int i = tid; i < kBackupSlots; i += 256) {
+        const int node = s_key[i];
+        if (node < 0) continue;
+        const int cnt = s_cnt[i];
+        atomicAdd(f.N + node, cnt);
+        unsafeAtomicAdd(f.W + node, s_w[i]);
+        if (vl > 0) vl_sub_clamp(f.VL + node, (vl + 1) * cnt);
+        else vl_dec_if_positive(f.VL + node, cnt);
     }
 }
 
