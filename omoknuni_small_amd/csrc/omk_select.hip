@@ -10,12 +10,13 @@
 // node all come through its parent.  So a work item is (node, the list of traversals that
 // reached it, in traversal-index order); ONE 64-lane wavefront owns the item and loads the
 // children once (coalesced, one child per lane per round).  The visitors are then
-// partitioned by chosen child (stable, so still in traversal order) into the work items
-// of the next level's launch; the wavefront walks on itself with a group that stays together
-// (or, for small groups, with a part that holds at least three quarters of it), and lone
-// visitors go to the single-visitor walk.
+// partitioned by chosen child (stable, so still in traversal order): the wavefront walks on
+// itself with the largest part, the other parts with several visitors become new items, and
+// lone visitors go to the single-visitor walk.
 //
 // Which child each visitor chooses:
+//  * one winner: if the best child's score for the LAST visitor still beats every other
+//    child's first score and its own scores never increase, every visitor takes it.
 //  * few visitors: they are played one after another on register-resident statistics --
 //    score, DPP arg-max with lowest-index tie-break, bump the chosen child's virtual loss,
 //    next visitor.  That is the serial order itself.
@@ -23,18 +24,28 @@
 //    batch depends on nothing but j.  If every child's scores do not increase with j, the
 //    serial winner sequence is the merge of these descending lists, i.e. the m best
 //    entries (i, j) in the order (score descending, candidate position ascending, j
-//    ascending).  In batches of up to 2048 entries: a bisection on the score threshold
-//    finds how many entries each child contributes, the entries are evaluated in parallel
-//    into LDS, a stable radix sort puts them in winner order.  Nothing is assumed:
-//    afterwards the wavefront checks, on the exact binary32 values, (i) that every child's
-//    taken entries and its first untaken entry do not increase and (ii) that the last
-//    taken entry still comes before every child's first untaken one.  Under (i) and (ii)
-//    the serial loop provably produces exactly this sequence; if either fails the node is
-//    replayed one visitor at a time.
+//    ascending).  In batches of up to 2048 entries: a search on the score threshold finds
+//    how many entries each child contributes (estimated by the closed-form inverse of the
+//    score, then counted exactly), the entries are evaluated in parallel into LDS, a stable
+//    radix sort puts them in winner order.  Nothing is assumed: afterwards the wavefront
+//    checks, on the exact binary32 values, (i) that every child's taken entries and its
+//    first untaken entry do not increase and (ii) that the last taken entry still comes
+//    before every child's first untaken one.  Under (i) and (ii) the serial loop provably
+//    produces exactly this sequence; if either fails the node is replayed one visitor at a
+//    time.  A long run of one child (its score hardly moves with virtual loss) is emitted
+//    without sorting.
+//  * a thousand visitors or more: the node is cut into slices of its winner order that
+//    several wavefronts settle side by side, and the partition is shared out the same way
+//    (see select_group).
 //
-// Two kernels: the multi-visitor kernel (LDS heavy, one launch per tree level) and the
-// single-visitor walk (no LDS, high occupancy, one launch): a visitor that is alone at a
-// node stays alone to its leaf, so it needs no level synchronisation at all.
+// Scheduling.  Two kernels.  The multi-visitor kernel is persistent: blocks of four
+// wavefronts, the first of which (the owner) takes tickets of a device-side work queue,
+// waits (bounded) until the item with that number is published, and processes it; the
+// other three help it with the batch work of larger nodes through block barriers.  Items
+// depend only on their ancestors, so there is no barrier between tree levels: the time of
+// a selection is the longest chain of crowded nodes.  The single-visitor walk (no LDS,
+// high occupancy, one launch afterwards) takes the visitors that are alone at a node: they
+// stay alone to their leaf.
 #include <algorithm>
 
 #include "omk_internal.h"
