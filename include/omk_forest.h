@@ -108,6 +108,14 @@ int omk_forest_get_stream(omk_forest *f, void **hip_stream_out);
 int omk_forest_upload(omk_forest *f, const omk_soa_view *h_view);
 /* Copies N, W, P, VL (and rN, rW) back; structure pointers of the view are ignored. */
 int omk_forest_download(omk_forest *f, omk_soa_view *h_view);
+/* Nodes the forest holds now (it grows with omk_expand_batch) and the room it was created
+ * with.  Either pointer may be NULL. */
+int omk_forest_node_count(omk_forest *f, int64_t *h_nodes, int64_t *h_capacity);
+/* Copies the structure back: first child id, child count (MCTSNode::getChildren().size(),
+ * 0 = isLeaf, src/mcts/mcts_node.cpp:442-444) and action (getAction) of every node; n_nodes
+ * must be the current node count; any pointer may be NULL. */
+int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_child_begin, int32_t *h_child_count,
+                                  int32_t *h_action);
 int omk_sync(omk_forest *f);
 
 /* ---- batch: the per-search buffers of executeBatchedTreeSearch
@@ -142,6 +150,25 @@ int omk_revert_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_
                         int32_t stride, int32_t max_len, int32_t virtual_loss);
 int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len,
                      const float *d_values, int32_t n, int32_t stride, int32_t max_len, int32_t virtual_loss);
+
+/* Leaf expansion for the leaves of the last selection: MCTSNode::expand
+ * (src/mcts/mcts_node.cpp:238-436) followed by setPriorProbabilities (:512-593), as the backup
+ * phase does before it backs the values up (src/mcts/mcts_engine_batch_tree_simple.cpp:249-259).
+ * The game rules stay on the host: simulation t offers the legal moves
+ * h_moves[h_move_begin[t] .. h_move_begin[t+1]) of its leaf state (the state it replayed from
+ * omk_batch_read); an empty list means a terminal state, the node stays a leaf.  A leaf
+ * reached by several simulations is expanded once, with the list of the first of them in
+ * index order that offers moves; a node that already has children is left alone; at most
+ * 1000 moves are used (the reference's limit).  One child per move in the order given (the
+ * reference shuffles with a random seed: every order is one of its outcomes), zero
+ * statistics, action = the move.  Priors: h_policy NULL -> 1 / children (expand's uniform
+ * prior); else row t of h_policy has action_space entries and the prior is
+ * clamp(policy[move], 0, 1), or 0.01 for a move outside the action space.  New node ids are
+ * handed out from the current node count on, in simulation order; OMK_ERR_CAPACITY (and no
+ * change) when the forest's capacity would be exceeded.  h_first_child (NULL or [n]): first
+ * new id for the simulation whose list was used, else -1.  Waits for the stream. */
+int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
+                     int32_t action_space, int32_t *h_first_child);
 
 /* Leaf gather (mcts_engine_batch_tree_simple.cpp:114,166-184): waits for the stream and
  * returns, per traversal, the path (row of max_depth+1 ids, -1 padded), its length, the

@@ -51,6 +51,21 @@ struct omk_forest {
     int children = 0;       // live batches and tables created on this forest
     bool released = false;  // omk_forest_destroy was called while children were alive
 
+    ForestMut mut() const {
+        ForestMut m;
+        m.span = span;
+        m.N = N;
+        m.W = W;
+        m.P = P;
+        m.VL = VL;
+        m.rN = has_rave ? rN : nullptr;
+        m.rW = has_rave ? rW : nullptr;
+        m.legal = has_legal ? legal : nullptr;
+        m.action = has_action ? action : nullptr;
+        m.hash = has_hash ? hash : nullptr;
+        return m;
+    }
+
     ForestDev dev() const {
         ForestDev d;
         d.span = span;
@@ -98,6 +113,8 @@ struct omk_batch {
     int32_t n_cus = 0;
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
+    void *exp_buf = nullptr;  // staging of an expansion: jobs, moves, priors, status
+    size_t exp_bytes = 0;
 };
 
 struct omk_tt {
@@ -309,6 +326,40 @@ int omk_forest_download(omk_forest *f, omk_soa_view *v) {
     return OMK_OK;
 }
 
+int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_child_begin, int32_t *h_child_count,
+                                  int32_t *h_action) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_download_structure: null forest");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_download_structure: nothing uploaded");
+    if (n_nodes != f->n_nodes)
+        return fail(OMK_ERR_INVALID, "omk_forest_download_structure: room for %lld nodes, forest has %lld",
+                    (long long)n_nodes, (long long)f->n_nodes);
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    if (h_action) {
+        if (f->has_action) {
+            HIP_TRY(hipMemcpy(h_action, f->action, (size_t)n_nodes * 4, hipMemcpyDeviceToHost));
+        } else {
+            for (int64_t i = 0; i < n_nodes; i++) h_action[i] = (int32_t)i;
+        }
+    }
+    if (h_child_begin || h_child_count) {
+        std::vector<int2> sp((size_t)n_nodes);
+        HIP_TRY(hipMemcpy(sp.data(), f->span, (size_t)n_nodes * sizeof(int2), hipMemcpyDeviceToHost));
+        for (int64_t i = 0; i < n_nodes; i++) {
+            if (h_child_begin) h_child_begin[i] = sp[(size_t)i].x;
+            if (h_child_count) h_child_count[i] = sp[(size_t)i].y;
+        }
+    }
+    return OMK_OK;
+}
+
+int omk_forest_node_count(omk_forest *f, int64_t *h_nodes, int64_t *h_capacity) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_node_count: null forest");
+    if (h_nodes) *h_nodes = f->n_nodes;
+    if (h_capacity) *h_capacity = f->capacity;
+    return OMK_OK;
+}
+
 // ---------------------------------------------------------------- batch
 
 int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, omk_batch **out) {
@@ -370,7 +421,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q, b->q_ready, b->hctx};
+                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -557,6 +608,109 @@ int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_pat
     if (int rc = check_paths_args("omk_backup_paths", f, d_paths, d_path_len, n, stride, max_len)) return rc;
     if (!d_values) return fail(OMK_ERR_INVALID, "omk_backup_paths: null values");
     HIP_TRY(launch_backup(f->dev(), d_paths, d_path_len, d_values, n, stride, max_len, virtual_loss, f->stream));
+    return OMK_OK;
+}
+
+int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
+                     int32_t action_space, int32_t *h_first_child) {
+    if (!b || !h_move_begin || !h_moves) return fail(OMK_ERR_INVALID, "omk_expand_batch: null argument");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_expand_batch: no selected paths");
+    if (h_policy && action_space <= 0)
+        return fail(OMK_ERR_INVALID, "omk_expand_batch: a policy needs action_space > 0 (got %d)", action_space);
+    omk_forest *f = b->f;
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    const int n = b->n;
+    std::vector<int32_t> leaf((size_t)n);
+    HIP_TRY(hipMemcpyAsync(leaf.data(), b->leaf, (size_t)n * 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    // one job per distinct leaf: the first traversal (in index order) that offers moves wins
+    std::vector<ExpandJob> jobs;
+    std::vector<int32_t> job_of((size_t)n, -1), moves;
+    std::vector<float> priors;
+    std::vector<int32_t> seen;  // leaves with a job, kept sorted by leaf id via the index below
+    {
+        std::vector<std::pair<int32_t, int32_t>> order;  // (leaf, traversal) of every offer
+        for (int t = 0; t < n; t++) {
+            if (h_move_begin[t + 1] < h_move_begin[t])
+                return fail(OMK_ERR_INVALID, "omk_expand_batch: move_begin decreases at traversal %d", t);
+            if (h_move_begin[t + 1] > h_move_begin[t] && leaf[(size_t)t] >= 0) order.emplace_back(leaf[(size_t)t], t);
+        }
+        std::sort(order.begin(), order.end());
+        std::vector<int32_t> winners;
+        for (size_t i = 0; i < order.size(); i++)
+            if (i == 0 || order[i].first != order[i - 1].first) winners.push_back(order[i].second);
+        std::sort(winners.begin(), winners.end());  // ids are handed out in traversal order
+        int64_t cursor = f->n_nodes;
+        bool sorted = true;
+        int mf = f->max_fanout;
+        for (int32_t t : winners) {
+            int32_t cnt = h_move_begin[t + 1] - h_move_begin[t];
+            if (cnt > 1000) cnt = 1000;  // MCTSNode::expand: max_reasonable_moves
+            ExpandJob j;
+            j.leaf = leaf[(size_t)t];
+            j.begin = (int32_t)cursor;
+            j.count = cnt;
+            j.off = (int32_t)moves.size();
+            float prev = 2.0f;
+            for (int32_t i = 0; i < cnt; i++) {
+                const int32_t mv = h_moves[h_move_begin[t] + i];
+                float prior;
+                if (!h_policy) {
+                    prior = 1.0f / (float)cnt;  // expand(): uniform prior
+                } else if (mv >= 0 && mv < action_space) {
+                    prior = h_policy[(size_t)t * (size_t)action_space + (size_t)mv];
+                    prior = prior > 0.0f ? prior : 0.0f;  // setPriorProbabilities: clamp to [0, 1]
+                    prior = prior < 1.0f ? prior : 1.0f;
+                } else {
+                    prior = 0.01f;  // move outside the action space
+                }
+                if (prior > prev) sorted = false;
+                prev = prior;
+                moves.push_back(mv);
+                priors.push_back(prior);
+            }
+            job_of[(size_t)t] = (int32_t)jobs.size();
+            jobs.push_back(j);
+            cursor += cnt;
+            mf = std::max(mf, (int)cnt);
+        }
+        if (cursor > f->capacity)
+            return fail(OMK_ERR_CAPACITY, "omk_expand_batch: %lld nodes needed, capacity %lld", (long long)cursor,
+                        (long long)f->capacity);
+        if (cursor > INT32_MAX) return fail(OMK_ERR_CAPACITY, "omk_expand_batch: node ids exceed 32 bits");
+        if (h_first_child)
+            for (int t = 0; t < n; t++) h_first_child[t] = -1;
+        if (jobs.empty()) return OMK_OK;
+        // staging: jobs | moves | priors | status
+        const size_t nj = jobs.size(), nm = moves.size();
+        const size_t bytes = nj * sizeof(ExpandJob) + nm * 8 + nj * 4;
+        if (bytes > b->exp_bytes) {
+            if (b->exp_buf) HIP_TRY(hipFree(b->exp_buf));
+            b->exp_buf = nullptr;
+            b->exp_bytes = 0;
+            HIP_TRY(hipMalloc(&b->exp_buf, bytes * 2));
+            b->exp_bytes = bytes * 2;
+        }
+        char *base = (char *)b->exp_buf;
+        ExpandJob *d_jobs = (ExpandJob *)base;
+        int32_t *d_moves = (int32_t *)(base + nj * sizeof(ExpandJob));
+        float *d_priors = (float *)(d_moves + nm);
+        int32_t *d_status = (int32_t *)(d_priors + nm);
+        HIP_TRY(hipMemcpyAsync(d_jobs, jobs.data(), nj * sizeof(ExpandJob), hipMemcpyHostToDevice, s));
+        HIP_TRY(hipMemcpyAsync(d_moves, moves.data(), nm * 4, hipMemcpyHostToDevice, s));
+        HIP_TRY(hipMemcpyAsync(d_priors, priors.data(), nm * 4, hipMemcpyHostToDevice, s));
+        HIP_TRY(launch_expand(f->mut(), d_jobs, (int)nj, d_moves, d_priors, d_status, f->n_nodes, cursor, s));
+        std::vector<int32_t> status(nj);
+        HIP_TRY(hipMemcpyAsync(status.data(), d_status, nj * 4, hipMemcpyDeviceToHost, s));
+        HIP_TRY(hipStreamSynchronize(s));
+        f->n_nodes = cursor;
+        f->max_fanout = mf;
+        if (!sorted) f->prior_sorted = false;
+        if (h_first_child)
+            for (int t = 0; t < n; t++)
+                if (job_of[(size_t)t] >= 0) h_first_child[t] = status[(size_t)job_of[(size_t)t]];
+    }
     return OMK_OK;
 }
 

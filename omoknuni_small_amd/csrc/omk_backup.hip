@@ -130,6 +130,58 @@ __global__ __launch_bounds__(256) void k_export(ForestDev f, const int32_t *path
     }
 }
 
+// ---- leaf expansion: MCTSNode::expand + setPriorProbabilities
+// (src/mcts/mcts_node.cpp:238-436, :512-593) for a batch of leaves ----
+
+// Bits of the legal mask for ids that did not exist before: the tail of the last old word
+// and every later word up to the new end start out clear.
+__global__ void k_expand_mask(uint32_t *legal, int64_t old_nodes, int64_t new_nodes) {
+    const int64_t w0 = old_nodes >> 5, w1 = (new_nodes + 31) >> 5;
+    for (int64_t w = w0 + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; w < w1;
+         w += (int64_t)gridDim.x * blockDim.x) {
+        if (w == w0 && (old_nodes & 31)) legal[w] &= (1u << (old_nodes & 31)) - 1u;
+        else legal[w] = 0u;
+    }
+}
+
+// One wavefront per leaf.  The children are written first, the leaf's child range last: a
+// node is a leaf exactly while its child count is 0.  A leaf that already has children
+// (the selection stopped at it because of the depth bound) is left alone; the ids reserved
+// for it become unreachable nodes with zero statistics.
+__global__ __launch_bounds__(64) void k_expand(ForestMut f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
+                                               const float *priors, int32_t *status) {
+    const int j = blockIdx.x;
+    if (j >= n_jobs) return;
+    const ExpandJob job = jobs[j];
+    const bool fresh = f.span[job.leaf].y == 0;
+    for (int i = threadIdx.x; i < job.count; i += 64) {
+        const int id = job.begin + i;
+        f.N[id] = 0;
+        f.W[id] = 0.0f;
+        f.P[id] = fresh ? priors[job.off + i] : 0.0f;
+        f.VL[id] = 0;
+        if (f.rN) f.rN[id] = 0;
+        if (f.rW) f.rW[id] = 0.0f;
+        f.span[id] = int2{0, 0};
+        if (f.action) f.action[id] = moves[job.off + i];
+        if (f.hash) f.hash[id] = 0ull;
+        if (f.legal && fresh) atomicOr(f.legal + ((uint32_t)id >> 5), 1u << ((uint32_t)id & 31u));
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (fresh) f.span[job.leaf] = int2{job.begin, job.count};
+        status[j] = fresh ? job.begin : -1;
+    }
+}
+
+hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
+                         const float *priors, int32_t *status, int64_t old_nodes, int64_t new_nodes, hipStream_t s) {
+    if (n_jobs <= 0) return hipSuccess;
+    if (f.legal) hipLaunchKernelGGL(k_expand_mask, dim3(64), dim3(256), 0, s, f.legal, old_nodes, new_nodes);
+    hipLaunchKernelGGL(k_expand, dim3(n_jobs), dim3(64), 0, s, f, jobs, n_jobs, moves, priors, status);
+    return hipGetLastError();
+}
+
 // plain copy of 4-byte words: the known-size kernel that hardware traffic counters are scaled by
 __global__ __launch_bounds__(256) void k_copy_words(uint32_t *dst, const uint32_t *src, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;

@@ -81,6 +81,47 @@ void ForestEngine::backPropagateBatch(const std::vector<float> &leaf_values) {
     check(omk_backup_batch(batch_, settings_.virtual_loss), "omk_backup_batch");
 }
 
+int64_t ForestEngine::nodeCount() const {
+    int64_t n = 0;
+    check(omk_forest_node_count(forest_, &n, nullptr), "omk_forest_node_count");
+    return n;
+}
+
+void ForestEngine::downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action) {
+    check(omk_forest_download_structure(forest_, n_nodes, child_begin, child_count, action),
+          "omk_forest_download_structure");
+}
+
+int64_t ForestEngine::expandLeafBatch(const std::vector<std::vector<int>> &legal_moves,
+                                      const std::vector<NetworkOutput> &outputs) {
+    if ((int)legal_moves.size() != last_n_) throw std::runtime_error("expandLeafBatch: one move list per simulation");
+    size_t action_space = 0;
+    bool have_policy = outputs.size() == legal_moves.size() && !outputs.empty();
+    if (have_policy) {
+        action_space = outputs[0].policy.size();
+        for (const auto &o : outputs)
+            if (o.policy.size() != action_space) have_policy = false;
+        if (action_space == 0) have_policy = false;
+    }
+    std::vector<int32_t> begin(legal_moves.size() + 1, 0), moves;
+    for (size_t i = 0; i < legal_moves.size(); i++) {
+        moves.insert(moves.end(), legal_moves[i].begin(), legal_moves[i].end());
+        begin[i + 1] = (int32_t)moves.size();
+    }
+    if (moves.empty()) moves.push_back(0);
+    std::vector<float> policy;
+    if (have_policy) {
+        policy.resize(outputs.size() * action_space);
+        for (size_t i = 0; i < outputs.size(); i++)
+            std::copy(outputs[i].policy.begin(), outputs[i].policy.end(), policy.begin() + i * action_space);
+    }
+    const int64_t before = nodeCount();
+    check(omk_expand_batch(batch_, begin.data(), moves.data(), have_policy ? policy.data() : nullptr,
+                           (int32_t)action_space, nullptr),
+          "omk_expand_batch");
+    return nodeCount() - before;
+}
+
 int ForestEngine::executeBatchedTreeSearch(int32_t root) {
     int completed = 0;
     std::vector<LeafItem> leaves;
@@ -92,6 +133,7 @@ int ForestEngine::executeBatchedTreeSearch(int32_t root) {
         if (out.size() != leaves.size()) throw std::runtime_error("inference function returned a short batch");
         values.resize(out.size());
         for (size_t i = 0; i < out.size(); i++) values[i] = out[i].value;
+        if (legal_moves_fn_) expandLeafBatch(legal_moves_fn_(leaves), out);  // reference :249-259
         backPropagateBatch(values);
         completed += n;
     }

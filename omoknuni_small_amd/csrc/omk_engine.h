@@ -5,6 +5,7 @@
 // (reference src/mcts/mcts_engine_batch_tree_simple.cpp:14-301):
 //   selectLeafBatch      phase 1 (:73-185) + leaf gather (:166-206): one LeafItem per simulation
 //   InferenceFunction    phase 2 (:212-236): the evaluator, called once per batch
+//   expandLeafBatch      phase 3, first half (:249-259): expand + setPriorProbabilities of the leaves
 //   backPropagateBatch   phase 3 (:276-281): update + revertVirtualLoss, sign flipped per ply
 // The reference hands the evaluator cloned game states; here a LeafItem carries the leaf
 // node and the move list to replay on a clone of the root state (what :170-178 does), so
@@ -51,6 +52,9 @@ struct LeafItem {
 };
 
 using InferenceFunction = std::function<std::vector<NetworkOutput>(const std::vector<LeafItem> &)>;
+// The legal moves of every leaf's state (IGameState::getLegalMoves on the state the host
+// replayed; an empty list = terminal state).  Game rules stay on the host.
+using LegalMovesFunction = std::function<std::vector<std::vector<int>>(const std::vector<LeafItem> &)>;
 
 class ForestEngine {
    public:
@@ -68,9 +72,17 @@ class ForestEngine {
     // Simulation i starts at roots[i]: independent trees searched side by side.
     void selectLeafBatch(const std::vector<int32_t> &roots, std::vector<LeafItem> &leaves);
     void backPropagateBatch(const std::vector<float> &leaf_values);
+    // Expands the leaves of the last selectLeafBatch on the device: one child per legal move,
+    // priors from the evaluator's policy (uniform when a policy is empty or absent: all
+    // policies of a batch must have the same size).  Returns the nodes added.
+    int64_t expandLeafBatch(const std::vector<std::vector<int>> &legal_moves, const std::vector<NetworkOutput> &outputs);
+    void setLegalMovesFunction(LegalMovesFunction fn) { legal_moves_fn_ = std::move(fn); }
+    int64_t nodeCount() const;
+    void downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action);
 
-    // The whole loop of executeBatchedTreeSearch without the expansion step: batches of
-    // settings.batch_size until num_simulations are done.  Returns simulations run.
+    // The whole loop of executeBatchedTreeSearch: batches of settings.batch_size until
+    // num_simulations are done; leaves are expanded when a legal-moves function is set.
+    // Returns simulations run.
     int executeBatchedTreeSearch(int32_t root);
 
     const MCTSSettings &settings() const { return settings_; }
@@ -80,6 +92,7 @@ class ForestEngine {
     void ensureBatch(int n);
 
     InferenceFunction inference_fn_;
+    LegalMovesFunction legal_moves_fn_;
     MCTSSettings settings_;
     omk_forest *forest_ = nullptr;
     omk_batch *batch_ = nullptr;

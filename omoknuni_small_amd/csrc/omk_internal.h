@@ -96,6 +96,32 @@ hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t
 
 hipError_t launch_copy_words(void *dst, const void *src, int64_t n_words, hipStream_t s);
 
+// The same arrays for the one operation that writes the structure (leaf expansion).
+struct ForestMut {
+    int2 *span;
+    int32_t *N;
+    float *W;
+    float *P;
+    int32_t *VL;
+    int32_t *rN;
+    float *rW;
+    uint32_t *legal;
+    int32_t *action;
+    uint64_t *hash;
+};
+
+// One leaf to expand: its children get the ids [begin, begin + count) and the moves / priors
+// moves[off .. off + count), priors[off .. off + count).
+struct ExpandJob {
+    int32_t leaf;
+    int32_t begin;
+    int32_t count;
+    int32_t off;
+};
+
+hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
+                         const float *priors, int32_t *status, int64_t old_nodes, int64_t new_nodes, hipStream_t s);
+
 struct TTSlot {
     unsigned long long key;
     int32_t node;

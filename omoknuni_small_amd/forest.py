@@ -22,7 +22,8 @@ u64p = C.POINTER(C.c_uint64)
 
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
-    "omk_forest_upload", "omk_forest_download", "omk_sync", "omk_batch_create", "omk_batch_destroy",
+    "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
+    "omk_expand_batch", "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
@@ -111,8 +112,9 @@ class Forest:
         _check(self._lib.omk_forest_create(C.byref(desc), C.byref(self._h)))
 
     @classmethod
-    def from_soa(cls, soa, device=0):
-        f = cls(len(soa["N"]), device=device, has_rave=soa.get("rN") is not None)
+    def from_soa(cls, soa, device=0, capacity=None):
+        """capacity > len(N) leaves room for Batch.expand() to add nodes."""
+        f = cls(max(len(soa["N"]), int(capacity or 0)), device=device, has_rave=soa.get("rN") is not None)
         f.upload(soa)
         return f
 
@@ -157,9 +159,24 @@ class Forest:
         _check(self._lib.omk_forest_upload(self._h, C.byref(v)))
         self.n_nodes = n
 
+    def node_count(self):
+        """(nodes now, capacity): the forest grows with Batch.expand()."""
+        n, cap = C.c_int64(), C.c_int64()
+        _check(self._lib.omk_forest_node_count(self._h, C.byref(n), C.byref(cap)))
+        self.n_nodes = int(n.value)
+        return int(n.value), int(cap.value)
+
+    def download_structure(self):
+        """Returns dict(child_begin, child_count, action) of the current nodes."""
+        n, _ = self.node_count()
+        out = dict(child_begin=np.empty(n, np.int32), child_count=np.empty(n, np.int32), action=np.empty(n, np.int32))
+        _check(self._lib.omk_forest_download_structure(self._h, C.c_int64(n), _ptr(out["child_begin"], i32p),
+                                                       _ptr(out["child_count"], i32p), _ptr(out["action"], i32p)))
+        return out
+
     def download(self):
         """Returns dict(N, W, P, VL[, rN, rW]) as numpy arrays."""
-        n = self.n_nodes
+        n, _ = self.node_count()
         out = dict(N=np.empty(n, np.int32), W=np.empty(n, np.float32), P=np.empty(n, np.float32),
                    VL=np.empty(n, np.int32))
         if self.has_rave:
@@ -255,6 +272,21 @@ class Batch:
         _check(self._lib.omk_batch_read(self._h, _ptr(paths, i32p), _ptr(plen, i32p), _ptr(leaf, i32p),
                                         _ptr(actions, i32p)))
         return paths, plen, leaf, actions
+
+    def expand(self, move_begin, moves, policy=None, action_space=0):
+        """Expands the leaves of the last select(): move_begin [n+1] / moves are the legal moves
+        every traversal offers for its leaf (empty = terminal), policy None or [n, action_space].
+        Returns first_child per traversal (-1 where nothing was added)."""
+        mb = np.ascontiguousarray(move_begin, dtype=np.int32)
+        mv = np.ascontiguousarray(moves, dtype=np.int32)
+        if len(mv) == 0:
+            mv = np.zeros(1, np.int32)
+        pol = None if policy is None else np.ascontiguousarray(policy, dtype=np.float32)
+        first = np.empty(len(mb) - 1, np.int32)
+        _check(self._lib.omk_expand_batch(self._h, _ptr(mb, i32p), _ptr(mv, i32p), _ptr(pol, f32p),
+                                          C.c_int32(int(action_space)), _ptr(first, i32p)))
+        self.forest.node_count()
+        return first
 
     def truncated(self):
         c = C.c_int32()

@@ -318,3 +318,62 @@ int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_
     }
     return hits;
 }
+
+/* ---- leaf expansion (mcts_node.cpp:238-436, :512-593; call site
+ * mcts_engine_batch_tree_simple.cpp:249-259) ---- */
+int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
+                         int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                         uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
+                         const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child) {
+    /* first pass: how many nodes would be added (a leaf counts once: child_count is set below,
+     * so a dry run has to remember the leaves it has seen) */
+    int64_t need = 0;
+    for (int32_t t = 0; t < B; t++) {
+        int32_t cnt = move_begin[t + 1] - move_begin[t];
+        if (cnt <= 0 || leaf[t] < 0 || child_count[leaf[t]] != 0) continue;
+        int seen = 0;
+        for (int32_t u = 0; u < t && !seen; u++)
+            seen = leaf[u] == leaf[t] && move_begin[u + 1] - move_begin[u] > 0;
+        if (seen) continue;
+        need += cnt > 1000 ? 1000 : cnt;
+    }
+    if (n_nodes + need > capacity) return -1;
+    for (int32_t t = 0; t < B; t++) {
+        if (first_child) first_child[t] = -1;
+        int32_t cnt = move_begin[t + 1] - move_begin[t];
+        if (cnt <= 0 || leaf[t] < 0) continue;         /* terminal: stays a leaf */
+        int32_t node = leaf[t];
+        if (child_count[node] != 0) continue;           /* already expanded: first caller won */
+        if (cnt > 1000) cnt = 1000;                     /* max_reasonable_moves */
+        const int32_t begin = (int32_t)n_nodes;
+        for (int32_t i = 0; i < cnt; i++) {
+            const int32_t id = begin + i;
+            const int32_t mv = moves[move_begin[t] + i];
+            float prior;
+            if (!policy) {
+                prior = 1.0f / (float)cnt;              /* expand(): uniform_prior */
+            } else if (mv >= 0 && mv < action_space) {
+                prior = policy[(int64_t)t * action_space + mv];
+                prior = prior > 0.0f ? prior : 0.0f;    /* std::min(1.0f, std::max(0.0f, prob)) */
+                prior = prior < 1.0f ? prior : 1.0f;
+            } else {
+                prior = 0.01f;                          /* action out of bounds */
+            }
+            N[id] = 0;
+            W[id] = 0.0f;
+            P[id] = prior;
+            VL[id] = 0;
+            if (rN) rN[id] = 0;
+            if (rW) rW[id] = 0.0f;
+            child_begin[id] = 0;
+            child_count[id] = 0;
+            if (action) action[id] = mv;
+            if (legal) legal[(uint32_t)id >> 5] |= 1u << ((uint32_t)id & 31u);
+        }
+        child_begin[node] = begin;
+        child_count[node] = cnt;
+        n_nodes += cnt;
+        if (first_child) first_child[t] = begin;
+    }
+    return n_nodes;
+}

@@ -103,6 +103,34 @@ void ref_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *path_len
 void ref_gather_actions(const ref_tree *t, const int32_t *paths, const int32_t *path_len,
                         int32_t B, int32_t stride, int32_t *actions);
 
+/* Leaf expansion as the backup phase of executeBatchedTreeSearch does it for the leaves of a
+ * batch (src/mcts/mcts_engine_batch_tree_simple.cpp:249-259): MCTSNode::expand
+ * (src/mcts/mcts_node.cpp:238-436) followed by setPriorProbabilities (:512-593).
+ *   - traversal t offers the legal moves moves[move_begin[t] .. move_begin[t+1]) of its leaf;
+ *     an empty list is a terminal state: the node stays a leaf (:257-259, :282-284);
+ *   - a leaf reached by several traversals is expanded once, by the first of them in index
+ *     order that offers moves (is_expanded_ compare-exchange, :263-265: the first caller
+ *     wins; one thread in index order is the deterministic schedule);
+ *   - a node that already has children is left alone (same compare-exchange);
+ *   - at most 1000 moves are used (max_reasonable_moves, :289-293);
+ *   - one child per move, in the order given (the reference shuffles the moves with a
+ *     random_device seed, :357-364, so every order is one of its outcomes), with zero
+ *     statistics, action = the move (:396-404);
+ *   - priors: without a policy the uniform 1/children of expand (:426-429); with a policy
+ *     row of action_space entries, clamp(policy[move], 0, 1), and 0.01 for a move outside
+ *     the action space (:537-558).
+ * The arrays hold room for `capacity` nodes; new ids are handed out in traversal order from
+ * n_nodes on.  first_child[t] (may be NULL) = first new id for the traversal whose list was
+ * used, else -1.  Returns the node count afterwards, or -1 when capacity would be exceeded
+ * (nothing is changed then).
+ * PARITY UNPINNED where the reference is random (child order) or silent (nothing in its tests
+ * fixes the priors); pinned: children = legal moves, terminal stays leaf, actions in range
+ * (tests/mcts/mcts_node_test.cpp:124-170), and the prior rules restated above. */
+int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
+                         int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                         uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
+                         const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child);
+
 /* Open-addressing table: 2^log2_slots slots of 16 bytes, linear probing,
  * home slot = (key * 0x9E3779B97F4A7C15) >> (64 - log2_slots), empty key = ~0. */
 typedef struct ref_tt_slot {

@@ -183,6 +183,52 @@ class RefTree:
         lib().ref_backup_batch(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), _ptr(values, f32p),
                                B, stride, int(amount))
 
+    def expand_batch(self, leaf, move_begin, moves, policy=None, action_space=0):
+        """MCTSNode::expand + setPriorProbabilities for the leaves of a batch (see ref_cpu.h).
+        Grows the arrays; returns first_child per traversal (-1 where nothing was added)."""
+        leaf = np.ascontiguousarray(leaf, dtype=np.int32)
+        move_begin = np.ascontiguousarray(move_begin, dtype=np.int32)
+        moves = np.ascontiguousarray(moves, dtype=np.int32)
+        B = len(leaf)
+        cap = self.n + int(np.minimum(np.diff(move_begin), 1000).clip(min=0).sum())
+
+        def grow(a, dtype, n=cap):
+            if a is None:
+                return None
+            out = np.zeros(n, dtype=dtype)
+            out[:len(a)] = a
+            return out
+
+        self.N, self.W, self.P, self.VL = (grow(self.N, np.int32), grow(self.W, np.float32),
+                                           grow(self.P, np.float32), grow(self.VL, np.int32))
+        self.rN, self.rW = grow(self.rN, np.int32), grow(self.rW, np.float32)
+        self.child_begin, self.child_count = grow(self.child_begin, np.int32), grow(self.child_count, np.int32)
+        self.action = grow(self.action, np.int32)
+        self.legal = grow(self.legal, np.uint32, (cap + 31) // 32)
+        if self.legal is not None and self.n & 31:
+            self.legal[self.n >> 5] &= np.uint32((1 << (self.n & 31)) - 1)  # bits of ids that do not exist yet
+        pol = None if policy is None else np.ascontiguousarray(policy, dtype=np.float32)
+        first = np.empty(B, dtype=np.int32)
+        fn = lib().ref_expand_batch
+        fn.restype = C.c_int64
+        n_after = fn(C.c_int64(self.n), C.c_int64(cap), _ptr(self.N, i32p), _ptr(self.W, f32p), _ptr(self.P, f32p),
+                     _ptr(self.VL, i32p), _ptr(self.rN, i32p), _ptr(self.rW, f32p), _ptr(self.child_begin, i32p),
+                     _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p), _ptr(leaf, i32p),
+                     B, _ptr(move_begin, i32p), _ptr(moves, i32p), _ptr(pol, f32p), int(action_space),
+                     _ptr(first, i32p))
+        assert n_after >= 0
+        self.n = int(n_after)
+        for name in ("N", "W", "P", "VL", "rN", "rW", "child_begin", "child_count", "action"):
+            a = getattr(self, name)
+            if a is not None:
+                setattr(self, name, a[:self.n].copy())
+        if self.legal is not None:
+            self.legal = self.legal[:(self.n + 31) // 32].copy()
+        self._c = _Tree(self.n, _ptr(self.N, i32p), _ptr(self.W, f32p), _ptr(self.P, f32p), _ptr(self.VL, i32p),
+                        _ptr(self.rN, i32p), _ptr(self.rW, f32p), _ptr(self.child_begin, i32p),
+                        _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p))
+        return first
+
     def gather_actions(self, paths, path_len):
         paths, path_len, B, stride = self._paths_args(paths, path_len)
         out = np.empty((B, stride - 1), dtype=np.int32)

@@ -1,0 +1,133 @@
+"""GPU parity of leaf expansion (omk_expand_batch) and of search steps on a tree that grows on
+the device: select -> leaf gather -> expand -> backup, every array against the CPU checker
+after every phase.  Structure, priors, actions, N and virtual loss bit-exact; W within 1e-5."""
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+from tests.helpers import random_tree
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_same_forest(f, ref, what):
+    st = f.download()
+    sx = f.download_structure()
+    assert len(st["N"]) == ref.n, what
+    assert (sx["child_begin"] == ref.child_begin).all() and (sx["child_count"] == ref.child_count).all(), what
+    assert (sx["action"] == ref.action).all(), what
+    assert st["P"].tobytes() == ref.P.tobytes(), what
+    assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all(), what
+    err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
+    assert err.max() <= 1e-5, what
+    return st
+
+
+def offers(rng, leaves, action_space, terminal_frac=0.1, max_moves=40):
+    """Legal moves per traversal, a function of the leaf so that two traversals at one leaf
+    offer the same state's moves, plus a policy row per traversal."""
+    begin, moves = [0], []
+    for lf in leaves:
+        r = np.random.default_rng(int(lf) * 7919 + 13)
+        if r.random() < terminal_frac:
+            k = 0
+        else:
+            k = int(r.integers(1, max_moves + 1))
+        moves.extend(r.choice(action_space, size=k, replace=False).tolist())
+        begin.append(len(moves))
+    policy = rng.random((len(leaves), action_space)).astype(np.float32)
+    policy /= policy.sum(axis=1, keepdims=True)
+    return np.array(begin, np.int32), np.array(moves, np.int32), policy
+
+
+@pytest.mark.parametrize("rave,B", [(False, 96), (True, 700)])
+def test_tree_grows_on_the_device(rave, B):
+    import omoknuni_small_amd as omk
+    A = 81
+    soa = dict(N=np.zeros(1, np.int32), W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=np.zeros(1, np.int32),
+               child_begin=np.zeros(1, np.int32), child_count=np.zeros(1, np.int32), action=np.full(1, -1, np.int32))
+    if rave:
+        soa["rN"] = np.zeros(1, np.int32)
+        soa["rW"] = np.zeros(1, np.float32)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa, capacity=400_000)
+    D, vl = 12, 3
+    b = omk.Batch(f, B, D)
+    roots = np.zeros(B, np.int32)
+    b.set_roots(roots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0, max_depth=D)
+    rng = np.random.default_rng(4)
+    for step in range(14):
+        rpaths, rlen, rleaf, near = ref.select_batch(roots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, gact = b.read()
+        bad = np.nonzero((gpaths != rpaths).any(axis=1) | (glen != rlen) | (gleaf != rleaf))[0]
+        assert len(bad) == 0, "step %d: %d paths differ (near ties flagged %d)" % (step, len(bad), int((near >= 0).sum()))
+        begin, moves, policy = offers(rng, rleaf, A)
+        pol = policy if step % 3 else None          # every third step: no policy, uniform priors
+        rfirst = ref.expand_batch(rleaf, begin, moves, policy=pol, action_space=A)
+        gfirst = b.expand(begin, moves, policy=pol, action_space=A)
+        assert (gfirst == rfirst).all(), "step %d: new ids differ" % step
+        assert_same_forest(f, ref, "after expansion, step %d" % step)
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, values, vl)
+        b.set_values(values)
+        b.backup(vl)
+        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        ref.W[:] = st["W"]
+    assert ref.n > 1000
+
+
+def test_expand_on_an_uploaded_tree_with_mask_and_shared_leaves():
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(77, n_expand=60, fanout=(2, 9), max_depth=5, mask_frac=0.2)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa, capacity=len(soa["N"]) + 5000)
+    B, D = 300, 8
+    b = omk.Batch(f, B, D)
+    troots = np.full(B, roots[0], np.int32)
+    b.set_roots(troots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=D)
+    rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp)
+    b.select(sp)
+    _, _, gleaf, _ = b.read()
+    assert (gleaf == rleaf).all()
+    assert len(np.unique(rleaf)) < B            # several traversals share a leaf
+    begin, moves, policy = offers(np.random.default_rng(1), rleaf, 50)
+    policy[:, 7] = 1.5                          # clamped to 1
+    policy[:, 8] = -0.5                         # clamped to 0
+    moves[::11] = 60                            # outside the action space: default prior
+    rfirst = ref.expand_batch(rleaf, begin, moves, policy=policy, action_space=50)
+    gfirst = b.expand(begin, moves, policy=policy, action_space=50)
+    assert (gfirst == rfirst).all()
+    assert_same_forest(f, ref, "after expansion")
+    assert (f.download_structure()["child_count"] == ref.child_count).all()
+    # the mask now covers the new nodes: select again and compare
+    values = np.zeros(B, np.float32)
+    ref.backup_batch(rpaths, rlen, values, 3)
+    b.set_values(values)
+    b.backup(3)
+    rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp)
+    b.select(sp)
+    gpaths, glen, gleaf, _ = b.read()
+    assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
+
+
+def test_expand_beyond_capacity_changes_nothing():
+    import omoknuni_small_amd as omk
+    soa = dict(N=np.zeros(1, np.int32), W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=np.zeros(1, np.int32),
+               child_begin=np.zeros(1, np.int32), child_count=np.zeros(1, np.int32), action=np.full(1, -1, np.int32))
+    f = omk.Forest.from_soa(soa, capacity=4)
+    b = omk.Batch(f, 2, 4)
+    b.set_roots(np.zeros(2, np.int32))
+    b.select(omk.SelectParams())
+    b.read()
+    with pytest.raises(omk.OmkError) as e:
+        b.expand([0, 5, 5], [0, 1, 2, 3, 4])
+    assert e.value.code == -3                    # OMK_ERR_CAPACITY
+    assert f.node_count() == (1, 4)
+    assert f.download_structure()["child_count"].tolist() == [0]
+    first = b.expand([0, 3, 3], [0, 1, 2])
+    assert first.tolist() == [1, -1] and f.node_count()[0] == 4

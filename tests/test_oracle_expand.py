@@ -1,0 +1,76 @@
+"""The checker's leaf expansion against what the reference fixes about MCTSNode::expand and
+setPriorProbabilities: its own unit tests (tests/mcts/mcts_node_test.cpp:124-170: children =
+legal moves, the node stops being a leaf, actions in range; :175-200: a terminal state is not
+expanded) and the rules read off src/mcts/mcts_node.cpp:238-436, :512-593 (uniform prior of
+expand, clamp to [0,1], 0.01 for a move outside the action space, first caller wins, 1000-move
+limit).  The order of the children is random in the reference; the checker keeps the order
+given, which is one of its outcomes."""
+import numpy as np
+
+from oracle import ref_cpu as R
+
+
+def leaf_tree(n=1):
+    z = np.zeros(n, np.int32)
+    return R.RefTree(N=z + 5, W=np.zeros(n, np.float32), P=np.ones(n, np.float32), VL=z, child_begin=z, child_count=z,
+                     action=z - 1)
+
+
+def test_three_legal_moves_give_three_children():
+    t = leaf_tree()
+    first = t.expand_batch([0], [0, 3], [2, 0, 1])
+    assert first.tolist() == [1] and t.n == 4
+    assert t.child_begin[0] == 1 and t.child_count[0] == 3          # not a leaf any more
+    assert t.action[1:4].tolist() == [2, 0, 1]                      # one child per move, each in range
+    assert (t.N[1:4] == 0).all() and (t.W[1:4] == 0).all() and (t.VL[1:4] == 0).all()
+    assert (t.child_count[1:4] == 0).all()                          # children are leaves
+    assert np.allclose(t.P[1:4], np.float32(1.0) / np.float32(3.0), rtol=0, atol=0)
+    assert t.N[0] == 5                                              # the node's own statistics are untouched
+
+
+def test_terminal_state_is_not_expanded():
+    t = leaf_tree()
+    first = t.expand_batch([0], [0, 0], [])
+    assert first.tolist() == [-1] and t.n == 1 and t.child_count[0] == 0
+
+
+def test_priors_follow_the_policy_with_clamp_and_default():
+    t = leaf_tree()
+    policy = np.array([[-0.2, 0.25, 1.7, 0.5]], np.float32)
+    t.expand_batch([0], [0, 5], [0, 1, 2, 3, 9], policy=policy, action_space=4)
+    assert t.P[1:6].tolist() == [0.0, 0.25, 1.0, 0.5, np.float32(0.01)]
+
+
+def test_first_traversal_wins_a_shared_leaf_and_ids_follow_traversal_order():
+    t = leaf_tree(3)
+    # traversals: 0 -> leaf 2, 1 -> leaf 1 (terminal), 2 -> leaf 2 again, 3 -> leaf 0
+    first = t.expand_batch([2, 1, 2, 0], [0, 2, 2, 5, 6], [7, 8, 1, 2, 3, 4])
+    assert first.tolist() == [3, -1, -1, 5]
+    assert (t.child_begin[2], t.child_count[2]) == (3, 2) and t.action[3:5].tolist() == [7, 8]
+    assert t.child_count[1] == 0
+    assert (t.child_begin[0], t.child_count[0]) == (5, 1) and t.action[5] == 4
+    assert t.n == 6
+
+
+def test_expanded_node_is_left_alone():
+    t = leaf_tree()
+    t.expand_batch([0], [0, 2], [0, 1])
+    before = (t.child_begin.copy(), t.child_count.copy(), t.P.copy())
+    first = t.expand_batch([0], [0, 3], [5, 6, 7])
+    assert first.tolist() == [-1] and t.n == 3
+    assert (t.child_begin == before[0]).all() and (t.child_count == before[1]).all() and (t.P == before[2]).all()
+
+
+def test_move_list_is_cut_at_the_reference_limit():
+    t = leaf_tree()
+    t.expand_batch([0], [0, 1500], np.arange(1500))
+    assert t.child_count[0] == 1000 and t.n == 1001 and t.action[1000] == 999
+
+
+def test_selection_descends_into_new_children():
+    t = leaf_tree()
+    t.expand_batch([0], [0, 3], [0, 1, 2], policy=np.array([[0.1, 0.7, 0.2]], np.float32), action_space=3)
+    p = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=4)
+    paths, plen, leaf, _ = t.select_batch(np.zeros(2, np.int32), p)
+    assert plen.tolist() == [2, 2]
+    assert leaf[0] == 2           # all children unvisited: the largest prior wins (sqrt(N_parent) > 0)
