@@ -16,6 +16,8 @@
  *   ref_update            src/mcts/mcts_node_virtual_loss.cpp:54-71
  *   ref_select_batch      src/mcts/mcts_engine_batch_tree_simple.cpp:73-185 (one thread, i ascending)
  *   ref_backup_batch      src/mcts/mcts_engine_batch_tree_simple.cpp:242-282 (i ascending)
+ *   ref_expand_batch      src/mcts/mcts_node.cpp:238-436, :512-593 (MCTSNode::expand, setPriorProbabilities),
+ *                         call site src/mcts/mcts_engine_batch_tree_simple.cpp:249-259
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
  *
@@ -32,7 +34,10 @@
  *   - the progressive-widening eligibility filter (pw != 0): top ceil(sqrt(N_parent))
  *     children by prior, ties to the lower child index;
  *   - the open-addressing transposition table (the reference delegates to the
- *     absent third-party parallel-hashmap v1.3.8); checked against a brute-force map.
+ *     absent third-party parallel-hashmap v1.3.8); checked against a brute-force map;
+ *   - the ORDER of the children that leaf expansion creates (the reference shuffles the
+ *     legal moves with a random seed; the order offered is kept here).  The rest of
+ *     expansion is pinned by tests/test_oracle_expand.py.
  *
  * Must be compiled with -ffp-contract=off and without -ffast-math: the reference
  * translation unit is built for baseline x86-64 (no FMA), IEEE binary32, round to nearest.
