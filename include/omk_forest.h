@@ -151,6 +151,17 @@ int omk_revert_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_
 int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len,
                      const float *d_values, int32_t n, int32_t stride, int32_t max_len, int32_t virtual_loss);
 
+/* The search result's move probabilities (MCTSEngine::getActionProbabilities,
+ * src/mcts/mcts_engine_tree.cpp:388-465) from the visit counts of `root`'s children, laid
+ * out over the action space: temperature < 0.01 puts 1 on the first child with the largest
+ * count; otherwise (count / max_count) ^ (1 / temperature) normalised, uniform when every
+ * count is 0.  Waits for the stream, reads the children's counts and actions back and does
+ * the arithmetic on the host, in the reference's order (it is a few hundred numbers per
+ * search).  h_children (may be NULL) receives the number of children; with none the output
+ * is all zero. */
+int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperature, int32_t action_space,
+                                    float *h_probabilities, int32_t *h_children);
+
 /* Leaf expansion for the leaves of the last selection: MCTSNode::expand
  * (src/mcts/mcts_node.cpp:238-436) followed by setPriorProbabilities (:512-593), as the backup
  * phase does before it backs the values up (src/mcts/mcts_engine_batch_tree_simple.cpp:249-259).

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -349,6 +350,81 @@ int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_chi
             if (h_child_begin) h_child_begin[i] = sp[(size_t)i].x;
             if (h_child_count) h_child_count[i] = sp[(size_t)i].y;
         }
+    }
+    return OMK_OK;
+}
+
+int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperature, int32_t action_space,
+                                    float *h_probabilities, int32_t *h_children) {
+    if (!f || !h_probabilities) return fail(OMK_ERR_INVALID, "omk_forest_action_probabilities: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_action_probabilities: nothing uploaded");
+    if (root < 0 || root >= f->n_nodes || action_space <= 0)
+        return fail(OMK_ERR_INVALID, "omk_forest_action_probabilities: root %d, action space %d", root, action_space);
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    int2 sp;
+    HIP_TRY(hipMemcpy(&sp, f->span + root, sizeof(sp), hipMemcpyDeviceToHost));
+    for (int32_t a = 0; a < action_space; a++) h_probabilities[a] = 0.0f;
+    if (h_children) *h_children = 0;
+    const int32_t cb = sp.x, cc = sp.y;
+    if (cc <= 0) return OMK_OK;
+    std::vector<int32_t> n((size_t)cc), act((size_t)cc);
+    HIP_TRY(hipMemcpy(n.data(), f->N + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
+    if (f->has_action) {
+        HIP_TRY(hipMemcpy(act.data(), f->action + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
+    } else {
+        for (int32_t i = 0; i < cc; i++) act[(size_t)i] = cb + i;
+    }
+    std::vector<uint32_t> legal;
+    const int64_t w0 = (int64_t)cb >> 5, w1 = ((int64_t)cb + cc + 31) >> 5;
+    if (f->has_legal) {
+        legal.resize((size_t)(w1 - w0));
+        HIP_TRY(hipMemcpy(legal.data(), f->legal + w0, legal.size() * 4, hipMemcpyDeviceToHost));
+    }
+    auto is_child = [&](int32_t i) {
+        if (!f->has_legal) return true;
+        const int64_t id = (int64_t)cb + i;
+        return ((legal[(size_t)((id >> 5) - w0)] >> (id & 31)) & 1u) != 0u;
+    };
+    // MCTSEngine::getActionProbabilities, statement by statement
+    int32_t children = 0, max_idx = -1;
+    float max_count = 0.0f;
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_child(i)) continue;
+        children++;
+        const float c = (float)n[(size_t)i];
+        if (max_idx < 0 || c > max_count) {  // std::max_element: the first of the largest
+            max_count = c;
+            max_idx = i;
+        }
+    }
+    if (h_children) *h_children = children;
+    if (children == 0) return OMK_OK;
+    const bool near_zero = temperature < 0.01f;
+    float sum = 0.0f;
+    if (!near_zero && max_count > 0.0f)
+        for (int32_t i = 0; i < cc; i++) {
+            if (!is_child(i)) continue;
+            const float c = (float)n[(size_t)i];
+            float scaled = 0.0f;
+            if (c > 0.0f) scaled = powf(c / max_count, 1.0f / temperature);
+            sum += scaled;
+        }
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_child(i)) continue;
+        float prob;
+        if (near_zero) {
+            prob = i == max_idx ? 1.0f : 0.0f;
+        } else if (max_count <= 0.0f || !(sum > 0.0f)) {
+            prob = 1.0f / (float)children;
+        } else {
+            const float c = (float)n[(size_t)i];
+            float scaled = 0.0f;
+            if (c > 0.0f) scaled = powf(c / max_count, 1.0f / temperature);
+            prob = scaled / sum;
+        }
+        const int32_t a = act[(size_t)i];
+        if (a >= 0 && a < action_space) h_probabilities[a] = prob;
     }
     return OMK_OK;
 }

@@ -81,6 +81,15 @@ void ForestEngine::backPropagateBatch(const std::vector<float> &leaf_values) {
     check(omk_backup_batch(batch_, settings_.virtual_loss), "omk_backup_batch");
 }
 
+std::vector<float> ForestEngine::getActionProbabilities(int32_t root, float temperature, int action_space) {
+    std::vector<float> probs((size_t)action_space, 0.0f);
+    int32_t children = 0;
+    check(omk_forest_action_probabilities(forest_, root, temperature, action_space, probs.data(), &children),
+          "omk_forest_action_probabilities");
+    if (children == 0) probs.clear();  // the reference returns an empty vector for a root without children
+    return probs;
+}
+
 int64_t ForestEngine::nodeCount() const {
     int64_t n = 0;
     check(omk_forest_node_count(forest_, &n, nullptr), "omk_forest_node_count");

@@ -77,6 +77,9 @@ class ForestEngine {
     // policies of a batch must have the same size).  Returns the nodes added.
     int64_t expandLeafBatch(const std::vector<std::vector<int>> &legal_moves, const std::vector<NetworkOutput> &outputs);
     void setLegalMovesFunction(LegalMovesFunction fn) { legal_moves_fn_ = std::move(fn); }
+    // SearchResult.probabilities (reference MCTSEngine::getActionProbabilities,
+    // src/mcts/mcts_engine_tree.cpp:388-465): visit counts of root's children, temperature.
+    std::vector<float> getActionProbabilities(int32_t root, float temperature, int action_space);
     int64_t nodeCount() const;
     void downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action);
 

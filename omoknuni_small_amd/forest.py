@@ -23,7 +23,7 @@ u64p = C.POINTER(C.c_uint64)
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
-    "omk_expand_batch", "omk_sync", "omk_batch_create", "omk_batch_destroy",
+    "omk_expand_batch", "omk_forest_action_probabilities", "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
@@ -165,6 +165,14 @@ class Forest:
         _check(self._lib.omk_forest_node_count(self._h, C.byref(n), C.byref(cap)))
         self.n_nodes = int(n.value)
         return int(n.value), int(cap.value)
+
+    def action_probabilities(self, root, temperature, action_space):
+        """MCTSEngine::getActionProbabilities from the root's children; (probabilities, children)."""
+        out = np.empty(int(action_space), np.float32)
+        n = C.c_int32()
+        _check(self._lib.omk_forest_action_probabilities(self._h, C.c_int32(int(root)), C.c_float(temperature),
+                                                         C.c_int32(int(action_space)), _ptr(out, f32p), C.byref(n)))
+        return out, int(n.value)
 
     def download_structure(self):
         """Returns dict(child_begin, child_count, action) of the current nodes."""

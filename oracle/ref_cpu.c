@@ -377,3 +377,59 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
     }
     return n_nodes;
 }
+
+/* ---- MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465) ---- */
+int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperature, int32_t action_space,
+                                 float *out) {
+    for (int32_t a = 0; a < action_space; a++) out[a] = 0.0f;
+    const int32_t cb = t->child_begin[root], cc = t->child_count[root];
+    /* the children: slots of the range whose legal bit is set */
+    int32_t n = 0;
+    for (int32_t i = 0; i < cc; i++) {
+        const int32_t id = cb + i;
+        if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+        n++;
+    }
+    if (n == 0) return 0;
+    float max_count = 0.0f;
+    int32_t max_idx = -1;
+    for (int32_t i = 0; i < cc; i++) {
+        const int32_t id = cb + i;
+        if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+        const float c = (float)t->N[id];
+        if (max_idx < 0 || c > max_count) { /* std::max_element: first of the largest */
+            max_count = c;
+            max_idx = id;
+        }
+    }
+    float sum = 0.0f;
+    const int near_zero = temperature < 0.01f;
+    if (!near_zero && max_count > 0.0f) {
+        for (int32_t i = 0; i < cc; i++) {
+            const int32_t id = cb + i;
+            if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+            const float c = (float)t->N[id];
+            float scaled = 0.0f;
+            if (c > 0.0f) scaled = powf(c / max_count, 1.0f / temperature);
+            sum += scaled;
+        }
+    }
+    for (int32_t i = 0; i < cc; i++) {
+        const int32_t id = cb + i;
+        if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+        float prob;
+        if (near_zero) {
+            prob = id == max_idx ? 1.0f : 0.0f;
+        } else if (max_count <= 0.0f || !(sum > 0.0f)) {
+            prob = 1.0f / (float)n; /* 1.0f / counts.size() */
+        } else {
+            const float c = (float)t->N[id];
+            float scaled = 0.0f;
+            if (c > 0.0f) scaled = powf(c / max_count, 1.0f / temperature);
+            prob = scaled / sum;
+        }
+        const int32_t a = t->action ? t->action[id] : id;
+        if (a >= 0 && a < action_space) out[a] = prob;
+    }
+    return n;
+}

@@ -18,6 +18,7 @@
  *   ref_backup_batch      src/mcts/mcts_engine_batch_tree_simple.cpp:242-282 (i ascending)
  *   ref_expand_batch      src/mcts/mcts_node.cpp:238-436, :512-593 (MCTSNode::expand, setPriorProbabilities),
  *                         call site src/mcts/mcts_engine_batch_tree_simple.cpp:249-259
+ *   ref_action_probabilities  src/mcts/mcts_engine_tree.cpp:388-465 (MCTSEngine::getActionProbabilities)
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
  *
@@ -135,6 +136,18 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
                          int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
                          uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
                          const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child);
+
+/* MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465): the search
+ * result's move probabilities from the root's children.  counts = float(N_child);
+ * temperature < 0.01: 1 for the FIRST child with the largest count, 0 elsewhere; else
+ * (count / max_count) ^ (1 / temperature) for count > 0, normalised by their sum in child
+ * order; uniform 1 / children when every count is 0 (or the sum is 0).  The result is laid
+ * out over the action space: out[action_i] = probability_i for 0 <= action_i < action_space
+ * (a later child with the same action overwrites an earlier one), 0 elsewhere.  Returns the
+ * number of children, 0 when the root has none (the reference returns an empty vector; out
+ * is left all zero).  Slots whose legal bit is clear are not children. */
+int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperature, int32_t action_space,
+                                 float *out);
 
 /* Open-addressing table: 2^log2_slots slots of 16 bytes, linear probing,
  * home slot = (key * 0x9E3779B97F4A7C15) >> (64 - log2_slots), empty key = ~0. */

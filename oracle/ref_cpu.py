@@ -229,6 +229,13 @@ class RefTree:
                         _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p))
         return first
 
+    def action_probabilities(self, root, temperature, action_space):
+        """MCTSEngine::getActionProbabilities over the root's children; (probabilities, children)."""
+        out = np.empty(int(action_space), dtype=np.float32)
+        n = lib().ref_action_probabilities(C.byref(self._c), int(root), C.c_float(temperature), int(action_space),
+                                           _ptr(out, f32p))
+        return out, int(n)
+
     def gather_actions(self, paths, path_len):
         paths, path_len, B, stride = self._paths_args(paths, path_len)
         out = np.empty((B, stride - 1), dtype=np.int32)

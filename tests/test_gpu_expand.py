@@ -131,3 +131,21 @@ def test_expand_beyond_capacity_changes_nothing():
     assert f.download_structure()["child_count"].tolist() == [0]
     first = b.expand([0, 3, 3], [0, 1, 2])
     assert first.tolist() == [1, -1] and f.node_count()[0] == 4
+
+
+@pytest.mark.parametrize("mask_frac", [0.0, 0.3])
+def test_action_probabilities_match_the_checker(mask_frac):
+    """MCTSEngine::getActionProbabilities through the C ABI: bit-exact (the arithmetic runs on
+    the host in the reference's order; the counts come from the device)."""
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(31, n_expand=50, fanout=(3, 30), max_depth=4, mask_frac=mask_frac, n_max=500)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    A = 40
+    nodes = [int(roots[0])] + [int(i) for i in np.nonzero(soa["child_count"] > 0)[0][:10]] + \
+            [int(np.nonzero(soa["child_count"] == 0)[0][0])]
+    for node in nodes:
+        for temp in (0.001, 0.5, 1.0, 2.0):
+            rp, rn = ref.action_probabilities(node, temp, A)
+            gp, gn = f.action_probabilities(node, temp, A)
+            assert gn == rn and gp.tobytes() == rp.tobytes(), (node, temp)

@@ -74,3 +74,49 @@ def test_selection_descends_into_new_children():
     paths, plen, leaf, _ = t.select_batch(np.zeros(2, np.int32), p)
     assert plen.tolist() == [2, 2]
     assert leaf[0] == 2           # all children unvisited: the largest prior wins (sqrt(N_parent) > 0)
+
+
+# ---- MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465) ----
+
+def counts_tree(counts, actions=None):
+    k = len(counts)
+    z = np.zeros(k + 1, np.int32)
+    cb, cc = z.copy(), z.copy()
+    cb[0], cc[0] = 1, k
+    act = np.concatenate([[-1], np.arange(k) if actions is None else actions]).astype(np.int32)
+    return R.RefTree(N=np.concatenate([[sum(counts)], counts]).astype(np.int32), W=np.zeros(k + 1, np.float32),
+                     P=np.ones(k + 1, np.float32), VL=z, child_begin=cb, child_count=cc, action=act)
+
+
+def test_probabilities_near_zero_temperature_pick_the_first_maximum():
+    p, n = counts_tree([3, 9, 9, 1]).action_probabilities(0, 0.001, 6)
+    assert n == 4 and p.tolist() == [0, 1, 0, 0, 0, 0]
+
+
+def test_probabilities_at_temperature_one_are_proportional_to_visits():
+    p, _ = counts_tree([1, 2, 5, 0]).action_probabilities(0, 1.0, 4)
+    # (count/max)^(1/1) normalised in binary32, in child order
+    s = np.float32(0)
+    scaled = [np.float32(np.float32(c) / np.float32(5)) for c in (1, 2, 5)]
+    for x in scaled:
+        s = np.float32(s + x)
+    assert p.tolist() == [np.float32(x / s) for x in scaled] + [0.0]
+    assert abs(float(p.sum()) - 1.0) < 1e-6
+
+
+def test_probabilities_sharpen_with_low_temperature():
+    p, _ = counts_tree([2, 4]).action_probabilities(0, 0.5, 2)
+    assert np.allclose(p, [0.2, 0.8], rtol=1e-6)      # (1/2)^2 : 1
+
+
+def test_probabilities_uniform_when_nothing_was_visited_and_empty_without_children():
+    p, n = counts_tree([0, 0, 0, 0]).action_probabilities(0, 1.0, 5)
+    assert n == 4 and p.tolist() == [0.25, 0.25, 0.25, 0.25, 0.0]
+    t = counts_tree([1, 2])
+    p, n = t.action_probabilities(1, 1.0, 3)          # a leaf
+    assert n == 0 and p.tolist() == [0.0, 0.0, 0.0]
+
+
+def test_probabilities_are_laid_out_by_action_and_skip_actions_outside_the_space():
+    p, _ = counts_tree([1, 1, 2], actions=[4, 9, 0]).action_probabilities(0, 1.0, 6)
+    assert p[4] == 0.25 and p[0] == 0.5 and p.sum() == 0.75   # action 9 is outside: dropped
