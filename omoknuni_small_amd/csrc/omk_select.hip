@@ -119,7 +119,7 @@ struct Kids {
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
 // so that it sits at the same place for every fan-out class.
-enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2 };
+enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3 };
 struct TeamCmd {
     int op;
     int rounds;  // R of the node's fan-out class: 1, or the kernel's RMAX
@@ -129,6 +129,10 @@ struct TeamCmd {
     int cur;     // which of the two buffers holds the ordered batch
     float ep;
     uint32_t uvl;
+    // kOpRun: a run of `total` entries of child `best` from its visit btk on
+    int best, btk, bn, bvl;
+    float bw, bp, bq2;
+    uint32_t hk, hp, sk, spos;
 };
 
 // Scratch in LDS of one block of the multi-visitor kernel (one node at a time).
@@ -633,6 +637,39 @@ __device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds,
     team_sync<NT>();
 }
 
+// A run of L entries of one child (visits btk .. btk + L - 1), about to be emitted as the
+// next L winners at ranks goff ..: every entry must have a real key and must not come before
+// its predecessor (the first one's predecessor is the child's current head (hk, hp), i.e.
+// itself), and the last one must still come before the others' best (sk, spos).  The
+// entries are written whether or not the checks hold; red[2] bit 2 reports a failure.
+template <int R, bool RAVE, int NT>
+__device__ __forceinline__ void batch_run(const SelectArgs &a, WaveLds<R> &lds, int tid, int L, int goff, int best,
+                                          int btk, int bn, float bw, float bp, int bvl, float bq2, float ep,
+                                          uint32_t uvl, uint32_t hk, uint32_t hp, uint32_t sk, uint32_t spos) {
+    const int per = (L + NT - 1) / NT;
+    const int j0 = tid * per < L ? tid * per : L;
+    const int j1 = j0 + per < L ? j0 + per : L;
+    bool bad_run = false;
+    if (j0 < j1) {
+        uint32_t pk = hk, pp = hp;
+        if (j0 > 0) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, btk + j0 - 1, best, pk, pp);
+        for (int j = j0; j < j1; j++) {
+            uint32_t kk, p2;
+            entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, btk + j, best, kk, p2);
+            if (kk == 0u || comes_before(kk, p2, pk, pp)) bad_run = true;
+            if (j == L - 1 && sk != 0u && !comes_before(kk, p2, sk, spos)) bad_run = true;
+            pk = kk;
+            pp = p2;
+        }
+    }
+    for (int j = tid; j < L; j += NT) {
+        a.sc_child[goff + j] = best;
+        a.sc_occ[goff + j] = btk + j;
+    }
+    if (__ballot(bad_run) != 0ull && (tid & 63) == 0) atomicOr(&lds.red[2], 4u);
+    team_sync<NT>();
+}
+
 // The visitors of a crowded node in batches (see the file header).  On success cnt[r]
 // holds the visitors of every child and sc_child / sc_occ hold (child, visit number) of
 // every visitor; returns false when the node has to be replayed one visitor at a time
@@ -778,34 +815,47 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     hi_l = new_hi < hi_l ? new_hi : hi_l;
                 }
                 const int L = lo_l;
-                // every entry of the run: a real key, never before its predecessor
-                bool bad_run = false;
-                uint32_t carry_k = hi_key, carry_p = hi_pos;
-                for (int base = 0; base < L; base += kWave) {
-                    const int j = base + lane;
-                    uint32_t kk = 0u, pp = 0xFFFFFFFFu;
-                    if (j < L) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + j, best, kk, pp);
-                    uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-                    uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
-                    if (lane == 0) {
-                        pk = carry_k;
-                        ppos = carry_p;
-                    }
-                    if (j < L && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad_run = true;
-                    if (j < L && j == L - 1 && sk != 0u && !comes_before(kk, pp, sk, spos)) bad_run = true;
-                    carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-                    carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
-                }
-                // the entry after the run must not come before the run's last one either
+                // the entry after the run must not come before the run's last one
                 uint32_t nk, np2, lk_, lp_;
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L, best, nk, np2);
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L - 1, best, lk_, lp_);
-                if (nk != 0u && comes_before(nk, np2, lk_, lp_)) bad_run = true;
-                if (__ballot(bad_run) == 0ull) {
-                    for (int j = lane; j < L; j += kWave) {
-                        a.sc_child[off + done + j] = best;
-                        a.sc_occ[off + done + j] = btk + j;
+                bool bad_run = nk != 0u && comes_before(nk, np2, lk_, lp_);
+                // every entry of the run is checked and written; a long run with the helpers
+                if (!bad_run) {
+                    if (lane == 0) lds.red[2] = 0u;
+                    if (L >= 2 * kTeamMin) {
+                        if (lane == 0) {
+                            TeamCmd &cm = lds.cmd;
+                            cm.op = kOpRun;
+                            cm.rounds = R;
+                            cm.total = L;
+                            cm.goff = off + done;
+                            cm.ep = c.ep;
+                            cm.uvl = uvl;
+                            cm.best = best;
+                            cm.btk = btk;
+                            cm.bn = bn;
+                            cm.bvl = bvl;
+                            cm.bw = bw;
+                            cm.bp = bp;
+                            cm.bq2 = bq2;
+                            cm.hk = hi_key;
+                            cm.hp = hi_pos;
+                            cm.sk = sk;
+                            cm.spos = spos;
+                        }
+                        __syncthreads();
+                        batch_run<R, RAVE, kTeam>(a, lds, lane, L, off + done, best, btk, bn, bw, bp, bvl, bq2, c.ep, uvl,
+                                                  hi_key, hi_pos, sk, spos);
+                        __syncthreads();
+                    } else {
+                        wave_sync_memory();
+                        batch_run<R, RAVE, kWave>(a, lds, lane, L, off + done, best, btk, bn, bw, bp, bvl, bq2, c.ep, uvl,
+                                                  hi_key, hi_pos, sk, spos);
                     }
+                    bad_run = (lds.red[2] & 4u) != 0u;
+                }
+                if (!bad_run) {
                     if (lane == bl) {
 #pragma unroll
                         for (int r = 0; r < R; r++)
@@ -889,11 +939,15 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         int ct[R];
         total = 0;
         int tries = 0;
+        uint32_t T_forced = 0u;  // threshold imposed for the next round instead of searching one
+        bool allow_above = true;
         for (;;) {
-            if (++tries > 6) OMK_FAIL(5);
+            if (++tries > 8) OMK_FAIL(5);
+            const uint32_t T_now = T_forced;  // imposed for this round only
+            T_forced = 0u;
             // bisection on the score with the estimated counts only (no exact evaluation)
             float flo = key_score(lo_key), fhi = key_score(hi_key);
-            for (int it = 0; it < 22; it++) {
+            for (int it = 0; it < 22 && T_now == 0u; it++) {
                 const float mid = 0.5f * (flo + fhi);
                 int est = 0;
 #pragma unroll
@@ -913,7 +967,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     }
                 }
             }
-            uint32_t T = score_key(flo);
+            uint32_t T = T_now != 0u ? T_now : score_key(flo);
             if (T < lo_key) T = lo_key;
             if (T > hi_key) T = hi_key;
             const float tau = key_score(T);
@@ -978,6 +1032,14 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 const uint32_t gmx = wave_max_u32((uint32_t)mx);
                 const int who = (int)wave_min_u32((uint32_t)mx == gmx ? (uint32_t)mi : 0xFFFFFFFFu);
                 const int excess = total - kBatchCap;
+                // One child floods the batch with entries AT the threshold (a score that hardly
+                // moves with virtual loss).  Take the entries strictly above it first, a small
+                // batch; the run of that child is then emitted without sorting.
+                if ((int)gmx > excess && allow_above && T < hi_key) {
+                    allow_above = false;
+                    T_forced = T + 1u;
+                    continue;
+                }
                 if ((int)gmx <= excess) {
                     target -= excess + margin;  // no single child absorbs it: aim higher instead
                     if (target < 1) target = 1;
@@ -988,6 +1050,10 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     if (ac[r] == who) ct[r] -= excess;
                 capped_child = who;
                 total = kBatchCap;
+            }
+            if (T_now != 0u) {
+                if (total < 1) continue;  // nothing above: back to the flooded threshold, capped
+                break;                    // may not finish the node: the run comes next
             }
             if (can_finish && total < remaining) {
                 target += (remaining - total) + margin;  // not enough to finish: aim lower
@@ -1118,14 +1184,107 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
     return true;
 }
 
-// For a heavy node: a score threshold at or above which about `target` of the node's
-// entries lie (estimated), and EXACTLY how many entries of every own child lie at or above
-// it (ct, at most m each).  Every wavefront that asks for the same target gets the same
-// threshold: the computation is deterministic and depends on the node's state only.
+// The children of a node that can contribute entries at or above a lower bound, listed
+// densely (one per lane and round) so that work on them costs one round per 64 ACTIVE
+// children instead of one per 64 children.
+template <int R>
+struct ActiveSet {
+    int rounds;
+    int c[R];  // child index, -1 = none
+    int n[R];
+    int vl[R];
+    float w[R], p[R], q2[R];
+    uint32_t head[R];
+};
+
+// Exact number of entries of every active child at or above threshold T (at most m each):
+// the closed-form estimate, then the two entries around it are tested with the exact
+// arithmetic; if the estimate is further off, gallop away from it and bisect the rest.
+template <int R, bool RAVE>
+__device__ __forceinline__ void active_counts(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t T, int m,
+                                              int (&out)[R]) {
+    const float tau = key_score(T);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        out[r] = 0;
+        if (r < s.rounds && s.c[r] >= 0 && s.head[r] >= T) {
+            int lo_c = 1, hi_c = m;  // the first entry itself is at or above T
+            int g = predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, tau, m);
+            g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
+            uint32_t kk, pp;
+            if (g > lo_c) {
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g - 1, s.c[r], kk, pp);
+                if (kk >= T) lo_c = g;
+                else hi_c = g - 1;
+            }
+            if (lo_c == g && g < hi_c) {
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g, s.c[r], kk, pp);
+                if (kk >= T) lo_c = g + 1;
+                else hi_c = g;
+            }
+            if (lo_c < hi_c) {
+                const bool up = lo_c > g;
+                for (int step = 2; lo_c < hi_c; step <<= 1) {
+                    int t = up ? lo_c + step : hi_c - step + 1;
+                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+                    entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
+                    const bool ge = kk >= T;
+                    if (ge) lo_c = t;
+                    else hi_c = t - 1;
+                    if (ge != up) break;
+                }
+            }
+            while (lo_c < hi_c) {
+                int t = (lo_c + hi_c + 1) >> 1;
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
+                if (kk >= T) lo_c = t;
+                else hi_c = t - 1;
+            }
+            out[r] = lo_c;
+        }
+    }
+}
+
+// A threshold at or above which about `target` of the node's entries lie, by bisection on
+// the key itself over ESTIMATED counts.  All targets of a node bisect the SAME interval
+// [lo_key, hi_key] for the same number of steps at most, so their thresholds come out
+// ordered like the targets (two searches see the same midpoints until they part, and from
+// then on one interval lies above the other; a search that stops early inside a window
+// narrower than the distance between two targets is passed below by every later target).
+// Bisecting keys, not scores, keeps thresholds apart even where thousands of entries crowd
+// into a sliver of the score range.
+template <int R, bool RAVE>
+__device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t lo_key,
+                                                     uint32_t hi_key, int target, int window, int m) {
+    uint32_t klo = lo_key, khi = hi_key;  // est(klo) >= target is taken for granted, est(khi) < target
+    for (int it = 0; it < 24 && khi - klo > 1u; it++) {
+        const uint32_t kmid = klo + ((khi - klo) >> 1);
+        const float mid = key_score(kmid);
+        int est = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (r < s.rounds && s.c[r] >= 0) est += predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, mid, m);
+        const int e = wave_sum_i32(est);
+        if (e >= target) {
+            klo = kmid;
+            if (e <= target + window) break;
+        } else {
+            khi = kmid;
+        }
+    }
+    return klo;
+}
+
+// For a slice of a heavy node: the thresholds of the cumulative targets target_hi and
+// target_lo (0 = not wanted) and EXACTLY how many entries of every own child lie at or above
+// each (ct_hi, ct_lo; at most m each).  Every wavefront that asks for the same target of the
+// same node gets the same threshold: the computation is deterministic and depends on the
+// node's state only.  Uses the LDS scratch.
 template <int R, bool RAVE>
 __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const NodeCtx &c, int lane,
-                                                 const Kids<R, RAVE> &k, int m, int target, int (&ct)[R],
-                                                 uint32_t &T_out) {
+                                                 const Kids<R, RAVE> &k, WaveLds<R> &lds, int m, int window,
+                                                 int target_hi, int target_lo, int (&ct_hi)[R], int (&ct_lo)[R],
+                                                 uint32_t &T_hi, uint32_t &T_lo) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     uint32_t headk[R];
@@ -1151,9 +1310,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     if (hi_key == 0u) return false;
     const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
     // The best child alone has m entries at or above the key of its m-th visit: a lower bound
-    // for every threshold of the node.  All targets bisect the SAME interval, so that their
-    // thresholds come out ordered like the targets (two searches see the same midpoints until
-    // they part, and from then on one interval lies above the other).
+    // for every threshold of the node.
     uint32_t lo_key = 0u;
     {
         uint32_t kk = 0u, pp = 0u;
@@ -1166,73 +1323,72 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     }
     if (lo_key == 0u) lo_key = 1u;
     if (lo_key > hi_key) return false;
-    // bisection on the key itself, down to neighbouring binary32 values: where thousands of
-    // entries crowd into a sliver of the score range (a child whose score hardly moves with
-    // virtual loss) the thresholds of different targets still come apart
-    uint32_t klo = lo_key, khi = hi_key;  // est(klo) >= target is taken for granted, est(khi) < target
-    while (khi - klo > 1u) {
-        const uint32_t kmid = klo + ((khi - klo) >> 1);
-        const float mid = key_score(kmid);
-        int est = 0;
-#pragma unroll
-        for (int r = 0; r < R; r++)
-            if (k.part[r] && headk[r] >= lo_key)
-                est += predict_count<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, mid, m);
-        const int e = wave_sum_i32(est);
-        if (e >= target) {
-            klo = kmid;
-            // Close enough.  The window is narrower than the distance between the targets of
-            // two slices, so the order of the thresholds is kept: a search for a later target
-            // that reaches this midpoint goes below it.
-            if (e <= target + (kSliceEntries >> 3)) break;
-        } else {
-            khi = kmid;
-        }
-    }
-    const uint32_t T = klo;
-    const float tau = key_score(T);
+    // the active children, densely
+    int n_act = 0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        ct[r] = 0;
-        if (k.part[r] && headk[r] >= T) {
-            const int i = r * kWave + lane;
-            int lo_c = 1, hi_c = m;  // the first entry itself is at or above T
-            int g = predict_count<RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tau, m);
-            g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
-            uint32_t kk, pp;
-            if (g > lo_c) {
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, g - 1, i, kk, pp);
-                if (kk >= T) lo_c = g;
-                else hi_c = g - 1;
-            }
-            if (lo_c == g && g < hi_c) {
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, g, i, kk, pp);
-                if (kk >= T) lo_c = g + 1;
-                else hi_c = g;
-            }
-            if (lo_c < hi_c) {
-                const bool up = lo_c > g;
-                for (int step = 2; lo_c < hi_c; step <<= 1) {
-                    int t = up ? lo_c + step : hi_c - step + 1;
-                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
-                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, t - 1, i, kk, pp);
-                    const bool ge = kk >= T;
-                    if (ge) lo_c = t;
-                    else hi_c = t - 1;
-                    if (ge != up) break;
-                }
-            }
-            while (lo_c < hi_c) {
-                int t = (lo_c + hi_c + 1) >> 1;
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, t - 1, i, kk, pp);
-                if (kk >= T) lo_c = t;
-                else hi_c = t - 1;
-            }
-            ct[r] = lo_c;
+        const int i = r * kWave + lane;
+        const bool act = k.part[r] && headk[r] != 0u && headk[r] >= lo_key;
+        const uint64_t am = __ballot(act);
+        if (act) lds.pay2[1][n_act + __popcll(am & ((1ull << lane) - 1ull))] = (uint32_t)i;
+        n_act += __popcll(am);
+        lds.key[1][i] = headk[r];
+        lds.st_n[i] = k.n[r];
+        lds.st_w[i] = k.w[r];
+        lds.st_p[i] = k.p[r];
+        lds.st_vl[i] = k.vl[r];
+        lds.st_q2[i] = k.q2[r];
+        lds.pay[i] = 0u;
+    }
+    wave_sync_memory();
+    ActiveSet<R> s;
+    s.rounds = (n_act + kWave - 1) / kWave;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        s.c[r] = -1;
+        s.n[r] = 0;
+        s.vl[r] = 0;
+        s.w[r] = s.p[r] = s.q2[r] = 0.0f;
+        s.head[r] = 0u;
+        if (r < s.rounds && r * kWave + lane < n_act) {
+            const int ci = (int)lds.pay2[1][r * kWave + lane];
+            s.c[r] = ci;
+            s.n[r] = lds.st_n[ci];
+            s.w[r] = lds.st_w[ci];
+            s.p[r] = lds.st_p[ci];
+            s.vl[r] = lds.st_vl[ci];
+            s.q2[r] = lds.st_q2[ci];
+            s.head[r] = lds.key[1][ci];
         }
     }
-    if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
-    T_out = T;
+    int cta[R];
+    T_hi = 0xFFFFFFFFu;
+    T_lo = 0u;
+#pragma unroll
+    for (int r = 0; r < R; r++) ct_hi[r] = ct_lo[r] = 0;
+    if (target_hi > 0) {
+        T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m);
+        active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
+        wave_sync_memory();
+#pragma unroll
+        for (int r = 0; r < R; r++) ct_hi[r] = (int)lds.pay[r * kWave + lane];
+        wave_sync_memory();
+    }
+    if (target_lo > 0) {
+        T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m);
+        active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
+        wave_sync_memory();
+#pragma unroll
+        for (int r = 0; r < R; r++) ct_lo[r] = (int)lds.pay[r * kWave + lane];
+        wave_sync_memory();
+    }
+    if (a.stats && lane == 0) atomicAdd(a.stats + 5, (target_hi > 0) + (target_lo > 0));
     return true;
 }
 
@@ -1431,16 +1587,18 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             bool ok = true;
             int rank_hi = 0, rank_lo = m;
             uint32_t T_hi = 0xFFFFFFFFu, T_lo = 0u;
-            if (slice > 0) {
-                ok = threshold_counts<R, RAVE>(a, c, lane, k, m, slice * S, ct_hi, T_hi);
-                if (!ok) OMK_NOTE(20);
+            // the window inside which a threshold search may stop early: narrower than the
+            // distance between the targets of two slices
+            ok = threshold_counts<R, RAVE>(a, c, lane, k, lds, m, S >> 2, slice > 0 ? slice * S : 0,
+                                           last ? 0 : (slice + 1) * S, ct_hi, ct_lo, T_hi, T_lo);
+            if (!ok) OMK_NOTE(20);
+            if (ok && slice > 0) {
                 int sum = 0;
 #pragma unroll
                 for (int r = 0; r < R; r++) sum += ct_hi[r];
                 rank_hi = wave_sum_i32(sum);
             }
             if (ok && !last) {
-                ok = threshold_counts<R, RAVE>(a, c, lane, k, m, (slice + 1) * S, ct_lo, T_lo);
                 int sum = 0;
                 bool bad = false;
 #pragma unroll
@@ -1449,7 +1607,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     if (ct_lo[r] < ct_hi[r]) bad = true;
                 }
                 rank_lo = wave_sum_i32(sum);
-                if (!ok) OMK_NOTE(21);
                 if (T_lo > T_hi || __ballot(bad) != 0ull) {
                     ok = false;
                     OMK_NOTE(22);
@@ -1881,8 +2038,23 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
 template <int R, bool RAVE>
 __device__ __forceinline__ void team_help(const SelectArgs &a, WaveLds<R> &lds, int tid, int op, int total, int keep,
                                           int goff, int cur, float ep, uint32_t uvl) {
-    if (op == kOpOrder) batch_order<R, RAVE, kTeam>(lds, tid, total, ep, uvl);
-    else if (op == kOpEmit) batch_emit<R, kTeam>(a, lds, tid, total, keep, goff, cur);
+    if (op == kOpOrder) {
+        batch_order<R, RAVE, kTeam>(lds, tid, total, ep, uvl);
+    } else if (op == kOpEmit) {
+        batch_emit<R, kTeam>(a, lds, tid, total, keep, goff, cur);
+    } else if (op == kOpRun) {
+        const TeamCmd &cm = lds.cmd;
+        const int best = __builtin_amdgcn_readfirstlane(cm.best), btk = __builtin_amdgcn_readfirstlane(cm.btk);
+        const int bn = __builtin_amdgcn_readfirstlane(cm.bn), bvl = __builtin_amdgcn_readfirstlane(cm.bvl);
+        const float bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(cm.bw)));
+        const float bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(cm.bp)));
+        const float bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(cm.bq2)));
+        const uint32_t hk = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.hk);
+        const uint32_t hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.hp);
+        const uint32_t sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.sk);
+        const uint32_t spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.spos);
+        batch_run<R, RAVE, kTeam>(a, lds, tid, total, goff, best, btk, bn, bw, bp, bvl, bq2, ep, uvl, hk, hp, sk, spos);
+    }
 }
 
 template <int RMAX, bool RAVE>
