@@ -162,6 +162,22 @@ int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_pat
 int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperature, int32_t action_space,
                                     float *h_probabilities, int32_t *h_children);
 
+/* Tree reuse between moves (MCTSEngine::searchWithTreeReuse,
+ * src/mcts/mcts_engine_search.cpp:1029-1075): the node to search from after `last_action` was
+ * played is the first child of `root` with that action (-1 in *h_child when there is none:
+ * the reference then starts a fresh search).  Node ids stay valid: pass the child to
+ * omk_batch_set_roots and go on. */
+int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, int32_t *h_child);
+/* Drops everything but the subtree of new_root (what the reference achieves by clearing the
+ * siblings' children, :1049-1055) and renumbers that subtree to ids 0..k-1: breadth-first,
+ * siblings contiguous in their old order, new_root = 0, so selections come out the same.
+ * *h_nodes_after = k; h_old_of_new (NULL or room for the old node count) receives the old id
+ * of every new node.  Paths of earlier selections, roots of batches and node ids stored in
+ * transposition tables refer to the old numbering: set roots again, clear the tables.  The
+ * renumbering is computed on the host from the child ranges (read back once); the
+ * statistics are moved on the device. */
+int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new);
+
 /* Leaf expansion for the leaves of the last selection: MCTSNode::expand
  * (src/mcts/mcts_node.cpp:238-436) followed by setPriorProbabilities (:512-593), as the backup
  * phase does before it backs the values up (src/mcts/mcts_engine_batch_tree_simple.cpp:249-259).

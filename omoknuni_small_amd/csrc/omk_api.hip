@@ -429,6 +429,119 @@ int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperatu
     return OMK_OK;
 }
 
+int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, int32_t *h_child) {
+    if (!f || !h_child) return fail(OMK_ERR_INVALID, "omk_forest_reroot_child: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_reroot_child: nothing uploaded");
+    if (root < 0 || root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_reroot_child: root %d", root);
+    *h_child = -1;
+    if (last_action < 0) return OMK_OK;
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    int2 sp;
+    HIP_TRY(hipMemcpy(&sp, f->span + root, sizeof(sp), hipMemcpyDeviceToHost));
+    if (sp.y <= 0) return OMK_OK;
+    std::vector<int32_t> act((size_t)sp.y);
+    if (f->has_action) {
+        HIP_TRY(hipMemcpy(act.data(), f->action + sp.x, (size_t)sp.y * 4, hipMemcpyDeviceToHost));
+    } else {
+        for (int32_t i = 0; i < sp.y; i++) act[(size_t)i] = sp.x + i;
+    }
+    std::vector<uint32_t> legal;
+    const int64_t w0 = (int64_t)sp.x >> 5, w1 = ((int64_t)sp.x + sp.y + 31) >> 5;
+    if (f->has_legal) {
+        legal.resize((size_t)(w1 - w0));
+        HIP_TRY(hipMemcpy(legal.data(), f->legal + w0, legal.size() * 4, hipMemcpyDeviceToHost));
+    }
+    for (int32_t i = 0; i < sp.y; i++) {
+        const int64_t id = (int64_t)sp.x + i;
+        if (f->has_legal && !((legal[(size_t)((id >> 5) - w0)] >> (id & 31)) & 1u)) continue;
+        if (act[(size_t)i] == last_action) {
+            *h_child = (int32_t)id;
+            break;
+        }
+    }
+    return OMK_OK;
+}
+
+int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_compact: null forest");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact: nothing uploaded");
+    if (new_root < 0 || new_root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_compact: root %d", new_root);
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    HIP_TRY(hipStreamSynchronize(s));
+    const int64_t n = f->n_nodes;
+    std::vector<int2> span((size_t)n);
+    HIP_TRY(hipMemcpy(span.data(), f->span, (size_t)n * sizeof(int2), hipMemcpyDeviceToHost));
+    // breadth-first order of the subtree; children are appended in visiting order, so the
+    // first child of new node i is 1 + the children of all new nodes before it
+    std::vector<int32_t> order, new_begin;
+    order.reserve(1024);
+    order.push_back(new_root);
+    for (size_t head = 0; head < order.size(); head++) {
+        const int2 sp = span[(size_t)order[head]];
+        new_begin.push_back(sp.y > 0 ? (int32_t)order.size() : 0);
+        for (int32_t i = 0; i < sp.y; i++) order.push_back(sp.x + i);
+        if ((int64_t)order.size() > n) return fail(OMK_ERR_STRUCTURE, "omk_forest_compact: the child ranges do not form a tree");
+    }
+    const int64_t k = (int64_t)order.size();
+    // the legal mask of the new numbering, on the host (one bit per node)
+    std::vector<uint32_t> new_legal;
+    if (f->has_legal) {
+        std::vector<uint32_t> legal((size_t)((n + 31) / 32));
+        HIP_TRY(hipMemcpy(legal.data(), f->legal, legal.size() * 4, hipMemcpyDeviceToHost));
+        new_legal.assign((size_t)((k + 31) / 32), 0u);
+        for (int64_t i = 0; i < k; i++) {
+            const uint32_t old = (uint32_t)order[(size_t)i];
+            if ((legal[old >> 5] >> (old & 31u)) & 1u) new_legal[(size_t)(i >> 5)] |= 1u << (i & 31);
+        }
+    }
+    // device: map, new child starts, and one scratch array that every field passes through
+    int32_t *d_map = nullptr, *d_begin = nullptr;
+    uint64_t *d_tmp = nullptr;
+    hipError_t e = hipMalloc((void **)&d_map, (size_t)k * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_begin, (size_t)k * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_tmp, (size_t)k * 8);
+    auto cleanup = [&]() {
+        if (d_map) (void)hipFree(d_map);
+        if (d_begin) (void)hipFree(d_begin);
+        if (d_tmp) (void)hipFree(d_tmp);
+    };
+    if (e == hipSuccess) e = hipMemcpyAsync(d_map, order.data(), (size_t)k * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_begin, new_begin.data(), (size_t)k * 4, hipMemcpyHostToDevice, s);
+    auto move_words = [&](void *arr) {
+        if (e != hipSuccess || !arr) return;
+        e = launch_gather_words((uint32_t *)d_tmp, (const uint32_t *)arr, d_map, k, s);
+        if (e == hipSuccess) e = hipMemcpyAsync(arr, d_tmp, (size_t)k * 4, hipMemcpyDeviceToDevice, s);
+    };
+    move_words(f->N);
+    move_words(f->W);
+    move_words(f->P);
+    move_words(f->VL);
+    if (f->has_rave) {
+        move_words(f->rN);
+        move_words(f->rW);
+    }
+    if (f->has_action) move_words(f->action);
+    if (e == hipSuccess && f->has_hash) {
+        e = launch_gather_dwords(d_tmp, f->hash, d_map, k, s);
+        if (e == hipSuccess) e = hipMemcpyAsync(f->hash, d_tmp, (size_t)k * 8, hipMemcpyDeviceToDevice, s);
+    }
+    if (e == hipSuccess) {
+        e = launch_gather_span((int2 *)d_tmp, f->span, d_map, d_begin, k, s);
+        if (e == hipSuccess) e = hipMemcpyAsync(f->span, d_tmp, (size_t)k * sizeof(int2), hipMemcpyDeviceToDevice, s);
+    }
+    if (e == hipSuccess && f->has_legal)
+        e = hipMemcpyAsync(f->legal, new_legal.data(), new_legal.size() * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    cleanup();
+    if (e != hipSuccess) return fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
+    f->n_nodes = k;
+    if (h_nodes_after) *h_nodes_after = k;
+    if (h_old_of_new) memcpy(h_old_of_new, order.data(), (size_t)k * 4);
+    return OMK_OK;
+}
+
 int omk_forest_node_count(omk_forest *f, int64_t *h_nodes, int64_t *h_capacity) {
     if (!f) return fail(OMK_ERR_INVALID, "omk_forest_node_count: null forest");
     if (h_nodes) *h_nodes = f->n_nodes;

@@ -182,6 +182,46 @@ hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, 
     return hipGetLastError();
 }
 
+// ---- compaction after re-rooting: gathers through the old-id-of-new-id map ----
+__global__ __launch_bounds__(256) void k_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < k) dst[i] = src[map[i]];
+}
+
+__global__ __launch_bounds__(256) void k_gather_dwords(uint64_t *dst, const uint64_t *src, const int32_t *map,
+                                                       int64_t k) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < k) dst[i] = src[map[i]];
+}
+
+__global__ __launch_bounds__(256) void k_gather_span(int2 *dst, const int2 *src, const int32_t *map,
+                                                     const int32_t *new_begin, int64_t k) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < k) {
+        const int cc = src[map[i]].y;
+        dst[i] = int2{cc > 0 ? new_begin[i] : 0, cc};
+    }
+}
+
+hipError_t launch_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k, hipStream_t s) {
+    if (k <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_gather_words, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, s, dst, src, map, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_dwords(uint64_t *dst, const uint64_t *src, const int32_t *map, int64_t k, hipStream_t s) {
+    if (k <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_gather_dwords, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, s, dst, src, map, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_span(int2 *dst, const int2 *src, const int32_t *map, const int32_t *new_begin, int64_t k,
+                              hipStream_t s) {
+    if (k <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_gather_span, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, s, dst, src, map, new_begin, k);
+    return hipGetLastError();
+}
+
 // plain copy of 4-byte words: the known-size kernel that hardware traffic counters are scaled by
 __global__ __launch_bounds__(256) void k_copy_words(uint32_t *dst, const uint32_t *src, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;

@@ -122,6 +122,13 @@ struct ExpandJob {
 hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
                          const float *priors, int32_t *status, int64_t old_nodes, int64_t new_nodes, hipStream_t s);
 
+// Compaction: new node i takes the statistics of old node map[i]; its child range keeps its
+// length and starts at new_begin[i].
+hipError_t launch_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k, hipStream_t s);
+hipError_t launch_gather_dwords(uint64_t *dst, const uint64_t *src, const int32_t *map, int64_t k, hipStream_t s);
+hipError_t launch_gather_span(int2 *dst, const int2 *src, const int32_t *map, const int32_t *new_begin, int64_t k,
+                              hipStream_t s);
+
 struct TTSlot {
     unsigned long long key;
     int32_t node;

@@ -23,7 +23,8 @@ u64p = C.POINTER(C.c_uint64)
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
-    "omk_expand_batch", "omk_forest_action_probabilities", "omk_sync", "omk_batch_create", "omk_batch_destroy",
+    "omk_expand_batch", "omk_forest_action_probabilities", "omk_forest_reroot_child", "omk_forest_compact",
+    "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
@@ -165,6 +166,23 @@ class Forest:
         _check(self._lib.omk_forest_node_count(self._h, C.byref(n), C.byref(cap)))
         self.n_nodes = int(n.value)
         return int(n.value), int(cap.value)
+
+    def reroot_child(self, root, last_action):
+        """searchWithTreeReuse: the first child of root reached by last_action, or -1."""
+        c = C.c_int32()
+        _check(self._lib.omk_forest_reroot_child(self._h, C.c_int32(int(root)), C.c_int32(int(last_action)),
+                                                 C.byref(c)))
+        return int(c.value)
+
+    def compact(self, new_root):
+        """Keeps the subtree of new_root, renumbered breadth-first from 0; returns the old id of
+        every new node."""
+        n_old, _ = self.node_count()
+        order = np.empty(n_old, np.int32)
+        k = C.c_int64()
+        _check(self._lib.omk_forest_compact(self._h, C.c_int32(int(new_root)), C.byref(k), _ptr(order, i32p)))
+        self.n_nodes = int(k.value)
+        return order[:self.n_nodes].copy()
 
     def action_probabilities(self, root, temperature, action_space):
         """MCTSEngine::getActionProbabilities from the root's children; (probabilities, children)."""

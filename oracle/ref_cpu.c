@@ -433,3 +433,27 @@ int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperat
     }
     return n;
 }
+
+/* ---- tree reuse (src/mcts/mcts_engine_search.cpp:1029-1075) ---- */
+int32_t ref_reroot_child(const ref_tree *t, int32_t root, int32_t last_action) {
+    if (last_action < 0) return -1; /* :1039 */
+    const int32_t cb = t->child_begin[root], cc = t->child_count[root];
+    for (int32_t i = 0; i < cc; i++) {
+        const int32_t id = cb + i;
+        if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+        const int32_t a = t->action ? t->action[id] : id;
+        if (a == last_action) return id;
+    }
+    return -1;
+}
+
+int64_t ref_compact_order(const ref_tree *t, int32_t new_root, int32_t *old_of_new) {
+    int64_t head = 0, tail = 0;
+    old_of_new[tail++] = new_root;
+    while (head < tail) {
+        const int32_t old = old_of_new[head++];
+        const int32_t cb = t->child_begin[old], cc = t->child_count[old];
+        for (int32_t i = 0; i < cc; i++) old_of_new[tail++] = cb + i; /* empty slots keep their place */
+    }
+    return tail;
+}

@@ -19,6 +19,7 @@
  *   ref_expand_batch      src/mcts/mcts_node.cpp:238-436, :512-593 (MCTSNode::expand, setPriorProbabilities),
  *                         call site src/mcts/mcts_engine_batch_tree_simple.cpp:249-259
  *   ref_action_probabilities  src/mcts/mcts_engine_tree.cpp:388-465 (MCTSEngine::getActionProbabilities)
+ *   ref_reroot_child      src/mcts/mcts_engine_search.cpp:1029-1075 (searchWithTreeReuse)
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
  *
@@ -148,6 +149,19 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
  * is left all zero).  Slots whose legal bit is clear are not children. */
 int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperature, int32_t action_space,
                                  float *out);
+
+/* Tree reuse between moves (MCTSEngine::searchWithTreeReuse,
+ * src/mcts/mcts_engine_search.cpp:1029-1075): the new root is the FIRST child of the old root
+ * whose action is last_action (:1041-1043, children in order); everything else of the old
+ * tree is dropped.  Returns the child's id, or -1 when there is none (the reference then
+ * falls back to a fresh search). */
+int32_t ref_reroot_child(const ref_tree *t, int32_t root, int32_t last_action);
+/* The subtree of new_root renumbered so that it fills ids 0..k-1: breadth-first, siblings
+ * contiguous and in their old order (so selections come out the same), new_root = 0.
+ * old_of_new[i] receives the old id of new node i (room for n_nodes entries); returns k.
+ * (The reference keeps pointers, so it has no numbering to preserve: this only reclaims the
+ * arrays of the dropped siblings.) */
+int64_t ref_compact_order(const ref_tree *t, int32_t new_root, int32_t *old_of_new);
 
 /* Open-addressing table: 2^log2_slots slots of 16 bytes, linear probing,
  * home slot = (key * 0x9E3779B97F4A7C15) >> (64 - log2_slots), empty key = ~0. */

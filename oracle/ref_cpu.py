@@ -229,6 +229,33 @@ class RefTree:
                         _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p))
         return first
 
+    def reroot_child(self, root, last_action):
+        return int(lib().ref_reroot_child(C.byref(self._c), int(root), int(last_action)))
+
+    def compacted(self, new_root):
+        """The subtree of new_root as a new RefTree with ids 0..k-1 (breadth-first, sibling order
+        kept) and the old id of every new node."""
+        order = np.empty(self.n, dtype=np.int32)
+        fn = lib().ref_compact_order
+        fn.restype = C.c_int64
+        k = int(fn(C.byref(self._c), int(new_root), _ptr(order, i32p)))
+        order = order[:k].copy()
+        # first child of new node i: children were appended in visiting order
+        cc = self.child_count[order]
+        cb = np.zeros(k, np.int32)
+        cb[cc > 0] = (1 + np.concatenate([[0], np.cumsum(cc)[:-1]]))[cc > 0]
+        legal = None
+        if self.legal is not None:
+            bits = (self.legal[order >> 5] >> (order & 31).astype(np.uint32)) & 1
+            pad = np.zeros((k + 31) // 32 * 32, np.uint8)
+            pad[:k] = bits
+            legal = np.packbits(pad.reshape(-1, 32), axis=1, bitorder="little").view("<u4").reshape(-1).copy()
+        t = RefTree(self.N[order], self.W[order], self.P[order], self.VL[order], cb, cc,
+                    action=None if self.action is None else self.action[order],
+                    rN=None if self.rN is None else self.rN[order], rW=None if self.rW is None else self.rW[order],
+                    legal=legal)
+        return t, order
+
     def action_probabilities(self, root, temperature, action_space):
         """MCTSEngine::getActionProbabilities over the root's children; (probabilities, children)."""
         out = np.empty(int(action_space), dtype=np.float32)

@@ -149,3 +149,37 @@ def test_action_probabilities_match_the_checker(mask_frac):
             rp, rn = ref.action_probabilities(node, temp, A)
             gp, gn = f.action_probabilities(node, temp, A)
             assert gn == rn and gp.tobytes() == rp.tobytes(), (node, temp)
+
+
+@pytest.mark.parametrize("mask_frac,rave", [(0.0, False), (0.25, True)])
+def test_reroot_and_compaction_match_the_checker(mask_frac, rave):
+    """Tree reuse between moves: the child reached by the move becomes the root, the rest is
+    dropped, the subtree is renumbered; searching goes on and still matches."""
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(41, n_expand=150, fanout=(2, 12), max_depth=6, mask_frac=mask_frac, rave=rave, n_max=300)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    root = int(roots[0])
+    # the move: the action of the most visited child of the root
+    kids = np.arange(soa["child_begin"][root], soa["child_begin"][root] + soa["child_count"][root])
+    if "legal" in soa:
+        kids = kids[((soa["legal"][kids >> 5] >> (kids & 31).astype(np.uint32)) & 1) == 1]
+    move = int(soa["action"][kids[np.argmax(soa["N"][kids])]])
+    rc, gc = ref.reroot_child(root, move), f.reroot_child(root, move)
+    assert gc == rc >= 0
+    assert f.reroot_child(root, 10_000) == ref.reroot_child(root, 10_000) == -1
+    ref2, order = ref.compacted(rc)
+    gorder = f.compact(gc)
+    assert (gorder == order).all() and f.node_count()[0] == ref2.n
+    assert_same_forest(f, ref2, "after compaction")
+    # search on from the new root
+    B, D = 200, 8
+    b = omk.Batch(f, B, D)
+    b.set_roots(np.zeros(B, np.int32))
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3, use_rave=rave, rave_k=1000.0)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, use_rave=rave, rave_k=1000.0, max_depth=D)
+    rpaths, rlen, rleaf, _ = ref2.select_batch(np.zeros(B, np.int32), rp)
+    b.select(sp)
+    gpaths, glen, gleaf, _ = b.read()
+    assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
+    assert (f.download()["VL"] == ref2.VL).all()

@@ -120,3 +120,42 @@ def test_probabilities_uniform_when_nothing_was_visited_and_empty_without_childr
 def test_probabilities_are_laid_out_by_action_and_skip_actions_outside_the_space():
     p, _ = counts_tree([1, 1, 2], actions=[4, 9, 0]).action_probabilities(0, 1.0, 6)
     assert p[4] == 0.25 and p[0] == 0.5 and p.sum() == 0.75   # action 9 is outside: dropped
+
+
+# ---- tree reuse (src/mcts/mcts_engine_search.cpp:1029-1075) ----
+
+def test_reroot_picks_the_first_child_with_the_action():
+    t = counts_tree([1, 2, 3, 4], actions=[7, 5, 7, 2])
+    assert t.reroot_child(0, 7) == 1          # children in order: the first match
+    assert t.reroot_child(0, 2) == 4
+    assert t.reroot_child(0, 9) == -1         # no such child: the reference starts afresh
+    assert t.reroot_child(0, -1) == -1        # last_action < 0: no reuse
+    assert t.reroot_child(1, 7) == -1         # a leaf has no children
+
+
+def test_compaction_keeps_the_subtree_in_breadth_first_sibling_order():
+    from tests.helpers import random_tree
+    soa, roots = random_tree(5, n_expand=30, fanout=(2, 6), max_depth=4)
+    t = R.RefTree.from_soa(soa)
+    kid = int(soa["child_begin"][roots[0]]) + 1
+    t2, order = t.compacted(kid)
+    assert order[0] == kid and len(set(order.tolist())) == len(order)
+    # every kept node keeps its statistics, and children stay contiguous in the old order
+    assert (t2.N == t.N[order]).all() and (t2.child_count == t.child_count[order]).all()
+    for i in range(t2.n):
+        for j in range(t2.child_count[i]):
+            assert order[t2.child_begin[i] + j] == t.child_begin[order[i]] + j
+    # exactly the descendants of the new root were kept
+    keep, stack = set(), [kid]
+    while stack:
+        x = stack.pop()
+        keep.add(x)
+        stack.extend(range(t.child_begin[x], t.child_begin[x] + t.child_count[x]))
+    assert keep == set(order.tolist())
+    # the same selections, node for node, before and after
+    p = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=6)
+    pa, la, _, _ = R.RefTree.from_soa(soa).select_batch(np.full(40, kid, np.int32), p)
+    pb, lb, _, _ = t2.select_batch(np.zeros(40, np.int32), p)
+    assert (la == lb).all()
+    for i in range(40):
+        assert (order[pb[i, :lb[i]]] == pa[i, :la[i]]).all()
