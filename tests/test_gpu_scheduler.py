@@ -142,3 +142,37 @@ def test_bounded_wait_reports_and_recovers():
     gpaths, glen, gleaf, _ = b.read()
     assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
     assert (f.download()["VL"] == ref.VL).all()
+
+
+def test_no_virtual_loss_with_thousands_of_visitors():
+    """Without virtual loss nothing changes between visitors: all of them follow the first one
+    down the same path, thousands per node (shared partition, no slices)."""
+    soa, roots = layered_forest(12, [90, 30, 8])
+    st = select_both(soa, np.zeros(5000, np.int32), 5, vl=0)
+    assert st["sliced_nodes"] == 0, st   # slices need virtual loss; the partition is still shared
+
+
+def test_two_selections_in_a_row_accumulate_virtual_loss():
+    """select, select again without a backup in between (virtual loss of the first is still on
+    the tree), then revert both: counters return to where they started."""
+    import omoknuni_small_amd as omk
+    soa, roots = layered_forest(13, [70, 25], rave=True)
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, use_rave=True, rave_k=1000.0, max_depth=3)
+    f = omk.Forest.from_soa(soa)
+    B = 2500
+    b1, b2 = omk.Batch(f, B, 3), omk.Batch(f, B, 3)
+    troots = np.zeros(B, np.int32)
+    b1.set_roots(troots)
+    b2.set_roots(troots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3, use_rave=True, rave_k=1000.0)
+    r1 = ref.select_batch(troots, rp)
+    b1.select(sp)
+    r2 = ref.select_batch(troots, rp)
+    b2.select(sp)
+    g1, g2 = b1.read(), b2.read()
+    assert (g1[0] == r1[0]).all() and (g2[0] == r2[0]).all()
+    assert (f.download()["VL"] == ref.VL).all() and ref.VL.max() > 0
+    b2.revert_vl(3)
+    b1.revert_vl(3)
+    assert (f.download()["VL"] == 0).all()
