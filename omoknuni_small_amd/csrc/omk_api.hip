@@ -726,7 +726,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.hctx_n = b->counters + 2 * kSchedStep + 64;
     a.hctx_cap = b->hctx_cap;
     static_assert(kHeavyCtxInts >= 16 + OMK_MAX_FANOUT, "context too small");
-#ifdef OMK_PHASE_TIMERS
+#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
     a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
     a.trace_n = b->counters + 24;
     a.trace_cap = (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 8);
@@ -960,7 +960,7 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     return OMK_OK;
 }
 
-#ifdef OMK_PHASE_TIMERS
+#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
 // measurement builds only: the per-node timeline of the last selection (4 x int64 per node)
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
     if (int rc = use_device(b->f)) return rc;

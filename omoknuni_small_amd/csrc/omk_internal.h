@@ -58,7 +58,7 @@ struct SelectArgs {
     int32_t poll_sleep;    // s_sleep(32) units between two polls of a waiting wavefront
     int32_t q_cap;
     int32_t epoch;         // number of this select call on the batch, > 0
-#ifdef OMK_PHASE_TIMERS
+#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
     long long *trace;      // per processed node: start, end (100 MHz clock), visitors | depth << 32, node
     int32_t *trace_n;
     int32_t trace_cap;

@@ -73,6 +73,9 @@ enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
 
 // Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
 // multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
+#if defined(OMK_PHASE_TIMERS) && !defined(OMK_TRACE)
+#define OMK_TRACE
+#endif
 #ifdef OMK_PHASE_TIMERS
 #define OMK_FAIL(code)                                                      \
     do {                                                                    \
@@ -1983,7 +1986,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             const int depth = it.depth;
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
             int32_t *seg_out = a.seg[depth & 1];
-#ifdef OMK_PHASE_TIMERS
+#ifdef OMK_TRACE
             const long long tr0 = wall_clock64();
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
@@ -1997,7 +2000,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                 else
                     status = select_group<RMAX, RAVE>(f, a, c, lane, it, seg_in, seg_out, s_lds, next);
             }
-#ifdef OMK_PHASE_TIMERS
+#ifdef OMK_TRACE
             if (lane == 0) {
                 int ti = atomicAdd(a.trace_n, 1);
                 if (ti < a.trace_cap) {
@@ -2143,7 +2146,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         a.sched_wait[0] = open0;
         a.sched_wait[1] = 0;
         *a.hctx_n = 0;
-#ifdef OMK_PHASE_TIMERS
+#ifdef OMK_TRACE
         *a.trace_n = 0;
 #endif
     }
@@ -2175,7 +2178,7 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
         const int most = n_traversals / 2;
         if (grid > most) grid = most;
         if (grid < 1) grid = 1;
-#ifdef OMK_PHASE_TIMERS
+#ifdef OMK_TRACE
         if (a.dbg_grid > 0 && grid > a.dbg_grid) grid = a.dbg_grid;
 #endif
         hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kTeam), 0, s, f, a);
