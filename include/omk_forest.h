@@ -197,6 +197,15 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
 int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
                      int32_t action_space, int32_t *h_first_child);
 
+/* The RAVE statistics of MCTSEngine::backPropagate (src/mcts/mcts_engine_tree.cpp:288-331 with
+ * MCTSNode::updateRAVE, src/mcts/mcts_node.cpp:631-643) for the paths of the last selection
+ * and the values of omk_batch_set_values: every child of a path node whose action occurs
+ * among the actions of the path's nodes gets rave_count += 1 and rave_value_sum += the
+ * node's signed value (sign as in the backup), once per child.  The reference's live
+ * batched loop never calls this (its RAVE counts stay zero); it is offered for engines
+ * that do.  Needs a forest created with RAVE arrays.  Asynchronous on the forest's stream. */
+int omk_backup_rave_batch(omk_batch *b);
+
 /* Leaf gather (mcts_engine_batch_tree_simple.cpp:114,166-184): waits for the stream and
  * returns, per traversal, the path (row of max_depth+1 ids, -1 padded), its length, the
  * leaf node and the move list to replay on a clone of the root state (row of max_depth

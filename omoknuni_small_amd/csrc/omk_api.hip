@@ -760,6 +760,16 @@ int omk_backup_batch(omk_batch *b, int32_t virtual_loss) {
     return OMK_OK;
 }
 
+int omk_backup_rave_batch(omk_batch *b) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_backup_rave_batch: null batch");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_backup_rave_batch: no selected paths");
+    if (!b->f->has_rave) return fail(OMK_ERR_INVALID, "omk_backup_rave_batch: the forest has no RAVE arrays");
+    if (int rc = use_device(b->f)) return rc;
+    HIP_TRY(launch_rave_backup(b->f->mut(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
+                               b->f->stream));
+    return OMK_OK;
+}
+
 int omk_revert_vl(omk_batch *b, int32_t virtual_loss) {
     if (!b) return fail(OMK_ERR_INVALID, "omk_revert_vl: null batch");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_revert_vl: no selected paths");

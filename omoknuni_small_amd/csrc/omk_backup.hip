@@ -182,6 +182,49 @@ hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, 
     return hipGetLastError();
 }
 
+// ---- RAVE statistics of MCTSEngine::backPropagate (src/mcts/mcts_engine_tree.cpp:288-331,
+// MCTSNode::updateRAVE src/mcts/mcts_node.cpp:631-643): every child of a path node whose
+// action occurs among the path's actions gets rN += 1, rW += the node's signed value ----
+constexpr int kRaveMaxLen = 4097;  // longest path the ABI accepts
+
+// One wavefront per (traversal, depth): the path's actions go to LDS, the node's children are
+// spread over the lanes.
+__global__ __launch_bounds__(64) void k_rave_backup(ForestMut f, const int32_t *paths, const int32_t *path_len,
+                                                    const float *values, int n, int stride) {
+    __shared__ int s_pa[kRaveMaxLen];
+    const int t = blockIdx.x, d = blockIdx.y, lane = threadIdx.x;
+    const int len = path_len[t];
+    if (d >= len) return;
+    const int node = paths[(size_t)d * stride + t];
+    const int2 sp = f.span[node];
+    if (sp.y <= 0) return;
+    for (int e = lane; e < len; e += 64) {
+        const int pn = paths[(size_t)e * stride + t];
+        s_pa[e] = f.action ? f.action[pn] : pn;
+    }
+    __syncthreads();
+    float v = values[t];
+    if ((len - 1 - d) & 1) v = -v;  // the leaf's children see +value, every ply up flips it
+    for (int i = lane; i < sp.y; i += 64) {
+        const int id = sp.x + i;
+        if (f.legal && !((f.legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+        const int a = f.action ? f.action[id] : id;
+        bool hit = false;
+        for (int e = 0; e < len && !hit; e++) hit = s_pa[e] != -1 && s_pa[e] == a;
+        if (hit) {
+            atomicAdd(f.rN + id, 1);
+            unsafeAtomicAdd(f.rW + id, v);
+        }
+    }
+}
+
+hipError_t launch_rave_backup(const ForestMut &f, const int32_t *paths, const int32_t *path_len, const float *values,
+                              int n, int stride, int max_len, hipStream_t s) {
+    if (n <= 0 || max_len <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_rave_backup, dim3(n, max_len), dim3(64), 0, s, f, paths, path_len, values, n, stride);
+    return hipGetLastError();
+}
+
 // ---- compaction after re-rooting: gathers through the old-id-of-new-id map ----
 __global__ __launch_bounds__(256) void k_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;

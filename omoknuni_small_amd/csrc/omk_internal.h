@@ -122,6 +122,9 @@ struct ExpandJob {
 hipError_t launch_expand(const ForestMut &f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
                          const float *priors, int32_t *status, int64_t old_nodes, int64_t new_nodes, hipStream_t s);
 
+hipError_t launch_rave_backup(const ForestMut &f, const int32_t *paths, const int32_t *path_len, const float *values,
+                              int n, int stride, int max_len, hipStream_t s);
+
 // Compaction: new node i takes the statistics of old node map[i]; its child range keeps its
 // length and starts at new_begin[i].
 hipError_t launch_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k, hipStream_t s);

@@ -26,7 +26,7 @@ EXPORTS = [
     "omk_expand_batch", "omk_forest_action_probabilities", "omk_forest_reroot_child", "omk_forest_compact",
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
-    "omk_revert_vl", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
+    "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
@@ -284,6 +284,10 @@ class Batch:
 
     def backup(self, virtual_loss):
         _check(self._lib.omk_backup_batch(self._h, int(virtual_loss)))
+
+    def backup_rave(self):
+        """RAVE statistics of backPropagate for the selected paths and the values set."""
+        _check(self._lib.omk_backup_rave_batch(self._h))
 
     def revert_vl(self, virtual_loss):
         _check(self._lib.omk_revert_vl(self._h, int(virtual_loss)))

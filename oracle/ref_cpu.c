@@ -457,3 +457,33 @@ int64_t ref_compact_order(const ref_tree *t, int32_t new_root, int32_t *old_of_n
     }
     return tail;
 }
+
+/* ---- RAVE statistics of backPropagate (src/mcts/mcts_engine_tree.cpp:288-331) ---- */
+void ref_rave_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *path_len, const float *values,
+                           int32_t B, int32_t stride) {
+    if (!t->rN || !t->rW) return;
+    for (int32_t i = 0; i < B; i++) {
+        const int32_t *path = paths + (int64_t)i * stride;
+        const int32_t len = path_len[i];
+        int invert = 0;
+        for (int32_t d = len - 1; d >= 0; d--) { /* leaf to root */
+            const int32_t node = path[d];
+            const float v = invert ? -values[i] : values[i];
+            const int32_t cb = t->child_begin[node], cc = t->child_count[node];
+            for (int32_t c = 0; c < cc; c++) {
+                const int32_t id = cb + c;
+                if (t->legal && !((t->legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u)) continue;
+                const int32_t a = t->action ? t->action[id] : id;
+                for (int32_t e = 0; e < len; e++) {
+                    const int32_t pa = t->action ? t->action[path[e]] : path[e];
+                    if (pa != -1 && pa == a) {
+                        t->rN[id] += 1;
+                        t->rW[id] += v;
+                        break; /* once per child */
+                    }
+                }
+            }
+            invert = !invert;
+        }
+    }
+}

@@ -19,6 +19,8 @@
  *   ref_expand_batch      src/mcts/mcts_node.cpp:238-436, :512-593 (MCTSNode::expand, setPriorProbabilities),
  *                         call site src/mcts/mcts_engine_batch_tree_simple.cpp:249-259
  *   ref_action_probabilities  src/mcts/mcts_engine_tree.cpp:388-465 (MCTSEngine::getActionProbabilities)
+ *   ref_rave_backup_batch src/mcts/mcts_engine_tree.cpp:288-331 (RAVE part of backPropagate; not dispatched
+ *                         by the reference's live search loop)
  *   ref_reroot_child      src/mcts/mcts_engine_search.cpp:1029-1075 (searchWithTreeReuse)
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
@@ -149,6 +151,17 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
  * is left all zero).  Slots whose legal bit is clear are not children. */
 int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperature, int32_t action_space,
                                  float *out);
+
+/* The RAVE part of MCTSEngine::backPropagate (src/mcts/mcts_engine_tree.cpp:288-331, with
+ * MCTSNode::updateRAVE, src/mcts/mcts_node.cpp:631-643), for a batch of paths in index order.
+ * The reference only runs it from a search loop that is not dispatched any more; it is
+ * restated for completeness.  path_actions = the actions of all nodes of the path that have
+ * one (action != -1, :296-300).  Going from the leaf to the root, with the value's sign
+ * flipped per ply as in the backup, every child of the path node whose action occurs in
+ * path_actions gets rave_count += 1 and rave_value_sum += the node's signed value, once per
+ * child (:310-324).  Slots whose legal bit is clear are not children.  Touches rN / rW only. */
+void ref_rave_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *path_len, const float *values,
+                           int32_t B, int32_t stride);
 
 /* Tree reuse between moves (MCTSEngine::searchWithTreeReuse,
  * src/mcts/mcts_engine_search.cpp:1029-1075): the new root is the FIRST child of the old root

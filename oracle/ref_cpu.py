@@ -229,6 +229,12 @@ class RefTree:
                         _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p))
         return first
 
+    def rave_backup_batch(self, paths, path_len, values):
+        paths, path_len, B, stride = self._paths_args(paths, path_len)
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        lib().ref_rave_backup_batch(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), _ptr(values, f32p),
+                                    B, stride)
+
     def reroot_child(self, root, last_action):
         return int(lib().ref_reroot_child(C.byref(self._c), int(root), int(last_action)))
 

@@ -183,3 +183,39 @@ def test_reroot_and_compaction_match_the_checker(mask_frac, rave):
     gpaths, glen, gleaf, _ = b.read()
     assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
     assert (f.download()["VL"] == ref2.VL).all()
+
+
+def test_rave_backup_matches_the_checker():
+    """The RAVE part of MCTSEngine::backPropagate (not run by the reference's live loop; offered
+    for engines that do): rN exact, rW within 1e-5."""
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(52, n_expand=120, fanout=(3, 14), max_depth=6, mask_frac=0.15, rave=True, n_max=200)
+    # small action space, so that sibling subtrees share actions (what RAVE is about)
+    soa["action"] = np.where(soa["action"] >= 0, soa["action"] % 9, soa["action"]).astype(np.int32)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    B, D = 500, 7
+    b = omk.Batch(f, B, D)
+    troots = np.full(B, roots[0], np.int32)
+    b.set_roots(troots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3, use_rave=True, rave_k=50.0)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, use_rave=True, rave_k=50.0, max_depth=D)
+    rng = np.random.default_rng(2)
+    for step in range(3):
+        rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths == rpaths).all(), "step %d" % step
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        b.set_values(values)
+        ref.rave_backup_batch(rpaths, rlen, values)
+        b.backup_rave()
+        ref.backup_batch(rpaths, rlen, values, 3)
+        b.backup(3)
+        st = f.download()
+        assert (st["rN"] == ref.rN).all() and ref.rN.sum() > soa["rN"].sum()
+        err = np.abs(st["rW"].astype(np.float64) - ref.rW) / np.maximum(np.abs(ref.rW), 1.0)
+        assert err.max() <= 1e-5
+        assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all()
+        ref.W[:] = st["W"]
+        ref.rW[:] = st["rW"]

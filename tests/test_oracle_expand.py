@@ -159,3 +159,19 @@ def test_compaction_keeps_the_subtree_in_breadth_first_sibling_order():
     assert (la == lb).all()
     for i in range(40):
         assert (order[pb[i, :lb[i]]] == pa[i, :la[i]]).all()
+
+
+# ---- RAVE statistics of backPropagate (src/mcts/mcts_engine_tree.cpp:288-331) ----
+
+def test_rave_backup_updates_children_whose_action_is_on_the_path():
+    # root(0) -> children 1,2,3 with actions 5,6,7; node 1 -> children 4,5 with actions 6,9
+    z = lambda *v: np.array(v, np.int32)
+    t = R.RefTree(N=z(3, 1, 1, 1, 0, 0), W=np.zeros(6, np.float32), P=np.ones(6, np.float32), VL=z(0, 0, 0, 0, 0, 0),
+                  child_begin=z(1, 4, 0, 0, 0, 0), child_count=z(3, 2, 0, 0, 0, 0), action=z(-1, 5, 6, 7, 6, 9),
+                  rN=np.zeros(6, np.int32), rW=np.zeros(6, np.float32))
+    # one path root -> 1 -> 4: its actions are {5, 6} (the root's -1 does not count)
+    t.rave_backup_batch(np.array([[0, 1, 4]], np.int32), [3], [0.5])
+    # at the leaf (4): no children.  at node 1 (sign flipped once): child 4 (action 6) matches, child 5 does not.
+    # at the root (flipped twice): children 1 (action 5) and 2 (action 6) match, child 3 does not.
+    assert t.rN.tolist() == [0, 1, 1, 0, 1, 0]
+    assert t.rW.tolist() == [0.0, 0.5, 0.5, 0.0, -0.5, 0.0]
