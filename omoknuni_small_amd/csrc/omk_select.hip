@@ -56,7 +56,7 @@ constexpr int kRunMin = 4;                // visitors from which the one-winner 
 constexpr int kWaterLevelMin = 24;        // visitors from which the parallel path is tried
 constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in the sort payload
 constexpr int kBatchCap = 2048;           // entries put in winner order at a time (LDS resident)
-constexpr int kSortBits = 4;              // radix digit of that sort
+constexpr int kSortBits = 6;              // widest radix digit of that sort (one lane per digit value)
 constexpr int kSortBins = 1 << kSortBits;
 constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-visitor kernel: one owner that
                                           // takes the items, three helpers for the batch work of its node
@@ -151,15 +151,53 @@ struct WaveLds {
     int st_vl[R * kWave];
     float st_q2[R * kWave];
     int st_j0[R * kWave];  // visits already settled / visit count, by phase
-    int hist[kSortBins * kTeam + kSortBins * kTeam / 16];  // sort: one counter per (digit value, thread), padded
+    int hist[kSortBins * (kBatchCap / kWave + 1) > R * kWave ? kSortBins * (kBatchCap / kWave + 1) : R * kWave];  // sort: entries per (digit value, block of 64); emit: visits per child
     uint32_t pay[R * kWave];      // per child: entries of the batch
     uint32_t key[2][kBatchCap];   // entries of the batch being ordered: inverted score key ...
     uint32_t pay2[2][kBatchCap];  // ... and pass flag, child, visit number; two buffers, ping-pong
 };
 
-template <int R, bool RAVE>
+// AHEAD: ask for the statistics of every child in range before the legality bits are known
+// (one memory round trip instead of two; reads the statistics of illegal children too, so
+// only where latency matters more than traffic).
+template <int R, bool RAVE, bool AHEAD = false>
 __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
                                           Kids<R, RAVE> &k) {
+    if (AHEAD) {
+        int rn[R];
+        float rw[R];
+        uint32_t word[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int i = r * kWave + lane;
+            const bool in = i < nelig;
+            const int id = cb + i;
+            word[r] = in && f.legal ? f.legal[(uint32_t)id >> 5] : 0xFFFFFFFFu;
+            k.n[r] = in ? f.N[id] : 0;
+            k.w[r] = in ? f.W[id] : 0.0f;
+            k.p[r] = in ? f.P[id] : 0.0f;
+            k.vl[r] = in ? f.VL[id] : 0;
+            rn[r] = RAVE && in ? f.rN[id] : 0;
+            rw[r] = RAVE && in ? f.rW[id] : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int i = r * kWave + lane;
+            const int id = cb + i;
+            const bool in = i < nelig && ((word[r] >> ((uint32_t)id & 31u)) & 1u);
+            k.part[r] = in;
+            if (!in) {
+                k.n[r] = 0;
+                k.w[r] = 0.0f;
+                k.p[r] = 0.0f;
+                k.vl[r] = 0;
+                rn[r] = 0;
+                rw[r] = 0.0f;
+            }
+            k.q2[r] = RAVE ? combined_value(k.n[r], k.w[r], rn[r], rw[r], rave_k) : 0.0f;
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         int i = r * kWave + lane;
@@ -471,130 +509,93 @@ __device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, 
 
     // Stable radix sort, in LDS.  Order wanted: key descending, then candidate position
     // ascending, then visit number.  The entries start in (child, visit) order; least
-    // significant digit first, a pass on the scan kind (only when both kinds occur:
-    // candidates of the first scan sit before those of the second) and then the key digits,
-    // over the bits of the key range.  One pass: every thread owns a contiguous block of the
-    // current order, counts its digits in registers (sixteen 8-bit counters), a scan over
-    // (digit value, thread) turns the counts into start positions, kept in LDS per (digit
-    // value, thread), and every thread moves its block in order.  No two threads share a
-    // counter, so the order inside a digit value is (thread, position in block): stable.
-    // A small batch (two entries per lane at most) is ranked by comparing every entry with
-    // every other one instead, through lane reads.
+    // significant digit first: a one-bit pass on the scan kind (only when both kinds occur:
+    // candidates of the first scan sit before those of the second), then the bits of the key
+    // range in digits of up to kSortBits bits.  One pass: the current order is cut in blocks
+    // of 64 entries, one per lane of a wavefront; inside a block every lane finds the lanes
+    // that hold the same digit value (one ballot per bit), which gives its rank among them
+    // and their number; the numbers go to a table indexed (digit value, block), an
+    // exclusive scan over the table in that order gives every (value, block) group its start,
+    // and every lane moves its entry to start + rank: stable.
     const uint32_t range = kmax - kmin;
     const int nbits = range == 0u ? 0 : 32 - __clz((int)range);
+    constexpr int kWaves = NT / kWave;
+    constexpr int kRounds = NT == kWave ? 4 : kBatchCap / NT;  // blocks a wavefront can be given
+    static_assert(kTeamMin <= 4 * kWave, "a lone wavefront orders fewer than four blocks");
+    const int wave = tid >> 6;
+    const int nblocks = (total + kWave - 1) >> 6;
+    const int nb1 = nblocks | 1;  // odd table stride: the lanes of a wavefront hit different LDS banks
     int cur = 0;
-    if (NT == kWave && total <= 2 * kWave) {
-        // entry q of the batch: (key, kind bit | q) compared as a pair; entries lane and 64 + lane
-        const bool in0 = lane < total, in1 = kWave + lane < total;
-        const uint32_t k0 = in0 ? lds.key[0][lane] : 0xFFFFFFFFu, k1 = in1 ? lds.key[0][kWave + lane] : 0xFFFFFFFFu;
-        const uint32_t p0 = in0 ? lds.pay2[0][lane] : 0u, p1 = in1 ? lds.pay2[0][kWave + lane] : 0u;
-        const uint32_t t0 = in0 ? (p0 & 0x80000000u) | (uint32_t)lane : 0xFFFFFFFFu;
-        const uint32_t t1 = in1 ? (p1 & 0x80000000u) | (uint32_t)(kWave + lane) : 0xFFFFFFFFu;
-        int rank0 = 0, rank1 = 0;
-        const int n0 = total < kWave ? total : kWave;
-        for (int s = 0; s < n0; s++) {
-            const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k0, s);
-            const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t0, s);
-            rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
-            rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
-        }
-        for (int s = 0; s < total - kWave; s++) {
-            const uint32_t ks = (uint32_t)__builtin_amdgcn_readlane((int)k1, s);
-            const uint32_t ts = (uint32_t)__builtin_amdgcn_readlane((int)t1, s);
-            rank0 += (ks < k0 || (ks == k0 && ts < t0)) ? 1 : 0;
-            rank1 += (ks < k1 || (ks == k1 && ts < t1)) ? 1 : 0;
-        }
-        if (in0) {
-            lds.key[1][rank0] = k0;
-            lds.pay2[1][rank0] = p0;
-        }
-        if (in1) {
-            lds.key[1][rank1] = k1;
-            lds.pay2[1][rank1] = p1;
-        }
-        cur = 1;
-    } else {
-        const int wave = tid >> 6;
-        for (int sh = mixed ? -kSortBits : 0; sh < nbits; sh += kSortBits) {
-            const uint32_t *src_k = lds.key[cur], *src_p = lds.pay2[cur];
-            uint32_t *dst_k = lds.key[cur ^ 1], *dst_p = lds.pay2[cur ^ 1];
-            uint64_t c_lo = 0ull, c_hi = 0ull;  // counters of digit values 0..7 and 8..15
-            for (int q = q0; q < q1; q += 4) {
-                uint32_t v[4];
+    const int key_passes = (nbits + kSortBits - 1) / kSortBits;
+    const int bits_even = key_passes > 0 ? (nbits + key_passes - 1) / key_passes : 0;
+    for (int pass = mixed ? -1 : 0; pass < key_passes; pass++) {
+        const int sh = pass * bits_even;
+        const int bits = pass < 0 ? 1 : (nbits - sh < bits_even ? nbits - sh : bits_even);
+        const int ndig = 1 << bits;
+        const uint32_t *src_k = lds.key[cur], *src_p = lds.pay2[cur];
+        uint32_t *dst_k = lds.key[cur ^ 1], *dst_p = lds.pay2[cur ^ 1];
+        uint32_t kk[kRounds], pp[kRounds];
+        int dig[kRounds], rank[kRounds];
 #pragma unroll
-                for (int u = 0; u < 4; u++) v[u] = q + u < q1 ? (sh < 0 ? src_p[q + u] : src_k[q + u]) : 0u;
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    if (q + u < q1) {
-                        const uint32_t d = sh < 0 ? v[u] >> 31 : ((v[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
-                        const uint64_t one = 1ull << ((d & 7u) * 8u);
-                        if (d & 8u) c_hi += one;
-                        else c_lo += one;
-                    }
+        for (int r = 0; r < kRounds; r++) {
+            const int blk = wave + r * kWaves;
+            if (blk < nblocks) {  // uniform per wavefront
+                const int q = blk * kWave + lane;
+                const bool valid = q < total;
+                kk[r] = valid ? src_k[q] : 0u;
+                pp[r] = valid ? src_p[q] : 0u;
+                const uint32_t d = pass < 0 ? pp[r] >> 31 : ((kk[r] - kmin) >> sh) & (uint32_t)(ndig - 1);
+                uint64_t same = __ballot(valid);
+                for (int bb = 0; bb < bits; bb++) {
+                    const bool one = (d >> bb) & 1u;
+                    const uint64_t bal = __ballot(one);
+                    same &= one ? bal : ~bal;
                 }
+                dig[r] = (int)d;
+                rank[r] = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32),
+                                                         __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
+                if (lane < ndig) {
+                    lds.hist[lane * nb1 + blk] = 0;
+                    if (blk == 0 && nb1 != nblocks) lds.hist[lane * nb1 + nblocks] = 0;  // the pad column
+                }
+                wave_sync_memory();
+                if (valid && rank[r] == 0) lds.hist[(int)d * nb1 + blk] = __popcll(same);
             }
-            // Start positions: exclusive prefix of the counts in (digit value, thread) order.
-            // The counts go to LDS in that order with one pad word per sixteen, every thread
-            // then owns sixteen consecutive ones (stride 17: conflict-free), sums them, one
-            // scan over the sums of the team, and the prefixes go back to the same places.
-#pragma unroll
-            for (int b = 0; b < kSortBins; b++) {
-                const int e = b * NT + tid;
-                lds.hist[e + (e >> 4)] = (int)(((b < 8 ? c_lo : c_hi) >> ((b & 7) * 8)) & 0xFFull);
-            }
-            team_sync<NT>();
-            {
-                int h[16];
-                int lsum = 0;
-#pragma unroll
-                for (int t = 0; t < 16; t++) {
-                    h[t] = lds.hist[tid * 17 + t];
-                    lsum += h[t];
-                }
-                const int inc = wave_inclusive_sum(lsum, lane);
-                int run = inc - lsum;
-                if (NT > kWave) {
-                    if (lane == kWave - 1) lds.wsum[wave] = inc;
-                    team_sync<NT>();
-                    for (int w = 0; w < wave; w++) run += lds.wsum[w];
-                }
-#pragma unroll
-                for (int t = 0; t < 16; t++) {
-                    lds.hist[tid * 17 + t] = run;
-                    run += h[t];
-                }
-            }
-            team_sync<NT>();
-            // the counters are private to their thread from here on
-            for (int q = q0; q < q1; q += 4) {
-                uint32_t kk[4], pp[4];
-                int pos[4];
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    kk[u] = q + u < q1 ? src_k[q + u] : 0u;
-                    pp[u] = q + u < q1 ? src_p[q + u] : 0u;
-                }
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    pos[u] = 0;
-                    if (q + u < q1) {
-                        const uint32_t d = sh < 0 ? pp[u] >> 31 : ((kk[u] - kmin) >> sh) & (uint32_t)(kSortBins - 1);
-                        const int e = (int)d * NT + tid;
-                        pos[u] = __hip_atomic_fetch_add(&lds.hist[e + (e >> 4)], 1, __ATOMIC_RELAXED,
-                                                        __HIP_MEMORY_SCOPE_WAVEFRONT);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    if (q + u < q1) {
-                        dst_k[pos[u]] = kk[u];
-                        dst_p[pos[u]] = pp[u];
-                    }
-                }
-            }
-            team_sync<NT>();
-            cur ^= 1;
         }
+        team_sync<NT>();
+        {
+            // exclusive scan of the table: every thread owns `own` consecutive counters
+            const int n_tab = ndig * nb1;
+            const int own = (n_tab + NT - 1) / NT;
+            const int t0 = tid * own < n_tab ? tid * own : n_tab;
+            const int t1 = t0 + own < n_tab ? t0 + own : n_tab;
+            int lsum = 0;
+            for (int t = t0; t < t1; t++) lsum += lds.hist[t];
+            const int inc = wave_inclusive_sum(lsum, lane);
+            int run = inc - lsum;
+            if (NT > kWave) {
+                if (lane == kWave - 1) lds.wsum[wave] = inc;
+                team_sync<NT>();
+                for (int w = 0; w < wave; w++) run += lds.wsum[w];
+            }
+            for (int t = t0; t < t1; t++) {
+                const int h = lds.hist[t];
+                lds.hist[t] = run;
+                run += h;
+            }
+        }
+        team_sync<NT>();
+#pragma unroll
+        for (int r = 0; r < kRounds; r++) {
+            const int blk = wave + r * kWaves;
+            if (blk < nblocks && blk * kWave + lane < total) {
+                const int pos = lds.hist[dig[r] * nb1 + blk] + rank[r];
+                dst_k[pos] = kk[r];
+                dst_p[pos] = pp[r];
+            }
+        }
+        team_sync<NT>();
+        cur ^= 1;
     }
     team_sync<NT>();
     return cur;
@@ -1510,7 +1511,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     const int off = item.off, m = item.m, depth = item.depth;
     Kids<R, RAVE> k;
     int cnt[R];
-    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, a.rave_k, k);
+    load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
 #pragma unroll
     for (int r = 0; r < R; r++) {
         score_round<R, RAVE>(k, r, c.ep);
@@ -1742,10 +1743,33 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // where the walk goes on: ask for that node's child range now, it arrives during the scatter
     int2 keep_span = int2{0, 0};
     if (keep >= 0) keep_span = f.span[c.cb + keep];
+    // the queue slots this node needs, asked for with one atomic per queue: a slot in the
+    // single-visitor queue for every child with one visitor (in child order), a slot in the
+    // work queue for every other child with visitors that this wavefront does not keep
+    int n_lone = 0, n_push = 0;
+    uint64_t has[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        const uint64_t lm1 = __ballot(cnt[r] == 1);
+        lds.st_vl[i] = n_lone + __popcll(lm1 & ((1ull << lane) - 1ull));
+        n_lone += __popcll(lm1);
+        has[r] = __ballot(cnt[r] > 1 && i != keep);
+        n_push += __popcll(has[r]);
+    }
+    int lone0 = 0, slot0 = -1;
+    bool have_slots = false;
+    if (!as_scatter && (m < kHeavyMin || R * kWave > kHeavyFanout)) {
+        // not a node whose scatter is shared out: the answers arrive during the next steps
+        if (lane == 0) {
+            if (n_lone > 0) lone0 = atomicAdd(a.n_singles, n_lone);
+            if (n_push > 0) slot0 = atomicAdd(a.sched_tail, n_push);
+        }
+        have_slots = true;
+    }
     int carry = 0;
     int keep_np = 0;
     int excl[R];
-    int n_lone = 0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         int inc = wave_inclusive_sum(cnt[r], lane);
@@ -1755,7 +1779,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         lds.st_j0[i] = cnt[r];
         lds.st_n[i] = k.n[r];
         if (i == keep) keep_np = k.n[r];
-        n_lone += __popcll(__ballot(cnt[r] == 1));
         carry += __builtin_amdgcn_readlane(inc, 63);
     }
     wave_sync_memory();
@@ -1770,6 +1793,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             part = slice;
             n_parts = n_slices;
             shared = true;
+            lone0 = a.hctx[(size_t)hid * kHeavyCtxInts + 3];
+            have_slots = true;  // the wavefront that finishes the scatter asks for the work queue's
         } else if (m >= kHeavyMin) {
             if (hid < 0) {
                 int id = a.hctx_cap;
@@ -1787,7 +1812,13 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
 #pragma unroll
                     for (int r = 0; r < R; r++) ctx[16 + r * kWave + lane] = cnt[r];
-                    if (lane == 0) ctx[2] = K2;
+                    if (lane == 0 && n_lone > 0) lone0 = atomicAdd(a.n_singles, n_lone);
+                    lone0 = __builtin_amdgcn_readfirstlane(lone0);
+                    have_slots = true;
+                    if (lane == 0) {
+                        ctx[2] = K2;
+                        ctx[3] = lone0;
+                    }
                     if (lane < K2 - 1) {
                         Item it = item;
                         it.pad[0] = 2;
@@ -1812,6 +1843,11 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             r1 = r0 + per < m ? r0 + per : m;
         }
     }
+    if (!have_slots && lane == 0) {  // a heavy node that could not share its scatter
+        if (n_lone > 0) lone0 = atomicAdd(a.n_singles, n_lone);
+        if (n_push > 0) slot0 = atomicAdd(a.sched_tail, n_push);
+    }
+    lone0 = __builtin_amdgcn_readfirstlane(lone0);
     int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
     // kScatterUnroll chunks of 64 visitors at a time: their loads are issued together, so the
     // loop pays the memory latency once per group of chunks instead of once per chunk
@@ -1839,19 +1875,11 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             if (base + u * kWave >= r1) break;
             const bool in = base + u * kWave + lane < r1;
             const int t = tt[u], i = ii[u];
-            bool lone = false;
             if (in) {
                 path_next[t] = c.cb + i;
                 seg_out[off + lds.offs[i] + oo[u]] = t;
-                lone = lds.st_j0[i] == 1;
-            }
-            // a visitor that is now alone goes to the single-visitor walk
-            uint64_t lm = __ballot(lone);
-            if (lm != 0ull) {
-                int s0 = 0;
-                if (lane == 0) s0 = atomicAdd(a.n_singles, __popcll(lm));
-                s0 = __builtin_amdgcn_readfirstlane(s0);
-                if (lone) {
+                // a visitor that is now alone goes to the single-visitor walk
+                if (lds.st_j0[i] == 1) {
                     Item it;
                     it.node = c.cb + i;
                     it.off = t;
@@ -1859,7 +1887,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     it.np = lds.st_n[i];
                     it.depth = depth + 1;
                     it.pad[0] = it.pad[1] = it.pad[2] = 0;
-                    a.singles_q[s0 + __popcll(lm & ((1ull << lane) - 1ull))] = it;
+                    a.singles_q[lone0 + lds.st_vl[i]] = it;
                 }
             }
         }
@@ -1878,35 +1906,33 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // wavefront does not keep become items of the queue: everything they refer to is written,
     // make it visible to the whole device, then mark them ready
     int myslot[R];
-    int n_pushed = 0;
+    const int n_pushed = n_push;
+    if (n_push > 0) {
+        // a shared scatter: the wavefront that finishes it asks for the slots
+        if (shared && lane == 0) slot0 = atomicAdd(a.sched_tail, n_push);
+        slot0 = __builtin_amdgcn_readfirstlane(slot0);
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int i = r * kWave + lane;
         myslot[r] = -1;
-        uint64_t has = __ballot(cnt[r] > 1 && i != keep);
-        int nnew = __popcll(has);
-        n_pushed += nnew;
-        if (nnew > 0) {
-            int slot0 = 0;
-            if (lane == 0) slot0 = atomicAdd(a.sched_tail, nnew);
-            slot0 = __builtin_amdgcn_readfirstlane(slot0);
-            if (cnt[r] > 1 && i != keep) {
-                int slot = slot0 + __popcll(has & ((1ull << lane) - 1ull));
-                if (slot < a.q_cap) {
-                    Item it;
-                    it.node = c.cb + i;
-                    it.off = off + excl[r];
-                    it.m = cnt[r];
-                    it.np = k.n[r];
-                    it.depth = depth + 1;
-                    it.pad[0] = it.pad[1] = it.pad[2] = 0;
-                    a.items_q[slot] = it;
-                    myslot[r] = slot;
-                } else {
-                    atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
-                }
+        if (cnt[r] > 1 && i != keep) {
+            int slot = slot0 + __popcll(has[r] & ((1ull << lane) - 1ull));
+            if (slot < a.q_cap) {
+                Item it;
+                it.node = c.cb + i;
+                it.off = off + excl[r];
+                it.m = cnt[r];
+                it.np = k.n[r];
+                it.depth = depth + 1;
+                it.pad[0] = it.pad[1] = it.pad[2] = 0;
+                a.items_q[slot] = it;
+                myslot[r] = slot;
+            } else {
+                atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
             }
         }
+        slot0 += __popcll(has[r]);
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
     }
     if (n_pushed > 0) {
