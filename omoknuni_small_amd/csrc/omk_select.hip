@@ -122,7 +122,7 @@ struct Kids {
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
 // so that it sits at the same place for every fan-out class.
-enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3 };
+enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3, kOpPartition = 4 };
 struct TeamCmd {
     int op;
     int rounds;  // R of the node's fan-out class: 1, or the kernel's RMAX
@@ -136,6 +136,20 @@ struct TeamCmd {
     int best, btk, bn, bvl;
     float bw, bp, bq2;
     uint32_t hk, hp, sk, spos;
+    // kOpPartition: the node whose visitors a helper shares out while the owner walks on
+    int j_cb, j_off, j_m, j_depth, j_keep, j_run_child;
+};
+
+// What that helper reads, at the same place for every fan-out class: the owner's next node
+// uses the scratch of its own class (WaveLds) meanwhile, and leaves this alone until the
+// helper is done.
+template <int RMAX>
+struct PartLds {
+    int offs[RMAX * kWave];  // start of every child's segment in the node's visitor list
+    int cnt[RMAX * kWave];   // visitors of every child
+    int np[RMAX * kWave];    // visit count of every child (its children's N_parent)
+    int lone[RMAX * kWave];  // rank of the child among those with one visitor
+    uint32_t order[kHeavyMin];  // (child, visit number) of every visitor in winner order (ordinary nodes only)
 };
 
 // Scratch in LDS of one block of the multi-visitor kernel (one node at a time).
@@ -394,6 +408,16 @@ __device__ __forceinline__ int predict_count(int n, float w, float p, int vl, fl
     return cnt >= (float)cap ? cap : (int)cnt;
 }
 
+// The owner may have left the partition of its previous node with a helper: the block
+// barrier that ends that request is still open.  Everything that needs the helpers, the
+// visitor lists that partition writes, or the LDS it reads, closes it first.
+__device__ __forceinline__ void close_pending(bool &pending) {
+    if (pending) {
+        __syncthreads();
+        pending = false;
+    }
+}
+
 template <int NT>
 __device__ __forceinline__ void team_sync() {
     if (NT == kWave) wave_sync_memory();
@@ -606,8 +630,8 @@ __device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, 
 // has after them, and checks the order of the whole batch, kept or not (what is dropped
 // must come after what is kept): red[2] bit 2 on failure.
 template <int R, int NT>
-__device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds, int tid, int total, int keep,
-                                           int goff, int cur) {
+__device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds, uint32_t *order, int tid, int total,
+                                           int keep, int goff, int cur) {
     constexpr int F = R * kWave;
     const uint32_t *skey = lds.key[cur], *spay = lds.pay2[cur];
     for (int i = tid; i < F; i += NT) lds.hist[i] = 0;
@@ -619,9 +643,11 @@ __device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds,
         const int child = (int)((pay >> 21) & 1023u);
         const int j = (int)(pay & 0x1FFFFFu);
         if (q < keep) {
-            if (goff >= 0) {  // else the caller reads the order from LDS
+            if (goff >= 0) {
                 a.sc_child[goff + q] = child;
                 a.sc_occ[goff + q] = j;
+            } else {  // the node's only batch: the partition reads the order from LDS
+                order[q] = pay;
             }
             atomicMax(&lds.hist[child], j + 1);
         }
@@ -693,7 +719,7 @@ template <int R, bool RAVE>
 __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
                                             int off, int rank0, int todo, const int (&tk0)[R], WaveLds<R> &lds,
                                             int (&cnt)[R], bool allow_lds, int &lds_cur, bool use_preset,
-                                            const int (&preset)[R]) {
+                                            const int (&preset)[R], uint32_t *order, bool &pending) {
     lds_cur = -1;
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
@@ -828,6 +854,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 if (!bad_run) {
                     if (lane == 0) lds.red[2] = 0u;
                     if (L >= 2 * kTeamMin) {
+                        close_pending(pending);
                         if (lane == 0) {
                             TeamCmd &cm = lds.cmd;
                             cm.op = kOpRun;
@@ -1094,6 +1121,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const bool team = total >= kTeamMin;
         int cur;
         if (team) {
+            close_pending(pending);
             if (lane == 0) {
                 lds.cmd.op = kOpOrder;
                 lds.cmd.rounds = R;
@@ -1127,6 +1155,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         // a node that this one batch settles keeps its winner order in LDS for the partition
         const bool only_batch = allow_lds && done == 0 && keep == m;
         if (team) {
+            close_pending(pending);
             if (lane == 0) {
                 lds.cmd.op = kOpEmit;
                 lds.cmd.rounds = R;
@@ -1136,12 +1165,13 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 lds.cmd.cur = cur;
             }
             __syncthreads();
-            batch_emit<R, kTeam>(a, lds, lane, total, keep, only_batch ? -1 : off + done, cur);
+            batch_emit<R, kTeam>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
             __syncthreads();
         } else {
-            batch_emit<R, kWave>(a, lds, lane, total, keep, only_batch ? -1 : off + done, cur);
+            if (only_batch) close_pending(pending);  // the previous node's partition may still read the order
+            batch_emit<R, kWave>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
         }
-        if (only_batch) lds_cur = cur;
+        if (only_batch) lds_cur = 0;
         bool bad = (lds.red[2] & 4u) != 0u;
         wave_sync_memory();
         {
@@ -1503,12 +1533,15 @@ struct Continuation {
 // wavefront that finishes last (a counter in the node's context) partitions the visitors
 // and walks on, every other returns kStepParked.  Any failed check sends the whole node
 // back to the one-wavefront path.
-template <int R, bool RAVE>
+template <int R, bool RAVE, int RMAX>
 __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                             const Item &item, const int32_t *seg_in, int32_t *seg_out,
-                                            WaveLds<R> &lds, Continuation &next) {
+                                            WaveLds<R> &lds, PartLds<RMAX> &pl, bool &pending, Continuation &next) {
     OMK_T0();
     const int off = item.off, m = item.m, depth = item.depth;
+    // a heavy node is settled and shared out by several wavefronts, which read its visitor
+    // list: it must be complete before any of them is called in
+    if (m >= kHeavyMin) close_pending(pending);
     Kids<R, RAVE> k;
     int cnt[R];
     load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
@@ -1626,7 +1659,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 #pragma unroll
                         for (int r = 0; r < R; r++) between[r] = ct_lo[r] - ct_hi[r];
                         ok = water_level<R, RAVE>(a, c, lane, k, off, rank_hi, todo, ct_hi, lds, cnt, false, unused_cur,
-                                                  !last, between);
+                                                  !last, between, pl.order, pending);
                     }
                 } else {
 #pragma unroll
@@ -1668,7 +1701,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         int zero[R];
 #pragma unroll
         for (int r = 0; r < R; r++) zero[r] = 0;
-        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt, m < kHeavyMin, lds_cur, false, zero);
+        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt, m < kHeavyMin, lds_cur, false, zero,
+                                       pl.order, pending);
         if (!settled) st_replay = 1;
     }
     if (!settled) {
@@ -1676,6 +1710,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         run_child = -1;
         lds_cur = -1;
         const bool seq_lds = m < kHeavyMin;  // few enough visitors to keep their order in LDS
+        if (seq_lds) close_pending(pending);  // the previous node's partition may still read that buffer
         for (int done = 0; done < m; done++) {
             int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
             if (i < 0) return kStepLeaf;  // no child takes part: uniform, and then for every visitor
@@ -1708,7 +1743,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 }
                 lane_best<R, RAVE>(k, lane, bk, bpos);
                 if (seq_lds) {
-                    lds.pay2[0][done] = ((uint32_t)i << 21) | (uint32_t)occ;
+                    pl.order[done] = ((uint32_t)i << 21) | (uint32_t)occ;
                 } else {
                     a.sc_child[off + done] = i;
                     a.sc_occ[off + done] = occ;
@@ -1728,6 +1763,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     }
 
     // ---- partition of the visitors by chosen child ----
+    // this node's visitor list is written by the previous node's partition
+    close_pending(pending);
     // (1) from the visits per child: the segment of every child, in LDS for all lanes
     uint32_t lmax = 0u;
 #pragma unroll
@@ -1743,6 +1780,51 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // where the walk goes on: ask for that node's child range now, it arrives during the scatter
     int2 keep_span = int2{0, 0};
     if (keep >= 0) keep_span = f.span[c.cb + keep];
+    // A node of ordinary size whose winner order is at hand: a helper wavefront of the block
+    // shares out the visitors and publishes the other children (partition_async), this one
+    // walks on into the kept child at once.  What the kept child needs of that work, its
+    // visitor list, it needs last (close_pending).
+    if (!as_scatter && !as_slice && m < kHeavyMin && (run_child >= 0 || lds_cur >= 0)) {
+        int carry = 0, ex_keep = 0, np_keep = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int inc = wave_inclusive_sum(cnt[r], lane);
+            const int ex = carry + inc - cnt[r];
+            const int i = r * kWave + lane;
+            pl.offs[i] = ex;
+            pl.cnt[i] = cnt[r];
+            pl.np[i] = k.n[r];
+            if (i == keep) {
+                ex_keep = ex;
+                np_keep = k.n[r];
+            }
+            carry += __builtin_amdgcn_readlane(inc, 63);
+        }
+        if (lane == 0) {
+            TeamCmd &cm = lds.cmd;
+            cm.op = kOpPartition;
+            cm.rounds = R;
+            cm.j_cb = c.cb;
+            cm.j_off = off;
+            cm.j_m = m;
+            cm.j_depth = depth;
+            cm.j_keep = keep;
+            cm.j_run_child = run_child;
+        }
+        __syncthreads();  // the request is open until close_pending
+        pending = true;
+        next.node = -1;
+        if (keep >= 0) {
+            next.node = c.cb + keep;
+            next.off = off + __builtin_amdgcn_readlane(ex_keep, keep & 63);
+            next.m = (int)gmax;
+            next.np = __builtin_amdgcn_readlane(np_keep, keep & 63);
+            next.span = keep_span;
+        }
+        OMK_TICK(14);
+        return kStepDescended;
+    }
+
     // the queue slots this node needs, asked for with one atomic per queue: a slot in the
     // single-visitor queue for every child with one visitor (in child order), a slot in the
     // work queue for every other child with visitors that this wavefront does not keep
@@ -1862,7 +1944,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 ii[u] = run_child;
                 oo[u] = j;
             } else if (lds_cur >= 0) {
-                const uint32_t pay = in ? lds.pay2[lds_cur][j] : 0u;
+                const uint32_t pay = in ? pl.order[j] : 0u;
                 ii[u] = (int)((pay >> 21) & 1023u);
                 oo[u] = (int)(pay & 0x1FFFFFu);
             } else {
@@ -1967,7 +2049,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 // A block is a team: its first wavefront (the owner) runs this loop, the other wavefronts
 // wait at a block barrier until the owner shares out the batch work of a node (team_help).
 template <int RMAX, bool RAVE>
-__device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs &a, WaveLds<RMAX> &s_lds, int lane) {
+__device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs &a, WaveLds<RMAX> &s_lds,
+                                           PartLds<RMAX> &s_part, bool &pending, int lane) {
     for (;;) {
         int ticket = 0;
         if (lane == 0) ticket = atomicAdd(a.sched_head, 1);
@@ -2021,10 +2104,11 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             next.node = -1;
             if (c.cc > 0 && depth < a.max_depth) {
                 if (c.cc <= kWave)
-                    status = select_group<1, RAVE>(f, a, c, lane, it, seg_in, seg_out,
-                                                   reinterpret_cast<WaveLds<1> &>(s_lds), next);
+                    status = select_group<1, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out,
+                                                         reinterpret_cast<WaveLds<1> &>(s_lds), s_part, pending, next);
                 else
-                    status = select_group<RMAX, RAVE>(f, a, c, lane, it, seg_in, seg_out, s_lds, next);
+                    status = select_group<RMAX, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out, s_lds, s_part, pending,
+                                                            next);
             }
 #ifdef OMK_TRACE
             if (lane == 0) {
@@ -2039,6 +2123,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
 #endif
             if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
             if (status == kStepLeaf) {
+                close_pending(pending);  // the visitor list comes from the previous node's partition
                 for (int j = lane; j < it.m; j += kWave) {
                     int t = seg_in[it.off + j];
                     a.leaf[t] = it.node;
@@ -2063,14 +2148,117 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
     }
 }
 
+// The partition of a settled node of ordinary size, by one helper wavefront, from what the
+// owner left in LDS (the request, PartLds): next path entry and place in the chosen child's
+// segment for every visitor, lone visitors to the single-visitor queue, virtual loss of the
+// chosen children, and the children with several visitors that the owner does not keep
+// become items of the work queue.
+template <int R, int RMAX>
+__device__ __forceinline__ void partition_async(const ForestDev &f, const SelectArgs &a, const TeamCmd &cm,
+                                                PartLds<RMAX> &pl, int lane) {
+    const int cb = __builtin_amdgcn_readfirstlane(cm.j_cb), off = __builtin_amdgcn_readfirstlane(cm.j_off);
+    const int m = __builtin_amdgcn_readfirstlane(cm.j_m), depth = __builtin_amdgcn_readfirstlane(cm.j_depth);
+    const int keep = __builtin_amdgcn_readfirstlane(cm.j_keep);
+    const int run_child = __builtin_amdgcn_readfirstlane(cm.j_run_child);
+    int cnt[R];
+    uint64_t has[R];
+    int n_lone = 0, n_push = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        cnt[r] = pl.cnt[i];
+        const uint64_t lm1 = __ballot(cnt[r] == 1);
+        pl.lone[i] = n_lone + __popcll(lm1 & ((1ull << lane) - 1ull));
+        n_lone += __popcll(lm1);
+        has[r] = __ballot(cnt[r] > 1 && i != keep);
+        n_push += __popcll(has[r]);
+    }
+    int lone0 = 0, slot0 = 0;
+    if (lane == 0) {
+        if (n_lone > 0) lone0 = atomicAdd(a.n_singles, n_lone);
+        if (n_push > 0) slot0 = atomicAdd(a.sched_tail, n_push);
+    }
+    wave_sync_memory();
+    lone0 = __builtin_amdgcn_readfirstlane(lone0);
+    const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
+    int32_t *seg_out = a.seg[depth & 1];
+    int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
+    for (int base = 0; base < m; base += kScatterUnroll * kWave) {
+        int tt[kScatterUnroll];
+        uint32_t pay[kScatterUnroll];
+#pragma unroll
+        for (int u = 0; u < kScatterUnroll; u++) {
+            const int j = base + u * kWave + lane;
+            const bool in = j < m;
+            tt[u] = in ? seg_in[off + j] : 0;
+            pay[u] = run_child >= 0 ? ((uint32_t)run_child << 21) | (uint32_t)j : (in ? pl.order[j] : 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < kScatterUnroll; u++) {
+            if (base + u * kWave + lane < m) {
+                const int t = tt[u], i = (int)((pay[u] >> 21) & 1023u), occ = (int)(pay[u] & 0x1FFFFFu);
+                path_next[t] = cb + i;
+                seg_out[off + pl.offs[i] + occ] = t;
+                if (pl.cnt[i] == 1) {
+                    Item it;
+                    it.node = cb + i;
+                    it.off = t;
+                    it.m = 1;
+                    it.np = pl.np[i];
+                    it.depth = depth + 1;
+                    it.pad[0] = it.pad[1] = it.pad[2] = 0;
+                    a.singles_q[lone0 + pl.lone[i]] = it;
+                }
+            }
+        }
+    }
+    slot0 = __builtin_amdgcn_readfirstlane(slot0);
+    int myslot[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        myslot[r] = -1;
+        if (cnt[r] > 1 && i != keep) {
+            const int slot = slot0 + __popcll(has[r] & ((1ull << lane) - 1ull));
+            if (slot < a.q_cap) {
+                Item it;
+                it.node = cb + i;
+                it.off = off + pl.offs[i];
+                it.m = cnt[r];
+                it.np = pl.np[i];
+                it.depth = depth + 1;
+                it.pad[0] = it.pad[1] = it.pad[2] = 0;
+                a.items_q[slot] = it;
+                myslot[r] = slot;
+            } else {
+                atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
+            }
+        }
+        slot0 += __popcll(has[r]);
+        if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
+    }
+    if (n_push > 0) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (myslot[r] >= 0)
+                __hip_atomic_store(a.q_ready + myslot[r], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);  // lone visitors leave the multi-visitor items
+}
+
 // What a helper wavefront does with one request of its owner.
-template <int R, bool RAVE>
-__device__ __forceinline__ void team_help(const SelectArgs &a, WaveLds<R> &lds, int tid, int op, int total, int keep,
-                                          int goff, int cur, float ep, uint32_t uvl) {
-    if (op == kOpOrder) {
+template <int R, bool RAVE, int RMAX>
+__device__ __forceinline__ void team_help(const ForestDev &f, const SelectArgs &a, WaveLds<R> &lds, PartLds<RMAX> &pl,
+                                          int tid, int op, int total, int keep, int goff, int cur, float ep,
+                                          uint32_t uvl) {
+    uint32_t *order = pl.order;
+    if (op == kOpPartition) {
+        if ((tid >> 6) == 1) partition_async<R, RMAX>(f, a, lds.cmd, pl, tid & 63);
+    } else if (op == kOpOrder) {
         batch_order<R, RAVE, kTeam>(lds, tid, total, ep, uvl);
     } else if (op == kOpEmit) {
-        batch_emit<R, kTeam>(a, lds, tid, total, keep, goff, cur);
+        batch_emit<R, kTeam>(a, lds, order, tid, total, keep, goff, cur);
     } else if (op == kOpRun) {
         const TeamCmd &cm = lds.cmd;
         const int best = __builtin_amdgcn_readfirstlane(cm.best), btk = __builtin_amdgcn_readfirstlane(cm.btk);
@@ -2089,10 +2277,13 @@ __device__ __forceinline__ void team_help(const SelectArgs &a, WaveLds<R> &lds, 
 template <int RMAX, bool RAVE>
 __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs a) {
     __shared__ WaveLds<RMAX> s_lds;
+    __shared__ PartLds<RMAX> s_part;
     const int tid = threadIdx.x;
     if (tid < kWave) {
         // every path out of the owner's loop comes back here: the helpers are always released
-        owner_loop<RMAX, RAVE>(f, a, s_lds, tid);
+        bool pending = false;
+        owner_loop<RMAX, RAVE>(f, a, s_lds, s_part, pending, tid);
+        close_pending(pending);
         if (tid == 0) s_lds.cmd.op = kOpExit;
         __syncthreads();
         return;
@@ -2109,9 +2300,10 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
         if (rounds == 1)
-            team_help<1, RAVE>(a, reinterpret_cast<WaveLds<1> &>(s_lds), tid, op, total, keep, goff, cur, ep, uvl);
+            team_help<1, RAVE, RMAX>(f, a, reinterpret_cast<WaveLds<1> &>(s_lds), s_part, tid, op, total, keep, goff, cur,
+                                     ep, uvl);
         else
-            team_help<RMAX, RAVE>(a, s_lds, tid, op, total, keep, goff, cur, ep, uvl);
+            team_help<RMAX, RAVE, RMAX>(f, a, s_lds, s_part, tid, op, total, keep, goff, cur, ep, uvl);
         __syncthreads();  // the request is done
     }
 }
