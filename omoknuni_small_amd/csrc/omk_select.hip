@@ -750,6 +750,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
     OMK_T0();
     for (int done = 0; done < m;) {
         const int remaining = m - done;
+#ifdef OMK_TRACE
+        if (lane == 0) lds.red[3] += 1u;  // batches and runs of this node, for the timeline
+#endif
 
         // ---- 1. threshold and exact per-child counts ----
         uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
@@ -886,6 +889,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     }
                     bad_run = (lds.red[2] & 4u) != 0u;
                 }
+#ifdef OMK_TRACE
+                if (!bad_run && lane == 0) lds.red[3] += 0x100u;  // runs emitted without sorting
+#endif
                 if (!bad_run) {
                     if (lane == bl) {
 #pragma unroll
@@ -1100,6 +1106,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (ac[r] >= 0) lds.pay[ac[r]] = (uint32_t)ct[r];
         wave_sync_memory();
         }  // !preset_done
+#ifdef OMK_TRACE
+        if (lane == 0) lds.red[3] = (lds.red[3] & 0xFFFFu) | ((uint32_t)total << 16);  // entries of the last batch
+#endif
         int nb[R];  // entries of every own child in this batch
 #pragma unroll
         for (int r = 0; r < R; r++) nb[r] = (int)lds.pay[r * kWave + lane];
@@ -1544,14 +1553,28 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     if (m >= kHeavyMin) close_pending(pending);
     Kids<R, RAVE> k;
     int cnt[R];
-    load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
+    uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
+    if (item.pad[0] == 2) {
+        // a part of a heavy node's partition: of the children only the visit counts are needed
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        score_round<R, RAVE>(k, r, c.ep);
-        cnt[r] = 0;
+        for (int r = 0; r < R; r++) {
+            const int i = r * kWave + lane;
+            k.n[r] = i < c.nelig ? f.N[c.cb + i] : 0;
+            k.w[r] = k.p[r] = k.q2[r] = 0.0f;
+            k.vl[r] = 0;
+            k.k1[r] = k.k2[r] = 0u;
+            k.part[r] = false;
+            cnt[r] = 0;
+        }
+    } else {
+        load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            score_round<R, RAVE>(k, r, c.ep);
+            cnt[r] = 0;
+        }
+        lane_best<R, RAVE>(k, lane, bk, bpos);
     }
-    uint32_t bk, bpos;
-    lane_best<R, RAVE>(k, lane, bk, bpos);
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
     OMK_TICK(12);
 
@@ -2097,6 +2120,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             int32_t *seg_out = a.seg[depth & 1];
 #ifdef OMK_TRACE
             const long long tr0 = wall_clock64();
+            if (lane == 0) s_lds.red[3] = 0u;
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
             int status = kStepLeaf;
@@ -2117,7 +2141,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                     a.trace[4 * ti + 0] = tr0;
                     a.trace[4 * ti + 1] = wall_clock64();
                     a.trace[4 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
-                    a.trace[4 * ti + 3] = it.node;
+                    a.trace[4 * ti + 3] = (long long)it.node | ((long long)s_lds.red[3] << 32);
                 }
             }
 #endif

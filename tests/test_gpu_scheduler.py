@@ -176,3 +176,46 @@ def test_two_selections_in_a_row_accumulate_virtual_loss():
     b2.revert_vl(3)
     b1.revert_vl(3)
     assert (f.download()["VL"] == 0).all()
+
+
+def chain_forest(seed, depth, fan, dominate):
+    """A spine of `depth` nodes: every spine node has `fan` children, one of which (the next
+    spine node) carries most of the prior when `dominate`; the other children are leaves or
+    have one level of children of their own."""
+    rng = np.random.default_rng(seed)
+    N, W, P, cb, cc, act = [1000], [0.0], [0.0], [0], [0], [-1]
+    spine = 0
+    for d in range(depth):
+        first = len(N)
+        cb[spine], cc[spine] = first, fan
+        nxt = int(rng.integers(fan))
+        pr = rng.dirichlet(np.ones(fan)).astype(np.float32)
+        if dominate:
+            pr = (pr * 0.05).astype(np.float32)
+            pr[nxt] = np.float32(0.95)
+        for i in range(fan):
+            n = int(rng.integers(0, 30))
+            N.append(n); W.append(float(np.float32(rng.uniform(-n, n)))); P.append(float(pr[i]))
+            cb.append(0); cc.append(0); act.append(i)
+        # some siblings get children too, so that visitors pushed off the spine walk on
+        for i in range(fan):
+            if i != nxt and rng.random() < 0.3:
+                c = first + i
+                cb[c], cc[c] = len(N), 3
+                for j in range(3):
+                    N.append(int(rng.integers(0, 5))); W.append(0.0); P.append(1.0 / 3); cb.append(0); cc.append(0); act.append(j)
+        N[spine] = max(N[spine], sum(N[first:first + fan]) + 1)
+        spine = first + nxt
+    soa = dict(N=np.array(N, np.int32), W=np.array(W, np.float32), P=np.array(P, np.float32),
+               VL=np.zeros(len(N), np.int32), child_begin=np.array(cb, np.int32), child_count=np.array(cc, np.int32),
+               action=np.array(act, np.int32))
+    return soa
+
+
+@pytest.mark.parametrize("dominate,fan,B", [(True, 5, 700), (True, 70, 900), (False, 9, 1000), (True, 5, 30)])
+def test_long_chains_of_crowded_nodes(dominate, fan, B):
+    # level after level the owner wavefront walks on into the kept child while a helper shares
+    # out the visitors of the node before; the spine ends in a leaf right after such a hand-over
+    soa = chain_forest(11, 40, fan, dominate)
+    st = select_both(soa, np.zeros(B, np.int32), 50, steps=3)
+    assert st["replayed_nodes"] == 0, st
