@@ -61,8 +61,8 @@ constexpr int kSortBins = 1 << kSortBits;
 constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-visitor kernel: one owner that
                                           // takes the items, three helpers for the batch work of its node
 constexpr int kTeam = kTeamWaves * 64;
-constexpr int kTeamMin = 192;             // batch entries from which the helpers are called in
-constexpr int kSliceEntries = 512;        // visitors per slice of such a node, about
+constexpr int kTeamMin = 96;              // batch entries from which the helpers are called in
+constexpr int kSliceEntries = 256;        // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
