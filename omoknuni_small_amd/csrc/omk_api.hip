@@ -107,6 +107,7 @@ struct omk_batch {
     bool stats_on = false;
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
     int32_t *hctx = nullptr;     // contexts of heavy nodes
+    int32_t *list_flag = nullptr;  // per visitor-list start: which depth's list is complete
     int32_t hctx_cap = 0;
     int32_t q_cap = 0;
     int32_t epoch = 0;           // select calls so far
@@ -579,6 +580,7 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     b->q_cap = (int32_t)((B / 2 + B / 16 + 64) * (max_depth + 1));
     b->hctx_cap = (int32_t)std::min<int64_t>(4096, (B / kHeavyMin) * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->hctx, (int64_t)b->hctx_cap * kHeavyCtxInts);
+    if (e == hipSuccess) e = dalloc(&b->list_flag, B);
     if (e == hipSuccess) e = dalloc(&b->items_q, b->q_cap);
     if (e == hipSuccess) e = dalloc(&b->q_ready, b->q_cap);
     if (e == hipSuccess) e = hipMemset(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4);
@@ -587,8 +589,8 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg0, B);
     if (e == hipSuccess) e = dalloc(&b->seg[0], B);
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
-    if (e == hipSuccess) e = dalloc(&b->sc_child, B);
-    if (e == hipSuccess) e = dalloc(&b->sc_occ, B);
+    if (e == hipSuccess) e = dalloc(&b->sc_child, 2 * B);  // two halves, alternating with the depth
+    if (e == hipSuccess) e = dalloc(&b->sc_occ, 2 * B);
     if (e == hipSuccess) e = dalloc(&b->counters, 4 * kSchedStep);
     if (e == hipSuccess) e = hipMemset(b->counters, 0, 4 * kSchedStep * 4);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&b->n_cus, hipDeviceAttributeMultiprocessorCount, f->device);
@@ -610,7 +612,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf};
+                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf, b->list_flag};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -725,6 +727,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.hctx = b->hctx;
     a.hctx_n = b->counters + 2 * kSchedStep + 64;
     a.hctx_cap = b->hctx_cap;
+    a.list_flag = b->list_flag;
     static_assert(kHeavyCtxInts >= 16 + OMK_MAX_FANOUT, "context too small");
 #if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
     a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
@@ -927,14 +930,25 @@ int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t 
     if (h_actions) HIP_TRY(hipMemcpyAsync(h_actions, b->out_actions, (size_t)n * D * 4, hipMemcpyDeviceToHost, s));
     if (h_path_len) HIP_TRY(hipMemcpyAsync(h_path_len, b->path_len, (size_t)n * 4, hipMemcpyDeviceToHost, s));
     if (h_leaf) HIP_TRY(hipMemcpyAsync(h_leaf, b->leaf, (size_t)n * 4, hipMemcpyDeviceToHost, s));
-    int32_t aborted = 0;
-    HIP_TRY(hipMemcpyAsync(&aborted, b->counters + 3 * kSchedStep + 1, 4, hipMemcpyDeviceToHost, s));
+    int32_t ab[4] = {0, 0, 0, 0};  // abort flag and what the wavefront that raised it was waiting for
+    HIP_TRY(hipMemcpyAsync(ab, b->counters + 3 * kSchedStep + 1, sizeof(ab), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
-    if (aborted)
+    if (ab[0] == 1)
         return fail(OMK_ERR_STATE,
-                    "omk_batch_read: the selection gave up (%s); its paths are incomplete, revert the virtual "
+                    "omk_batch_read: the selection gave up (a wavefront waited longer than the spin limit for item %d "
+                    "of the work queue, %d handed out, %d visitors open); its paths are incomplete, revert the virtual "
                     "losses with omk_forest_upload or omk_revert_vl_paths over known paths",
-                    aborted == 1 ? "a wavefront waited longer than the spin limit" : "work queue overflow");
+                    ab[1], ab[2], ab[3]);
+    if (ab[0] == 3)
+        return fail(OMK_ERR_STATE,
+                    "omk_batch_read: the selection gave up (a wavefront waited longer than the spin limit for the "
+                    "visitor list at %d of depth %d, complete to depth %d); its paths are incomplete, revert the "
+                    "virtual losses with omk_forest_upload or omk_revert_vl_paths over known paths",
+                    ab[1], ab[2], ab[3]);
+    if (ab[0])
+        return fail(OMK_ERR_STATE,
+                    "omk_batch_read: the selection gave up (work queue overflow); its paths are incomplete, revert "
+                    "the virtual losses with omk_forest_upload or omk_revert_vl_paths over known paths");
     return OMK_OK;
 }
 

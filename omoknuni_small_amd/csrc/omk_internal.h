@@ -54,6 +54,8 @@ struct SelectArgs {
     int32_t *hctx;         // contexts of heavy nodes, kHeavyCtxInts each: [0] slices still running,
                            // [1] a slice failed a check, [16 + i] visits of child i
     int32_t *hctx_n;       // contexts handed out
+    int32_t *list_flag;    // per visitor-list start: depth of the deepest item whose list, starting there,
+                           // is complete (items of kind 3 are published before their list is written)
     int32_t hctx_cap;
     int32_t poll_sleep;    // s_sleep(32) units between two polls of a waiting wavefront
     int32_t q_cap;
@@ -66,7 +68,7 @@ struct SelectArgs {
 #endif
     int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
-    int32_t *sc_child;     // per visitor: chosen child index
+    int32_t *sc_child;     // per visitor: chosen child index (two halves of `stride`, alternating with the depth)
     int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child
     int32_t *paths;        // level-major [max_depth+1][stride]
     int32_t *path_len;

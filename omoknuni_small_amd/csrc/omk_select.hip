@@ -418,6 +418,39 @@ __device__ __forceinline__ void close_pending(bool &pending) {
     }
 }
 
+// An item of kind 3 was published before its visitor list was written (the children of a
+// heavy node, whose visitors several wavefronts share out): wait for the list.  Bounded like
+// every wait; false when the selection is given up.
+__device__ __forceinline__ bool wait_list(const SelectArgs &a, int off, int depth, int lane) {
+    bool ok = false;
+    for (int spins = 0;; spins++) {
+        int v = 0, ab = 0;
+        if (lane == 0) {
+            v = __hip_atomic_load(a.list_flag + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v < depth && (spins & 3) == 3)
+                ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        v = __builtin_amdgcn_readfirstlane(v);
+        ab = __builtin_amdgcn_readfirstlane(ab);
+        if (v >= depth) {
+            ok = true;
+            break;
+        }
+        if (ab) break;
+        if (spins >= a.spin_limit) {
+            if (lane == 0 && atomicCAS(a.sched_wait + 1, 0, 3) == 0) {
+                a.sched_wait[2] = off;  // which list never came, for the error message
+                a.sched_wait[3] = depth;
+                a.sched_wait[4] = v;
+            }
+            break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return ok;
+}
+
 template <int NT>
 __device__ __forceinline__ void team_sync() {
     if (NT == kWave) wave_sync_memory();
@@ -1550,6 +1583,13 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     const int off = item.off, m = item.m, depth = item.depth;
     // a heavy node is settled and shared out by several wavefronts, which read its visitor
     // list: it must be complete before any of them is called in
+    // where this node's winner order goes in sc_child / sc_occ when it does not fit LDS: the
+    // two halves alternate with the depth, because the children of a heavy node are at work
+    // while wavefronts still read the order of their parent
+    const int soff = off + (depth & 1) * a.stride;
+    // the visitor list of an item of kind 3, and of the slices of one, may not be there yet:
+    // whoever shares out the visitors waits for it (below), settling them does not need it
+    bool list_ok = !(item.pad[0] == 3 || (item.pad[0] == 1 && ((item.pad[2] >> 30) & 1)));
     if (m >= kHeavyMin) close_pending(pending);
     Kids<R, RAVE> k;
     int cnt[R];
@@ -1586,7 +1626,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     int run_child = -1, lds_cur = -1;
     bool as_slice = item.pad[0] == 1;
     const bool as_scatter = item.pad[0] == 2;
-    int hid = item.pad[0] != 0 ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF, n_slices = item.pad[2] >> 16;
+    int hid = as_slice || as_scatter ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF, n_slices = (item.pad[2] >> 16) & 0x3FFF;
     if (as_scatter) {
         // a part of the partition of a heavy node: the visits per child are in its context
         const int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
@@ -1595,7 +1635,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         settled = true;
     }
     if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
-        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, off, m, m >= kHeavyMin, cnt, run_child);
+        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kHeavyMin, cnt, run_child);
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
@@ -1618,7 +1658,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         Item it = item;
                         it.pad[0] = 1;
                         it.pad[1] = id;
-                        it.pad[2] = (lane + 1) | (K << 16);
+                        it.pad[2] = (lane + 1) | (K << 16) | (list_ok ? 0 : 1 << 30);
                         a.items_q[slot0 + lane] = it;
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -1681,7 +1721,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         int between[R];  // entries of every child between the two thresholds
 #pragma unroll
                         for (int r = 0; r < R; r++) between[r] = ct_lo[r] - ct_hi[r];
-                        ok = water_level<R, RAVE>(a, c, lane, k, off, rank_hi, todo, ct_hi, lds, cnt, false, unused_cur,
+                        ok = water_level<R, RAVE>(a, c, lane, k, soff, rank_hi, todo, ct_hi, lds, cnt, false, unused_cur,
                                                   !last, between, pl.order, pending);
                     }
                 } else {
@@ -1724,7 +1764,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         int zero[R];
 #pragma unroll
         for (int r = 0; r < R; r++) zero[r] = 0;
-        settled = water_level<R, RAVE>(a, c, lane, k, off, 0, m, zero, lds, cnt, m < kHeavyMin, lds_cur, false, zero,
+        settled = water_level<R, RAVE>(a, c, lane, k, soff, 0, m, zero, lds, cnt, m < kHeavyMin, lds_cur, false, zero,
                                        pl.order, pending);
         if (!settled) st_replay = 1;
     }
@@ -1741,8 +1781,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 // no virtual loss: nothing changes between visitors, they all follow the first
                 if (!seq_lds) {
                     for (int j = lane; j < m; j += kWave) {
-                        a.sc_child[off + j] = i;
-                        a.sc_occ[off + j] = j;
+                        a.sc_child[soff + j] = i;
+                        a.sc_occ[soff + j] = j;
                     }
                 }
                 if (lane == (i & 63)) {
@@ -1768,8 +1808,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 if (seq_lds) {
                     pl.order[done] = ((uint32_t)i << 21) | (uint32_t)occ;
                 } else {
-                    a.sc_child[off + done] = i;
-                    a.sc_occ[off + done] = occ;
+                    a.sc_child[soff + done] = i;
+                    a.sc_occ[soff + done] = occ;
                 }
             }
         }
@@ -1788,6 +1828,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // ---- partition of the visitors by chosen child ----
     // this node's visitor list is written by the previous node's partition
     close_pending(pending);
+    if (!list_ok) {
+        if (!wait_list(a, off, depth, lane)) return kStepParked;
+        list_ok = true;
+    }
     // (1) from the visits per child: the segment of every child, in LDS for all lanes
     uint32_t lmax = 0u;
 #pragma unroll
@@ -1909,11 +1953,23 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             }
             const int K2 = (m + kScatterPart - 1) / kScatterPart < kMaxSlices ? (m + kScatterPart - 1) / kScatterPart
                                                                              : kMaxSlices;
+            // The children with several visitors are published together with the parts, before
+            // their lists exist (kind 3: they wait for list_flag where they need the list; the
+            // parts sit before them in the queue, so whatever a waiting child depends on has
+            // been taken by a wavefront that does not wait).  None is kept: the wavefront that
+            // finishes the scatter is any of those that took a part.
+            uint64_t kids[R];
+            int n_kids = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                kids[r] = __ballot(cnt[r] > 1);
+                n_kids += __popcll(kids[r]);
+            }
             if (hid >= 0) {
                 int slot0 = 0;
-                if (lane == 0) slot0 = atomicAdd(a.sched_tail, K2 - 1);
+                if (lane == 0) slot0 = atomicAdd(a.sched_tail, K2 - 1 + n_kids);
                 slot0 = __builtin_amdgcn_readfirstlane(slot0);
-                if (slot0 + K2 - 1 <= a.q_cap) {
+                if (slot0 + K2 - 1 + n_kids <= a.q_cap) {
                     int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
 #pragma unroll
                     for (int r = 0; r < R; r++) ctx[16 + r * kWave + lane] = cnt[r];
@@ -1931,10 +1987,37 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         it.pad[2] = (lane + 1) | (K2 << 16);
                         a.items_q[slot0 + lane] = it;
                     }
+                    int kslot[R];
+                    int kbase = slot0 + K2 - 1;
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int i = r * kWave + lane;
+                        kslot[r] = -1;
+                        if (cnt[r] > 1) {
+                            Item it;
+                            it.node = c.cb + i;
+                            it.off = off + excl[r];
+                            it.m = cnt[r];
+                            it.np = k.n[r];
+                            it.depth = depth + 1;
+                            it.pad[0] = 3;
+                            it.pad[1] = it.pad[2] = 0;
+                            kslot[r] = kbase + __popcll(kids[r] & ((1ull << lane) - 1ull));
+                            a.items_q[kslot[r]] = it;
+                        }
+                        kbase += __popcll(kids[r]);
+                        if (cnt[r] > 0 && a.vl > 0)
+                            atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
+                    }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
                     if (lane < K2 - 1)
                         __hip_atomic_store(a.q_ready + slot0 + lane, a.epoch, __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                        if (kslot[r] >= 0)
+                            __hip_atomic_store(a.q_ready + kslot[r], a.epoch, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
                     n_parts = K2;
                     shared = true;
                 } else if (lane == 0) {
@@ -1971,8 +2054,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 ii[u] = (int)((pay >> 21) & 1023u);
                 oo[u] = (int)(pay & 0x1FFFFFu);
             } else {
-                ii[u] = in ? a.sc_child[off + j] : 0;
-                oo[u] = in ? a.sc_occ[off + j] : 0;
+                ii[u] = in ? a.sc_child[soff + j] : 0;
+                oo[u] = in ? a.sc_occ[soff + j] : 0;
             }
         }
 #pragma unroll
@@ -2005,6 +2088,18 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         before = __builtin_amdgcn_readfirstlane(before);
         if (before != 1) return kStepParked;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // every part is written, and the children are in the queue already: tell them that
+        // their lists are complete
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (cnt[r] > 1)
+                __hip_atomic_store(a.list_flag + off + excl[r], depth + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);
+        next.node = -1;
+        wave_sync_memory();
+        OMK_TICK(14);
+        return kStepDescended;
     }
 
     // (3) virtual loss of the chosen children, and the parts with several visitors that this
@@ -2013,8 +2108,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     int myslot[R];
     const int n_pushed = n_push;
     if (n_push > 0) {
-        // a shared scatter: the wavefront that finishes it asks for the slots
-        if (shared && lane == 0) slot0 = atomicAdd(a.sched_tail, n_push);
         slot0 = __builtin_amdgcn_readfirstlane(slot0);
     }
 #pragma unroll
@@ -2098,7 +2191,11 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             }
             if (open <= 0 || ab) break;
             if (spins >= a.spin_limit) {
-                if (lane == 0) atomicExch(a.sched_wait + 1, 1);
+                if (lane == 0 && atomicCAS(a.sched_wait + 1, 0, 1) == 0) {
+                    a.sched_wait[2] = ticket;  // which item never came, for the error message
+                    a.sched_wait[3] = *a.sched_tail;
+                    a.sched_wait[4] = open;
+                }
                 break;
             }
             for (int z = 0; z < a.poll_sleep; z++) __builtin_amdgcn_s_sleep(32);
@@ -2148,6 +2245,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
             if (status == kStepLeaf) {
                 close_pending(pending);  // the visitor list comes from the previous node's partition
+                if (it.pad[0] == 3 && !wait_list(a, it.off, depth, lane)) break;
                 for (int j = lane; j < it.m; j += kWave) {
                     int t = seg_in[it.off + j];
                     a.leaf[t] = it.node;
@@ -2402,6 +2500,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
     for (int i = gid; i < n_traversals; i += step) {
         a.path_len[i] = 0;
         a.leaf[i] = -1;
+        a.list_flag[i] = 0;
     }
 }
 
