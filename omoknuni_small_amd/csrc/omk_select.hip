@@ -781,8 +781,15 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
     }
 
     OMK_T0();
+    // Set when the threshold search finds the unsettled entries piled up on ONE key in several
+    // children and nothing above it (children exactly tied on a plateau): among equal keys the
+    // lowest position wins for as long as its key stays there, so the next winners are a run of
+    // the best child however short, and the next round takes it.
+    bool force_run = false;
     for (int done = 0; done < m;) {
         const int remaining = m - done;
+        const int run_min = force_run ? 1 : kRunShortcutMin;
+        force_run = false;
 #ifdef OMK_TRACE
         if (lane == 0) lds.red[3] += 1u;  // batches and runs of this node, for the timeline
 #endif
@@ -827,7 +834,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         // When the best child's next entries stay ahead of every other child's next entry (its
         // score hardly moves with virtual loss, e.g. a RAVE blend that dominates), they are the
         // next winners one after another: count them, check them, emit them without sorting.
-        if (remaining >= kRunShortcutMin) {
+        if (remaining >= run_min) {
             uint32_t ok2 = 0u, opos2 = 0xFFFFFFFFu;
 #pragma unroll
             for (int r = 0; r < R; r++)
@@ -859,12 +866,12 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             const int btk = __builtin_amdgcn_readlane(ttk, bl);
             // probe: does the run reach kRunShortcutMin entries at all?
             uint32_t pk_, pp_;
-            entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + kRunShortcutMin - 1, best, pk_, pp_);
+            entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + run_min - 1, best, pk_, pp_);
             if (pk_ != 0u && (sk == 0u || comes_before(pk_, pp_, sk, spos))) {
                 // largest L <= remaining whose last entry still comes before the others' best
                 // (64 candidate lengths at a time, one per lane; the entries are checked one by
                 // one below, so this search only has to propose)
-                int lo_l = kRunShortcutMin, hi_l = remaining;
+                int lo_l = run_min, hi_l = remaining;
                 while (lo_l < hi_l) {
                     const int step = (hi_l - lo_l + kWave - 1) / kWave;
                     const int cand = lo_l + (lane + 1) * step;
@@ -940,6 +947,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 }
             }
         }
+        if (run_min == 1) OMK_FAIL(11);  // the run that had to be there was refused
         const int want = remaining < kBatchCap ? remaining : kBatchCap;
         // lower bound of any useful threshold: the best child alone has `want` entries at or
         // above the key of its want-th next visit
@@ -1011,14 +1019,18 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         int tries = 0;
         uint32_t T_forced = 0u;  // threshold imposed for the next round instead of searching one
         bool allow_above = true;
+        bool several_flood = false;  // no single child accounts for the excess at the flooded key
         for (;;) {
             if (++tries > 8) OMK_FAIL(5);
             const uint32_t T_now = T_forced;  // imposed for this round only
             T_forced = 0u;
-            // bisection on the score with the estimated counts only (no exact evaluation)
-            float flo = key_score(lo_key), fhi = key_score(hi_key);
-            for (int it = 0; it < 22 && T_now == 0u; it++) {
-                const float mid = 0.5f * (flo + fhi);
+            // bisection on the KEY (not the score: entries may crowd into a sliver of the score
+            // range that halving a wide score interval never resolves) with the estimated counts
+            // only, no exact evaluation
+            uint32_t klo = lo_key, khi = hi_key;
+            for (int it = 0; it < 32 && T_now == 0u && khi - klo > 1u; it++) {
+                const uint32_t kmid = klo + ((khi - klo) >> 1);
+                const float mid = key_score(kmid);
                 int est = 0;
 #pragma unroll
                 for (int r = 0; r < R; r++)
@@ -1026,18 +1038,18 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                         est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, child_cap);
                 const int e = wave_sum_i32(est);
                 if (e >= target) {
-                    flo = mid;
+                    klo = kmid;
                     // close enough: a quarter more entries than aimed at cost less than more steps
                     if (e <= target + (target >> 2) && e <= kBatchCap - margin) break;
                 } else {
-                    fhi = mid;
+                    khi = kmid;
                     if (!can_finish && e >= target - (target >> 2)) {
-                        flo = mid;  // a batch that cannot finish anyway may as well be a little smaller
+                        klo = kmid;  // a batch that cannot finish anyway may as well be a little smaller
                         break;
                     }
                 }
             }
-            uint32_t T = T_now != 0u ? T_now : score_key(flo);
+            uint32_t T = T_now != 0u ? T_now : klo;
             if (T < lo_key) T = lo_key;
             if (T > hi_key) T = hi_key;
             const float tau = key_score(T);
@@ -1105,10 +1117,17 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 // One child floods the batch with entries AT the threshold (a score that hardly
                 // moves with virtual loss).  Take the entries strictly above it first, a small
                 // batch; the run of that child is then emitted without sorting.
-                if ((int)gmx > excess && allow_above && T < hi_key) {
+                if (allow_above && T < hi_key && ((int)gmx > excess || tries >= 3)) {
+                    // (after a few rounds of aiming higher in vain the key is taken to be flooded by
+                    // several children at once)
+                    several_flood = (int)gmx <= excess;
                     allow_above = false;
                     T_forced = T + 1u;
                     continue;
+                }
+                if ((int)gmx <= excess && T >= hi_key && tries >= 3) {
+                    force_run = true;  // several children exactly tied at the very top
+                    break;
                 }
                 if ((int)gmx <= excess) {
                     target -= excess + margin;  // no single child absorbs it: aim higher instead
@@ -1122,8 +1141,13 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 total = kBatchCap;
             }
             if (T_now != 0u) {
-                if (total < 1) continue;  // nothing above: back to the flooded threshold, capped
-                break;                    // may not finish the node: the run comes next
+                if (total < 1) {
+                    // nothing above the flooded key: if it is flooded by one child, back to it, capped;
+                    // if by several, exactly tied, the best of them runs first
+                    if (several_flood) force_run = true;
+                    else continue;
+                }
+                break;  // may not finish the node: the run comes next
             }
             if (can_finish && total < remaining) {
                 target += (remaining - total) + margin;  // not enough to finish: aim lower
@@ -1133,6 +1157,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (total < 1) OMK_FAIL(7);
             break;
         }
+        if (force_run) continue;
         // hand the counts back to the lanes that own the children
 #pragma unroll
         for (int r = 0; r < R; r++)
