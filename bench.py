@@ -14,9 +14,11 @@ traversal is selected AND backed up inside the timed region).  `roofline` prices
 selection kernel against HBM bandwidth with algorithmic bytes (what one selection step
 has to read: the statistics of the children that take part, the node header, the legal
 mask bits, the virtual-loss update), measured with HIP events on the stream the kernels
-run on.  `cpu_baseline` times the CPU checker (a restatement of the reference's serial
-selection / backup loops) on the host cores of the same machine, on a bounded number of
-steps of the same workload.
+run on.  `cpu_baseline` times the CPU checker on the host cores of the same machine, on a
+bounded number of steps of the same workload: the serial array restatement of the
+reference's selection / backup loops (one core) and the same arithmetic over the
+reference's own node layout (heap nodes, one cache line per atomic field) with its OpenMP
+loops, at one thread and at the host's share of cores; `value` is the fastest of them.
 """
 import argparse
 import ctypes as C
@@ -289,17 +291,56 @@ def main():
             done += 1
             if done >= K + args.warmup:
                 break
+        soa_rate = B * done / (sel_s + bak_s)
         out["cpu_baseline"] = {
-            "value": B * done / (sel_s + bak_s),
+            "value": soa_rate,
             "unit": "traversals/s",
             "cores": 1,
             "kind": "port",
             "sample": "%d steps of the same workload (same forest, roots and leaf values) through the "
                       "serial CPU restatement of selectChild / applyVirtualLoss / update / revertVirtualLoss" % done,
-            "select_traversals_per_s": B * done / sel_s,
-            "backups_per_s": B * done / bak_s,
+            "soa_serial_select_traversals_per_s": B * done / sel_s,
+            "soa_serial_backups_per_s": B * done / bak_s,
             "host_cores_visible": os.cpu_count(),
         }
+        # The same arithmetic over the reference's own layout and threading: heap nodes with one
+        # cache line per atomic field, shared_ptr child vectors, OpenMP loops with
+        # schedule(dynamic, 1).  Timed with one thread and with the host's share of cores; the
+        # faster of the three figures becomes `value` (with several threads the traversal
+        # order, hence the result, depends on the schedule, as the reference's does).
+        if len(soa["N"]) <= 20_000_000:
+            from oracle import ref_ptr as RP
+            t_build = time.perf_counter()
+            pt = RP.PtrTree(soa)
+            t_build = time.perf_counter() - t_build
+            n_thr = max(1, min(16, os.cpu_count() or 1))
+            kw = dict(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                      rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+            rates = {}
+            for thr in sorted({1, n_thr}):
+                tot, steps_done = 0.0, 0
+                t_start = time.perf_counter()
+                while steps_done < 2 or (time.perf_counter() - t_start) < args.cpu_seconds / 2:
+                    _, _, s_s, b_s = pt.step(troots, values, threads=thr, **kw)
+                    tot += s_s + b_s
+                    steps_done += 1
+                    if steps_done >= K + args.warmup:
+                        break
+                rates[thr] = B * steps_done / tot
+            pt.close()
+            cb = out["cpu_baseline"]
+            cb["soa_serial_traversals_per_s"] = soa_rate
+            cb["pointer_tree_traversals_per_s"] = {str(k): v for k, v in rates.items()}
+            cb["pointer_tree_node_bytes"] = RP.PtrTree.node_bytes()
+            cb["pointer_tree_build_s"] = t_build
+            best_thr = max(rates, key=rates.get)
+            if rates[best_thr] > soa_rate:
+                cb["value"] = rates[best_thr]
+                cb["cores"] = best_thr
+                cb["sample"] = ("steps of the same workload (same forest, roots and leaf values) through the CPU "
+                                "restatement over the reference's node layout (heap nodes, one cache line per "
+                                "atomic) and OpenMP loops, %d thread(s); the serial array checker and the "
+                                "one-thread figure are given beside it" % best_thr)
         del rtt
     print(json.dumps(out))
 
