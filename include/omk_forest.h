@@ -151,6 +151,16 @@ int omk_revert_vl_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_
 int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_path_len,
                      const float *d_values, int32_t n, int32_t stride, int32_t max_len, int32_t virtual_loss);
 
+/* Dirichlet noise on the priors of `root`'s children (MCTSEngine::addDirichletNoise,
+ * src/mcts/mcts_engine_eval.cpp:78-110): the caller draws one gamma(alpha, 1) sample per
+ * child with its own generator, as the reference does with std::gamma_distribution on the
+ * engine's random engine (:83-90); the library normalises them (their float sum in order;
+ * uniform 1/children when it is not positive) and sets
+ * prior = (1 - epsilon) * prior + epsilon * noise, child by child in the reference's
+ * order.  n_gamma must be the number of children (legal slots).  A root without children
+ * is left alone.  Waits for the stream; the arithmetic is done on the host. */
+int omk_forest_add_root_noise(omk_forest *f, int32_t root, const float *h_gamma, int32_t n_gamma, float epsilon);
+
 /* The search result's move probabilities (MCTSEngine::getActionProbabilities,
  * src/mcts/mcts_engine_tree.cpp:388-465) from the visit counts of `root`'s children, laid
  * out over the action space: temperature < 0.01 puts 1 on the first child with the largest

@@ -355,6 +355,55 @@ int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_chi
     return OMK_OK;
 }
 
+int omk_forest_add_root_noise(omk_forest *f, int32_t root, const float *h_gamma, int32_t n_gamma, float epsilon) {
+    if (!f || !h_gamma) return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_add_root_noise: nothing uploaded");
+    if (root < 0 || root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: root %d", root);
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    int2 sp;
+    HIP_TRY(hipMemcpy(&sp, f->span + root, sizeof(sp), hipMemcpyDeviceToHost));
+    const int32_t cb = sp.x, cc = sp.y;
+    if (cc <= 0) return OMK_OK;  // no children to add noise to (mcts_engine_eval.cpp:78-80)
+    std::vector<float> prior((size_t)cc);
+    HIP_TRY(hipMemcpy(prior.data(), f->P + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
+    std::vector<uint32_t> legal;
+    const int64_t w0 = (int64_t)cb >> 5, w1 = ((int64_t)cb + cc + 31) >> 5;
+    if (f->has_legal) {
+        legal.resize((size_t)(w1 - w0));
+        HIP_TRY(hipMemcpy(legal.data(), f->legal + w0, legal.size() * 4, hipMemcpyDeviceToHost));
+    }
+    auto is_child = [&](int32_t i) {
+        if (!f->has_legal) return true;
+        const int64_t id = (int64_t)cb + i;
+        return ((legal[(size_t)((id >> 5) - w0)] >> (id & 31)) & 1u) != 0u;
+    };
+    int32_t children = 0;
+    for (int32_t i = 0; i < cc; i++) children += is_child(i) ? 1 : 0;
+    if (children == 0) return OMK_OK;
+    if (n_gamma != children)
+        return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: %d samples for %d children", n_gamma, children);
+    // MCTSEngine::addDirichletNoise from the normalisation on, statement by statement
+    float sum = 0.0f;
+    for (int32_t j = 0; j < children; j++) sum = sum + h_gamma[j];
+    std::vector<float> noise(h_gamma, h_gamma + children);
+    if (sum > 0.0f) {
+        for (auto &x : noise) x /= sum;
+    } else {
+        const float uniform_noise = 1.0f / (float)children;
+        for (auto &x : noise) x = uniform_noise;
+    }
+    int32_t j = 0;
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_child(i)) continue;
+        const float keep = (1.0f - epsilon) * prior[(size_t)i];
+        const float add = epsilon * noise[(size_t)j++];
+        prior[(size_t)i] = keep + add;
+    }
+    HIP_TRY(hipMemcpy(f->P + cb, prior.data(), (size_t)cc * 4, hipMemcpyHostToDevice));
+    return OMK_OK;
+}
+
 int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperature, int32_t action_space,
                                     float *h_probabilities, int32_t *h_children) {
     if (!f || !h_probabilities) return fail(OMK_ERR_INVALID, "omk_forest_action_probabilities: null argument");

@@ -90,6 +90,11 @@ std::vector<float> ForestEngine::getActionProbabilities(int32_t root, float temp
     return probs;
 }
 
+void ForestEngine::addDirichletNoise(int32_t root, const std::vector<float> &gamma_samples, float epsilon) {
+    check(omk_forest_add_root_noise(forest_, root, gamma_samples.data(), (int32_t)gamma_samples.size(), epsilon),
+          "omk_forest_add_root_noise");
+}
+
 int64_t ForestEngine::nodeCount() const {
     int64_t n = 0;
     check(omk_forest_node_count(forest_, &n, nullptr), "omk_forest_node_count");

@@ -80,6 +80,10 @@ class ForestEngine {
     // SearchResult.probabilities (reference MCTSEngine::getActionProbabilities,
     // src/mcts/mcts_engine_tree.cpp:388-465): visit counts of root's children, temperature.
     std::vector<float> getActionProbabilities(int32_t root, float temperature, int action_space);
+    // Dirichlet noise on the root's priors (reference MCTSEngine::addDirichletNoise,
+    // src/mcts/mcts_engine_eval.cpp:78-110): one gamma(alpha, 1) sample per child, drawn by
+    // the caller's generator as the reference draws them from its own.
+    void addDirichletNoise(int32_t root, const std::vector<float> &gamma_samples, float epsilon);
     int64_t nodeCount() const;
     void downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action);
 

@@ -41,9 +41,14 @@
 // Scheduling.  Two kernels.  The multi-visitor kernel is persistent: blocks of four
 // wavefronts, the first of which (the owner) takes tickets of a device-side work queue,
 // waits (bounded) until the item with that number is published, and processes it; the
-// other three help it with the batch work of larger nodes through block barriers.  Items
-// depend only on their ancestors, so there is no barrier between tree levels: the time of
-// a selection is the longest chain of crowded nodes.  The single-visitor walk (no LDS,
+// other three help it through block barriers: with the batch work of larger nodes, and one of
+// them shares out the visitors of a settled node (the partition) while the owner already
+// walks on into the kept child.  Items depend only on their ancestors, so there is no barrier
+// between tree levels: the time of a selection is the longest chain of crowded nodes.
+// Settling a node needs only the NUMBER of its visitors; the list of their traversal ids is
+// needed last, for the node's own partition.  The children of a heavy node are therefore
+// published before their lists are written (item kind 3) and wait for a "list complete" word
+// where they need it.  The single-visitor walk (no LDS,
 // high occupancy, one launch afterwards) takes the visitors that are alone at a node: they
 // stay alone to their leaf.
 #include <algorithm>

@@ -379,6 +379,30 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
 }
 
 /* ---- MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465) ---- */
+/* src/mcts/mcts_engine_eval.cpp:78-110 (MCTSEngine::addDirichletNoise) from the samples on:
+ * gamma[] holds one gamma(alpha, 1) draw per child of root, in child order (the reference
+ * draws them from std::gamma_distribution on its engine, :83-90).  Returns the number of
+ * children, or -1 when n_gamma does not match it. */
+int32_t ref_add_root_noise(ref_tree *t, int32_t root, const float *gamma, int32_t n_gamma, float epsilon) {
+    const int32_t cb = t->child_begin[root], cc = t->child_count[root];
+    int32_t children = 0;
+    for (int32_t i = 0; i < cc; i++) children += is_legal(t, cb + i) ? 1 : 0;
+    if (children == 0) return 0; /* :78-80 */
+    if (n_gamma != children) return -1;
+    float sum = 0.0f; /* std::accumulate(..., 0.0f): left to right */
+    for (int32_t j = 0; j < children; j++) sum = sum + gamma[j];
+    int32_t j = 0;
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_legal(t, cb + i)) continue;
+        float n = sum > 0.0f ? gamma[j] / sum : 1.0f / (float)children; /* :93-101 */
+        float keep = (1.0f - epsilon) * t->P[cb + i];
+        float add = epsilon * n;
+        t->P[cb + i] = keep + add; /* :104-110 */
+        j++;
+    }
+    return children;
+}
+
 int32_t ref_action_probabilities(const ref_tree *t, int32_t root, float temperature, int32_t action_space,
                                  float *out) {
     for (int32_t a = 0; a < action_space; a++) out[a] = 0.0f;

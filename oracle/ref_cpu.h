@@ -19,6 +19,8 @@
  *   ref_expand_batch      src/mcts/mcts_node.cpp:238-436, :512-593 (MCTSNode::expand, setPriorProbabilities),
  *                         call site src/mcts/mcts_engine_batch_tree_simple.cpp:249-259
  *   ref_action_probabilities  src/mcts/mcts_engine_tree.cpp:388-465 (MCTSEngine::getActionProbabilities)
+ *   ref_add_root_noise    src/mcts/mcts_engine_eval.cpp:78-110 (MCTSEngine::addDirichletNoise, from the
+ *                         gamma samples on)
  *   ref_rave_backup_batch src/mcts/mcts_engine_tree.cpp:288-331 (RAVE part of backPropagate; not dispatched
  *                         by the reference's live search loop)
  *   ref_reroot_child      src/mcts/mcts_engine_search.cpp:1029-1075 (searchWithTreeReuse)
@@ -139,6 +141,9 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
                          int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
                          uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
                          const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child);
+
+/* Dirichlet noise on the root's priors from caller-drawn gamma samples (see ref_cpu.c). */
+int32_t ref_add_root_noise(ref_tree *t, int32_t root, const float *gamma, int32_t n_gamma, float epsilon);
 
 /* MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465): the search
  * result's move probabilities from the root's children.  counts = float(N_child);

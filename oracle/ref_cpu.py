@@ -269,6 +269,16 @@ class RefTree:
                                            _ptr(out, f32p))
         return out, int(n)
 
+    def add_root_noise(self, root, gamma, epsilon):
+        """MCTSEngine::addDirichletNoise from the gamma samples on; returns the number of children."""
+        gamma = np.ascontiguousarray(gamma, dtype=np.float32)
+        L = lib()
+        L.ref_add_root_noise.restype = C.c_int32
+        n = L.ref_add_root_noise(C.byref(self._c), C.c_int32(int(root)), _ptr(gamma, f32p), C.c_int32(len(gamma)),
+                                 C.c_float(epsilon))
+        assert n >= 0, "sample count does not match the number of children"
+        return int(n)
+
     def gather_actions(self, paths, path_len):
         paths, path_len, B, stride = self._paths_args(paths, path_len)
         out = np.empty((B, stride - 1), dtype=np.int32)

@@ -219,3 +219,21 @@ def test_rave_backup_matches_the_checker():
         assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all()
         ref.W[:] = st["W"]
         ref.rW[:] = st["rW"]
+
+
+def test_root_noise_matches_the_checker():
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(61, n_expand=40, fanout=(5, 60), max_depth=3, mask_frac=0.25)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    rng = np.random.default_rng(4)
+    for node in (int(roots[0]), int(np.nonzero(soa["child_count"] > 0)[0][-1])):
+        cb, cc = int(soa["child_begin"][node]), int(soa["child_count"][node])
+        ids = np.arange(cb, cb + cc)
+        n_children = int(((soa["legal"][ids >> 5] >> (ids & 31).astype(np.uint32)) & 1).sum())
+        gamma = rng.gamma(0.3, 1.0, n_children).astype(np.float32)
+        assert ref.add_root_noise(node, gamma, 0.25) == n_children
+        f.add_root_noise(node, gamma, 0.25)
+        assert (f.download()["P"] == ref.P).all()  # same operations in the same order: bit-exact
+    with pytest.raises(omk.OmkError):
+        f.add_root_noise(int(roots[0]), np.ones(1, np.float32), 0.25)

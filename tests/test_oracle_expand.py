@@ -175,3 +175,20 @@ def test_rave_backup_updates_children_whose_action_is_on_the_path():
     # at the root (flipped twice): children 1 (action 5) and 2 (action 6) match, child 3 does not.
     assert t.rN.tolist() == [0, 1, 1, 0, 1, 0]
     assert t.rW.tolist() == [0.0, 0.5, 0.5, 0.0, -0.5, 0.0]
+
+
+# ---- Dirichlet noise on the root priors (src/mcts/mcts_engine_eval.cpp:78-110) ----
+
+def test_root_noise_mixes_normalised_samples_into_the_priors():
+    z = lambda *v: np.array(v, np.int32)
+    t = R.RefTree(N=z(1, 0, 0, 0, 0), W=np.zeros(5, np.float32), P=np.array([0, .5, .25, .125, .125], np.float32),
+                  VL=z(0, 0, 0, 0, 0), child_begin=z(1, 0, 0, 0, 0), child_count=z(4, 0, 0, 0, 0))
+    assert t.add_root_noise(0, [1.0, 3.0, 0.0, 4.0], 0.25) == 4
+    # noise = samples / 8 = .125 .375 0 .5 ; prior = .75 * prior + .25 * noise  (all exact in binary32)
+    assert t.P.tolist() == [0.0, 0.40625, 0.28125, 0.09375, 0.21875]
+    assert abs(float(t.P[1:].sum()) - 1.0) < 1e-6   # a distribution stays one
+    # samples that sum to zero: uniform noise (:98-101)
+    t.add_root_noise(0, [0.0, 0.0, 0.0, 0.0], 0.5)
+    assert t.P.tolist() == [0.0, 0.328125, 0.265625, 0.171875, 0.234375]
+    # a root without children is left alone (:78-80)
+    assert t.add_root_noise(2, [], 0.25) == 0
