@@ -73,6 +73,8 @@ constexpr int kRunShortcutMin = 128;      // entries from which a run of one chi
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
 constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
+constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
+                                          // is shared out like a heavy node's instead of left to one helper
 
 enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
 
@@ -1665,7 +1667,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         settled = true;
     }
     if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
-        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kHeavyMin, cnt, run_child);
+        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child);
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
@@ -1881,7 +1883,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // shares out the visitors and publishes the other children (partition_async), this one
     // walks on into the kept child at once.  What the kept child needs of that work, its
     // visitor list, it needs last (close_pending).
-    if (!as_scatter && !as_slice && m < kHeavyMin && (run_child >= 0 || lds_cur >= 0)) {
+    if (!as_scatter && !as_slice && ((m < kHeavyMin && lds_cur >= 0) || (run_child >= 0 && m < kRunShareMin))) {
         int carry = 0, ex_keep = 0, np_keep = 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
