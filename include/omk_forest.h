@@ -183,9 +183,10 @@ int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, in
  * siblings contiguous in their old order, new_root = 0, so selections come out the same.
  * *h_nodes_after = k; h_old_of_new (NULL or room for the old node count) receives the old id
  * of every new node.  Paths of earlier selections, roots of batches and node ids stored in
- * transposition tables refer to the old numbering: set roots again, clear the tables.  The
- * renumbering is computed on the host from the child ranges (read back once); the
- * statistics are moved on the device. */
+ * transposition tables refer to the old numbering: set roots again, clear the tables.  All
+ * of it runs on the device: the renumbering level by level (child counts of a level, an
+ * exclusive scan, the children's ids written to the next level), then one gather per array;
+ * the host only reads the size of every level. */
 int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new);
 
 /* Leaf expansion for the leaves of the last selection: MCTSNode::expand

@@ -521,44 +521,48 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
     hipStream_t s = f->stream;
     HIP_TRY(hipStreamSynchronize(s));
     const int64_t n = f->n_nodes;
-    std::vector<int2> span((size_t)n);
-    HIP_TRY(hipMemcpy(span.data(), f->span, (size_t)n * sizeof(int2), hipMemcpyDeviceToHost));
-    // breadth-first order of the subtree; children are appended in visiting order, so the
-    // first child of new node i is 1 + the children of all new nodes before it
-    std::vector<int32_t> order, new_begin;
-    order.reserve(1024);
-    order.push_back(new_root);
-    for (size_t head = 0; head < order.size(); head++) {
-        const int2 sp = span[(size_t)order[head]];
-        new_begin.push_back(sp.y > 0 ? (int32_t)order.size() : 0);
-        for (int32_t i = 0; i < sp.y; i++) order.push_back(sp.x + i);
-        if ((int64_t)order.size() > n) return fail(OMK_ERR_STRUCTURE, "omk_forest_compact: the child ranges do not form a tree");
-    }
-    const int64_t k = (int64_t)order.size();
-    // the legal mask of the new numbering, on the host (one bit per node)
-    std::vector<uint32_t> new_legal;
-    if (f->has_legal) {
-        std::vector<uint32_t> legal((size_t)((n + 31) / 32));
-        HIP_TRY(hipMemcpy(legal.data(), f->legal, legal.size() * 4, hipMemcpyDeviceToHost));
-        new_legal.assign((size_t)((k + 31) / 32), 0u);
-        for (int64_t i = 0; i < k; i++) {
-            const uint32_t old = (uint32_t)order[(size_t)i];
-            if ((legal[old >> 5] >> (old & 31u)) & 1u) new_legal[(size_t)(i >> 5)] |= 1u << (i & 31);
-        }
-    }
-    // device: map, new child starts, and one scratch array that every field passes through
-    int32_t *d_map = nullptr, *d_begin = nullptr;
+    // breadth-first order of the subtree, on the device: d_map[new id] = old id, d_begin[new id]
+    // = new id of its first child.  One level per round; the levels' sizes come back to the
+    // host (a handful of bytes per level).
+    int32_t *d_map = nullptr, *d_begin = nullptr, *d_cc = nullptr, *d_scan = nullptr;
+    uint32_t *d_legal = nullptr;
     uint64_t *d_tmp = nullptr;
-    hipError_t e = hipMalloc((void **)&d_map, (size_t)k * 4);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_begin, (size_t)k * 4);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_tmp, (size_t)k * 8);
+    void *d_scan_tmp = nullptr;
+    size_t scan_bytes = 0;
+    hipError_t e = bfs_scan_bytes(n, &scan_bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_map, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_begin, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_cc, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_scan, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc(&d_scan_tmp, scan_bytes > 0 ? scan_bytes : 4);
     auto cleanup = [&]() {
-        if (d_map) (void)hipFree(d_map);
-        if (d_begin) (void)hipFree(d_begin);
-        if (d_tmp) (void)hipFree(d_tmp);
+        for (void *p : {(void *)d_map, (void *)d_begin, (void *)d_cc, (void *)d_scan, (void *)d_legal, (void *)d_tmp,
+                        d_scan_tmp})
+            if (p) (void)hipFree(p);
     };
-    if (e == hipSuccess) e = hipMemcpyAsync(d_map, order.data(), (size_t)k * 4, hipMemcpyHostToDevice, s);
-    if (e == hipSuccess) e = hipMemcpyAsync(d_begin, new_begin.data(), (size_t)k * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_map, &new_root, 4, hipMemcpyHostToDevice, s);
+    int64_t lo = 0, hi = 1;
+    bool not_a_tree = false;
+    while (e == hipSuccess && hi > lo) {
+        int64_t total = 0;
+        e = launch_bfs_level(f->span, d_map, d_begin, lo, hi - lo, n - hi, d_cc, d_scan, d_scan_tmp, scan_bytes, &total, s);
+        if (e == hipSuccess && total > n - hi) {
+            not_a_tree = true;
+            break;
+        }
+        lo = hi;
+        hi += total;
+    }
+    if (e != hipSuccess || not_a_tree) {
+        (void)hipStreamSynchronize(s);
+        cleanup();
+        if (not_a_tree) return fail(OMK_ERR_STRUCTURE, "omk_forest_compact: the child ranges do not form a tree");
+        return fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
+    }
+    const int64_t k = hi;
+    // one scratch array that every field passes through
+    e = hipMalloc((void **)&d_tmp, (size_t)k * 8);
+    if (e == hipSuccess && f->has_legal) e = hipMalloc((void **)&d_legal, (size_t)((k + 31) / 32) * 4);
     auto move_words = [&](void *arr) {
         if (e != hipSuccess || !arr) return;
         e = launch_gather_words((uint32_t *)d_tmp, (const uint32_t *)arr, d_map, k, s);
@@ -581,14 +585,17 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
         e = launch_gather_span((int2 *)d_tmp, f->span, d_map, d_begin, k, s);
         if (e == hipSuccess) e = hipMemcpyAsync(f->span, d_tmp, (size_t)k * sizeof(int2), hipMemcpyDeviceToDevice, s);
     }
-    if (e == hipSuccess && f->has_legal)
-        e = hipMemcpyAsync(f->legal, new_legal.data(), new_legal.size() * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess && f->has_legal) {
+        e = launch_gather_legal(d_legal, f->legal, d_map, k, s);
+        if (e == hipSuccess)
+            e = hipMemcpyAsync(f->legal, d_legal, (size_t)((k + 31) / 32) * 4, hipMemcpyDeviceToDevice, s);
+    }
+    if (e == hipSuccess && h_old_of_new) e = hipMemcpyAsync(h_old_of_new, d_map, (size_t)k * 4, hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
     cleanup();
     if (e != hipSuccess) return fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
     f->n_nodes = k;
     if (h_nodes_after) *h_nodes_after = k;
-    if (h_old_of_new) memcpy(h_old_of_new, order.data(), (size_t)k * 4);
     return OMK_OK;
 }
 

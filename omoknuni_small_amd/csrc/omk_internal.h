@@ -129,6 +129,12 @@ hipError_t launch_rave_backup(const ForestMut &f, const int32_t *paths, const in
 
 // Compaction: new node i takes the statistics of old node map[i]; its child range keeps its
 // length and starts at new_begin[i].
+// Breadth-first renumbering of a subtree, level by level (omk_compact.hip).
+hipError_t bfs_scan_bytes(int64_t max_items, size_t *bytes);
+hipError_t launch_bfs_level(const int2 *span, int32_t *order, int32_t *new_begin, int64_t lo, int64_t cnt,
+                            int64_t room, int32_t *cc, int32_t *scan, void *temp, size_t temp_bytes,
+                            int64_t *h_total, hipStream_t s);
+hipError_t launch_gather_legal(uint32_t *dst, const uint32_t *src, const int32_t *order, int64_t k, hipStream_t s);
 hipError_t launch_gather_words(uint32_t *dst, const uint32_t *src, const int32_t *map, int64_t k, hipStream_t s);
 hipError_t launch_gather_dwords(uint64_t *dst, const uint64_t *src, const int32_t *map, int64_t k, hipStream_t s);
 hipError_t launch_gather_span(int2 *dst, const int2 *src, const int32_t *map, const int32_t *new_begin, int64_t k,
