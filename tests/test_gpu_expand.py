@@ -237,3 +237,41 @@ def test_root_noise_matches_the_checker():
         assert (f.download()["P"] == ref.P).all()  # same operations in the same order: bit-exact
     with pytest.raises(omk.OmkError):
         f.add_root_noise(int(roots[0]), np.ones(1, np.float32), 0.25)
+
+
+def test_compaction_of_deep_and_wide_shapes_and_of_a_broken_structure():
+    """The level-by-level renumbering on shapes that stress it: a path-like tree (one node per
+    level for hundreds of levels), one very wide level, the whole tree from its root; and child
+    ranges that loop back, which are refused."""
+    import omoknuni_small_amd as omk
+    # a spine 300 levels deep with a few leaves on the way, then a node with 900 children
+    N, cb, cc = [1], [0], [0]
+    spine = 0
+    for d in range(300):
+        fan = 3 if d % 7 == 0 else 1
+        cb[spine], cc[spine] = len(N), fan
+        first = len(N)
+        for _ in range(fan):
+            N.append(d + 1); cb.append(0); cc.append(0)
+        spine = first + fan - 1
+    cb[spine], cc[spine] = len(N), 900
+    for i in range(900):
+        N.append(i); cb.append(0); cc.append(0)
+    n = len(N)
+    soa = dict(N=np.array(N, np.int32), W=np.arange(n, dtype=np.float32), P=np.full(n, 0.5, np.float32),
+               VL=np.zeros(n, np.int32), child_begin=np.array(cb, np.int32), child_count=np.array(cc, np.int32),
+               action=np.arange(n, dtype=np.int32))
+    ref = R.RefTree.from_soa(soa)
+    for new_root in (0, int(cb[0]) + 2, spine):
+        f = omk.Forest.from_soa(soa)
+        ref2, order = ref.compacted(new_root)
+        gorder = f.compact(new_root)
+        assert len(gorder) == len(order) and (gorder == order).all(), new_root
+        assert_same_forest(f, ref2, "subtree of %d" % new_root)
+    # a child range that points back at the root: not a tree
+    bad = dict(soa)
+    bad["child_begin"] = soa["child_begin"].copy()
+    bad["child_count"] = soa["child_count"].copy()
+    bad["child_begin"][n - 1], bad["child_count"][n - 1] = 0, 2
+    with pytest.raises(omk.OmkError):  # the upload already refuses it (a node with two parents)
+        omk.Forest.from_soa(bad).compact(0)
