@@ -956,18 +956,22 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         }
         if (run_min == 1) OMK_FAIL(11);  // the run that had to be there was refused
         const int want = remaining < kBatchCap ? remaining : kBatchCap;
-        // lower bound of any useful threshold: the best child alone has `want` entries at or
-        // above the key of its want-th next visit
+        // lower bound of any useful threshold: a child alone has `want` entries at or above the
+        // key of its want-th next visit; the best such key over all children (the child that
+        // holds out longest, which need not be the one with the best next entry)
         uint32_t lo_key = 0u;
         {
-            uint32_t kk = 0u, pp = 0u;
+            uint32_t lmax = 0u;
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                if (r == (best >> 6))
-                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk[r] + want - 1, best, kk,
-                                       pp);
+                if (k.part[r] && headk[r] != 0u) {
+                    uint32_t kk, pp;
+                    entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, tk[r] + want - 1,
+                                       r * kWave + lane, kk, pp);
+                    lmax = umax32(lmax, kk);
+                }
             }
-            lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
+            lo_key = wave_max_u32(lmax);
         }
         if (lo_key == 0u) lo_key = 1u;
         if (lo_key > hi_key) OMK_FAIL(3);  // scores rose along the best child's list
@@ -1416,18 +1420,20 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     uint32_t hi_key, hi_pos;
     wave_best(lbk, lbp, hi_key, hi_pos);
     if (hi_key == 0u) return false;
-    const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
-    // The best child alone has m entries at or above the key of its m-th visit: a lower bound
-    // for every threshold of the node.
+    // A child alone has m entries at or above the key of its m-th visit: the best such key over
+    // all children is a lower bound for every threshold of the node.
     uint32_t lo_key = 0u;
     {
-        uint32_t kk = 0u, pp = 0u;
+        uint32_t lmax = 0u;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if (r == (best >> 6))
-                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, m - 1, best, kk, pp);
+            if (k.part[r] && headk[r] != 0u) {
+                uint32_t kk, pp;
+                entry_key<R, RAVE>(k.n[r], k.w[r], k.p[r], k.vl[r], k.q2[r], c.ep, uvl, m - 1, r * kWave + lane, kk, pp);
+                lmax = umax32(lmax, kk);
+            }
         }
-        lo_key = (uint32_t)__builtin_amdgcn_readlane((int)kk, best & 63);
+        lo_key = wave_max_u32(lmax);
     }
     if (lo_key == 0u) lo_key = 1u;
     if (lo_key > hi_key) return false;
