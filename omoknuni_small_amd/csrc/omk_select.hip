@@ -1030,7 +1030,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         int tries = 0;
         uint32_t T_forced = 0u;  // threshold imposed for the next round instead of searching one
         bool allow_above = true;
-        bool several_flood = false;  // no single child accounts for the excess at the flooded key
         for (;;) {
             if (++tries > 8) OMK_FAIL(5);
             const uint32_t T_now = T_forced;  // imposed for this round only
@@ -1131,13 +1130,12 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 if (allow_above && T < hi_key && ((int)gmx > excess || tries >= 3)) {
                     // (after a few rounds of aiming higher in vain the key is taken to be flooded by
                     // several children at once)
-                    several_flood = (int)gmx <= excess;
                     allow_above = false;
                     T_forced = T + 1u;
                     continue;
                 }
-                if ((int)gmx <= excess && T >= hi_key && tries >= 3) {
-                    force_run = true;  // several children exactly tied at the very top
+                if (T >= hi_key) {
+                    force_run = true;  // flooded at the best key itself: nothing lies above, the best child runs
                     break;
                 }
                 if ((int)gmx <= excess) {
@@ -1152,12 +1150,10 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 total = kBatchCap;
             }
             if (T_now != 0u) {
-                if (total < 1) {
-                    // nothing above the flooded key: if it is flooded by one child, back to it, capped;
-                    // if by several, exactly tied, the best of them runs first
-                    if (several_flood) force_run = true;
-                    else continue;
-                }
+                // nothing above the flooded key: every child's next entry is at that key or below,
+                // equal keys go by position, so the best child runs first, however short its run
+                // (the child that floods the key follows with a long one)
+                if (total < 1) force_run = true;
                 break;  // may not finish the node: the run comes next
             }
             if (can_finish && total < remaining) {
@@ -1369,7 +1365,7 @@ template <int R, bool RAVE>
 __device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t lo_key,
                                                      uint32_t hi_key, int target, int window, int m) {
     uint32_t klo = lo_key, khi = hi_key;  // est(klo) >= target is taken for granted, est(khi) < target
-    for (int it = 0; it < 24 && khi - klo > 1u; it++) {
+    for (int it = 0; it < 32 && khi - klo > 1u; it++) {
         const uint32_t kmid = klo + ((khi - klo) >> 1);
         const float mid = key_score(kmid);
         int est = 0;
