@@ -67,6 +67,8 @@ constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-v
                                           // takes the items, three helpers for the batch work of its node
 constexpr int kTeam = kTeamWaves * 64;
 constexpr int kTeamMin = 96;              // batch entries from which the helpers are called in
+// a batch of at most this many entries per thread is ordered by counting: a lone wavefront, the block
+constexpr int kCountSortLone = 2, kCountSortTeam = 1;
 constexpr int kSliceEntries = 256;        // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
@@ -174,8 +176,8 @@ struct WaveLds {
     int st_j0[R * kWave];  // visits already settled / visit count, by phase
     int hist[kSortBins * (kBatchCap / kWave + 1) > R * kWave ? kSortBins * (kBatchCap / kWave + 1) : R * kWave];  // sort: entries per (digit value, block of 64); emit: visits per child
     uint32_t pay[R * kWave];      // per child: entries of the batch
-    uint32_t key[2][kBatchCap];   // entries of the batch being ordered: inverted score key ...
-    uint32_t pay2[2][kBatchCap];  // ... and pass flag, child, visit number; two buffers, ping-pong
+    alignas(16) uint32_t key[2][kBatchCap];  // entries of the batch being ordered: inverted score key ...
+    alignas(16) uint32_t pay2[2][kBatchCap];  // ... and pass flag, child, visit number; two buffers, ping-pong
 };
 
 // AHEAD: ask for the statistics of every child in range before the legality bits are known
@@ -555,6 +557,10 @@ __device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, 
             atomicMax(&lds.red[1], kmax);
             atomicOr(&lds.red[2], flags);
         }
+        // a small batch is ordered by counting (below), four entries per LDS read: keys behind
+        // its last entry that never count
+        if (total <= (NT == kWave ? kCountSortLone : kCountSortTeam) * NT && tid < 4)
+            lds.key[0][total + tid] = 0xFFFFFFFFu;
         team_sync<NT>();
         // the run of the previous thread may end inside the same child: check the seam
         bool bad_seam = false;
@@ -570,6 +576,47 @@ __device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, 
     const uint32_t kmin = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[0]);
     const uint32_t kmax = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[1]);
     const bool mixed = ((uint32_t)__builtin_amdgcn_readfirstlane((int)lds.red[2]) & 3u) == 3u;
+
+    // A small batch (at most kCountSortLone / kCountSortTeam entries per thread): the rank of an
+    // entry is the number of entries that come before it, counted against every entry of the
+    // batch (one 16-byte LDS read serves four of them, the same address for all lanes).  Same
+    // order as the radix sort below: inverted key ascending, then scan kind, child and visit
+    // number, which is the payload as a number: key and payload are compared as one 64-bit
+    // number (children tied on a key are common, so the payload is not left to a second pass).
+    constexpr int kCountSortPerThread = NT == kWave ? kCountSortLone : kCountSortTeam;
+    if (total <= kCountSortPerThread * NT) {
+        const uint32_t *src_k = lds.key[0], *src_p = lds.pay2[0];
+        uint32_t mk[kCountSortPerThread], mp[kCountSortPerThread];
+        uint64_t mine[kCountSortPerThread];
+        int rk[kCountSortPerThread];
+#pragma unroll
+        for (int e = 0; e < kCountSortPerThread; e++) {
+            const int q = tid + e * NT;
+            mk[e] = q < total ? src_k[q] : 0xFFFFFFFFu;
+            mp[e] = q < total ? src_p[q] : 0xFFFFFFFFu;
+            mine[e] = ((uint64_t)mk[e] << 32) | mp[e];
+            rk[e] = 0;
+        }
+#pragma unroll 4
+        for (int q4 = 0; q4 < total; q4 += 4) {
+            const uint4 ok = *reinterpret_cast<const uint4 *>(src_k + q4);
+            const uint4 op = *reinterpret_cast<const uint4 *>(src_p + q4);
+            const uint64_t o0 = ((uint64_t)ok.x << 32) | op.x, o1 = ((uint64_t)ok.y << 32) | op.y;
+            const uint64_t o2 = ((uint64_t)ok.z << 32) | op.z, o3 = ((uint64_t)ok.w << 32) | op.w;
+#pragma unroll
+            for (int e = 0; e < kCountSortPerThread; e++)
+                rk[e] += (int)(o0 < mine[e]) + (int)(o1 < mine[e]) + (int)(o2 < mine[e]) + (int)(o3 < mine[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < kCountSortPerThread; e++) {
+            if (tid + e * NT < total) {
+                lds.key[1][rk[e]] = mk[e];
+                lds.pay2[1][rk[e]] = mp[e];
+            }
+        }
+        team_sync<NT>();
+        return 1;
+    }
 
     // Stable radix sort, in LDS.  Order wanted: key descending, then candidate position
     // ascending, then visit number.  The entries start in (child, visit) order; least
