@@ -252,6 +252,22 @@ typedef struct omk_tt_slot {
     int32_t depth;
 } omk_tt_slot;
 
+/* Position key of the state every selected leaf stands for: what the traversal loop obtains by
+ * cloning the root state, replaying the move list and calling getHash()
+ * (mcts_engine_batch_tree_simple.cpp:119-124 and :133-137), for a game whose stones stay where they
+ * are placed and whose sides alternate (GomokuState::compute_hash_signature_internal,
+ * src/games/gomoku/gomoku_state.cpp:947-957: the piece keys of all stones and the key of the side
+ * to move, XORed).  The caller passes the tables of the game's utils::ZobristHash
+ * (src/utils/zobrist_hash.cpp:9-36; they are seeded from the clock there, so they are the
+ * caller's): d_piece_keys[p * cells + action] = getPieceHash(p, action) for the two sides,
+ * d_player_keys[p] = getPlayerHash(p); and per traversal the root state's getHash() and its side to
+ * move (0 or 1 = current_player - 1).  d_out[t] = key of the leaf's state, ready for omk_tt_probe /
+ * omk_tt_insert.  All pointers are device memory; a move outside [0, cells) is an error.  A game
+ * with captures (Go) cannot be keyed from the move list alone and keeps its keys in the forest
+ * (omk_soa_view.hash, omk_tt_probe_leaves). */
+int omk_batch_leaf_keys(omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
+                        const uint64_t *d_root_keys, const int32_t *d_root_players, uint64_t *d_out);
+
 int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out);
 int omk_tt_destroy(omk_tt *tt);
 int omk_tt_clear(omk_tt *tt);

@@ -1128,6 +1128,28 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
     return OMK_OK;
 }
 
+int omk_batch_leaf_keys(omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
+                        const uint64_t *d_root_keys, const int32_t *d_root_players, uint64_t *d_out) {
+    if (!b || !d_piece_keys || !d_player_keys || !d_root_keys || !d_root_players || !d_out)
+        return fail(OMK_ERR_INVALID, "omk_batch_leaf_keys: null argument");
+    if (cells <= 0) return fail(OMK_ERR_INVALID, "omk_batch_leaf_keys: cells %d", cells);
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_leaf_keys: no selected paths");
+    omk_forest *f = b->f;
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    int32_t *d_status = b->counters + 32;  // a word of the batch's counter block that nothing else uses
+    int bad = 0;
+    HIP_TRY(hipMemcpyAsync(d_status, &bad, sizeof(bad), hipMemcpyHostToDevice, s));
+    HIP_TRY(launch_leaf_keys(f->dev(), b->paths, b->path_len, b->n, b->stride, d_piece_keys, cells, d_player_keys,
+                             d_root_keys, d_root_players, d_out, d_status, s));
+    HIP_TRY(hipMemcpyAsync(&bad, d_status, sizeof(bad), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (bad)
+        return fail(OMK_ERR_INVALID, "omk_batch_leaf_keys: %d paths hold a move outside [0, %d) or no node at all "
+                    "(their keys are ~0)", bad, cells);
+    return OMK_OK;
+}
+
 int omk_tt_upload(omk_tt *tt, const omk_tt_slot *h_slots) {
     if (!tt || !h_slots) return fail(OMK_ERR_INVALID, "omk_tt_upload: null argument");
     if (int rc = use_device(tt->f)) return rc;

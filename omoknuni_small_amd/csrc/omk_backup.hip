@@ -130,6 +130,44 @@ __global__ __launch_bounds__(256) void k_export(ForestDev f, const int32_t *path
     }
 }
 
+// ---- position keys of the selected leaves: GomokuState::compute_hash_signature_internal
+// (src/games/gomoku/gomoku_state.cpp:947-957) over the tables of utils::ZobristHash
+// (src/utils/zobrist_hash.cpp:9-36), for the state the traversal loop rebuilds by replaying its
+// move list (mcts_engine_batch_tree_simple.cpp:119-124,133-137) ----
+
+// A stone placed stays (no captures), so the key of the replayed state is the root state's key
+// with the piece keys of the path's moves folded in and the side-to-move key swapped: the mover
+// of ply k is the root's side to move when k is even.  One thread per traversal; the path is
+// stored level-major, so each level is a coalesced read.
+__global__ __launch_bounds__(256) void k_leaf_keys(ForestDev f, const int32_t *paths, const int32_t *path_len, int n,
+                                                   int stride, const uint64_t *piece, int cells,
+                                                   const uint64_t *player, const uint64_t *root_key,
+                                                   const int32_t *root_player, uint64_t *out, int *d_status) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    const int len = path_len[t];
+    const int p0 = root_player[t] & 1;
+    uint64_t h = root_key[t];
+    bool bad = false;
+    for (int d = 1; d < len; d++) {
+        const int node = paths[(size_t)d * stride + t];
+        if (node < 0 || node >= f.n_nodes) {  // never index the forest with an id it does not have
+            bad = true;
+            break;
+        }
+        const int act = f.action ? f.action[node] : node;
+        if (act < 0 || act >= cells) {
+            bad = true;
+            break;
+        }
+        h ^= piece[(size_t)((p0 + d - 1) & 1) * cells + act];
+    }
+    if (len >= 1 && ((len - 1) & 1)) h ^= player[p0] ^ player[p0 ^ 1];
+    if (len < 1) bad = true;
+    out[t] = bad ? ~0ull : h;
+    if (bad) atomicAdd(d_status, 1);
+}
+
 // ---- leaf expansion: MCTSNode::expand + setPriorProbabilities
 // (src/mcts/mcts_node.cpp:238-436, :512-593) for a batch of leaves ----
 
@@ -311,6 +349,15 @@ hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t
     int64_t total = (int64_t)n * (max_depth + 1);
     hipLaunchKernelGGL(k_export, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, f, paths, path_len, n,
                        stride, max_depth, out_paths, out_actions);
+    return hipGetLastError();
+}
+
+hipError_t launch_leaf_keys(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                            const uint64_t *piece, int cells, const uint64_t *player, const uint64_t *root_key,
+                            const int32_t *root_player, uint64_t *out, int *d_status, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_leaf_keys, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f, paths, path_len, n,
+                       stride, piece, cells, player, root_key, root_player, out, d_status);
     return hipGetLastError();
 }
 

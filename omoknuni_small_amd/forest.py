@@ -27,7 +27,7 @@ EXPORTS = [
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_leaf_keys", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
 ]
@@ -308,6 +308,34 @@ class Batch:
         _check(self._lib.omk_batch_read(self._h, _ptr(paths, i32p), _ptr(plen, i32p), _ptr(leaf, i32p),
                                         _ptr(actions, i32p)))
         return paths, plen, leaf, actions
+
+    def leaf_keys_dev(self, d_piece_keys, cells, d_player_keys, d_root_keys, d_root_players, d_out):
+        _check(self._lib.omk_batch_leaf_keys(self._h, C.c_void_p(d_piece_keys), C.c_int32(int(cells)),
+                                             C.c_void_p(d_player_keys), C.c_void_p(d_root_keys),
+                                             C.c_void_p(d_root_players), C.c_void_p(d_out)))
+
+    def leaf_keys(self, piece_keys, player_keys, root_keys, root_players):
+        """Position key of every selected leaf's state (getHash() of the root state after the path's
+        moves): piece_keys [2, cells] and player_keys [2] are the game's Zobrist tables, root_keys /
+        root_players [n] the root states' keys and sides to move (0 or 1)."""
+        f = self.forest
+        pk = np.ascontiguousarray(piece_keys, np.uint64)
+        assert pk.ndim == 2 and pk.shape[0] == 2
+        pl = np.ascontiguousarray(player_keys, np.uint64)
+        rk = np.ascontiguousarray(root_keys, np.uint64)
+        rp = np.ascontiguousarray(root_players, np.int32)
+        assert len(pl) == 2 and len(rk) == self.n and len(rp) == self.n
+        out = np.empty(self.n, np.uint64)
+        bufs = [f.dev_alloc(x.nbytes) for x in (pk, pl, rk, rp, out)]
+        try:
+            for d, x in zip(bufs[:4], (pk, pl, rk, rp)):
+                f.h2d(d, x)
+            self.leaf_keys_dev(bufs[0], pk.shape[1], bufs[1], bufs[2], bufs[3], bufs[4])
+            f.d2h(out, bufs[4])
+        finally:
+            for d in bufs:
+                f.dev_free(d)
+        return out
 
     def expand(self, move_begin, moves, policy=None, action_space=0):
         """Expands the leaves of the last select(): move_begin [n+1] / moves are the legal moves

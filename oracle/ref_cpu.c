@@ -511,3 +511,91 @@ void ref_rave_backup_batch(ref_tree *t, const int32_t *paths, const int32_t *pat
         }
     }
 }
+
+/* ---- position keys (src/utils/zobrist_hash.cpp:9-36,129-131; src/games/gomoku/gomoku_state.cpp:947-957) ---- */
+
+/* std::mt19937_64, the generator ZobristHash draws from (zobrist_hash.cpp:20): the published
+ * MT19937-64 recurrence (n = 312, m = 156, r = 31, a = 0xB5026F5AA96619E9, tempering
+ * 29/0x5555555555555555, 17/0x71D67FFFEDA60000, 37/0xFFF7EEE000000000, 43) and the seeding
+ * x_i = 6364136223846793005 * (x_{i-1} ^ (x_{i-1} >> 62)) + i of the C++ standard. */
+void ref_mt64_seed(ref_mt64 *g, uint64_t seed) {
+    g->mt[0] = seed;
+    for (int i = 1; i < 312; i++) g->mt[i] = 6364136223846793005ull * (g->mt[i - 1] ^ (g->mt[i - 1] >> 62)) + (uint64_t)i;
+    g->idx = 312;
+}
+
+uint64_t ref_mt64_next(ref_mt64 *g) {
+    if (g->idx >= 312) {
+        for (int i = 0; i < 312; i++) {
+            const uint64_t x = (g->mt[i] & 0xFFFFFFFF80000000ull) | (g->mt[(i + 1) % 312] & 0x7FFFFFFFull);
+            g->mt[i] = g->mt[(i + 156) % 312] ^ (x >> 1) ^ ((x & 1ull) ? 0xB5026F5AA96619E9ull : 0ull);
+        }
+        g->idx = 0;
+    }
+    uint64_t y = g->mt[g->idx++];
+    y ^= (y >> 29) & 0x5555555555555555ull;
+    y ^= (y << 17) & 0x71D67FFFEDA60000ull;
+    y ^= (y << 37) & 0xFFF7EEE000000000ull;
+    y ^= y >> 43;
+    return y;
+}
+
+/* ZobristHash::ZobristHash(boardSize, numPieceTypes, numPlayers, seed), zobrist_hash.cpp:9-36: one
+ * generator seeded with `seed` (an unsigned: 32 bits), piece tables first (piece-major,
+ * boardSize * boardSize keys each), then the player keys.  seed 0 means "from the clock" there
+ * and is refused here. */
+int ref_zobrist_tables(int32_t board_size, int32_t n_piece, int32_t n_players, uint32_t seed, uint64_t *piece,
+                       uint64_t *player) {
+    if (board_size <= 0 || n_piece < 0 || n_players <= 0 || seed == 0) return -1;
+    ref_mt64 g;
+    ref_mt64_seed(&g, (uint64_t)seed);
+    const int64_t per = (int64_t)board_size * board_size;
+    for (int32_t p = 0; p < n_piece; p++)
+        for (int64_t pos = 0; pos < per; pos++) piece[(int64_t)p * per + pos] = ref_mt64_next(&g);
+    for (int32_t p = 0; p < n_players; p++) player[p] = ref_mt64_next(&g);
+    return 0;
+}
+
+/* GomokuState::compute_hash_signature_internal, gomoku_state.cpp:947-957: for both sides, for every
+ * cell in ascending order, a stone of that side folds in getPieceHash(side, cell); then
+ * getPlayerHash(current_player - 1).  board[cell] = 0 empty, 1 BLACK, 2 WHITE. */
+uint64_t ref_position_key(const int8_t *board, int32_t cells, const uint64_t *piece, int64_t piece_stride,
+                          const uint64_t *player, int32_t current_player) {
+    uint64_t h = 0;
+    for (int32_t p_idx = 0; p_idx < 2; p_idx++)
+        for (int32_t action = 0; action < cells; action++)
+            if (board[action] == p_idx + 1) h ^= piece[(int64_t)p_idx * piece_stride + action];
+    h ^= player[current_player - 1];
+    return h;
+}
+
+/* The temp_state of the traversal loop (mcts_engine_batch_tree_simple.cpp:119-124,133-137): a
+ * clone of the root state, makeMove for every move of the path (make_move_internal,
+ * gomoku_state.cpp:963-980: the side to move places a stone, then the other side is to move),
+ * getHash() computed from the resulting board.  Returns the number of paths with a move that is
+ * off the board or on an occupied cell (their key is ~0). */
+int32_t ref_leaf_keys(const ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B, int32_t stride,
+                      const int8_t *root_boards, const int32_t *root_player, int32_t cells, const uint64_t *piece,
+                      int64_t piece_stride, const uint64_t *player, uint64_t *out) {
+    int32_t bad = 0;
+    int8_t *board = (int8_t *)malloc((size_t)cells);
+    for (int32_t i = 0; i < B; i++) {
+        memcpy(board, root_boards + (int64_t)i * cells, (size_t)cells);
+        int32_t cur = root_player[i];
+        int ok = path_len[i] >= 1;
+        for (int32_t d = 1; ok && d < path_len[i]; d++) {
+            const int32_t node = paths[(int64_t)i * stride + d];
+            const int32_t a = t->action ? t->action[node] : node;
+            if (a < 0 || a >= cells || board[a] != 0) {
+                ok = 0;
+                break;
+            }
+            board[a] = (int8_t)cur;
+            cur = cur == 1 ? 2 : 1;
+        }
+        out[i] = ok ? ref_position_key(board, cells, piece, piece_stride, player, cur) : ~0ull;
+        bad += !ok;
+    }
+    free(board);
+    return bad;
+}

@@ -24,6 +24,9 @@
  *   ref_rave_backup_batch src/mcts/mcts_engine_tree.cpp:288-331 (RAVE part of backPropagate; not dispatched
  *                         by the reference's live search loop)
  *   ref_reroot_child      src/mcts/mcts_engine_search.cpp:1029-1075 (searchWithTreeReuse)
+ *   ref_mt64_*, ref_zobrist_tables  src/utils/zobrist_hash.cpp:9-36,129-131 (std::mt19937_64 stream of the tables)
+ *   ref_position_key      src/games/gomoku/gomoku_state.cpp:947-957 (compute_hash_signature_internal)
+ *   ref_leaf_keys         src/mcts/mcts_engine_batch_tree_simple.cpp:119-124,133-137 (clone, replay, getHash)
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
  *
@@ -195,6 +198,25 @@ int ref_tt_insert(ref_tt_slot *slots, int32_t log2_slots, uint64_t key, int32_t 
 /* out_node[i] = node stored under keys[i] with depth >= min_depth, else -1; returns hits */
 int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_t *keys, int64_t n,
                      int32_t min_depth, int32_t *out_node);
+
+/* ---- position keys: utils::ZobristHash tables and GomokuState::getHash() of a replayed path ---- */
+typedef struct ref_mt64 {
+    uint64_t mt[312];
+    int idx;
+} ref_mt64;
+void ref_mt64_seed(ref_mt64 *g, uint64_t seed);
+uint64_t ref_mt64_next(ref_mt64 *g);
+/* piece[n_piece][board_size * board_size], player[n_players]; -1 for arguments the constructor rejects
+ * and for seed 0 (the reference then seeds from the clock) */
+int ref_zobrist_tables(int32_t board_size, int32_t n_piece, int32_t n_players, uint32_t seed, uint64_t *piece,
+                       uint64_t *player);
+/* board[cell] = 0 empty, 1 BLACK, 2 WHITE; current_player 1 or 2; piece[side * piece_stride + cell] */
+uint64_t ref_position_key(const int8_t *board, int32_t cells, const uint64_t *piece, int64_t piece_stride,
+                          const uint64_t *player, int32_t current_player);
+/* paths row-major [B][stride]; root_boards [B][cells]; root_player [B] in {1, 2}; returns bad paths */
+int32_t ref_leaf_keys(const ref_tree *t, const int32_t *paths, const int32_t *path_len, int32_t B, int32_t stride,
+                      const int8_t *root_boards, const int32_t *root_player, int32_t cells, const uint64_t *piece,
+                      int64_t piece_stride, const uint64_t *player, uint64_t *out);
 
 #ifdef __cplusplus
 }

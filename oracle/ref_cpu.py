@@ -77,6 +77,17 @@ def lib():
         L.ref_tt_insert.restype = C.c_int
         L.ref_tt_probe.argtypes = [C.c_void_p, C.c_int32, u64p, C.c_int64, C.c_int32, i32p]
         L.ref_tt_probe.restype = C.c_int64
+        L.ref_zobrist_tables.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_uint32, u64p, u64p]
+        L.ref_zobrist_tables.restype = C.c_int
+        L.ref_position_key.argtypes = [C.c_void_p, C.c_int32, u64p, C.c_int64, u64p, C.c_int32]
+        L.ref_position_key.restype = C.c_uint64
+        L.ref_leaf_keys.argtypes = [C.POINTER(_Tree), i32p, i32p, C.c_int32, C.c_int32, C.c_void_p, i32p, C.c_int32,
+                                    u64p, C.c_int64, u64p, u64p]
+        L.ref_leaf_keys.restype = C.c_int32
+        L.ref_mt64_seed.argtypes = [C.c_void_p, C.c_uint64]
+        L.ref_mt64_seed.restype = None
+        L.ref_mt64_next.argtypes = [C.c_void_p]
+        L.ref_mt64_next.restype = C.c_uint64
         _LIB = L
     return _LIB
 
@@ -301,3 +312,46 @@ class RefTT:
         hits = lib().ref_tt_probe(self.slots.ctypes.data, self.log2, _ptr(keys, u64p), len(keys), int(min_depth),
                                   _ptr(out, i32p))
         return out, int(hits)
+
+
+def mt19937_64(seed, count):
+    """The first `count` outputs of std::mt19937_64(seed)."""
+    g = (C.c_uint64 * 313)()
+    lib().ref_mt64_seed(g, int(seed))
+    return np.array([lib().ref_mt64_next(g) for _ in range(count)], dtype=np.uint64)
+
+
+def zobrist_tables(board_size, n_piece, n_players, seed):
+    """piece [n_piece, board_size**2], player [n_players] of ZobristHash(board_size, n_piece, n_players, seed)."""
+    piece = np.empty((n_piece, board_size * board_size), np.uint64)
+    player = np.empty(n_players, np.uint64)
+    rc = lib().ref_zobrist_tables(int(board_size), int(n_piece), int(n_players), int(seed), _ptr(piece, u64p),
+                                  _ptr(player, u64p))
+    if rc != 0:
+        raise ValueError("arguments the ZobristHash constructor rejects, or seed 0")
+    return piece, player
+
+
+def position_key(board, piece, player, current_player):
+    """compute_hash_signature_internal of a board (0 empty, 1 BLACK, 2 WHITE) with `current_player` to move."""
+    board = np.ascontiguousarray(board, np.int8)
+    piece = np.ascontiguousarray(piece, np.uint64)
+    player = np.ascontiguousarray(player, np.uint64)
+    return int(lib().ref_position_key(board.ctypes.data, len(board), _ptr(piece, u64p), piece.shape[1],
+                                      _ptr(player, u64p), int(current_player)))
+
+
+def leaf_keys(tree, paths, path_len, root_boards, root_player, piece, player):
+    """getHash() of every path's replayed state; (keys, number of bad paths)."""
+    paths = np.ascontiguousarray(paths, np.int32)
+    path_len = np.ascontiguousarray(path_len, np.int32)
+    root_boards = np.ascontiguousarray(root_boards, np.int8)
+    root_player = np.ascontiguousarray(root_player, np.int32)
+    piece = np.ascontiguousarray(piece, np.uint64)
+    player = np.ascontiguousarray(player, np.uint64)
+    B, cells = root_boards.shape
+    out = np.empty(B, np.uint64)
+    bad = lib().ref_leaf_keys(C.byref(tree._c), _ptr(paths, i32p), _ptr(path_len, i32p), B, paths.shape[1],
+                              root_boards.ctypes.data, _ptr(root_player, i32p), cells, _ptr(piece, u64p),
+                              piece.shape[1], _ptr(player, u64p), _ptr(out, u64p))
+    return out, int(bad)

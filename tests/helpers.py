@@ -90,3 +90,35 @@ def random_tree(seed, n_expand=40, fanout=(1, 12), max_depth=6, n_roots=1, mask_
         bits[:n] = np.array(legal, dtype=np.uint8)
         soa["legal"] = np.packbits(bits.reshape(-1, 32), axis=1, bitorder="little").view("<u4").reshape(-1).copy()
     return soa, np.array(roots, np.int32)
+
+
+def board_forest(seed, cells=225, root_stones=20, **kw):
+    """random_tree whose actions are moves of a stone-placing game on `cells` cells: every root gets a
+    random position (root_stones stones, sides alternating, so the side to move follows from the
+    parity), and the children of a node play distinct empty cells of the position the node stands
+    for.  Returns (soa, roots, root_boards [n_roots, cells] int8 with 0 empty / 1 / 2,
+    root_player [n_roots] in {1, 2})."""
+    soa, roots = random_tree(seed, **kw)
+    rng = np.random.default_rng(seed + 77)
+    cb, cc, act = soa["child_begin"], soa["child_count"], soa["action"]
+    boards = np.zeros((len(roots), cells), np.int8)
+    players = np.zeros(len(roots), np.int32)
+    for ri, root in enumerate(roots):
+        k = int(rng.integers(0, root_stones + 1))
+        for j, c in enumerate(rng.permutation(cells)[:k]):
+            boards[ri, c] = 1 + (j & 1)
+        players[ri] = 1 + (k & 1)
+        stack = [(int(root), set(np.nonzero(boards[ri])[0].tolist()))]
+        while stack:
+            node, used = stack.pop()
+            f = int(cc[node])
+            if f == 0:
+                continue
+            free = np.array(sorted(set(range(cells)) - used))
+            picks = rng.permutation(free)[:f]
+            assert len(picks) == f
+            for i in range(f):
+                child = int(cb[node]) + i
+                act[child] = int(picks[i])
+                stack.append((child, used | {int(picks[i])}))
+    return soa, roots, boards, players
