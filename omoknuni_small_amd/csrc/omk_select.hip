@@ -75,6 +75,7 @@ constexpr int kRunShortcutMin = 128;      // entries from which a run of one chi
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
 constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
+constexpr int kFastSinglesMax = 16384;    // traversals up to which the single-visitor kernel trades bytes for latency
 constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
                                           // is shared out like a heavy node's instead of left to one helper
 
@@ -127,6 +128,7 @@ struct Kids {
     uint32_t k1[R];
     uint32_t k2[R];
     bool part[R];
+    int2 sp[R];  // (child_begin, child_count) of the child, where load_kids is asked for it (SPAN)
 };
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
@@ -183,9 +185,12 @@ struct WaveLds {
 // AHEAD: ask for the statistics of every child in range before the legality bits are known
 // (one memory round trip instead of two; reads the statistics of illegal children too, so
 // only where latency matters more than traffic).
-template <int R, bool RAVE, bool AHEAD = false>
+// SPAN (with AHEAD): the child range of every child in range comes along, so that a walk that goes on into
+// one of them does not make one more dependent trip to memory for it.
+template <int R, bool RAVE, bool AHEAD = false, bool SPAN = false>
 __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
                                           Kids<R, RAVE> &k) {
+    static_assert(AHEAD || !SPAN, "the child ranges are only fetched by the look-ahead variant");
     if (AHEAD) {
         int rn[R];
         float rw[R];
@@ -202,6 +207,7 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
             k.vl[r] = in ? f.VL[id] : 0;
             rn[r] = RAVE && in ? f.rN[id] : 0;
             rw[r] = RAVE && in ? f.rW[id] : 0.0f;
+            if (SPAN) k.sp[r] = in ? f.span[id] : int2{0, 0};
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -331,11 +337,16 @@ __device__ __forceinline__ NodeCtx node_ctx(const ForestDev &f, const SelectArgs
 
 // One selection for a single visitor.  Returns the child index or -1; np_child receives
 // the visit count of the chosen child (the next node's N_parent).
-template <int R, bool RAVE>
+//
+// FAST: for a launch with few walkers, where a walk is as slow as its chain of dependent trips to
+// memory (child range, legality bits, statistics: three per level) and the memory system is idle:
+// statistics and child ranges of all children in range are asked for at once (one trip per level,
+// about 1.5 times the bytes); span_child then receives the chosen child's range.
+template <int R, bool RAVE, bool FAST>
 __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
-                                             int &np_child) {
+                                             int &np_child, int2 &span_child) {
     Kids<R, RAVE> k;
-    load_kids<R, RAVE>(f, c.cb, c.nelig, lane, a.rave_k, k);
+    load_kids<R, RAVE, FAST, FAST>(f, c.cb, c.nelig, lane, a.rave_k, k);
 #pragma unroll
     for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep);
     uint32_t bk, bpos;
@@ -348,6 +359,18 @@ __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArg
         if (r == (i >> 6)) nsel = k.n[r];
     }
     np_child = __builtin_amdgcn_readlane(nsel, i & 63);
+    if (FAST) {
+        int sx = 0, sy = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (r == (i >> 6)) {
+                sx = k.sp[r].x;
+                sy = k.sp[r].y;
+            }
+        }
+        span_child.x = __builtin_amdgcn_readlane(sx, i & 63);
+        span_child.y = __builtin_amdgcn_readlane(sy, i & 63);
+    }
     return i;
 }
 
@@ -2512,7 +2535,7 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
 }
 
 // Single visitors: the rest of the path is private to the visitor, one wavefront walks it.
-template <int RMAX, bool RAVE>
+template <int RMAX, bool RAVE, bool FAST>
 __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -2526,13 +2549,22 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
         np = f.N[node];
         if (lane == 0) a.paths[t] = node;
     }
+    // the widest fan-out class has no registers to spare for the child ranges
+    constexpr bool kFastWide = FAST && RMAX <= 6;
+    bool have_span = false;
+    int2 span = int2{0, 0};
     for (;;) {
-        NodeCtx c = node_ctx(f, a, node, np);
+        NodeCtx c = node_ctx(f, a, node, np, have_span, span);
         int i = -1;
         int np_child = 0;
         if (c.cc > 0 && d < a.max_depth) {
-            if (c.cc <= kWave) i = select_single<1, RAVE>(f, a, c, lane, np_child);
-            else i = select_single<RMAX, RAVE>(f, a, c, lane, np_child);
+            if (c.cc <= kWave) {
+                i = select_single<1, RAVE, FAST>(f, a, c, lane, np_child, span);
+                have_span = FAST;
+            } else {
+                i = select_single<RMAX, RAVE, kFastWide>(f, a, c, lane, np_child, span);
+                have_span = kFastWide;
+            }
         }
         if (i < 0) {
             if (lane == 0) {
@@ -2605,7 +2637,13 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
 #endif
         hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kTeam), 0, s, f, a);
     }
-    hipLaunchKernelGGL((k_select_singles<RMAX, RAVE>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
+    // Few walkers cannot keep the memory system busy: then the variant that spends bytes to save
+    // dependent trips (select_single, FAST).  The number of lone visitors is only known on the
+    // device; the number of traversals bounds it.
+    if (n_traversals <= kFastSinglesMax)
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, true>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
+    else
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, false>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
     return hipGetLastError();
 }
 
