@@ -85,6 +85,9 @@ struct omk_forest {
 };
 
 constexpr int kSchedStep = 1024;  // int32 words between two scheduler words: 4 KiB
+// Simulations cut by max_depth: two counters, used in turn (select calls of even / odd number).  Every
+// select clears the counter of the next one, so that a select of lone traversals needs no reset launch.
+constexpr int kTruncatedWord = 40;
 
 struct omk_batch {
     omk_forest *f = nullptr;
@@ -99,7 +102,8 @@ struct omk_batch {
     int32_t n_singles0 = 0;
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
-    // [0] simulations cut by max_depth, [1..16] work statistics, [17] single-visitor queue length;
+    // [1..16] work statistics, [17] single-visitor queue length, [32] status of omk_batch_leaf_keys,
+    // [40..41] simulations cut by max_depth (kTruncatedWord);
     // the scheduler words of the multi-visitor kernel follow at 4 KiB steps (kSchedStep), so
     // that each lies in a memory channel of its own
     int32_t *counters = nullptr;
@@ -773,7 +777,8 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.q_cap = b->q_cap;
     a.epoch = b->epoch;
     a.spin_limit = b->spin_limit;
-    a.truncated = b->counters + 0;
+    a.truncated = b->counters + kTruncatedWord + (b->epoch & 1);
+    a.truncated_next = b->counters + kTruncatedWord + ((b->epoch + 1) & 1);
     a.stats = b->stats_on ? b->counters + 1 : nullptr;
     a.n_singles = b->counters + 17;
     a.sched_head = b->counters + 1 * kSchedStep;
@@ -1012,7 +1017,8 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count) {
     if (!b || !h_count) return fail(OMK_ERR_INVALID, "omk_batch_truncated: null argument");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_truncated: no selected paths");
     if (int rc = use_device(b->f)) return rc;
-    HIP_TRY(hipMemcpyAsync(h_count, b->counters + 0, 4, hipMemcpyDeviceToHost, b->f->stream));
+    HIP_TRY(hipMemcpyAsync(h_count, b->counters + kTruncatedWord + (b->epoch & 1), 4, hipMemcpyDeviceToHost,
+                           b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     return OMK_OK;
 }

@@ -73,7 +73,8 @@ struct SelectArgs {
     int32_t *paths;        // level-major [max_depth+1][stride]
     int32_t *path_len;
     int32_t *leaf;
-    int32_t *truncated;
+    int32_t *truncated;       // simulations cut by max_depth in this select: zero when it starts ...
+    int32_t *truncated_next;  // ... because the select before it cleared it: the counter of the next select
     int32_t *stats;        // optional 8 counters describing how the work was done (nullptr = off)
     int32_t stride;
     int32_t max_depth;

@@ -128,7 +128,6 @@ struct Kids {
     uint32_t k1[R];
     uint32_t k2[R];
     bool part[R];
-    int2 sp[R];  // (child_begin, child_count) of the child, where load_kids is asked for it (SPAN)
 };
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
@@ -185,11 +184,12 @@ struct WaveLds {
 // AHEAD: ask for the statistics of every child in range before the legality bits are known
 // (one memory round trip instead of two; reads the statistics of illegal children too, so
 // only where latency matters more than traffic).
-// SPAN (with AHEAD): the child range of every child in range comes along, so that a walk that goes on into
-// one of them does not make one more dependent trip to memory for it.
+// SPAN (with AHEAD): the child range of every child in range comes along (sp[r], like the
+// statistics), so that a walk that goes on into one of them does not make one more dependent trip
+// to memory for it.
 template <int R, bool RAVE, bool AHEAD = false, bool SPAN = false>
 __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
-                                          Kids<R, RAVE> &k) {
+                                          Kids<R, RAVE> &k, int2 *sp = nullptr) {
     static_assert(AHEAD || !SPAN, "the child ranges are only fetched by the look-ahead variant");
     if (AHEAD) {
         int rn[R];
@@ -207,7 +207,7 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
             k.vl[r] = in ? f.VL[id] : 0;
             rn[r] = RAVE && in ? f.rN[id] : 0;
             rw[r] = RAVE && in ? f.rW[id] : 0.0f;
-            if (SPAN) k.sp[r] = in ? f.span[id] : int2{0, 0};
+            if (SPAN) sp[r] = in ? f.span[id] : int2{0, 0};
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -346,7 +346,8 @@ template <int R, bool RAVE, bool FAST>
 __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              int &np_child, int2 &span_child) {
     Kids<R, RAVE> k;
-    load_kids<R, RAVE, FAST, FAST>(f, c.cb, c.nelig, lane, a.rave_k, k);
+    int2 sp[R];
+    load_kids<R, RAVE, FAST, FAST>(f, c.cb, c.nelig, lane, a.rave_k, k, sp);
 #pragma unroll
     for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep);
     uint32_t bk, bpos;
@@ -364,8 +365,8 @@ __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArg
 #pragma unroll
         for (int r = 0; r < R; r++) {
             if (r == (i >> 6)) {
-                sx = k.sp[r].x;
-                sy = k.sp[r].y;
+                sx = sp[r].x;
+                sy = sp[r].y;
             }
         }
         span_child.x = __builtin_amdgcn_readlane(sx, i & 63);
@@ -2536,11 +2537,19 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
 
 // Single visitors: the rest of the path is private to the visitor, one wavefront walks it.
 template <int RMAX, bool RAVE, bool FAST>
-__global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a) {
+__global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a, int seeded) {
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (wave >= *a.n_singles) return;
-    const Item it = a.singles_q[wave];
+    // seeded > 0: every traversal of the batch is alone at its root and this is the only launch of
+    // the select (no reset launch, no multi-visitor launch): the walkers are the `seeded` entries
+    // the host prepared, and one thread leaves the scheduler words as a reset would have
+    if (seeded > 0 && wave == 0 && lane == 0) {
+        *a.n_singles = seeded;
+        *a.truncated_next = 0;
+        a.sched_wait[1] = 0;
+    }
+    if (wave >= (seeded > 0 ? seeded : *a.n_singles)) return;
+    const Item it = seeded > 0 ? a.singles0[wave] : a.singles_q[wave];
     int node = it.node;
     const int t = it.off;
     int d = it.depth;
@@ -2593,6 +2602,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
     const int step = gridDim.x * blockDim.x;
     if (gid == 0) {
         *a.truncated = 0;
+        *a.truncated_next = 0;
         *a.n_singles = n_singles0;
         *a.sched_head = 0;
         *a.sched_tail = n_items0;
@@ -2619,7 +2629,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
 
 template <int RMAX, bool RAVE>
 static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals,
-                                 int n_cus, hipStream_t s) {
+                                 int n_cus, int seeded, hipStream_t s) {
     if (n_items0 > 0) {
         // as many wavefronts as can be resident, but no more than there can be items at once
         // (an item has at least two visitors)
@@ -2639,22 +2649,31 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
     }
     // Few walkers cannot keep the memory system busy: then the variant that spends bytes to save
     // dependent trips (select_single, FAST).  The number of lone visitors is only known on the
-    // device; the number of traversals bounds it.
-    if (n_traversals <= kFastSinglesMax)
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, true>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
+    // device; the number of traversals bounds it.  Measured: it pays on a board layout (legal
+    // mask: three trips per level become one), not on a compact one (two become one).
+    if (n_traversals <= kFastSinglesMax && f.legal)
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, true>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a,
+                           seeded);
     else
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, false>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a);
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, false>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a,
+                           seeded);
     return hipGetLastError();
 }
 
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
                          int max_fanout, bool rave, int n_cus, hipStream_t s) {
-    int reset_blocks = (n_traversals + 255) / 256;
-    hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
-                       n_traversals - n_singles0, n_traversals);
-#define OMK_DISPATCH(RM)                                                                  \
-    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, s)        \
-                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, s)
+    // Every traversal alone at its root (one per tree: leaf-parallel self-play): the single-visitor
+    // kernel is the whole select and takes its walkers from the host's list; every walker writes its
+    // own leaf and path length, so nothing has to be cleared first.  Otherwise the reset launch.
+    const int seeded = n_items0 == 0 && n_singles0 == n_traversals && !a.stats ? n_singles0 : 0;
+    if (seeded == 0) {
+        int reset_blocks = (n_traversals + 255) / 256;
+        hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
+                           n_traversals - n_singles0, n_traversals);
+    }
+#define OMK_DISPATCH(RM)                                                                       \
+    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, seeded, s)     \
+                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, seeded, s)
     if (max_fanout <= 64) { OMK_DISPATCH(1); }
     if (max_fanout <= 256) { OMK_DISPATCH(4); }
     if (max_fanout <= 384) { OMK_DISPATCH(6); }
