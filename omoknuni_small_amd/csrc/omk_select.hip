@@ -338,16 +338,19 @@ __device__ __forceinline__ NodeCtx node_ctx(const ForestDev &f, const SelectArgs
 // One selection for a single visitor.  Returns the child index or -1; np_child receives
 // the visit count of the chosen child (the next node's N_parent).
 //
-// FAST: for a launch with few walkers, where a walk is as slow as its chain of dependent trips to
-// memory (child range, legality bits, statistics: three per level) and the memory system is idle:
-// statistics and child ranges of all children in range are asked for at once (one trip per level,
-// about 1.5 times the bytes); span_child then receives the chosen child's range.
-template <int R, bool RAVE, bool FAST>
+// A walk is a chain of dependent trips to memory: child range, legality bits, statistics, three per
+// level on a layout with a legal mask.  AHEAD asks for the statistics of all children in range
+// before the legality bits are known (two trips; the cache lines of the illegal ones are fetched
+// anyway).  FAST, for a launch with few walkers and an idle memory system, also asks for the child
+// ranges of all of them (one trip, about 1.5 times the bytes); span_child then receives the chosen
+// child's range.
+template <int R, bool RAVE, bool AHEAD, bool FAST>
 __device__ __forceinline__ int select_single(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                              int &np_child, int2 &span_child) {
+    static_assert(AHEAD || !FAST, "FAST includes AHEAD");
     Kids<R, RAVE> k;
     int2 sp[R];
-    load_kids<R, RAVE, FAST, FAST>(f, c.cb, c.nelig, lane, a.rave_k, k, sp);
+    load_kids<R, RAVE, AHEAD, FAST>(f, c.cb, c.nelig, lane, a.rave_k, k, sp);
 #pragma unroll
     for (int r = 0; r < R; r++) score_round<R, RAVE>(k, r, c.ep);
     uint32_t bk, bpos;
@@ -2536,8 +2539,10 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
 }
 
 // Single visitors: the rest of the path is private to the visitor, one wavefront walks it.
-template <int RMAX, bool RAVE, bool FAST>
+// MODE 0: plain loads; 1: AHEAD; 2: AHEAD and FAST (select_single).
+template <int RMAX, bool RAVE, int MODE>
 __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a, int seeded) {
+    constexpr bool AHEAD = MODE >= 1, FAST = MODE >= 2;
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     // seeded > 0: every traversal of the batch is alone at its root and this is the only launch of
@@ -2568,10 +2573,10 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
         int np_child = 0;
         if (c.cc > 0 && d < a.max_depth) {
             if (c.cc <= kWave) {
-                i = select_single<1, RAVE, FAST>(f, a, c, lane, np_child, span);
+                i = select_single<1, RAVE, AHEAD, FAST>(f, a, c, lane, np_child, span);
                 have_span = FAST;
             } else {
-                i = select_single<RMAX, RAVE, kFastWide>(f, a, c, lane, np_child, span);
+                i = select_single<RMAX, RAVE, AHEAD, kFastWide>(f, a, c, lane, np_child, span);
                 have_span = kFastWide;
             }
         }
@@ -2651,12 +2656,13 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_
     // dependent trips (select_single, FAST).  The number of lone visitors is only known on the
     // device; the number of traversals bounds it.  Measured: it pays on a board layout (legal
     // mask: three trips per level become one), not on a compact one (two become one).
-    if (n_traversals <= kFastSinglesMax && f.legal)
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, true>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a,
-                           seeded);
+    const dim3 grid((n_traversals + 3) / 4), block(256);
+    if (!f.legal)
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 0>), grid, block, 0, s, f, a, seeded);
+    else if (n_traversals <= kFastSinglesMax)
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 2>), grid, block, 0, s, f, a, seeded);
     else
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, false>), dim3((n_traversals + 3) / 4), dim3(256), 0, s, f, a,
-                           seeded);
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 1>), grid, block, 0, s, f, a, seeded);
     return hipGetLastError();
 }
 
