@@ -265,6 +265,10 @@ def main():
             "algorithmic_bytes_per_step": sel_bytes,
             "launches_per_step": launches_per_select,
             "avg_launch_us": sel_ms_step * 1e3 / launches_per_select,
+            "launch_covers": "the whole selection of a step, HIP events around it: " +
+                             ("k_select_reset + k_select_groups + k_select_singles" if has_groups
+                              else "k_select_singles alone (no reset launch when every traversal is alone at its root)")
+                             + "; rocprofv3's per-kernel averages add up to it",
             "backup_algorithmic_bytes_per_step": bak_bytes,
             "backup_achieved": bak_bytes / (bak_ms_step * 1e-3) / 1e9,
         },
