@@ -110,6 +110,7 @@ struct omk_batch {
     int32_t poll_sleep = 1;
     bool stats_on = false;
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
+    int32_t *single_ready = nullptr;  // the same per entry of the single-visitor queue
     int32_t *hctx = nullptr;     // contexts of heavy nodes
     int32_t *list_flag = nullptr;  // per visitor-list start: which depth's list is complete
     int32_t hctx_cap = 0;
@@ -651,8 +652,10 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->seg[1], B);
     if (e == hipSuccess) e = dalloc(&b->sc_child, 2 * B);  // two halves, alternating with the depth
     if (e == hipSuccess) e = dalloc(&b->sc_occ, 2 * B);
-    if (e == hipSuccess) e = dalloc(&b->counters, 4 * kSchedStep);
-    if (e == hipSuccess) e = hipMemset(b->counters, 0, 4 * kSchedStep * 4);
+    if (e == hipSuccess) e = dalloc(&b->counters, 5 * kSchedStep);
+    if (e == hipSuccess) e = hipMemset(b->counters, 0, 5 * kSchedStep * 4);
+    if (e == hipSuccess) e = dalloc(&b->single_ready, max_traversals);
+    if (e == hipSuccess) e = hipMemset(b->single_ready, 0, (size_t)std::max(max_traversals, 1) * 4);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&b->n_cus, hipDeviceAttributeMultiprocessorCount, f->device);
     if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
@@ -672,7 +675,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf, b->list_flag};
+                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf, b->list_flag, b->single_ready};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -770,6 +773,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.seg[1] = b->seg[1];
     if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
         HIP_TRY(hipMemsetAsync(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4, f->stream));
+        HIP_TRY(hipMemsetAsync(b->single_ready, 0, (size_t)std::max(b->max_traversals, 1) * 4, f->stream));
         b->epoch = 0;
     }
     b->epoch++;
@@ -784,6 +788,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.sched_head = b->counters + 1 * kSchedStep;
     a.sched_tail = b->counters + 2 * kSchedStep;
     a.sched_wait = b->counters + 3 * kSchedStep;
+    a.singles_head = b->counters + 4 * kSchedStep;
+    a.single_ready = b->single_ready;
+    a.n_trav = b->n;
+    a.n_team_blocks = 0;
+    a.fast_singles = 0;
     a.poll_sleep = b->poll_sleep;
     a.hctx = b->hctx;
     a.hctx_n = b->counters + 2 * kSchedStep + 64;
@@ -1004,6 +1013,12 @@ int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t 
         return fail(OMK_ERR_STATE,
                     "omk_batch_read: the selection gave up (a wavefront waited longer than the spin limit for the "
                     "visitor list at %d of depth %d, complete to depth %d); its paths are incomplete, revert the "
+                    "virtual losses with omk_forest_upload or omk_revert_vl_paths over known paths",
+                    ab[1], ab[2], ab[3]);
+    if (ab[0] == 4)
+        return fail(OMK_ERR_STATE,
+                    "omk_batch_read: the selection gave up (a wavefront waited longer than the spin limit for entry %d "
+                    "of the single-visitor queue, %d written, %d visitors open); its paths are incomplete, revert the "
                     "virtual losses with omk_forest_upload or omk_revert_vl_paths over known paths",
                     ab[1], ab[2], ab[3]);
     if (ab[0])

@@ -67,6 +67,11 @@ struct SelectArgs {
     int32_t dbg_grid;      // cap on the blocks of the multi-visitor kernel (0 = none)
 #endif
     int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag
+    int32_t *single_ready;  // per entry of the single-visitor queue: number of the select call that wrote it
+    int32_t *singles_head;  // tickets of the walkers of the persistent launch
+    int32_t n_trav;         // traversals of the batch (entries the single-visitor queue can hold)
+    int32_t n_team_blocks;  // blocks of the persistent launch that are teams; the blocks behind them are walkers
+    int32_t fast_singles;   // the walkers use the variant of select_single that trades bytes for latency
     int32_t *seg[2];       // visitor lists of level L >= 1 live in seg[(L-1)&1]
     int32_t *sc_child;     // per visitor: chosen child index (two halves of `stride`, alternating with the depth)
     int32_t *sc_occ;       // per visitor: how many earlier visitors of the item chose the same child

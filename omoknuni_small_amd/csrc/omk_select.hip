@@ -2203,6 +2203,12 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         for (int r = 0; r < R; r++)
             if (cnt[r] > 1)
                 __hip_atomic_store(a.list_flag + off + excl[r], depth + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // ... and the walkers of the persistent launch that their lone visitors are there
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (cnt[r] == 1)
+                __hip_atomic_store(a.single_ready + lone0 + lds.st_vl[r * kWave + lane], a.epoch, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
         if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);
         next.node = -1;
         wave_sync_memory();
@@ -2241,12 +2247,16 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         slot0 += __popcll(has[r]);
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + c.cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
     }
-    if (n_pushed > 0) {
+    if (n_pushed > 0 || n_lone > 0) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
 #pragma unroll
-        for (int r = 0; r < R; r++)
+        for (int r = 0; r < R; r++) {
             if (myslot[r] >= 0)
                 __hip_atomic_store(a.q_ready + myslot[r], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (cnt[r] == 1)
+                __hip_atomic_store(a.single_ready + lone0 + lds.st_vl[r * kWave + lane], a.epoch, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);  // lone visitors leave the multi-visitor items
     next.node = -1;
@@ -2467,12 +2477,16 @@ __device__ __forceinline__ void partition_async(const ForestDev &f, const Select
         slot0 += __popcll(has[r]);
         if (cnt[r] > 0 && a.vl > 0) atomicAdd(f.VL + cb + i, (int)((uint32_t)a.vl * (uint32_t)cnt[r]));
     }
-    if (n_push > 0) {
+    if (n_push > 0 || n_lone > 0) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
 #pragma unroll
-        for (int r = 0; r < R; r++)
+        for (int r = 0; r < R; r++) {
             if (myslot[r] >= 0)
                 __hip_atomic_store(a.q_ready + myslot[r], a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (cnt[r] == 1)
+                __hip_atomic_store(a.single_ready + lone0 + pl.lone[r * kWave + lane], a.epoch, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);  // lone visitors leave the multi-visitor items
 }
@@ -2505,10 +2519,17 @@ __device__ __forceinline__ void team_help(const ForestDev &f, const SelectArgs &
 }
 
 template <int RMAX, bool RAVE>
+__device__ void walkers_loop(ForestDev f, SelectArgs a, int lane);
+
+template <int RMAX, bool RAVE>
 __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs a) {
     __shared__ WaveLds<RMAX> s_lds;
     __shared__ PartLds<RMAX> s_part;
     const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= a.n_team_blocks) {
+        walkers_loop<RMAX, RAVE>(f, a, tid & 63);
+        return;
+    }
     if (tid < kWave) {
         // every path out of the owner's loop comes back here: the helpers are always released
         bool pending = false;
@@ -2539,22 +2560,11 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
 }
 
 // Single visitors: the rest of the path is private to the visitor, one wavefront walks it.
-// MODE 0: plain loads; 1: AHEAD; 2: AHEAD and FAST (select_single).
+// One lone visitor from its item to its leaf.  MODE 0: plain loads; 1: AHEAD; 2: AHEAD and FAST
+// (select_single).
 template <int RMAX, bool RAVE, int MODE>
-__global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a, int seeded) {
+__device__ __forceinline__ void walk_single(const ForestDev &f, const SelectArgs &a, const Item &it, int lane) {
     constexpr bool AHEAD = MODE >= 1, FAST = MODE >= 2;
-    const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    // seeded > 0: every traversal of the batch is alone at its root and this is the only launch of
-    // the select (no reset launch, no multi-visitor launch): the walkers are the `seeded` entries
-    // the host prepared, and one thread leaves the scheduler words as a reset would have
-    if (seeded > 0 && wave == 0 && lane == 0) {
-        *a.n_singles = seeded;
-        *a.truncated_next = 0;
-        a.sched_wait[1] = 0;
-    }
-    if (wave >= (seeded > 0 ? seeded : *a.n_singles)) return;
-    const Item it = seeded > 0 ? a.singles0[wave] : a.singles_q[wave];
     int node = it.node;
     const int t = it.off;
     int d = it.depth;
@@ -2600,6 +2610,79 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
     }
 }
 
+// The kernel of a select whose traversals are all alone at their roots (one per tree): the
+// walkers are the `seeded` entries the host prepared, no other launch belongs to the select, and
+// one thread leaves the scheduler words as a reset would have.
+template <int RMAX, bool RAVE, int MODE>
+__global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs a, int seeded) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave == 0 && lane == 0) {
+        *a.n_singles = seeded;
+        *a.truncated_next = 0;
+        a.sched_wait[1] = 0;
+    }
+    if (wave >= seeded) return;
+    walk_single<RMAX, RAVE, MODE>(f, a, a.singles0[wave], lane);
+}
+
+// The walkers of the persistent launch: wavefronts of the blocks behind the teams take the lone
+// visitors one by one as the teams create them (a ticket, then the entry's ready word, set after
+// the release fence of whoever wrote the entry), so that a lone visitor walks while the chain of
+// crowded nodes is still being settled.  A walker leaves when no visitor is left in any
+// multi-visitor item (nothing more can come) and its ticket lies beyond the entries written.
+// The wait is bounded like every other.  Not inlined (the teams' code keeps its registers) and the
+// arguments by value (by reference, the kernel's own copies would have to live in memory, and every
+// use of them in the teams' code would become a load).
+template <int RMAX, bool RAVE>
+__device__ __noinline__ void walkers_loop(ForestDev f, SelectArgs a, int lane) {
+    for (;;) {
+        int ticket = 0;
+        if (lane == 0) ticket = atomicAdd(a.singles_head, 1);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        bool got = false;
+        for (int spins = 0;; spins++) {
+            int rdy = 0, open = 1, ab = 0, n = 0;
+            if (lane == 0) {
+                rdy = ticket < a.n_trav &&
+                      __hip_atomic_load(a.single_ready + ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
+                if (!rdy && (spins & 3) == 3) {
+                    open = __hip_atomic_load(a.sched_wait, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (open <= 0) {
+                        // every entry was counted before its writer let go of its visitors
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                        n = __hip_atomic_load(a.n_singles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (ticket < n) open = 1;  // counted, so its ready word is on its way
+                    }
+                }
+            }
+            rdy = __builtin_amdgcn_readfirstlane(rdy);
+            open = __builtin_amdgcn_readfirstlane(open);
+            ab = __builtin_amdgcn_readfirstlane(ab);
+            if (rdy) {
+                got = true;
+                break;
+            }
+            if (open <= 0 || ab) break;
+            if (spins >= a.spin_limit) {
+                if (lane == 0 && atomicCAS(a.sched_wait + 1, 0, 4) == 0) {
+                    a.sched_wait[2] = ticket;  // which entry never came, for the error message
+                    a.sched_wait[3] = *a.n_singles;
+                    a.sched_wait[4] = open;
+                }
+                break;
+            }
+            for (int z = 0; z < a.poll_sleep; z++) __builtin_amdgcn_s_sleep(32);
+        }
+        if (!got) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const Item it = a.singles_q[ticket];
+        if (a.fast_singles) walk_single<RMAX, RAVE, 2>(f, a, it, lane);
+        else walk_single<RMAX, RAVE, 0>(f, a, it, lane);
+    }
+}
+
 // Scheduler state, statistics, the work queue seeded with the items of the roots, and the
 // single-visitor queue seeded with the traversals that are alone at their root.
 __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0, int n_traversals) {
@@ -2610,6 +2693,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         *a.truncated_next = 0;
         *a.n_singles = n_singles0;
         *a.sched_head = 0;
+        *a.singles_head = 0;
         *a.sched_tail = n_items0;
         a.sched_wait[0] = open0;
         a.sched_wait[1] = 0;
@@ -2623,7 +2707,10 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         a.items_q[i] = a.items0[i];
         a.q_ready[i] = a.epoch;
     }
-    for (int i = gid; i < n_singles0; i += step) a.singles_q[i] = a.singles0[i];
+    for (int i = gid; i < n_singles0; i += step) {
+        a.singles_q[i] = a.singles0[i];
+        a.single_ready[i] = a.epoch;
+    }
     // a traversal that the selection does not finish (the kernel gave up) has an empty path
     for (int i = gid; i < n_traversals; i += step) {
         a.path_len[i] = 0;
@@ -2633,36 +2720,48 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
 }
 
 template <int RMAX, bool RAVE>
-static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a, int n_items0, int n_traversals,
-                                 int n_cus, int seeded, hipStream_t s) {
+static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n_items0, int n_traversals,
+                                 int n_cus, hipStream_t s) {
+    // Few walkers cannot keep the memory system busy: then the variant that spends bytes to save
+    // dependent trips (select_single, FAST).  The number of lone visitors is only known on the
+    // device; the number of traversals bounds it.  Measured: it pays on a board layout (legal
+    // mask: three trips per level become one), not on a compact one (two become one).
+    const bool fast = f.legal && n_traversals <= kFastSinglesMax;
     if (n_items0 > 0) {
-        // as many wavefronts as can be resident, but no more than there can be items at once
-        // (an item has at least two visitors)
+        // One persistent launch: teams for the multi-visitor items (as many as can be resident,
+        // but no more than there can be items at once: an item has at least two visitors) and,
+        // behind them, blocks of walkers for the lone visitors the teams create.
         int per_cu = 1;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_select_groups<RMAX, RAVE>, kTeam, 0) !=
                 hipSuccess ||
             per_cu < 1)
             per_cu = 1;
-        int grid = n_cus * per_cu;
-        const int most = n_traversals / 2;
-        if (grid > most) grid = most;
-        if (grid < 1) grid = 1;
+        int capacity = n_cus * per_cu;
 #ifdef OMK_TRACE
-        if (a.dbg_grid > 0 && grid > a.dbg_grid) grid = a.dbg_grid;
+        if (a0.dbg_grid > 0 && capacity > a0.dbg_grid) capacity = a0.dbg_grid;
 #endif
-        hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(grid), dim3(kTeam), 0, s, f, a);
+        if (capacity < 2) capacity = 2;
+        int walkers = n_traversals / 64;
+        if (walkers > capacity / 4) walkers = capacity / 4;
+        if (walkers < 1) walkers = 1;
+        int teams = capacity - walkers;
+        const int most = n_traversals / 2;
+        if (teams > most) teams = most;
+        if (teams < 1) teams = 1;
+        SelectArgs a = a0;
+        a.n_team_blocks = teams;
+        a.fast_singles = fast ? 1 : 0;
+        hipLaunchKernelGGL((k_select_groups<RMAX, RAVE>), dim3(teams + walkers), dim3(kTeam), 0, s, f, a);
+        return hipGetLastError();
     }
-    // Few walkers cannot keep the memory system busy: then the variant that spends bytes to save
-    // dependent trips (select_single, FAST).  The number of lone visitors is only known on the
-    // device; the number of traversals bounds it.  Measured: it pays on a board layout (legal
-    // mask: three trips per level become one), not on a compact one (two become one).
+    // every traversal is alone at its root: the walkers are the host's list
     const dim3 grid((n_traversals + 3) / 4), block(256);
     if (!f.legal)
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 0>), grid, block, 0, s, f, a, seeded);
-    else if (n_traversals <= kFastSinglesMax)
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 2>), grid, block, 0, s, f, a, seeded);
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 0>), grid, block, 0, s, f, a0, n_traversals);
+    else if (fast)
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 2>), grid, block, 0, s, f, a0, n_traversals);
     else
-        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 1>), grid, block, 0, s, f, a, seeded);
+        hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 1>), grid, block, 0, s, f, a0, n_traversals);
     return hipGetLastError();
 }
 
@@ -2670,16 +2769,17 @@ hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, 
                          int max_fanout, bool rave, int n_cus, hipStream_t s) {
     // Every traversal alone at its root (one per tree: leaf-parallel self-play): the single-visitor
     // kernel is the whole select and takes its walkers from the host's list; every walker writes its
-    // own leaf and path length, so nothing has to be cleared first.  Otherwise the reset launch.
-    const int seeded = n_items0 == 0 && n_singles0 == n_traversals && !a.stats ? n_singles0 : 0;
-    if (seeded == 0) {
+    // own leaf and path length, so nothing has to be cleared first (the statistics apart).
+    // Otherwise the reset launch.
+    const bool alone = n_items0 == 0 && n_singles0 == n_traversals;
+    if (!alone || a.stats) {
         int reset_blocks = (n_traversals + 255) / 256;
         hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
                            n_traversals - n_singles0, n_traversals);
     }
-#define OMK_DISPATCH(RM)                                                                       \
-    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, seeded, s)     \
-                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, seeded, s)
+#define OMK_DISPATCH(RM)                                                              \
+    return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, s)    \
+                : launch_kernels<RM, false>(f, a, n_items0, n_traversals, n_cus, s)
     if (max_fanout <= 64) { OMK_DISPATCH(1); }
     if (max_fanout <= 256) { OMK_DISPATCH(4); }
     if (max_fanout <= 384) { OMK_DISPATCH(6); }
