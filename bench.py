@@ -207,8 +207,9 @@ def main():
     batch.backup(vl)
     forest.sync()
     sel_bytes, bak_bytes, n_sel_steps = algorithmic_bytes(soa, meta, paths, plen, N_now)
-    # selection = 1 reset + 1 launch of the multi-visitor kernel (a persistent kernel over a work
-    # queue; only when any traversals share a root) + 1 launch of the single-visitor kernel; the
+    # selection = 1 reset + 1 persistent launch (teams over a work queue of multi-visitor items, and
+    # walkers for the lone visitors) when any traversals share a root, else 1 launch of the
+    # single-visitor kernel; the
     # roofline is quoted for the kernel that carries the work, with the whole selection phase
     # (HIP events around it on the forest's stream) as its launch duration
     has_groups = len(np.unique(troots)) < B
@@ -266,7 +267,7 @@ def main():
             "launches_per_step": launches_per_select,
             "avg_launch_us": sel_ms_step * 1e3 / launches_per_select,
             "launch_covers": "the whole selection of a step, HIP events around it: " +
-                             ("k_select_reset + k_select_groups + k_select_singles" if has_groups
+                             ("k_select_reset + k_select_groups (teams and walkers in one persistent launch)" if has_groups
                               else "k_select_singles alone (no reset launch when every traversal is alone at its root)")
                              + "; rocprofv3's per-kernel averages add up to it",
             "backup_algorithmic_bytes_per_step": bak_bytes,

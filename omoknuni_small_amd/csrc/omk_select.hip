@@ -75,6 +75,7 @@ constexpr int kRunShortcutMin = 128;      // entries from which a run of one chi
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
 constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
+constexpr int kMaxWalkerBlocks = 32;         // blocks of walkers of the persistent launch, at most
 constexpr int kFastSinglesMax = 16384;    // traversals up to which the single-visitor kernel trades bytes for latency
 constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
                                           // is shared out like a heavy node's instead of left to one helper
@@ -2743,6 +2744,7 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
         if (capacity < 2) capacity = 2;
         int walkers = n_traversals / 64;
         if (walkers > capacity / 4) walkers = capacity / 4;
+        if (walkers > kMaxWalkerBlocks) walkers = kMaxWalkerBlocks;  // idle walkers poll: more of them slow the teams
         if (walkers < 1) walkers = 1;
         int teams = capacity - walkers;
         const int most = n_traversals / 2;
