@@ -774,6 +774,8 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
         HIP_TRY(hipMemsetAsync(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4, f->stream));
         HIP_TRY(hipMemsetAsync(b->single_ready, 0, (size_t)std::max(b->max_traversals, 1) * 4, f->stream));
+        // the two depth-cap counters take turns by call parity, which this restart breaks once
+        HIP_TRY(hipMemsetAsync(b->counters + kTruncatedWord, 0, 2 * sizeof(int32_t), f->stream));
         b->epoch = 0;
     }
     b->epoch++;

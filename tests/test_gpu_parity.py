@@ -164,6 +164,32 @@ def test_depth_cap_truncates():
     assert n_near >= 0
 
 
+def test_depth_cap_counter_over_consecutive_selects():
+    """The count of depth-capped simulations is per select, whichever launches the select consists of:
+    lone traversals (one launch, no reset before it) twice in a row, then traversals that share
+    roots, then lone ones again."""
+    omk = _gpu()
+    soa, roots = random_tree(71, n_expand=120, fanout=(2, 4), max_depth=10, n_roots=6)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, 24, 2)
+    sp = omk.SelectParams(virtual_loss=0)
+
+    def run(troots):
+        b.set_roots(np.asarray(troots, np.int32))
+        b.select(sp)
+        _, plen, leaf, _ = b.read()
+        expect = int(((plen == 3) & (soa["child_count"][leaf] > 0)).sum())
+        assert expect > 0
+        assert b.truncated() == expect
+        return expect
+
+    alone = run(roots)
+    assert run(roots) == alone
+    run(np.repeat(roots, 4))
+    assert run(roots) == alone
+    run(roots[:3])
+
+
 def test_all_equal_scores_tie_to_lowest_index():
     # unvisited children with equal priors: every pick is an exact tie until virtual loss separates them
     k = 300
