@@ -7,18 +7,26 @@ backup of one value per leaf (update + revert virtual loss, sign flipped per ply
 the leaf-key table probes on the workload that has them.  Everything a step touches is
 resident in HBM before the timed region starts; nothing returns to the host inside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0..c4|wide]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c0..c4|wide] [--configs c0,c1,...|none]
 
-Prints ONE JSON line.  `value` is traversals per second over whole steps (every
-traversal is selected AND backed up inside the timed region).  `roofline` prices the
-selection kernel against HBM bandwidth with algorithmic bytes (what one selection step
-has to read: the statistics of the children that take part, the node header, the legal
-mask bits, the virtual-loss update), measured with HIP events on the stream the kernels
-run on.  `cpu_baseline` times the CPU checker on the host cores of the same machine, on a
-bounded number of steps of the same workload: the serial array restatement of the
-reference's selection / backup loops (one core) and the same arithmetic over the
-reference's own node layout (heap nodes, one cache line per atomic field) with its OpenMP
-loops, at one thread and at the host's share of cores; `value` is the fastest of them.
+Prints ONE JSON line.  The top-level fields are those of --workload (default c3, the
+"batch 4096" configuration the metric is quoted on); `per_config` holds the same measurement
+for every other benchmark configuration (c0 .. c4), each on its own full-size forest.
+
+`value` is traversals per second over whole steps (every traversal is selected AND backed up
+inside the timed region; the K timed steps run back to back).  `roofline` prices the selection
+against HBM bandwidth with algorithmic bytes (what one selection step has to read: the
+statistics of the children that take part, the node header, the legal mask bits, the
+virtual-loss update), summed over the K timed steps: after the timed run the statistics are
+put back to where they were when it started and the same K steps are run again with the paths
+read back after each one.  Durations come from HIP events on the stream the kernels run on.
+`parity` compares one more step on the very forest that was timed with the CPU checker (paths,
+leaves, N, virtual loss exact; W relative error; near ties as the checker counts them; table
+probes).  `cpu_baseline` times the CPU checker on the host cores of the same machine, on a
+bounded number of steps of the same workload: the serial array restatement of the reference's
+selection / backup loops (one core) and the same arithmetic over the reference's own node
+layout (heap nodes, one cache line per atomic field) with its OpenMP loops, at one thread and
+at the host's share of cores; `value` is the fastest of them.
 """
 import argparse
 import ctypes as C
@@ -33,6 +41,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+BENCH_CONFIGS = ["c0", "c1", "c2", "c3", "c4"]
 
 
 class HipEvents:
@@ -49,6 +58,9 @@ class HipEvents:
         ev = C.c_void_p()
         self._ok(self.hip.hipEventCreate(C.byref(ev)), "hipEventCreate")
         return ev
+
+    def destroy(self, ev):
+        self.hip.hipEventDestroy(ev)
 
     def record(self, ev, stream):
         self._ok(self.hip.hipEventRecord(ev, C.c_void_p(stream)), "hipEventRecord")
@@ -74,27 +86,340 @@ def legal_children_per_node(soa):
     return cs[np.minimum(cb + cc, n)] - cs[np.minimum(cb, n)]
 
 
-def algorithmic_bytes(soa, meta, paths, plen, N_now):
+class ByteModel:
     """Bytes one step has to move, by the per-unit model:
     selection step at a node with L participating children of F slots:
         L*16 (N, W, P, VL)  [+ L*8 RAVE]  + ceil(F/8) mask bytes (dense slots only)
         + 16 (child range, N_parent, flags) + 8 (virtual-loss update of the chosen child)
     backup of a path node: 24 (N, W, VL read-modify-write), + 4 per leaf value + 4 per path entry."""
-    L = legal_children_per_node(soa)
-    cc = soa["child_count"].astype(np.int64)
-    per_child = 24 if meta.get("has_rave") else 16
-    n_t, row = paths.shape
-    d_idx = np.arange(row)[None, :]
-    sel_mask = d_idx < (plen[:, None] - 1)  # a selection happens at every path node but the leaf
-    nodes = paths[sel_mask]
-    Lsel = L[nodes]
-    if meta.get("pw"):
-        k = np.ceil(np.sqrt(np.maximum(N_now[nodes].astype(np.float64), 1.0))).astype(np.int64)
-        Lsel = np.minimum(Lsel, np.maximum(k, 1))
-    mask_bytes = (cc[nodes] + 7) // 8 if soa.get("legal") is not None else 0
-    sel = int((Lsel * per_child + mask_bytes + 24).sum()) + int(4 * plen.sum())
-    bak = int(24 * plen.sum() + 4 * n_t + 4 * plen.sum())
-    return sel, bak, int(sel_mask.sum())
+
+    def __init__(self, soa, meta):
+        self.L = legal_children_per_node(soa)
+        self.cc = soa["child_count"].astype(np.int64)
+        self.per_child = 24 if meta.get("has_rave") else 16
+        self.pw = bool(meta.get("pw"))
+        self.dense = soa.get("legal") is not None
+
+    def step(self, paths, plen, N_at_select):
+        n_t, row = paths.shape
+        d_idx = np.arange(row)[None, :]
+        sel_mask = d_idx < (plen[:, None] - 1)  # a selection happens at every path node but the leaf
+        nodes = paths[sel_mask]
+        Lsel = self.L[nodes]
+        if self.pw:
+            k = np.ceil(np.sqrt(np.maximum(N_at_select[nodes].astype(np.float64), 1.0))).astype(np.int64)
+            Lsel = np.minimum(Lsel, np.maximum(k, 1))
+        mask_bytes = (self.cc[nodes] + 7) // 8 if self.dense else 0
+        sel = int((Lsel * self.per_child + mask_bytes + 24).sum()) + int(4 * plen.sum())
+        bak = int(24 * plen.sum() + 4 * n_t + 4 * plen.sum())
+        return sel, bak, int(sel_mask.sum())
+
+
+def visits_of(paths, plen, n_nodes):
+    """How often every node occurs on the paths of a step (what a backup adds to N)."""
+    row = paths.shape[1]
+    on_path = np.arange(row)[None, :] < plen[:, None]
+    return np.bincount(paths[on_path], minlength=n_nodes).astype(np.int32)
+
+
+def cpu_baseline(soa, meta, troots, values, seconds, max_steps):
+    """The CPU checker on the host's cores, on a bounded number of steps of the same workload."""
+    from oracle import ref_cpu as R
+    B, D, vl = len(troots), int(meta["max_depth"]), int(meta["virtual_loss"])
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                       rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+    done = 0
+    sel_s = bak_s = 0.0
+    t_start = time.perf_counter()
+    while done < 2 or (time.perf_counter() - t_start) < seconds / 2:
+        a = time.perf_counter()
+        rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
+        b = time.perf_counter()
+        ref.backup_batch(rpaths, rlen, values, vl)
+        c = time.perf_counter()
+        sel_s += b - a
+        bak_s += c - b
+        done += 1
+        if done >= max_steps:
+            break
+    del ref
+    soa_rate = B * done / (sel_s + bak_s)
+    out = {
+        "value": soa_rate,
+        "unit": "traversals/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "%d steps of the same workload (same forest, roots and leaf values) through the "
+                  "serial CPU restatement of selectChild / applyVirtualLoss / update / revertVirtualLoss" % done,
+        "soa_serial_select_traversals_per_s": B * done / sel_s,
+        "soa_serial_backups_per_s": B * done / bak_s,
+        "soa_serial_traversals_per_s": soa_rate,
+        "host_cores_visible": os.cpu_count(),
+    }
+    # The same arithmetic over the reference's own layout and threading: heap nodes with one
+    # cache line per atomic field, shared_ptr child vectors, OpenMP loops with
+    # schedule(dynamic, 1).  Timed with one thread and with the host's share of cores; the
+    # faster of the three figures becomes `value` (with several threads the traversal
+    # order, hence the result, depends on the schedule, as the reference's does).
+    if len(soa["N"]) <= 20_000_000:
+        from oracle import ref_ptr as RP
+        t_build = time.perf_counter()
+        pt = RP.PtrTree(soa)
+        t_build = time.perf_counter() - t_build
+        n_thr = max(1, min(16, os.cpu_count() or 1))
+        kw = dict(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                  rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+        rates = {}
+        for thr in sorted({1, n_thr}):
+            tot, steps_done = 0.0, 0
+            t_start = time.perf_counter()
+            while steps_done < 2 or (time.perf_counter() - t_start) < seconds / 4:
+                _, _, s_s, b_s = pt.step(troots, values, threads=thr, **kw)
+                tot += s_s + b_s
+                steps_done += 1
+                if steps_done >= max_steps:
+                    break
+            rates[thr] = B * steps_done / tot
+        pt.close()
+        out["pointer_tree_traversals_per_s"] = {str(k): v for k, v in rates.items()}
+        out["pointer_tree_node_bytes"] = RP.PtrTree.node_bytes()
+        out["pointer_tree_build_s"] = t_build
+        best_thr = max(rates, key=rates.get)
+        if rates[best_thr] > soa_rate:
+            out["value"] = rates[best_thr]
+            out["cores"] = best_thr
+            out["sample"] = ("steps of the same workload (same forest, roots and leaf values) through the CPU "
+                             "restatement over the reference's node layout (heap nodes, one cache line per "
+                             "atomic) and OpenMP loops, %d thread(s); the serial array checker and the "
+                             "one-thread figure are given beside it" % best_thr)
+    return out
+
+
+def parity_check(omk, soa, meta, forest, batch, tt, tt_ids, troots, values, params, steps=1):
+    """`steps` more steps on the forest that was just timed, on the device and through the CPU checker
+    (started from the device's current statistics), compared phase by phase."""
+    from oracle import ref_cpu as R
+    B, D, vl = len(troots), int(meta["max_depth"]), int(meta["virtual_loss"])
+    now = forest.download()
+    cur = dict(soa)
+    cur.update(N=now["N"], W=now["W"], VL=now["VL"])
+    ref = R.RefTree.from_soa(cur)
+    rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                       rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+    out = dict(checked_steps=steps, traversals_per_step=B, mismatched_traversals=0, move_lists_equal=True,
+               N_equal=True, VL_equal=True, W_max_rel_err=0.0, near_tie_traversals=0,
+               mismatches_outside_near_ties=0)
+    if tt is not None:
+        ref_tt = R.RefTT(4)
+        ref_tt.log2 = tt.log2
+        ref_tt.slots = tt.download()
+        out["tt_probes_equal"] = True
+        out["tt_hits"] = 0
+    for _ in range(steps):
+        rpaths, rlen, rleaf, near = ref.select_batch(troots, rp)
+        batch.select(params)
+        gpaths, glen, gleaf, gact = batch.read()
+        bad = (gpaths != rpaths).any(axis=1) | (glen != rlen) | (gleaf != rleaf)
+        out["mismatched_traversals"] += int(bad.sum())
+        out["mismatches_outside_near_ties"] += int((bad & (near < 0)).sum())
+        out["near_tie_traversals"] += int((near >= 0).sum())
+        out["move_lists_equal"] &= bool((gact == ref.gather_actions(rpaths, rlen)).all())
+        st = forest.download()
+        out["VL_equal"] &= bool((st["VL"] == ref.VL).all())
+        if tt is not None:
+            got = tt.probe_leaves(batch)
+            want, hits = ref_tt.probe(soa["hash"][rleaf])
+            out["tt_probes_equal"] &= bool((got == want).all())
+            out["tt_hits"] += hits
+        ref.backup_batch(rpaths, rlen, values, vl)
+        batch.backup(vl)
+        st = forest.download()
+        out["N_equal"] &= bool((st["N"] == ref.N).all())
+        out["VL_equal"] &= bool((st["VL"] == ref.VL).all())
+        err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
+        out["W_max_rel_err"] = max(out["W_max_rel_err"], float(err.max()))
+        ref.W[:] = st["W"]
+    out["ok"] = bool(out["mismatches_outside_near_ties"] == 0 and out["move_lists_equal"] and out["N_equal"]
+                     and out["VL_equal"] and out["W_max_rel_err"] <= 1e-5 and out.get("tt_probes_equal", True))
+    return out
+
+
+def traffic_of(workload):
+    """HBM bytes per selection from the committed profiler summary (not measured in this run)."""
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(tfile):
+        return None, None
+    with open(tfile) as fh:
+        tj = json.load(fh)
+    if workload not in tj:
+        return None, None
+    return tj[workload].get("selection_bytes_per_launch"), (
+        "profiles/hbm_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `%s`, scaled by the 64 MiB copy "
+        "kernel; not measured in this run" % tj[workload].get("command", "bench.py --workload %s" % workload))
+
+
+def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parity=True):
+    """Everything bench.py reports about one workload."""
+    kw = {}
+    if scale != 1.0:
+        kw["nodes_per_tree"] = max(1000, int(synth.CONFIGS[name]["nodes_per_tree"] * scale))
+    t0 = time.time()
+    soa, roots, meta = synth.generate(name, seed=seed, **kw)
+    gen_s = time.time() - t0
+    n_nodes = len(soa["N"])
+    B = int(meta["n_traversals"])
+    D = int(meta["max_depth"])
+    vl = int(meta["virtual_loss"])
+    troots = synth.traversal_roots(roots, B)
+    values = np.random.default_rng(seed + 1).uniform(-1, 1, B).astype(np.float32)
+    params = omk.SelectParams(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                              rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")))
+
+    forest = omk.Forest.from_soa(soa)
+    batch = omk.Batch(forest, B, D)
+    batch.set_roots(troots)
+    batch.set_values(values)
+    tt = None
+    tt_ids = None
+    d_probe = 0
+    if meta.get("tt_log2"):
+        tt = omk.TranspositionTable(forest, int(meta["tt_log2"]))
+        n_ins = 1 << (int(meta["tt_log2"]) - 1)  # 50 % load
+        tt_ids = np.unique(np.linspace(0, meta["n_nodes"] - 1, n_ins).astype(np.int64))
+        tt.insert(soa["hash"][tt_ids], tt_ids.astype(np.int32))
+        d_probe = forest.dev_alloc(B * 4)
+
+    def step():
+        batch.select(params)
+        if tt is not None:
+            tt.probe_leaves_dev(batch, d_probe)
+        batch.backup(vl)
+
+    ev = HipEvents()
+    stream = forest.get_stream()
+    for _ in range(warmup):
+        step()
+    forest.sync()
+    ev.device_sync()
+    start = forest.download()  # the statistics the timed steps start from
+
+    K = steps
+    e_sel0 = [ev.create() for _ in range(K)]
+    e_sel1 = [ev.create() for _ in range(K)]
+    e_end = [ev.create() for _ in range(K)]
+    t_wall0 = time.perf_counter()
+    for i in range(K):
+        ev.record(e_sel0[i], stream)
+        batch.select(params)
+        ev.record(e_sel1[i], stream)
+        if tt is not None:
+            tt.probe_leaves_dev(batch, d_probe)
+        batch.backup(vl)
+        ev.record(e_end[i], stream)
+    forest.sync()
+    ev.device_sync()
+    wall_s = time.perf_counter() - t_wall0
+    total_ms = ev.elapsed_ms(e_sel0[0], e_end[K - 1])
+    sel_step = [ev.elapsed_ms(e_sel0[i], e_sel1[i]) for i in range(K)]
+    bak_step = [ev.elapsed_ms(e_sel1[i], e_end[i]) for i in range(K)]
+    for e in e_sel0 + e_sel1 + e_end:
+        ev.destroy(e)
+    sel_ms, bak_ms = sum(sel_step), sum(bak_step)
+
+    # The byte model over the K timed steps: back to the statistics they started from, the same K
+    # steps again, the paths read back after each (the value sums of a backup are atomic float adds,
+    # so a replayed W can differ from the timed run's in its last bits; the model counts children
+    # and path nodes, which that does not move).
+    replay = dict(soa)
+    replay.update(N=start["N"], W=start["W"], VL=start["VL"])
+    forest.upload(replay)
+    del replay
+    batch.set_roots(troots)
+    model = ByteModel(soa, meta)
+    N_host = start["N"].copy()
+    sel_bytes = bak_bytes = n_sel_steps = 0
+    path_nodes = 0
+    for i in range(K):
+        batch.select(params)
+        paths, plen, leaf, _ = batch.read()
+        s_b, b_b, n_s = model.step(paths, plen, N_host)
+        sel_bytes += s_b
+        bak_bytes += b_b
+        n_sel_steps += n_s
+        path_nodes += int(plen.sum())
+        if tt is not None:
+            tt.probe_leaves_dev(batch, d_probe)
+        batch.backup(vl)
+        N_host += visits_of(paths, plen, n_nodes)
+    forest.sync()
+    del start, N_host, model
+
+    par = parity_check(omk, soa, meta, forest, batch, tt, tt_ids, troots, values, params) if parity else None
+
+    # selection = 1 reset + 1 persistent launch (teams over a work queue of multi-visitor items, and
+    # walkers for the lone visitors) when any traversals share a root, else 1 launch of the
+    # single-visitor kernel; the roofline is quoted for the kernel that carries the work, with the
+    # whole selection phase (HIP events around it on the forest's stream) as its launch duration
+    has_groups = len(np.unique(troots)) < B
+    dominant = "k_select_groups" if has_groups else "k_select_singles"
+    sel_ms_step = sel_ms / K
+    bak_ms_step = bak_ms / K
+    achieved = sel_bytes / (sel_ms * 1e-3) / 1e9
+    traffic, traffic_source = traffic_of(name) if scale == 1.0 else (None, None)
+    res = {
+        "workload": "%s: %d tree(s) x %d nodes, %d traversals per step, depth <= %d, c_puct %.2f, virtual loss %d%s%s%s"
+                    % (name, meta["n_trees"], meta["nodes_per_tree"], B, D, meta["c_puct"], vl,
+                       ", RAVE k=%g" % meta["rave_k"] if meta.get("has_rave") else "",
+                       ", progressive widening" if meta.get("pw") else "",
+                       ", 2^%d-slot table probes" % meta["tt_log2"] if meta.get("tt_log2") else ""),
+        "traversals_per_step": B,
+        "steps": K,
+        "traversals_per_s": B * K / (total_ms * 1e-3),
+        "ms_per_step": total_ms / K,
+        "select_ms": sel_ms_step,
+        "backup_ms": bak_ms_step,
+        "select_ms_first_last": [sel_step[0], sel_step[-1]],
+        "select_traversals_per_s": B / (sel_ms_step * 1e-3),
+        "backups_per_s": B / (bak_ms_step * 1e-3),
+        "wall_ms_per_step": wall_s * 1e3 / K,
+        "mean_path_nodes": path_nodes / float(K * B),
+        "selection_steps_per_step": n_sel_steps / float(K),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dominant,
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
+            "algorithmic_bytes": sel_bytes / float(K),
+            "algorithmic_bytes_over": "the %d timed steps (replayed from their starting statistics, paths read "
+                                      "back after each)" % K,
+            "launches_per_step": 1,
+            "avg_launch_us": sel_ms_step * 1e3,
+            "launch_covers": "the whole selection of a step, HIP events around it: " +
+                             ("k_select_reset + k_select_groups (teams and walkers in one persistent launch)"
+                              if has_groups else
+                              "k_select_singles alone (no reset launch when every traversal is alone at its root)")
+                             + "; rocprofv3's per-kernel averages add up to it",
+            "backup_algorithmic_bytes": bak_bytes / float(K),
+            "backup_achieved": bak_bytes / (bak_ms * 1e-3) / 1e9,
+        },
+        "parity": par,
+        "generate_s": gen_s,
+        "seed": seed,
+    }
+    if d_probe:
+        forest.dev_free(d_probe)
+    if tt is not None:
+        tt.close()
+    batch.close()
+    forest.close()
+    if cpu_seconds > 0:
+        res["cpu_baseline"] = cpu_baseline(soa, meta, troots, values, cpu_seconds, K + warmup)
+    return res
 
 
 def main():
@@ -102,10 +427,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c0", "c1", "c2", "c3", "c4", "wide"])
+    ap.add_argument("--workload", default="c3", choices=BENCH_CONFIGS + ["wide"])
+    ap.add_argument("--configs", default=",".join(BENCH_CONFIGS),
+                    help="comma-separated workloads measured beside --workload into per_config ('none': only --workload)")
     ap.add_argument("--seed", type=int, default=2025)
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="budget of the CPU baseline leg of --workload (0 = skip); the other configurations get a third")
     ap.add_argument("--scale", type=float, default=1.0, help="scale nodes_per_tree (debugging only)")
+    ap.add_argument("--no-parity", action="store_true", help="skip the comparison with the CPU checker")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only run the plain copy kernel over this many MiB, 10 times (to scale profiler "
                          "traffic counters by) and exit")
@@ -129,224 +458,85 @@ def main():
         print(json.dumps({"copy_calibration_bytes_each_way": nbytes, "launches": 10}))
         return
 
-    kw = {}
-    if args.scale != 1.0:
-        kw["nodes_per_tree"] = max(1000, int(synth.CONFIGS[args.workload]["nodes_per_tree"] * args.scale))
-    t0 = time.time()
-    soa, roots, meta = synth.generate(args.workload, seed=args.seed, **kw)
-    gen_s = time.time() - t0
-    B = int(meta["n_traversals"])
-    D = int(meta["max_depth"])
-    vl = int(meta["virtual_loss"])
-    troots = synth.traversal_roots(roots, B)
-    values = np.random.default_rng(args.seed + 1).uniform(-1, 1, B).astype(np.float32)
-    params = omk.SelectParams(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
-                              rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")))
+    head = measure(omk, synth, args.workload, args.steps, args.warmup, args.seed, args.cpu_seconds, args.scale,
+                   parity=not args.no_parity)
 
-    forest = omk.Forest.from_soa(soa)
-    batch = omk.Batch(forest, B, D)
-    batch.set_roots(troots)
-    batch.set_values(values)
-    tt = None
-    d_probe = 0
-    if meta.get("tt_log2"):
-        tt = omk.TranspositionTable(forest, int(meta["tt_log2"]))
-        n_ins = 1 << (int(meta["tt_log2"]) - 1)  # 50 % load
-        ids = np.linspace(0, meta["n_nodes"] - 1, n_ins).astype(np.int64)
-        ids = np.unique(ids)
-        tt.insert(soa["hash"][ids], ids.astype(np.int32))
-        d_probe = forest.dev_alloc(B * 4)
-
-    def step():
-        batch.select(params)
-        if tt is not None:
-            tt.probe_leaves_dev(batch, d_probe)
-        batch.backup(vl)
-
-    ev = HipEvents()
-    stream = forest.get_stream()
-    for _ in range(args.warmup):
-        step()
-    forest.sync()
-    ev.device_sync()
-
-    K = args.steps
-    e_sel0 = [ev.create() for _ in range(K)]
-    e_sel1 = [ev.create() for _ in range(K)]
-    e_end = [ev.create() for _ in range(K)]
-    t_wall0 = time.perf_counter()
-    for i in range(K):
-        ev.record(e_sel0[i], stream)
-        batch.select(params)
-        ev.record(e_sel1[i], stream)
-        if tt is not None:
-            tt.probe_leaves_dev(batch, d_probe)
-        batch.backup(vl)
-        ev.record(e_end[i], stream)
-    forest.sync()
-    ev.device_sync()
-    wall_s = time.perf_counter() - t_wall0
-    total_ms = ev.elapsed_ms(e_sel0[0], e_end[K - 1])
-    sel_ms = sum(ev.elapsed_ms(e_sel0[i], e_sel1[i]) for i in range(K))
-    bak_ms = sum(ev.elapsed_ms(e_sel1[i], e_end[i]) for i in range(K))
-
-    # outside the timed region: three plain copies of 64 MiB, the known-size kernel that a
+    # outside every timed region: three plain copies of 64 MiB, the known-size kernel that a
     # profiler run of this command scales its traffic counters by
+    f = omk.Forest(16)
     cal_bytes = 64 << 20
-    d_src, d_dst = forest.dev_alloc(cal_bytes), forest.dev_alloc(cal_bytes)
+    d_src, d_dst = f.dev_alloc(cal_bytes), f.dev_alloc(cal_bytes)
     for _ in range(3):
-        forest.dev_copy(d_dst, d_src, cal_bytes)
-    forest.sync()
-    forest.dev_free(d_src)
-    forest.dev_free(d_dst)
-
-    # the byte model is evaluated on the paths of one more (untimed) step
-    batch.select(params)
-    paths, plen, leaf, _ = batch.read()
-    N_now = forest.download()["N"]
-    batch.backup(vl)
-    forest.sync()
-    sel_bytes, bak_bytes, n_sel_steps = algorithmic_bytes(soa, meta, paths, plen, N_now)
-    # selection = 1 reset + 1 persistent launch (teams over a work queue of multi-visitor items, and
-    # walkers for the lone visitors) when any traversals share a root, else 1 launch of the
-    # single-visitor kernel; the
-    # roofline is quoted for the kernel that carries the work, with the whole selection phase
-    # (HIP events around it on the forest's stream) as its launch duration
-    has_groups = len(np.unique(troots)) < B
-    dominant = "k_select_groups" if has_groups else "k_select_singles"
-    launches_per_select = 1
-    sel_ms_step = sel_ms / K
-    bak_ms_step = bak_ms / K
-    achieved = sel_bytes / (sel_ms_step * 1e-3) / 1e9
-    traffic = None
-    tfile = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tfile):
-        with open(tfile) as fh:
-            tj = json.load(fh)
-        if args.workload in tj and args.scale == 1.0:
-            traffic = tj[args.workload].get("selection_bytes_per_launch")
+        f.dev_copy(d_dst, d_src, cal_bytes)
+    f.sync()
+    f.dev_free(d_src)
+    f.dev_free(d_dst)
+    f.close()
 
     out = {
         "metric": "PUCT traversals/s (selection with virtual loss + value backup per step)",
-        "value": B * K / (total_ms * 1e-3),
+        "value": head["traversals_per_s"],
         "unit": "traversals/s",
         "n_gpus": 1,
-        "steps": K,
+        "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": total_ms / K,
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "%s: %d tree(s) x %d nodes, %d traversals per step, depth <= %d, c_puct %.2f, virtual loss %d%s%s%s"
-                        % (args.workload, meta["n_trees"], meta["nodes_per_tree"], B, D, meta["c_puct"], vl,
-                           ", RAVE k=%g" % meta["rave_k"] if meta.get("has_rave") else "",
-                           ", progressive widening" if meta.get("pw") else "",
-                           ", 2^%d-slot table probes" % meta["tt_log2"] if meta.get("tt_log2") else ""),
-            "traversals_per_step": B,
+            "workload": head["workload"],
+            "traversals_per_step": head["traversals_per_step"],
             "seed": args.seed,
-            "mean_path_nodes": float(plen.mean()),
-            "selection_steps_per_step": n_sel_steps,
+            "mean_path_nodes": head["mean_path_nodes"],
+            "selection_steps_per_step": head["selection_steps_per_step"],
         },
-        "select_traversals_per_s": B / (sel_ms_step * 1e-3),
-        "backups_per_s": B / (bak_ms_step * 1e-3),
-        "select_ms_per_step": sel_ms_step,
-        "backup_ms_per_step": bak_ms_step,
-        "wall_ms_per_step": wall_s * 1e3 / K,
-        "roofline": {
-            "bound": "hbm",
-            "kernel": dominant,
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": traffic,
-            "algorithmic_bytes_per_step": sel_bytes,
-            "launches_per_step": launches_per_select,
-            "avg_launch_us": sel_ms_step * 1e3 / launches_per_select,
-            "launch_covers": "the whole selection of a step, HIP events around it: " +
-                             ("k_select_reset + k_select_groups (teams and walkers in one persistent launch)" if has_groups
-                              else "k_select_singles alone (no reset launch when every traversal is alone at its root)")
-                             + "; rocprofv3's per-kernel averages add up to it",
-            "backup_algorithmic_bytes_per_step": bak_bytes,
-            "backup_achieved": bak_bytes / (bak_ms_step * 1e-3) / 1e9,
-        },
-        "generate_s": gen_s,
+        "select_traversals_per_s": head["select_traversals_per_s"],
+        "backups_per_s": head["backups_per_s"],
+        "select_ms_per_step": head["select_ms"],
+        "backup_ms_per_step": head["backup_ms"],
+        "wall_ms_per_step": head["wall_ms_per_step"],
+        "roofline": head["roofline"],
+        "parity": head["parity"],
+        "generate_s": head["generate_s"],
     }
+    if "cpu_baseline" in head:
+        out["cpu_baseline"] = head["cpu_baseline"]
 
-    if args.cpu_seconds > 0:
-        from oracle import ref_cpu as R
-        ref = R.RefTree.from_soa(soa)
-        rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
-                           rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
-        rtt = None
-        done = 0
-        sel_s = bak_s = 0.0
-        t_start = time.perf_counter()
-        while done < 2 or (time.perf_counter() - t_start) < args.cpu_seconds:
-            a = time.perf_counter()
-            rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
-            b = time.perf_counter()
-            ref.backup_batch(rpaths, rlen, values, vl)
-            c = time.perf_counter()
-            sel_s += b - a
-            bak_s += c - b
-            done += 1
-            if done >= K + args.warmup:
-                break
-        soa_rate = B * done / (sel_s + bak_s)
-        out["cpu_baseline"] = {
-            "value": soa_rate,
-            "unit": "traversals/s",
-            "cores": 1,
-            "kind": "port",
-            "sample": "%d steps of the same workload (same forest, roots and leaf values) through the "
-                      "serial CPU restatement of selectChild / applyVirtualLoss / update / revertVirtualLoss" % done,
-            "soa_serial_select_traversals_per_s": B * done / sel_s,
-            "soa_serial_backups_per_s": B * done / bak_s,
-            "host_cores_visible": os.cpu_count(),
+    names = [] if args.configs.strip().lower() in ("", "none") else [c.strip() for c in args.configs.split(",")]
+    per = {}
+    for name in names:
+        if name not in BENCH_CONFIGS + ["wide"]:
+            print("bench.py: unknown configuration %r in --configs" % name, file=sys.stderr)
+            sys.exit(2)
+        if name == args.workload:
+            r = head
+        else:
+            r = measure(omk, synth, name, args.steps, args.warmup, args.seed, args.cpu_seconds / 3.0, args.scale,
+                        parity=not args.no_parity)
+        per[name] = {
+            "workload": r["workload"],
+            "select_ms": r["select_ms"],
+            "backup_ms": r["backup_ms"],
+            "ms_per_step": r["ms_per_step"],
+            "traversals_per_s": r["traversals_per_s"],
+            "select_traversals_per_s": r["select_traversals_per_s"],
+            "backups_per_s": r["backups_per_s"],
+            "select_ms_first_last": r["select_ms_first_last"],
+            "roofline": {k: r["roofline"][k] for k in ("kernel", "achieved", "frac", "algorithmic_bytes",
+                                                        "backup_algorithmic_bytes", "backup_achieved", "traffic")},
+            "parity": r["parity"],
         }
-        # The same arithmetic over the reference's own layout and threading: heap nodes with one
-        # cache line per atomic field, shared_ptr child vectors, OpenMP loops with
-        # schedule(dynamic, 1).  Timed with one thread and with the host's share of cores; the
-        # faster of the three figures becomes `value` (with several threads the traversal
-        # order, hence the result, depends on the schedule, as the reference's does).
-        if len(soa["N"]) <= 20_000_000:
-            from oracle import ref_ptr as RP
-            t_build = time.perf_counter()
-            pt = RP.PtrTree(soa)
-            t_build = time.perf_counter() - t_build
-            n_thr = max(1, min(16, os.cpu_count() or 1))
-            kw = dict(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
-                      rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
-            rates = {}
-            for thr in sorted({1, n_thr}):
-                tot, steps_done = 0.0, 0
-                t_start = time.perf_counter()
-                while steps_done < 2 or (time.perf_counter() - t_start) < args.cpu_seconds / 2:
-                    _, _, s_s, b_s = pt.step(troots, values, threads=thr, **kw)
-                    tot += s_s + b_s
-                    steps_done += 1
-                    if steps_done >= K + args.warmup:
-                        break
-                rates[thr] = B * steps_done / tot
-            pt.close()
-            cb = out["cpu_baseline"]
-            cb["soa_serial_traversals_per_s"] = soa_rate
-            cb["pointer_tree_traversals_per_s"] = {str(k): v for k, v in rates.items()}
-            cb["pointer_tree_node_bytes"] = RP.PtrTree.node_bytes()
-            cb["pointer_tree_build_s"] = t_build
-            best_thr = max(rates, key=rates.get)
-            if rates[best_thr] > soa_rate:
-                cb["value"] = rates[best_thr]
-                cb["cores"] = best_thr
-                cb["sample"] = ("steps of the same workload (same forest, roots and leaf values) through the CPU "
-                                "restatement over the reference's node layout (heap nodes, one cache line per "
-                                "atomic) and OpenMP loops, %d thread(s); the serial array checker and the "
-                                "one-thread figure are given beside it" % best_thr)
-        del rtt
+        if "cpu_baseline" in r:
+            cb = r["cpu_baseline"]
+            per[name]["cpu_baseline"] = {k: cb[k] for k in ("value", "unit", "cores", "kind") if k in cb}
+            for k in ("soa_serial_traversals_per_s", "pointer_tree_traversals_per_s"):
+                if k in cb:
+                    per[name]["cpu_baseline"][k] = cb[k]
+    if per:
+        out["per_config"] = per
     print(json.dumps(out))
 
 

@@ -1136,7 +1136,7 @@ int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_dept
     if (!tt || !d_keys || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe: null argument");
     if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_probe: n %lld", (long long)n);
     if (int rc = use_device(tt->f)) return rc;
-    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, n, min_depth, d_out, tt->f->stream));
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, 0, n, min_depth, d_out, tt->f->stream));
     return OMK_OK;
 }
 
@@ -1146,7 +1146,7 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: no selected paths");
     if (!b->f->has_hash) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: the forest was uploaded without position keys");
     if (int rc = use_device(tt->f)) return rc;
-    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->n, min_depth, d_out,
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->f->n_nodes, b->n, min_depth, d_out,
                             tt->f->stream));
     return OMK_OK;
 }

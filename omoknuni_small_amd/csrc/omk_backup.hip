@@ -405,13 +405,14 @@ __global__ __launch_bounds__(256) void k_tt_insert(TTSlot *slots, int log2_slots
 }
 
 __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys,
-                                                  const int32_t *leaf, const uint64_t *node_hash, int64_t n,
-                                                  int min_depth, int32_t *out) {
+                                                  const int32_t *leaf, const uint64_t *node_hash, int64_t n_nodes,
+                                                  int64_t n, int min_depth, int32_t *out) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     unsigned long long key = kTTEmpty;
     if (keys) key = keys[i];
-    else if (leaf[i] >= 0) key = node_hash[leaf[i]];  // a traversal without a leaf finds nothing
+    // a traversal without a leaf finds nothing; never index the forest with an id it does not have
+    else if (leaf[i] >= 0 && leaf[i] < n_nodes) key = node_hash[leaf[i]];
     int found = -1;
     if (key != kTTEmpty) {
         uint64_t mask = (1ull << log2_slots) - 1ull;
@@ -437,10 +438,11 @@ hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s) {
 }
 
 hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
-                           const uint64_t *node_hash, int64_t n, int min_depth, int32_t *out, hipStream_t s) {
+                           const uint64_t *node_hash, int64_t n_nodes, int64_t n, int min_depth, int32_t *out,
+                           hipStream_t s) {
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_tt_probe, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, log2_slots, keys, leaf,
-                       node_hash, n, min_depth, out);
+                       node_hash, n_nodes, n, min_depth, out);
     return hipGetLastError();
 }
 

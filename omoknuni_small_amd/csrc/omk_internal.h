@@ -158,7 +158,9 @@ hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s);
 // d_status[0] += entries that found no free slot, d_status[1] += keys equal to the empty marker
 hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
                             const int32_t *depths, int64_t n, int *d_status, hipStream_t s);
+// keys == nullptr: the key of entry i is node_hash[leaf[i]] (nothing for a leaf outside [0, n_nodes))
 hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
-                           const uint64_t *node_hash, int64_t n, int min_depth, int32_t *out, hipStream_t s);
+                           const uint64_t *node_hash, int64_t n_nodes, int64_t n, int min_depth, int32_t *out,
+                           hipStream_t s);
 
 }  // namespace omk

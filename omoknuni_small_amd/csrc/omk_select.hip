@@ -48,9 +48,10 @@
 // Settling a node needs only the NUMBER of its visitors; the list of their traversal ids is
 // needed last, for the node's own partition.  The children of a heavy node are therefore
 // published before their lists are written (item kind 3) and wait for a "list complete" word
-// where they need it.  The single-visitor walk (no LDS,
-// high occupancy, one launch afterwards) takes the visitors that are alone at a node: they
-// stay alone to their leaf.
+// where they need it.  A visitor that is alone at a node stays alone to its leaf: blocks of
+// walkers behind the teams of the same persistent launch take such visitors as the teams
+// create them (one wavefront per walk, no LDS); a batch whose traversals are all alone at
+// their roots is one launch of the single-visitor kernel instead.
 #include <algorithm>
 
 #include "omk_internal.h"
@@ -294,6 +295,14 @@ template <int R, bool RAVE>
 __device__ __forceinline__ int wave_pick(const Kids<R, RAVE> &k, int lane, uint32_t bk, uint32_t bpos) {
     uint32_t m, pos;
     wave_best(bk, bpos, m, pos);
+    if (RAVE && m != 0u && pos >= (uint32_t)(R * kWave)) {
+        // a candidate of the second scan: the reference only runs that scan when the first one
+        // found a child (mcts_node.cpp:173-184); with no real first-scan score it falls back
+        bool any1 = false;
+#pragma unroll
+        for (int r = 0; r < R; r++) any1 |= k.k1[r] != 0u;
+        if (__ballot(any1) == 0ull) m = 0u;
+    }
     if (m != 0u) return (int)(pos >= (uint32_t)(R * kWave) ? pos - (uint32_t)(R * kWave) : pos);
     uint32_t mn = 0xFFFFFFFFu;  // order-preserving int -> uint
     bool any = false;
@@ -1721,6 +1730,18 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         for (int r = 0; r < R; r++) {
             score_round<R, RAVE>(k, r, c.ep);
             cnt[r] = 0;
+        }
+        if (RAVE) {
+            // no real score in the first scan: the reference never runs the second one
+            // (mcts_node.cpp:173-184); without keys every parallel path declines and the visitors
+            // are played one at a time, where wave_pick applies the same rule
+            bool any1 = false;
+#pragma unroll
+            for (int r = 0; r < R; r++) any1 |= k.k1[r] != 0u;
+            if (__ballot(any1) == 0ull) {
+#pragma unroll
+                for (int r = 0; r < R; r++) k.k2[r] = 0u;
+            }
         }
         lane_best<R, RAVE>(k, lane, bk, bpos);
     }

@@ -1,0 +1,79 @@
+"""GPU parity on the five benchmark workloads at their FULL size (the trees and batches the benchmark
+times: 200 k nodes / 64 traversals, 256 x 50 k / 256, 64 x 1 M / 1024, 4 M / 4096 with progressive
+widening, 16 M with RAVE / 16384 and the 2^24-slot table), two search steps each, against the CPU
+checker after every phase: paths, lengths, leaves, move lists, N and virtual loss bit-exact, W within
+1e-5 relative, table probes of the leaves' keys identical."""
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+
+pytestmark = pytest.mark.gpu
+
+W_RTOL = 1e-5
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("name", ["c0", "c1", "c3", "c4", "c2"])
+def test_full_size_workload(name):
+    import omoknuni_small_amd as omk
+    from omoknuni_small_amd import synth
+
+    soa, roots, meta = synth.generate(name, seed=2025)
+    B, D, vl = int(meta["n_traversals"]), int(meta["max_depth"]), int(meta["virtual_loss"])
+    rave, pw = bool(meta.get("has_rave")), bool(meta.get("pw"))
+    rave_k = float(meta.get("rave_k", 3000.0))
+    assert len(soa["N"]) == synth.CONFIGS[name]["n_trees"] * synth.CONFIGS[name]["nodes_per_tree"]
+    troots = synth.traversal_roots(roots, B)
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=rave, rave_k=rave_k, pw=pw, max_depth=D)
+    forest = omk.Forest.from_soa(soa)
+    batch = omk.Batch(forest, B, D)
+    batch.set_roots(troots)
+    sp = omk.SelectParams(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=rave, rave_k=rave_k, pw=pw)
+    tt = ref_slots = None
+    if meta.get("tt_log2"):
+        # the benchmark's table: 2^24 slots at 50 % load, keyed by the position keys of evenly spaced nodes
+        log2 = int(meta["tt_log2"])
+        ids = np.unique(np.linspace(0, meta["n_nodes"] - 1, 1 << (log2 - 1)).astype(np.int64)).astype(np.int32)
+        tt = omk.TranspositionTable(forest, log2)
+        tt.insert(soa["hash"][ids], ids)
+        # the checker probes the very slots the device built (their layout is checked against the
+        # checker's own inserts on smaller tables elsewhere) and a dict says what must be found
+        ref_tt = R.RefTT(4)
+        ref_tt.log2 = log2
+        ref_tt.slots = tt.download()
+        sorted_keys = np.sort(soa["hash"][ids])
+        order = np.argsort(soa["hash"][ids])
+    rng = np.random.default_rng(9)
+    near_total = 0
+    for step in range(2):
+        rpaths, rlen, rleaf, near = ref.select_batch(troots, rp)
+        near_total += int((near >= 0).sum())
+        batch.select(sp)
+        gpaths, glen, gleaf, gact = batch.read()
+        bad = np.nonzero((gpaths != rpaths).any(axis=1) | (glen != rlen) | (gleaf != rleaf))[0]
+        assert len(bad) == 0, "%s step %d: %d of %d paths differ (first %s)" % (name, step, len(bad), B, bad[:5])
+        assert (gact == ref.gather_actions(rpaths, rlen)).all()
+        assert batch.truncated() == int(((rlen == D + 1) & (ref.child_count[rleaf] > 0)).sum())
+        st = forest.download()
+        assert (st["VL"] == ref.VL).all(), "virtual loss after select, step %d" % step
+        if tt is not None:
+            got = tt.probe_leaves(batch)
+            want, hits = ref_tt.probe(soa["hash"][rleaf])
+            assert (got == want).all()
+            k = soa["hash"][rleaf]
+            pos = np.minimum(np.searchsorted(sorted_keys, k), len(sorted_keys) - 1)
+            by_search = np.where(sorted_keys[pos] == k, ids[order[pos]], -1).astype(np.int32)
+            assert (got == by_search).all()
+            assert 0 < hits < B
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, values, vl)
+        batch.set_values(values)
+        batch.backup(vl)
+        st = forest.download()
+        assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all(), "counters after backup, step %d" % step
+        err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
+        assert err.max() <= W_RTOL
+        ref.W[:] = st["W"]
+    print("%s: near-tie traversals flagged by the checker over 2 steps: %d" % (name, near_total))

@@ -131,6 +131,36 @@ def test_rave_two_pass(seed):
     run_both(soa, roots, np.zeros(96, np.int32), use_rave=True, rave_k=3000.0, c_puct=0.3, max_depth=6)
 
 
+@pytest.mark.parametrize("visitors", [1, 3, 40, 1500])
+def test_rave_second_scan_needs_a_first_scan_winner(visitors):
+    """Every first-scan score is NaN (unvisited children under virtual loss whose value sum is NaN)
+    while the RAVE blend of the second scan is finite: the reference skips the second scan and falls
+    back to the least-visited child, first minimum (mcts_node.cpp:173-184), for every visitor."""
+    kids = [[0, float("nan"), 0.2, 2, 5 + i, float(i)] for i in range(70)]
+    soa = star(10, kids, rave=True)
+    # one level further down the same situation among visited children (N > 0, W = NaN)
+    base = len(soa["N"])
+    extra = 5
+    soa["child_begin"][1] = base
+    soa["child_count"][1] = extra
+    app = lambda key, vals, dt: np.concatenate([soa[key], np.asarray(vals, dt)])
+    soa["N"] = app("N", [4, 2, 9, 2, 7], np.int32)
+    soa["W"] = app("W", [float("nan")] * extra, np.float32)
+    soa["P"] = app("P", [0.2] * extra, np.float32)
+    soa["VL"] = app("VL", [0] * extra, np.int32)
+    soa["rN"] = app("rN", [3, 3, 3, 3, 3], np.int32)
+    soa["rW"] = app("rW", [1.0, 2.0, 3.0, -1.0, 0.5], np.float32)
+    soa["child_begin"] = app("child_begin", [0] * extra, np.int32)
+    soa["child_count"] = app("child_count", [0] * extra, np.int32)
+    soa["action"] = app("action", list(range(extra)), np.int32)
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(use_rave=True, rave_k=1000.0, max_depth=3)
+    assert ref.select_child(0, rp) == 1 and ref.select_child(1, rp) == base + 1  # least visited, first minimum
+    # no backup: the value sums are NaN on purpose, which the W comparison cannot take
+    run_both(soa, np.array([0], np.int32), np.zeros(visitors, np.int32), use_rave=True, rave_k=1000.0, max_depth=3,
+             do_backup=False)
+
+
 @pytest.mark.parametrize("seed", [40, 41])
 def test_forest_of_trees(seed):
     soa, roots = random_tree(seed, n_expand=120, fanout=(3, 70), max_depth=6, n_roots=8)
