@@ -122,6 +122,17 @@ def visits_of(paths, plen, n_nodes):
     return np.bincount(paths[on_path], minlength=n_nodes).astype(np.int32)
 
 
+def exact_value_sums(paths, plen, values, n_nodes):
+    """What a backup adds to W of every node, in double precision: the leaf of a path takes +value,
+    every ply up flips the sign."""
+    row = paths.shape[1]
+    d_idx = np.arange(row)[None, :]
+    on_path = d_idx < plen[:, None]
+    sign = np.where(((plen[:, None] - 1 - d_idx) & 1) == 1, -1.0, 1.0)
+    contrib = (sign * values.astype(np.float64)[:, None])[on_path]
+    return np.bincount(paths[on_path], weights=contrib, minlength=n_nodes)
+
+
 def cpu_baseline(soa, meta, troots, values, seconds, max_steps):
     """The CPU checker on the host's cores, on a bounded number of steps of the same workload."""
     from oracle import ref_cpu as R
@@ -207,9 +218,12 @@ def parity_check(omk, soa, meta, forest, batch, tt, tt_ids, troots, values, para
     ref = R.RefTree.from_soa(cur)
     rp = R.make_params(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
                        rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")), max_depth=D)
+    # W: the device adds the values with float atomics in no fixed order, the checker one after the
+    # other in binary32 (the reference itself adds from OpenMP threads, in any order); each is
+    # compared with the exact sum, |W - exact| / max(|exact|, 1), and with each other
     out = dict(checked_steps=steps, traversals_per_step=B, mismatched_traversals=0, move_lists_equal=True,
-               N_equal=True, VL_equal=True, W_max_rel_err=0.0, near_tie_traversals=0,
-               mismatches_outside_near_ties=0)
+               N_equal=True, VL_equal=True, W_max_rel_err=0.0, W_max_rel_err_vs_serial_f32=0.0,
+               serial_f32_max_rel_err=0.0, near_tie_traversals=0, mismatches_outside_near_ties=0)
     if tt is not None:
         ref_tt = R.RefTT(4)
         ref_tt.log2 = tt.log2
@@ -232,13 +246,18 @@ def parity_check(omk, soa, meta, forest, batch, tt, tt_ids, troots, values, para
             want, hits = ref_tt.probe(soa["hash"][rleaf])
             out["tt_probes_equal"] &= bool((got == want).all())
             out["tt_hits"] += hits
+        exact = ref.W.astype(np.float64) + exact_value_sums(rpaths, rlen, values, len(ref.W))
         ref.backup_batch(rpaths, rlen, values, vl)
         batch.backup(vl)
         st = forest.download()
         out["N_equal"] &= bool((st["N"] == ref.N).all())
         out["VL_equal"] &= bool((st["VL"] == ref.VL).all())
-        err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
-        out["W_max_rel_err"] = max(out["W_max_rel_err"], float(err.max()))
+        scale = np.maximum(np.abs(exact), 1.0)
+        gw = st["W"].astype(np.float64)
+        out["W_max_rel_err"] = max(out["W_max_rel_err"], float((np.abs(gw - exact) / scale).max()))
+        out["serial_f32_max_rel_err"] = max(out["serial_f32_max_rel_err"], float((np.abs(ref.W - exact) / scale).max()))
+        out["W_max_rel_err_vs_serial_f32"] = max(out["W_max_rel_err_vs_serial_f32"],
+                                                 float((np.abs(gw - ref.W) / np.maximum(np.abs(ref.W), 1.0)).max()))
         ref.W[:] = st["W"]
     out["ok"] = bool(out["mismatches_outside_near_ties"] == 0 and out["move_lists_equal"] and out["N_equal"]
                      and out["VL_equal"] and out["W_max_rel_err"] <= 1e-5 and out.get("tt_probes_equal", True))

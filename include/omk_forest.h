@@ -104,7 +104,9 @@ int omk_forest_set_stream(omk_forest *f, void *hip_stream);
 /* The hipStream_t the forest's work is enqueued on (to record events on it). */
 int omk_forest_get_stream(omk_forest *f, void **hip_stream_out);
 /* Checks that the arrays describe a forest (ranges in bounds, every node the child of at
- * most one parent, fan-out <= OMK_MAX_FANOUT) and copies them to the device. */
+ * most one parent, fan-out <= OMK_MAX_FANOUT) and copies them to the device.  Uploading the same
+ * child ranges again (statistics put back) leaves batches usable; after an upload of another
+ * structure their roots and paths are stale: OMK_ERR_STATE until omk_batch_set_roots. */
 int omk_forest_upload(omk_forest *f, const omk_soa_view *h_view);
 /* Copies N, W, P, VL (and rN, rW) back; structure pointers of the view are ignored. */
 int omk_forest_download(omk_forest *f, omk_soa_view *h_view);
@@ -183,7 +185,8 @@ int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, in
  * siblings contiguous in their old order, new_root = 0, so selections come out the same.
  * *h_nodes_after = k; h_old_of_new (NULL or room for the old node count) receives the old id
  * of every new node.  Paths of earlier selections, roots of batches and node ids stored in
- * transposition tables refer to the old numbering: set roots again, clear the tables.  All
+ * transposition tables refer to the old numbering: set roots again (a batch refuses to select,
+ * back up, expand or read with OMK_ERR_STATE until then), clear the tables.  All
  * of it runs on the device: the renumbering level by level (child counts of a level, an
  * exclusive scan, the children's ids written to the next level), then one gather per array;
  * the host only reads the size of every level. */

@@ -40,6 +40,11 @@ struct omk_forest {
     bool uploaded = false;
     bool prior_sorted = false;
     int max_fanout = 0;
+    // Counts the changes that give node ids a new meaning (a compaction, an upload of a different
+    // structure): paths, roots and work items of a batch made before such a change are stale.
+    int64_t generation = 0;
+    uint64_t structure_sum = 0;  // checksum of the child ranges last uploaded
+    bool structure_changed = false;  // the device's child ranges are no longer the uploaded ones (expansion, compaction)
     hipStream_t own_stream = nullptr;
     hipStream_t stream = nullptr;
     // device arrays
@@ -95,6 +100,7 @@ struct omk_batch {
     int32_t max_depth = 0;
     int32_t stride = 0;
     int32_t n = 0;          // traversals bound by set_roots
+    int64_t generation = -1;  // the forest's generation when the roots were set
     bool selected = false;  // paths of a select are on the device
     int32_t *paths = nullptr, *path_len = nullptr, *leaf = nullptr;
     float *values = nullptr;
@@ -140,6 +146,15 @@ static int use_device(const omk_forest *f) {
     if (f->released) return fail(OMK_ERR_STATE, "the forest of this handle has been destroyed");
     HIP_TRY(hipSetDevice(f->device));
     (void)hipGetLastError();  // launches are checked with hipGetLastError: start from a clean slate
+    return OMK_OK;
+}
+
+// Roots, paths and work items of a batch are node ids: stale once the forest was compacted or a
+// different structure uploaded.
+static int fresh_batch(const char *who, const omk_batch *b) {
+    if (b->generation != b->f->generation)
+        return fail(OMK_ERR_STATE, "%s: the forest was compacted or uploaded with another structure since this "
+                    "batch's roots were set; call omk_batch_set_roots and select again", who);
     return OMK_OK;
 }
 
@@ -234,10 +249,11 @@ int omk_sync(omk_forest *f) {
 // correct when every node is the child of at most one parent, so it is checked here, on
 // the host, before anything reaches the device (it also keeps every child range in
 // bounds, which is what protects the kernels from wild reads).
-static int validate(const omk_soa_view *v, int64_t n, int *max_fanout, bool *prior_sorted) {
+static int validate(const omk_soa_view *v, int64_t n, int *max_fanout, bool *prior_sorted, uint64_t *structure_sum) {
     std::vector<uint8_t> is_child((size_t)n, 0);
     int mf = 0;
     bool sorted = true;
+    uint64_t h = 0xCBF29CE484222325ull ^ (uint64_t)n;  // checksum of (node, child range) of every expanded node
     for (int64_t i = 0; i < n; i++) {
         int32_t cc = v->child_count[i];
         if (cc == 0) continue;
@@ -256,9 +272,11 @@ static int validate(const omk_soa_view *v, int64_t n, int *max_fanout, bool *pri
             if (sorted && c > cb && !(v->P[c - 1] >= v->P[c])) sorted = false;
         }
         mf = std::max(mf, (int)cc);
+        h = (h ^ ((uint64_t)i * 0x9E3779B97F4A7C15ull + ((uint64_t)(uint32_t)cb << 32) + (uint32_t)cc)) * 0x100000001B3ull;
     }
     *max_fanout = mf;
     *prior_sorted = sorted && v->legal == nullptr;
+    *structure_sum = h;
     return OMK_OK;
 }
 
@@ -274,7 +292,8 @@ int omk_forest_upload(omk_forest *f, const omk_soa_view *v) {
         return fail(OMK_ERR_INVALID, "omk_forest_upload: the forest was created with RAVE, rN and rW are required");
     int mf = 0;
     bool sorted = false;
-    if (int rc = validate(v, n, &mf, &sorted)) return rc;
+    uint64_t ssum = 0;
+    if (int rc = validate(v, n, &mf, &sorted, &ssum)) return rc;
     if (int rc = use_device(f)) return rc;
 
     std::vector<int2> span((size_t)n);
@@ -308,6 +327,10 @@ int omk_forest_upload(omk_forest *f, const omk_soa_view *v) {
         if (!f->hash) HIP_TRY(dalloc(&f->hash, f->capacity));
         HIP_TRY(hipMemcpy(f->hash, v->hash, (size_t)n * 8, hipMemcpyHostToDevice));
     }
+    // the same structure again (statistics put back): node ids keep their meaning
+    if (!f->uploaded || f->structure_changed || n != f->n_nodes || ssum != f->structure_sum) f->generation++;
+    f->structure_sum = ssum;
+    f->structure_changed = false;
     f->n_nodes = n;
     f->max_fanout = mf;
     f->prior_sorted = sorted;
@@ -518,39 +541,33 @@ int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, in
     return OMK_OK;
 }
 
-int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new) {
-    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_compact: null forest");
-    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact: nothing uploaded");
-    if (new_root < 0 || new_root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_compact: root %d", new_root);
-    if (int rc = use_device(f)) return rc;
+// Device memory a compaction works in, beyond the forest's own arrays.
+struct CompactScratch {
+    int32_t *map = nullptr;    // [n] old id of every new node
+    int32_t *begin = nullptr;  // [n] new id of every new node's first child
+    int32_t *cc = nullptr;     // [n] child counts of the level at hand
+    int32_t *scan = nullptr;   // [n] their exclusive prefix
+    void *scan_tmp = nullptr;  // work space of the scan
+    size_t scan_bytes = 0;
+    uint64_t *tmp = nullptr;   // [n] the array every field passes through
+    uint32_t *legal = nullptr; // [(n + 31) / 32] the new legal mask
+};
+
+// The compaction itself, in scratch memory the caller provides (room for the forest's node count).
+static int compact_in(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new,
+                      const CompactScratch &sc) {
     hipStream_t s = f->stream;
-    HIP_TRY(hipStreamSynchronize(s));
     const int64_t n = f->n_nodes;
-    // breadth-first order of the subtree, on the device: d_map[new id] = old id, d_begin[new id]
+    // breadth-first order of the subtree, on the device: map[new id] = old id, begin[new id]
     // = new id of its first child.  One level per round; the levels' sizes come back to the
     // host (a handful of bytes per level).
-    int32_t *d_map = nullptr, *d_begin = nullptr, *d_cc = nullptr, *d_scan = nullptr;
-    uint32_t *d_legal = nullptr;
-    uint64_t *d_tmp = nullptr;
-    void *d_scan_tmp = nullptr;
-    size_t scan_bytes = 0;
-    hipError_t e = bfs_scan_bytes(n, &scan_bytes);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_map, (size_t)n * 4);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_begin, (size_t)n * 4);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_cc, (size_t)n * 4);
-    if (e == hipSuccess) e = hipMalloc((void **)&d_scan, (size_t)n * 4);
-    if (e == hipSuccess) e = hipMalloc(&d_scan_tmp, scan_bytes > 0 ? scan_bytes : 4);
-    auto cleanup = [&]() {
-        for (void *p : {(void *)d_map, (void *)d_begin, (void *)d_cc, (void *)d_scan, (void *)d_legal, (void *)d_tmp,
-                        d_scan_tmp})
-            if (p) (void)hipFree(p);
-    };
-    if (e == hipSuccess) e = hipMemcpyAsync(d_map, &new_root, 4, hipMemcpyHostToDevice, s);
+    hipError_t e = hipMemcpyAsync(sc.map, &new_root, 4, hipMemcpyHostToDevice, s);
     int64_t lo = 0, hi = 1;
     bool not_a_tree = false;
     while (e == hipSuccess && hi > lo) {
         int64_t total = 0;
-        e = launch_bfs_level(f->span, d_map, d_begin, lo, hi - lo, n - hi, d_cc, d_scan, d_scan_tmp, scan_bytes, &total, s);
+        e = launch_bfs_level(f->span, sc.map, sc.begin, lo, hi - lo, n - hi, sc.cc, sc.scan, sc.scan_tmp,
+                             sc.scan_bytes, &total, s);
         if (e == hipSuccess && total > n - hi) {
             not_a_tree = true;
             break;
@@ -560,18 +577,14 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
     }
     if (e != hipSuccess || not_a_tree) {
         (void)hipStreamSynchronize(s);
-        cleanup();
         if (not_a_tree) return fail(OMK_ERR_STRUCTURE, "omk_forest_compact: the child ranges do not form a tree");
         return fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
     }
     const int64_t k = hi;
-    // one scratch array that every field passes through
-    e = hipMalloc((void **)&d_tmp, (size_t)k * 8);
-    if (e == hipSuccess && f->has_legal) e = hipMalloc((void **)&d_legal, (size_t)((k + 31) / 32) * 4);
     auto move_words = [&](void *arr) {
         if (e != hipSuccess || !arr) return;
-        e = launch_gather_words((uint32_t *)d_tmp, (const uint32_t *)arr, d_map, k, s);
-        if (e == hipSuccess) e = hipMemcpyAsync(arr, d_tmp, (size_t)k * 4, hipMemcpyDeviceToDevice, s);
+        e = launch_gather_words((uint32_t *)sc.tmp, (const uint32_t *)arr, sc.map, k, s);
+        if (e == hipSuccess) e = launch_copy_words(arr, sc.tmp, k, s);
     };
     move_words(f->N);
     move_words(f->W);
@@ -583,25 +596,50 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
     }
     if (f->has_action) move_words(f->action);
     if (e == hipSuccess && f->has_hash) {
-        e = launch_gather_dwords(d_tmp, f->hash, d_map, k, s);
-        if (e == hipSuccess) e = hipMemcpyAsync(f->hash, d_tmp, (size_t)k * 8, hipMemcpyDeviceToDevice, s);
+        e = launch_gather_dwords(sc.tmp, f->hash, sc.map, k, s);
+        if (e == hipSuccess) e = launch_copy_words(f->hash, sc.tmp, k * 2, s);
     }
     if (e == hipSuccess) {
-        e = launch_gather_span((int2 *)d_tmp, f->span, d_map, d_begin, k, s);
-        if (e == hipSuccess) e = hipMemcpyAsync(f->span, d_tmp, (size_t)k * sizeof(int2), hipMemcpyDeviceToDevice, s);
+        e = launch_gather_span((int2 *)sc.tmp, f->span, sc.map, sc.begin, k, s);
+        if (e == hipSuccess) e = launch_copy_words(f->span, sc.tmp, k * 2, s);
     }
     if (e == hipSuccess && f->has_legal) {
-        e = launch_gather_legal(d_legal, f->legal, d_map, k, s);
-        if (e == hipSuccess)
-            e = hipMemcpyAsync(f->legal, d_legal, (size_t)((k + 31) / 32) * 4, hipMemcpyDeviceToDevice, s);
+        e = launch_gather_legal(sc.legal, f->legal, sc.map, k, s);
+        if (e == hipSuccess) e = launch_copy_words(f->legal, sc.legal, (k + 31) / 32, s);
     }
-    if (e == hipSuccess && h_old_of_new) e = hipMemcpyAsync(h_old_of_new, d_map, (size_t)k * 4, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess && h_old_of_new) e = hipMemcpyAsync(h_old_of_new, sc.map, (size_t)k * 4, hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
-    cleanup();
     if (e != hipSuccess) return fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
     f->n_nodes = k;
+    f->generation++;
+    f->structure_changed = true;
     if (h_nodes_after) *h_nodes_after = k;
     return OMK_OK;
+}
+
+int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_compact: null forest");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact: nothing uploaded");
+    if (new_root < 0 || new_root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_compact: root %d", new_root);
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    const int64_t n = f->n_nodes;
+    CompactScratch sc;
+    hipError_t e = bfs_scan_bytes(n, &sc.scan_bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&sc.map, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&sc.begin, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&sc.cc, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&sc.scan, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc(&sc.scan_tmp, sc.scan_bytes > 0 ? sc.scan_bytes : 4);
+    if (e == hipSuccess) e = hipMalloc((void **)&sc.tmp, (size_t)n * 8);
+    if (e == hipSuccess && f->has_legal) e = hipMalloc((void **)&sc.legal, (size_t)((n + 31) / 32) * 4);
+    int rc = e == hipSuccess ? compact_in(f, new_root, h_nodes_after, h_old_of_new, sc)
+                             : fail(OMK_ERR_HIP, "omk_forest_compact: %s", hipGetErrorString(e));
+    (void)hipStreamSynchronize(f->stream);
+    for (void *p : {(void *)sc.map, (void *)sc.begin, (void *)sc.cc, (void *)sc.scan, (void *)sc.legal, (void *)sc.tmp,
+                    sc.scan_tmp})
+        if (p) (void)hipFree(p);
+    return rc;
 }
 
 int omk_forest_node_count(omk_forest *f, int64_t *h_nodes, int64_t *h_capacity) {
@@ -728,6 +766,7 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
     b->n_items0 = (int32_t)items.size();
     b->n_singles0 = (int32_t)singles.size();
     b->n = n;
+    b->generation = f->generation;
     b->selected = false;
     return OMK_OK;
 }
@@ -757,6 +796,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     if (!b || !p) return fail(OMK_ERR_INVALID, "omk_select_batch: null argument");
     omk_forest *f = b->f;
     if (!f->uploaded || b->n <= 0) return fail(OMK_ERR_STATE, "omk_select_batch: upload a forest and set roots first");
+    if (int rc = fresh_batch("omk_select_batch", b)) return rc;
     if (p->use_rave && !f->has_rave)
         return fail(OMK_ERR_INVALID, "omk_select_batch: use_rave on a forest created without RAVE arrays");
     if (p->pw && !f->prior_sorted)
@@ -772,10 +812,10 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.seg[0] = b->seg[0];
     a.seg[1] = b->seg[1];
     if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
-        HIP_TRY(hipMemsetAsync(b->q_ready, 0, (size_t)std::max(b->q_cap, 1) * 4, f->stream));
-        HIP_TRY(hipMemsetAsync(b->single_ready, 0, (size_t)std::max(b->max_traversals, 1) * 4, f->stream));
+        HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
+        HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
         // the two depth-cap counters take turns by call parity, which this restart breaks once
-        HIP_TRY(hipMemsetAsync(b->counters + kTruncatedWord, 0, 2 * sizeof(int32_t), f->stream));
+        HIP_TRY(launch_fill_words(b->counters + kTruncatedWord, 0u, 2, f->stream));
         b->epoch = 0;
     }
     b->epoch++;
@@ -829,6 +869,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
 int omk_backup_batch(omk_batch *b, int32_t virtual_loss) {
     if (!b) return fail(OMK_ERR_INVALID, "omk_backup_batch: null batch");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_backup_batch: no selected paths");
+    if (int rc = fresh_batch("omk_backup_batch", b)) return rc;
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_backup(b->f->dev(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
                           virtual_loss, b->f->stream));
@@ -838,6 +879,7 @@ int omk_backup_batch(omk_batch *b, int32_t virtual_loss) {
 int omk_backup_rave_batch(omk_batch *b) {
     if (!b) return fail(OMK_ERR_INVALID, "omk_backup_rave_batch: null batch");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_backup_rave_batch: no selected paths");
+    if (int rc = fresh_batch("omk_backup_rave_batch", b)) return rc;
     if (!b->f->has_rave) return fail(OMK_ERR_INVALID, "omk_backup_rave_batch: the forest has no RAVE arrays");
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_rave_backup(b->f->mut(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
@@ -848,6 +890,7 @@ int omk_backup_rave_batch(omk_batch *b) {
 int omk_revert_vl(omk_batch *b, int32_t virtual_loss) {
     if (!b) return fail(OMK_ERR_INVALID, "omk_revert_vl: null batch");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_revert_vl: no selected paths");
+    if (int rc = fresh_batch("omk_revert_vl", b)) return rc;
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_revert_vl(b->f->dev(), b->paths, b->path_len, b->n, b->stride, b->max_depth + 1, virtual_loss,
                              b->f->stream));
@@ -889,6 +932,7 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
                      int32_t action_space, int32_t *h_first_child) {
     if (!b || !h_move_begin || !h_moves) return fail(OMK_ERR_INVALID, "omk_expand_batch: null argument");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_expand_batch: no selected paths");
+    if (int rc = fresh_batch("omk_expand_batch", b)) return rc;
     if (h_policy && action_space <= 0)
         return fail(OMK_ERR_INVALID, "omk_expand_batch: a policy needs action_space > 0 (got %d)", action_space);
     omk_forest *f = b->f;
@@ -979,6 +1023,7 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
         HIP_TRY(hipMemcpyAsync(status.data(), d_status, nj * 4, hipMemcpyDeviceToHost, s));
         HIP_TRY(hipStreamSynchronize(s));
         f->n_nodes = cursor;
+        f->structure_changed = true;  // ids keep their meaning, but an upload of the old arrays would not
         f->max_fanout = mf;
         if (!sorted) f->prior_sorted = false;
         if (h_first_child)
@@ -991,6 +1036,7 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
 int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t *h_leaf, int32_t *h_actions) {
     if (!b) return fail(OMK_ERR_INVALID, "omk_batch_read: null batch");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_read: no selected paths");
+    if (int rc = fresh_batch("omk_batch_read", b)) return rc;
     omk_forest *f = b->f;
     if (int rc = use_device(f)) return rc;
     hipStream_t s = f->stream;
@@ -1144,6 +1190,7 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
     if (!tt || !b || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe_leaves: null argument");
     if (tt->f != b->f) return fail(OMK_ERR_INVALID, "omk_tt_probe_leaves: table and batch belong to different forests");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: no selected paths");
+    if (int rc = fresh_batch("omk_tt_probe_leaves", b)) return rc;
     if (!b->f->has_hash) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: the forest was uploaded without position keys");
     if (int rc = use_device(tt->f)) return rc;
     HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->f->n_nodes, b->n, min_depth, d_out,
@@ -1157,6 +1204,7 @@ int omk_batch_leaf_keys(omk_batch *b, const uint64_t *d_piece_keys, int32_t cell
         return fail(OMK_ERR_INVALID, "omk_batch_leaf_keys: null argument");
     if (cells <= 0) return fail(OMK_ERR_INVALID, "omk_batch_leaf_keys: cells %d", cells);
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_leaf_keys: no selected paths");
+    if (int rc = fresh_batch("omk_batch_leaf_keys", b)) return rc;
     omk_forest *f = b->f;
     if (int rc = use_device(f)) return rc;
     hipStream_t s = f->stream;

@@ -50,6 +50,22 @@ __global__ __launch_bounds__(256) void k_gather_legal(uint32_t *dst, const uint3
     dst[w] = word;
 }
 
+// Plain fill kernel: used instead of hipMemsetAsync wherever a caller might capture the stream
+// into a graph.
+__global__ __launch_bounds__(256) void k_fill_words(uint32_t *dst, uint32_t value, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * 256;
+    for (; i < n; i += step) dst[i] = value;
+}
+
+hipError_t launch_fill_words(void *dst, uint32_t value, int64_t n_words, hipStream_t s) {
+    if (n_words <= 0) return hipSuccess;
+    int64_t blocks = (n_words + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_fill_words, dim3((unsigned)blocks), dim3(256), 0, s, (uint32_t *)dst, value, n_words);
+    return hipGetLastError();
+}
+
 hipError_t bfs_scan_bytes(int64_t max_items, size_t *bytes) {
     *bytes = 0;
     return hipcub::DeviceScan::ExclusiveSum(nullptr, *bytes, (const int32_t *)nullptr, (int32_t *)nullptr,
@@ -78,7 +94,7 @@ hipError_t launch_bfs_level(const int2 *span, int32_t *order, int32_t *new_begin
                            cnt, lo + cnt, scan);
         e = hipGetLastError();
     } else {
-        e = hipMemsetAsync(new_begin + lo, 0, (size_t)cnt * 4, s);
+        e = launch_fill_words(new_begin + lo, 0u, cnt, s);
     }
     return e;
 }

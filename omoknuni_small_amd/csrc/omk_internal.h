@@ -106,6 +106,7 @@ hipError_t launch_leaf_keys(const ForestDev &f, const int32_t *paths, const int3
                             const uint64_t *piece, int cells, const uint64_t *player, const uint64_t *root_key,
                             const int32_t *root_player, uint64_t *out, int *d_status, hipStream_t s);
 hipError_t launch_copy_words(void *dst, const void *src, int64_t n_words, hipStream_t s);
+hipError_t launch_fill_words(void *dst, uint32_t value, int64_t n_words, hipStream_t s);
 
 // The same arrays for the one operation that writes the structure (leaf expansion).
 struct ForestMut {

@@ -152,11 +152,15 @@ def test_bench_byte_model_on_a_known_tree():
     assert list(L[:2]) == [2, 2]
     paths = np.array([[0, 1, 4], [0, 1, 5], [0, 3, -1]], np.int32)
     plen = np.array([3, 3, 2], np.int32)
-    sel, bak, steps = bench.algorithmic_bytes(soa, {}, paths, plen, np.zeros(6, np.int32))
+    sel, bak, steps = bench.ByteModel(soa, {}).step(paths, plen, np.zeros(6, np.int32))
     assert steps == 5
     # per selection step: L*16 + ceil(F/8) + 24; per path entry written: 4
     assert sel == 3 * (2 * 16 + 1 + 24) + 2 * (2 * 16 + 1 + 24) + 4 * 8
     assert bak == 24 * 8 + 4 * 3 + 4 * 8
+    assert list(bench.visits_of(paths, plen, 6)) == [3, 2, 0, 1, 1, 1]
+    # the exact value sums of a backup: the leaf takes +v, every ply up flips the sign
+    add = bench.exact_value_sums(paths, plen, np.array([0.5, -0.25, 1.0], np.float32), 6)
+    assert list(add) == [0.5 - 0.25 - 1.0, -0.5 + 0.25, 0.0, 1.0, 0.5, -0.25]
 
 
 def test_golden_fixture_is_data_only():
