@@ -192,6 +192,17 @@ int omk_forest_reroot_child(omk_forest *f, int32_t root, int32_t last_action, in
  * the host only reads the size of every level. */
 int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new);
 
+/* omk_forest_compact for callers that cannot allocate device memory (code under HIP graph
+ * capture around it, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart
+ * in the reference.  Same arguments, same result, but every piece of device scratch memory (the
+ * breadth-first order, the per-level counts and their scan, the staging array the fields pass
+ * through) lives in one array inside the library that each GPU holds for the life of the process
+ * (about 25 MiB), and the call makes no hipMalloc / hipFree.  Limit: the forest may hold at most
+ * 2^20 = 1048576 nodes when it is called (OMK_ERR_CAPACITY beyond that, and nothing is changed).
+ * All calls on one GPU share that array: two calls that overlap in time on the same GPU, from
+ * whatever forests or threads, race; calls one after another need no clearing in between. */
+int omk_forest_compact_static(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new);
+
 /* Leaf expansion for the leaves of the last selection: MCTSNode::expand
  * (src/mcts/mcts_node.cpp:238-436) followed by setPriorProbabilities (:512-593), as the backup
  * phase does before it backs the values up (src/mcts/mcts_engine_batch_tree_simple.cpp:249-259).

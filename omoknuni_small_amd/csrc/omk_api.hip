@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -640,6 +641,79 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
                     sc.scan_tmp})
         if (p) (void)hipFree(p);
     return rc;
+}
+
+// ---- the same compaction for callers that cannot allocate ----
+//
+// All the scratch memory of a compaction of up to kStaticCompactNodes nodes, laid out in one
+// file-scope device array: every GPU the library runs on holds its own copy for the life of the
+// process.  In host code the array's name is only a handle for hipGetSymbolAddress; the address the
+// kernels get is looked up once per device (static_scratch) and kept.
+constexpr int64_t kStaticCompactNodes = 1ll << 20;
+constexpr size_t kStaticScanBytes = 1u << 20;  // work space of the level scan (a few KiB are used)
+constexpr size_t kStaticWords = (size_t)kStaticCompactNodes * 4;
+constexpr size_t kStaticOffMap = 0;
+constexpr size_t kStaticOffBegin = kStaticOffMap + kStaticWords;
+constexpr size_t kStaticOffCc = kStaticOffBegin + kStaticWords;
+constexpr size_t kStaticOffScan = kStaticOffCc + kStaticWords;
+constexpr size_t kStaticOffTmp = kStaticOffScan + kStaticWords;
+constexpr size_t kStaticOffLegal = kStaticOffTmp + 2 * kStaticWords;
+constexpr size_t kStaticOffScanTmp = kStaticOffLegal + kStaticWords / 32;
+constexpr size_t kStaticScratchBytes = kStaticOffScanTmp + kStaticScanBytes;
+static_assert(kStaticOffScanTmp % 256 == 0 && kStaticOffLegal % 256 == 0, "parts of the scratch keep its alignment");
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on every device, once known
+
+// The device address of the scratch array on the forest's device (which must be current).
+static int static_scratch(int device, unsigned char **out) {
+    if (device < 0 || device >= kMaxDevices) return fail(OMK_ERR_INVALID, "device %d: at most %d devices", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(OMK_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
+        g_scratch_ptr[device] = (unsigned char *)p;
+    }
+    *out = g_scratch_ptr[device];
+    return OMK_OK;
+}
+
+int omk_forest_compact_static(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, int32_t *h_old_of_new) {
+    if (!f) return fail(OMK_ERR_INVALID, "omk_forest_compact_static: null forest");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact_static: nothing uploaded");
+    if (new_root < 0 || new_root >= f->n_nodes)
+        return fail(OMK_ERR_INVALID, "omk_forest_compact_static: root %d", new_root);
+    if (f->n_nodes > kStaticCompactNodes)
+        return fail(OMK_ERR_CAPACITY,
+                    "omk_forest_compact_static: the forest holds %lld nodes, the static scratch memory serves at most "
+                    "%lld; use omk_forest_compact",
+                    (long long)f->n_nodes, (long long)kStaticCompactNodes);
+    if (int rc = use_device(f)) return rc;
+    unsigned char *base = nullptr;
+    if (int rc = static_scratch(f->device, &base)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    CompactScratch sc;
+    size_t need = 0;
+    HIP_TRY(bfs_scan_bytes(f->n_nodes, &need));
+    if (need > kStaticScanBytes)
+        return fail(OMK_ERR_CAPACITY, "omk_forest_compact_static: the level scan wants %zu bytes of work space, %zu are reserved",
+                    need, kStaticScanBytes);
+    // every part is written by this call before it is read (the order map from the root on, the
+    // counts and their scan per level, the staging array per field): nothing has to start at zero
+    sc.map = (int32_t *)(base + kStaticOffMap);
+    sc.begin = (int32_t *)(base + kStaticOffBegin);
+    sc.cc = (int32_t *)(base + kStaticOffCc);
+    sc.scan = (int32_t *)(base + kStaticOffScan);
+    sc.tmp = (uint64_t *)(base + kStaticOffTmp);
+    sc.legal = (uint32_t *)(base + kStaticOffLegal);
+    sc.scan_tmp = base + kStaticOffScanTmp;
+    sc.scan_bytes = kStaticScanBytes;
+    return compact_in(f, new_root, h_nodes_after, h_old_of_new, sc);
 }
 
 int omk_forest_node_count(omk_forest *f, int64_t *h_nodes, int64_t *h_capacity) {

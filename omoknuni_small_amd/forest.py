@@ -23,7 +23,7 @@ u64p = C.POINTER(C.c_uint64)
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
-    "omk_expand_batch", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_reroot_child", "omk_forest_compact",
+    "omk_expand_batch", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_reroot_child", "omk_forest_compact", "omk_forest_compact_static",
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
@@ -174,13 +174,14 @@ class Forest:
                                                  C.byref(c)))
         return int(c.value)
 
-    def compact(self, new_root):
+    def compact(self, new_root, static=False):
         """Keeps the subtree of new_root, renumbered breadth-first from 0; returns the old id of
-        every new node."""
+        every new node.  static: the variant that allocates nothing (at most 2^20 nodes)."""
         n_old, _ = self.node_count()
         order = np.empty(n_old, np.int32)
         k = C.c_int64()
-        _check(self._lib.omk_forest_compact(self._h, C.c_int32(int(new_root)), C.byref(k), _ptr(order, i32p)))
+        fn = self._lib.omk_forest_compact_static if static else self._lib.omk_forest_compact
+        _check(fn(self._h, C.c_int32(int(new_root)), C.byref(k), _ptr(order, i32p)))
         self.n_nodes = int(k.value)
         return order[:self.n_nodes].copy()
 
