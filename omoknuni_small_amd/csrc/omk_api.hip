@@ -1183,9 +1183,12 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     return OMK_OK;
 }
 
-#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
-// measurement builds only: the per-node timeline of the last selection (4 x int64 per node)
+// The per-node timeline of the last selection (4 x int64 per processed multi-visitor item), which
+// only a build with -DOMK_TRACE records.
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
+    if (!b || !h_trace || !h_n || max_entries < 0) return fail(OMK_ERR_INVALID, "omk_debug_trace: bad argument");
+#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_debug_trace: no selected paths");
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     HIP_TRY(hipMemcpy(h_n, b->counters + 24, 4, hipMemcpyDeviceToHost));
@@ -1193,8 +1196,11 @@ int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32
     if (n > 0) HIP_TRY(hipMemcpy(h_trace, b->out_paths, (size_t)n * 32, hipMemcpyDeviceToHost));
     *h_n = n;
     return OMK_OK;
-}
+#else
+    *h_n = 0;
+    return fail(OMK_ERR_UNSUPPORTED, "omk_debug_trace: this library was built without -DOMK_TRACE (make trace)");
 #endif
+}
 
 // ---------------------------------------------------------------- transposition table
 

@@ -27,7 +27,7 @@ EXPORTS = [
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_leaf_keys", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
 ]
@@ -67,7 +67,9 @@ class _BatchDev(C.Structure):
 
 
 def library_path():
-    return os.path.join(_HERE, "libomk_forest.so")
+    """libomk_forest.so beside this file, or another build of the same ABI named by OMK_FOREST_LIB
+    (the measurement build libomk_forest_trace.so)."""
+    return os.environ.get("OMK_FOREST_LIB") or os.path.join(_HERE, "libomk_forest.so")
 
 
 def load_library():
@@ -373,6 +375,15 @@ class Batch:
                 "replayed_nodes", "threshold_probes", "single_visitor_steps", "fail_code", "cyc_threshold",
                 "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "sliced_nodes")
         return dict(zip(keys, map(int, out)))
+
+    def debug_trace(self, max_entries=1 << 16):
+        """Timeline of the last select() from a library built with -DOMK_TRACE: int64 array [n, 4] of
+        (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | counters << 32."""
+        buf = np.zeros((int(max_entries), 4), np.int64)
+        n = C.c_int32()
+        _check(self._lib.omk_debug_trace(self._h, buf.ctypes.data_as(C.c_void_p), C.c_int32(int(max_entries)),
+                                         C.byref(n)))
+        return buf[:n.value].copy()
 
     def device(self):
         d = _BatchDev()

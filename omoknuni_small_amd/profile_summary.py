@@ -2,11 +2,17 @@
 
     python -m omoknuni_small_amd.profile_summary stats  <kernel_stats.csv>
     python -m omoknuni_small_amd.profile_summary pmc    <counter_collection.csv> <COUNTER> [copy_bytes]
+    OMK_FOREST_LIB=omoknuni_small_amd/libomk_forest_trace.so \
+    python -m omoknuni_small_amd.profile_summary timeline <workload> [warmup_steps]
 
 `stats` prints calls / total / average duration per kernel.  `pmc` prints, per kernel, the
 sum of a hardware counter over its dispatches; given the bytes the calibration copy kernel
 (k_copy_words) moved each way per launch, it also prints the counter-to-bytes factor that
-copy implies and every kernel's traffic in bytes scaled by it.
+copy implies and every kernel's traffic in bytes scaled by it.  `timeline` runs a benchmark
+workload on the GPU through the measurement build of the library (make -C csrc trace), which records
+when every multi-visitor work item of a selection was processed, and prints the chain of crowded
+nodes of one steady-state selection: per tree level the node with most visitors, when its wavefront
+started and ended, and what it did.
 """
 import csv
 import sys
@@ -50,11 +56,70 @@ def pmc(path, counter, copy_bytes=None):
         print(line)
 
 
+def timeline(workload, warmup=8):
+    import numpy as np
+    import omoknuni_small_amd as omk
+    from omoknuni_small_amd import synth
+
+    soa, roots, meta = synth.generate(workload, seed=2025)
+    B, D, vl = int(meta["n_traversals"]), int(meta["max_depth"]), int(meta["virtual_loss"])
+    troots = synth.traversal_roots(roots, B)
+    values = np.random.default_rng(2026).uniform(-1, 1, B).astype(np.float32)
+    sp = omk.SelectParams(c_puct=meta["c_puct"], virtual_loss=vl, use_rave=bool(meta.get("has_rave")),
+                          rave_k=float(meta.get("rave_k", 3000.0)), pw=bool(meta.get("pw")))
+    forest = omk.Forest.from_soa(soa)
+    batch = omk.Batch(forest, B, D)
+    batch.set_roots(troots)
+    batch.set_values(values)
+    for _ in range(int(warmup)):
+        batch.select(sp)
+        batch.backup(vl)
+    batch.select(sp)
+    tr = batch.debug_trace()
+    batch.backup(vl)
+    t0 = tr[:, 0].min()
+    start = (tr[:, 0] - t0) / 100.0  # microseconds
+    end = (tr[:, 1] - t0) / 100.0
+    m = (tr[:, 2] & 0xFFFFFFFF).astype(np.int64)
+    depth = ((tr[:, 2] >> 32) & 0xFFFFFFF).astype(np.int64)
+    kind = ((tr[:, 2] >> 60) & 7).astype(np.int64)
+    node = (tr[:, 3] & 0xFFFFFFFF).astype(np.int64)
+    ctr = (tr[:, 3] >> 32) & 0xFFFFFFFF
+    print("workload %s, selection number %d: %d multi-visitor items traced, span %.1f us (100 MHz clock)"
+          % (workload, int(warmup) + 1, len(tr), end.max()))
+    print("chain of crowded nodes: per level the node with most visitors (kinds: node = taken as a whole, "
+          "early = published before its visitor list was complete; a node cut into slices / scatter parts shows "
+          "their number and the span from the first start to the last end)")
+    print("%5s %9s %9s %7s %9s %9s %8s  %s" % ("level", "node", "visitors", "kind", "start_us", "end_us", "us", "work"))
+    names = {0: "node", 1: "slice", 2: "part", 3: "early"}
+    for d in range(int(depth.max()) + 1):
+        at = np.nonzero(depth == d)[0]
+        if len(at) == 0:
+            continue
+        top = at[np.argmax(m[at])]
+        same = at[node[at] == node[top]]
+        whole = same[(kind[same] == 0) | (kind[same] == 3)]
+        first = whole[0] if len(whole) else same[0]
+        s0, e1 = start[same].min(), end[same].max()
+        n_sl, n_pt = int((kind[same] == 1).sum()), int((kind[same] == 2).sum())
+        batches = int(sum(int(c) & 0xFF for c in ctr[same]))
+        runs = int(sum((int(c) >> 8) & 0xFF for c in ctr[same]))
+        work = "%d batch(es), %d run(s)" % (batches, runs)
+        if n_sl or n_pt:
+            work += ", %d slice item(s), %d scatter part(s)" % (n_sl, n_pt)
+        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f  %s" % (d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1,
+                                                       e1 - s0, work))
+    by_kind = ", ".join("%s %d" % (names[k], int((kind == k).sum())) for k in sorted(names))
+    print("items by kind: %s; visitors per item: median %d, largest %d" % (by_kind, int(np.median(m)), int(m.max())))
+
+
 if __name__ == "__main__":
     if len(sys.argv) >= 3 and sys.argv[1] == "stats":
         stats(sys.argv[2])
     elif len(sys.argv) >= 4 and sys.argv[1] == "pmc":
         pmc(sys.argv[2], sys.argv[3], int(sys.argv[4]) if len(sys.argv) > 4 else None)
+    elif len(sys.argv) >= 3 and sys.argv[1] == "timeline":
+        timeline(sys.argv[2], int(sys.argv[3]) if len(sys.argv) > 3 else 8)
     else:
         print(__doc__)
         sys.exit(2)

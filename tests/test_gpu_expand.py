@@ -275,3 +275,35 @@ def test_compaction_of_deep_and_wide_shapes_and_of_a_broken_structure():
     bad["child_begin"][n - 1], bad["child_count"][n - 1] = 0, 2
     with pytest.raises(omk.OmkError):  # the upload already refuses it (a node with two parents)
         omk.Forest.from_soa(bad).compact(0)
+
+
+def test_stale_batch_is_refused_after_compaction():
+    """Roots and paths are node ids: after a compaction a batch made before it says so."""
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(73, n_expand=80, fanout=(2, 8), max_depth=6)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, 50, 6)
+    b.set_roots(np.zeros(50, np.int32))
+    sp = omk.SelectParams()
+    b.select(sp)
+    f.compact(int(soa["child_begin"][0]))
+    for call in (lambda: b.select(sp), lambda: b.backup(3), lambda: b.read(), lambda: b.revert_vl(3)):
+        with pytest.raises(omk.OmkError) as e:
+            call()
+        assert e.value.code == -6
+    b.set_roots(np.zeros(50, np.int32))
+    b.select(sp)
+    b.read()
+    # an upload of the same child ranges as the last upload (statistics put back) keeps a batch
+    # usable; an upload of anything else does not
+    st = dict(f.download(), **f.download_structure())
+    f.upload(st)
+    b.set_roots(np.zeros(50, np.int32))
+    b.select(sp)
+    f.upload(st)
+    b.select(sp)
+    b.read()
+    f.upload(soa)
+    with pytest.raises(omk.OmkError) as e:
+        b.select(sp)
+    assert e.value.code == -6
