@@ -250,10 +250,15 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
  * them off omk_batch_stats returns zeros.  Diagnostics only; no counterpart in the reference. */
 int omk_batch_set_stats(omk_batch *b, int32_t enabled);
 /* Measurement aid, no counterpart in the reference: the timeline of the last select, one record
- * of four int64 per multi-visitor work item processed: start and end on the GPU's 100 MHz clock,
+ * of twelve int64 per multi-visitor work item processed: start and end on the GPU's 100 MHz clock,
  * visitors | depth << 32 | item kind << 60, node | (batches | runs << 8 | entries of the last
- * batch << 16) << 32.  Only a library built with -DOMK_TRACE (csrc/Makefile, target `trace`)
- * records it; any other build returns OMK_ERR_UNSUPPORTED and *h_n = 0. */
+ * batch << 16) << 32, then eight words holding two 32-bit phase times each (same clock; slots 0-7:
+ * threshold phase, -, evaluation and ordering, emission and checks, loading and scoring the
+ * children, the whole settling of the visitors, the partition, -; slots 8-15, parts of these: run
+ * probe, bounds and active children, threshold search, exact counts, one-winner check, -, -, -).
+ * h_trace has room for max_entries records.
+ * Only a library built with -DOMK_TRACE (csrc/Makefile, target `trace`) records it; any other
+ * build returns OMK_ERR_UNSUPPORTED and *h_n = 0. */
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n);
 /* The multi-visitor selection kernel is persistent: its wavefronts wait for work items that
  * other wavefronts publish.  Every wait is bounded; a wavefront that polls `polls` times in

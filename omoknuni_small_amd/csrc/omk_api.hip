@@ -918,7 +918,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
 #if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
     a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
     a.trace_n = b->counters + 24;
-    a.trace_cap = (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 8);
+    a.trace_cap = (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 24);
     a.dbg_grid = getenv("OMK_DBG_GRID") ? atoi(getenv("OMK_DBG_GRID")) : 0;
 #endif
     a.singles0 = b->singles0;
@@ -1183,7 +1183,7 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     return OMK_OK;
 }
 
-// The per-node timeline of the last selection (4 x int64 per processed multi-visitor item), which
+// The per-node timeline of the last selection (12 x int64 per processed multi-visitor item), which
 // only a build with -DOMK_TRACE records.
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
     if (!b || !h_trace || !h_n || max_entries < 0) return fail(OMK_ERR_INVALID, "omk_debug_trace: bad argument");
@@ -1192,8 +1192,8 @@ int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     HIP_TRY(hipMemcpy(h_n, b->counters + 24, 4, hipMemcpyDeviceToHost));
-    int32_t n = std::min(std::min(*h_n, max_entries), (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 8));
-    if (n > 0) HIP_TRY(hipMemcpy(h_trace, b->out_paths, (size_t)n * 32, hipMemcpyDeviceToHost));
+    int32_t n = std::min(std::min(*h_n, max_entries), (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 24));
+    if (n > 0) HIP_TRY(hipMemcpy(h_trace, b->out_paths, (size_t)n * 96, hipMemcpyDeviceToHost));
     *h_n = n;
     return OMK_OK;
 #else

@@ -105,6 +105,28 @@ enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
         if (a.stats && lane == 0) atomicAdd(a.stats + (slot), (int)((now_ - t_phase_) >> 4)); \
         t_phase_ = now_;                                                            \
     } while (0)
+#elif defined(OMK_TRACE)
+// timeline build: the owner wavefront adds up, per node, the time it spends in every phase
+// (100 MHz clock) in the block's LDS scratch; the node's trace record carries the sums
+#define OMK_FAIL(code) return false
+#define OMK_NOTE(code) \
+    do {               \
+    } while (0)
+#define OMK_T0() long long t_phase_ = wall_clock64()
+#define OMK_TICK(slot)                                                       \
+    do {                                                                     \
+        long long now_ = wall_clock64();                                     \
+        if (lane == 0) lds.tph[(slot)-8] += (uint32_t)(now_ - t_phase_);     \
+        t_phase_ = now_;                                                     \
+    } while (0)
+// finer stamps inside a phase, on a timer of their own
+#define OMK_S0() long long t_sub_ = wall_clock64()
+#define OMK_STAMP(slot)                                                  \
+    do {                                                                 \
+        long long now_ = wall_clock64();                                 \
+        if (lane == 0) lds.tph[(slot)] += (uint32_t)(now_ - t_sub_);     \
+        t_sub_ = now_;                                                   \
+    } while (0)
 #else
 #define OMK_FAIL(code) return false
 #define OMK_NOTE(code) \
@@ -115,6 +137,14 @@ enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
     } while (0)
 #define OMK_TICK(slot) \
     do {               \
+    } while (0)
+#endif
+#ifndef OMK_S0
+#define OMK_S0() \
+    do {         \
+    } while (0)
+#define OMK_STAMP(slot) \
+    do {                \
     } while (0)
 #endif
 
@@ -169,6 +199,9 @@ template <int R>
 struct WaveLds {
     TeamCmd cmd;
     uint32_t red[4];       // team reductions: smallest / largest inverted key, flags
+#ifdef OMK_TRACE
+    uint32_t tph[16];      // timeline build: time of the node at hand per phase
+#endif
     int wsum[kTeamWaves];  // team prefix scan: totals of the wavefronts
     int offs[R * kWave];   // exclusive prefix of the visit counts in child order
     int st_n[R * kWave];   // statistics of every child, readable by any lane
@@ -495,6 +528,62 @@ __device__ __forceinline__ bool wait_list(const SelectArgs &a, int off, int dept
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     return ok;
+}
+
+// A key in [lo_key, hi_key] whose estimated entry count est(key) (wave-uniform, non-increasing in
+// the key) lands in the window [target, acc_hi], or failing that in [acc_below, target); the largest
+// key found with est >= target otherwise.  est(lo_key) >= target and est(hi_key) < target are taken
+// for granted.  The count is close to a hyperbola in the score, alpha / (score + 1) - beta (every
+// child's next visits score about (W + N + c) / x - 1), so the search works in y = 1 / (score + 1),
+// where the count is nearly a straight line: false position between the ends of its bracket, with
+// the value of an end that stays put halved at every step that leaves it there (the Illinois rule:
+// the ends' counts are capped per child and would otherwise pin the interpolation), the first
+// step from made-up end values.  Halving the KEY interval instead takes a dozen steps whenever the
+// bracket straddles score zero, where the keys are densest.  Deterministic: the same arguments
+// give the same key on every wavefront.  Only efficiency depends on the result: whatever key comes
+// out, the caller counts exactly.
+template <typename Est>
+__device__ __forceinline__ uint32_t search_threshold(uint32_t lo_key, uint32_t hi_key, int target, int acc_hi,
+                                                     int acc_below, int &evals, Est est) {
+    uint32_t klo = lo_key, khi = hi_key;
+    auto y_of = [](uint32_t k) {
+        float d = key_score(k) + 1.0f;
+        d = d > 1e-6f ? d : 1e-6f;
+        return __frcp_rn(d);
+    };
+    float ylo = y_of(klo), yhi = y_of(khi);
+    const float aim = (float)target + 0.5f * (float)(acc_hi - target);
+    float flo = aim, fhi = -aim;  // count minus aim at the two ends: made up until an end has been evaluated
+    int last = 0;                 // which end the last step moved: +1 the low one, -1 the high one
+    for (int it = 0; it < 48 && khi - klo > 1u; it++) {
+        const float ym = (ylo * fhi - yhi * flo) * __frcp_rn(fhi - flo);
+        uint32_t kmid = score_key(__frcp_rn(ym) - 1.0f);
+        if (!(kmid > klo)) kmid = klo + 1u;
+        if (!(kmid < khi)) kmid = khi - 1u;
+        // the dense sliver: once false position stops moving off an end, halve the key interval
+        if (it >= 12) kmid = klo + ((khi - klo) >> 1);
+        const int e = est(kmid);
+        evals++;
+        if (e >= target) {
+            klo = kmid;
+            ylo = y_of(kmid);
+            flo = (float)e - aim;
+            if (e <= acc_hi) break;
+            if (last > 0) fhi *= 0.5f;
+            last = 1;
+        } else {
+            if (e >= acc_below) {
+                klo = kmid;
+                break;
+            }
+            khi = kmid;
+            yhi = y_of(kmid);
+            fhi = (float)e - aim;
+            if (last < 0) flo *= 0.5f;
+            last = -1;
+        }
+    }
+    return klo;
 }
 
 template <int NT>
@@ -886,6 +975,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
 #endif
 
         // ---- 1. threshold and exact per-child counts ----
+        OMK_S0();
         uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -1039,6 +1129,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             }
         }
         if (run_min == 1) OMK_FAIL(11);  // the run that had to be there was refused
+        OMK_STAMP(8);
         const int want = remaining < kBatchCap ? remaining : kBatchCap;
         // lower bound of any useful threshold: a child alone has `want` entries at or above the
         // key of its want-th next visit; the best such key over all children (the child that
@@ -1112,37 +1203,34 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         int ct[R];
         total = 0;
         int tries = 0;
+        OMK_STAMP(9);
         uint32_t T_forced = 0u;  // threshold imposed for the next round instead of searching one
         bool allow_above = true;
         for (;;) {
             if (++tries > 8) OMK_FAIL(5);
             const uint32_t T_now = T_forced;  // imposed for this round only
             T_forced = 0u;
-            // bisection on the KEY (not the score: entries may crowd into a sliver of the score
-            // range that halving a wide score interval never resolves) with the estimated counts
-            // only, no exact evaluation
-            uint32_t klo = lo_key, khi = hi_key;
-            for (int it = 0; it < 32 && T_now == 0u && khi - klo > 1u; it++) {
-                const uint32_t kmid = klo + ((khi - klo) >> 1);
-                const float mid = key_score(kmid);
-                int est = 0;
+            // a threshold with about `target` ESTIMATED entries at or above it (no exact evaluation
+            // yet): a quarter more than aimed at costs less than more search steps, and a batch that
+            // cannot finish the node anyway may as well be a little smaller
+            uint32_t klo = lo_key;
+            int n_evals = 0;
+            if (T_now == 0u) {
+                int acc_hi = target + (target >> 2);
+                if (acc_hi > kBatchCap - margin) acc_hi = kBatchCap - margin;
+                if (acc_hi < target) acc_hi = target;
+                const int acc_below = can_finish ? target : target - (target >> 2);
+                klo = search_threshold(lo_key, hi_key, target, acc_hi, acc_below, n_evals, [&](uint32_t kmid) {
+                    const float mid = key_score(kmid);
+                    int est = 0;
 #pragma unroll
-                for (int r = 0; r < R; r++)
-                    if (r < rounds && ac[r] >= 0)
-                        est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, child_cap);
-                const int e = wave_sum_i32(est);
-                if (e >= target) {
-                    klo = kmid;
-                    // close enough: a quarter more entries than aimed at cost less than more steps
-                    if (e <= target + (target >> 2) && e <= kBatchCap - margin) break;
-                } else {
-                    khi = kmid;
-                    if (!can_finish && e >= target - (target >> 2)) {
-                        klo = kmid;  // a batch that cannot finish anyway may as well be a little smaller
-                        break;
-                    }
-                }
+                    for (int r = 0; r < R; r++)
+                        if (r < rounds && ac[r] >= 0)
+                            est += predict_count<RAVE>(an[r], aw[r], ap[r], avl[r], aq2[r], c.ep, uvl, mid, child_cap);
+                    return wave_sum_i32(est);
+                });
             }
+            OMK_STAMP(10);
             uint32_t T = T_now != 0u ? T_now : klo;
             if (T < lo_key) T = lo_key;
             if (T > hi_key) T = hi_key;
@@ -1191,6 +1279,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 }
             }
             total = wave_sum_i32(sum);  // at most 64 * R * (capacity + 1)
+            OMK_STAMP(11);
             if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
             // A batch that does not fit is cut at the child with most entries (typically one
             // whose score hardly moves with virtual loss): it contributes fewer entries now,
@@ -1437,34 +1526,26 @@ __device__ __forceinline__ void active_counts(const ActiveSet<R> &s, float ep, u
     }
 }
 
-// A threshold at or above which about `target` of the node's entries lie, by bisection on
-// the key itself over ESTIMATED counts.  All targets of a node bisect the SAME interval
-// [lo_key, hi_key] for the same number of steps at most, so their thresholds come out
-// ordered like the targets (two searches see the same midpoints until they part, and from
-// then on one interval lies above the other; a search that stops early inside a window
-// narrower than the distance between two targets is passed below by every later target).
-// Bisecting keys, not scores, keeps thresholds apart even where thousands of entries crowd
-// into a sliver of the score range.
+// A threshold at or above which about `target` of the node's entries lie, found on ESTIMATED
+// counts (search_threshold).  The thresholds of a node's targets come out ordered like the
+// targets: a search either stops with its count inside [target, target + window], and the windows
+// of two targets are narrower than their distance, or it ends on the largest key whose count
+// still reaches the target; the counts do not increase with the key, so in every combination the
+// larger target gets the lower key.  (The estimate's fast arithmetic may break that monotonicity
+// by a hair; the caller checks the order of the thresholds and of the exact counts.)
 template <int R, bool RAVE>
 __device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t lo_key,
                                                      uint32_t hi_key, int target, int window, int m) {
-    uint32_t klo = lo_key, khi = hi_key;  // est(klo) >= target is taken for granted, est(khi) < target
-    for (int it = 0; it < 32 && khi - klo > 1u; it++) {
-        const uint32_t kmid = klo + ((khi - klo) >> 1);
+    int n_evals = 0;
+    return search_threshold(lo_key, hi_key, target, target + window, target, n_evals, [&](uint32_t kmid) {
         const float mid = key_score(kmid);
         int est = 0;
 #pragma unroll
         for (int r = 0; r < R; r++)
-            if (r < s.rounds && s.c[r] >= 0) est += predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, mid, m);
-        const int e = wave_sum_i32(est);
-        if (e >= target) {
-            klo = kmid;
-            if (e <= target + window) break;
-        } else {
-            khi = kmid;
-        }
-    }
-    return klo;
+            if (r < s.rounds && s.c[r] >= 0)
+                est += predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, mid, m);
+        return wave_sum_i32(est);
+    });
 }
 
 // For a slice of a heavy node: the thresholds of the cumulative targets target_hi and
@@ -1479,6 +1560,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
                                                  uint32_t &T_hi, uint32_t &T_lo) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
+    OMK_S0();
     uint32_t headk[R];
     uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
 #pragma unroll
@@ -1556,13 +1638,16 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
         }
     }
     int cta[R];
+    OMK_STAMP(9);
     T_hi = 0xFFFFFFFFu;
     T_lo = 0u;
 #pragma unroll
     for (int r = 0; r < R; r++) ct_hi[r] = ct_lo[r] = 0;
     if (target_hi > 0) {
         T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m);
+        OMK_STAMP(10);
         active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta);
+        OMK_STAMP(11);
 #pragma unroll
         for (int r = 0; r < R; r++)
             if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
@@ -1573,7 +1658,9 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     }
     if (target_lo > 0) {
         T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m);
+        OMK_STAMP(10);
         active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta);
+        OMK_STAMP(11);
 #pragma unroll
         for (int r = 0; r < R; r++)
             if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
@@ -1764,8 +1851,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         for (int r = 0; r < R; r++) cnt[r] = ctx[16 + r * kWave + lane];
         settled = true;
     }
+    OMK_S0();
     if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
         settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child);
+    OMK_STAMP(12);
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
@@ -2358,6 +2447,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
 #ifdef OMK_TRACE
             const long long tr0 = wall_clock64();
             if (lane == 0) s_lds.red[3] = 0u;
+            if (lane < 16) s_lds.tph[lane] = 0u;
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
             int status = kStepLeaf;
@@ -2375,10 +2465,12 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             if (lane == 0) {
                 int ti = atomicAdd(a.trace_n, 1);
                 if (ti < a.trace_cap) {
-                    a.trace[4 * ti + 0] = tr0;
-                    a.trace[4 * ti + 1] = wall_clock64();
-                    a.trace[4 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
-                    a.trace[4 * ti + 3] = (long long)it.node | ((long long)s_lds.red[3] << 32);
+                    a.trace[12 * ti + 0] = tr0;
+                    a.trace[12 * ti + 1] = wall_clock64();
+                    a.trace[12 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
+                    a.trace[12 * ti + 3] = (long long)it.node | ((long long)s_lds.red[3] << 32);
+                    for (int q = 0; q < 8; q++)
+                        a.trace[12 * ti + 4 + q] = (long long)s_lds.tph[2 * q] | ((long long)s_lds.tph[2 * q + 1] << 32);
                 }
             }
 #endif

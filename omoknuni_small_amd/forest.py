@@ -377,9 +377,10 @@ class Batch:
         return dict(zip(keys, map(int, out)))
 
     def debug_trace(self, max_entries=1 << 16):
-        """Timeline of the last select() from a library built with -DOMK_TRACE: int64 array [n, 4] of
-        (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | counters << 32."""
-        buf = np.zeros((int(max_entries), 4), np.int64)
+        """Timeline of the last select() from a library built with -DOMK_TRACE: int64 array [n, 12] of
+        (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | counters << 32 and
+        eight words of two 32-bit phase times each (see omk_debug_trace in the header)."""
+        buf = np.zeros((int(max_entries), 12), np.int64)
         n = C.c_int32()
         _check(self._lib.omk_debug_trace(self._h, buf.ctypes.data_as(C.c_void_p), C.c_int32(int(max_entries)),
                                          C.byref(n)))

@@ -3,7 +3,7 @@
     python -m omoknuni_small_amd.profile_summary stats  <kernel_stats.csv>
     python -m omoknuni_small_amd.profile_summary pmc    <counter_collection.csv> <COUNTER> [copy_bytes]
     OMK_FOREST_LIB=omoknuni_small_amd/libomk_forest_trace.so \
-    python -m omoknuni_small_amd.profile_summary timeline <workload> [warmup_steps]
+    python -m omoknuni_small_amd.profile_summary timeline <workload> [warmup_steps [level ...]]
 
 `stats` prints calls / total / average duration per kernel.  `pmc` prints, per kernel, the
 sum of a hardware counter over its dispatches; given the bytes the calibration copy kernel
@@ -12,7 +12,7 @@ copy implies and every kernel's traffic in bytes scaled by it.  `timeline` runs 
 workload on the GPU through the measurement build of the library (make -C csrc trace), which records
 when every multi-visitor work item of a selection was processed, and prints the chain of crowded
 nodes of one steady-state selection: per tree level the node with most visitors, when its wavefront
-started and ended, and what it did.
+started and ended, and what it did; for every level named, all items of that node.
 """
 import csv
 import sys
@@ -56,7 +56,7 @@ def pmc(path, counter, copy_bytes=None):
         print(line)
 
 
-def timeline(workload, warmup=8):
+def timeline(workload, warmup=8, levels=()):
     import numpy as np
     import omoknuni_small_amd as omk
     from omoknuni_small_amd import synth
@@ -90,7 +90,15 @@ def timeline(workload, warmup=8):
     print("chain of crowded nodes: per level the node with most visitors (kinds: node = taken as a whole, "
           "early = published before its visitor list was complete; a node cut into slices / scatter parts shows "
           "their number and the span from the first start to the last end)")
-    print("%5s %9s %9s %7s %9s %9s %8s  %s" % ("level", "node", "visitors", "kind", "start_us", "end_us", "us", "work"))
+    ph = np.stack([(tr[:, 4 + q // 2] >> (32 * (q % 2))) & 0xFFFFFFFF for q in range(16)], axis=1) / 100.0
+    print("phase columns (us of the owner wavefront, summed over the node's items): load = children loaded and "
+          "scored, thr = threshold search and exact counts, ord = entries evaluated and put in order, emit = "
+          "emission and checks, settle = all of the settling (includes thr, ord, emit), part = partition or its "
+          "hand-over; parts of thr (and of the thresholds a slice derives): probe = run probe, act = bounds and "
+          "active children, srch = threshold search, cnt = exact counts; 1win = the one-winner check")
+    print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s  %s" % (
+        "level", "node", "visitors", "kind", "start_us", "end_us", "us", "load", "thr", "ord", "emit", "settle", "part",
+        "probe", "act", "srch", "cnt", "1win", "work"))
     names = {0: "node", 1: "slice", 2: "part", 3: "early"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
@@ -107,8 +115,21 @@ def timeline(workload, warmup=8):
         work = "%d batch(es), %d run(s)" % (batches, runs)
         if n_sl or n_pt:
             work += ", %d slice item(s), %d scatter part(s)" % (n_sl, n_pt)
-        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f  %s" % (d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1,
-                                                       e1 - s0, work))
+        p = ph[same].sum(axis=0)
+        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
+            d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1, e1 - s0, p[4], p[0], p[2], p[3], p[5], p[6],
+            p[8], p[9], p[10], p[11], p[12], work))
+    for lv in levels:
+        at = np.nonzero(depth == lv)[0]
+        top = at[np.argmax(m[at])]
+        same = at[node[at] == node[top]]
+        same = same[np.argsort(start[same])]
+        print("items of node %d at level %d (slice / part number of a heavy node in `work`):" % (node[top], lv))
+        for i in same:
+            c = int(ctr[i])
+            print("  %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f  %d batch(es), %d run(s), last batch %d entries"
+                  % (names.get(int(kind[i]), "?"), start[i], end[i], end[i] - start[i], ph[i, 4], ph[i, 0], ph[i, 2], ph[i, 3],
+                     ph[i, 5], ph[i, 6], ph[i, 8], ph[i, 9], ph[i, 10], ph[i, 11], ph[i, 12], c & 0xFF, (c >> 8) & 0xFF, c >> 16))
     by_kind = ", ".join("%s %d" % (names[k], int((kind == k).sum())) for k in sorted(names))
     print("items by kind: %s; visitors per item: median %d, largest %d" % (by_kind, int(np.median(m)), int(m.max())))
 
@@ -119,7 +140,7 @@ if __name__ == "__main__":
     elif len(sys.argv) >= 4 and sys.argv[1] == "pmc":
         pmc(sys.argv[2], sys.argv[3], int(sys.argv[4]) if len(sys.argv) > 4 else None)
     elif len(sys.argv) >= 3 and sys.argv[1] == "timeline":
-        timeline(sys.argv[2], int(sys.argv[3]) if len(sys.argv) > 3 else 8)
+        timeline(sys.argv[2], int(sys.argv[3]) if len(sys.argv) > 3 else 8, [int(x) for x in sys.argv[4:]])
     else:
         print(__doc__)
         sys.exit(2)
