@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "omk_score.h"
+
 namespace omk {
 
 constexpr int kWave = 64;
@@ -92,57 +94,6 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, kWave);
     return v;
-}
-
-// Maps a score to an unsigned key with the same order as the float comparison used by
-// "score > best_score" (mcts_node.cpp:163,216).  A score that can never beat the initial
-// -infinity (NaN or -infinity itself) maps to 0, below every real key.
-__device__ __forceinline__ uint32_t score_key(float s) {
-    if (!(s > -__builtin_inff())) return 0u;
-    s = s + 0.0f;  // -0.0 and +0.0 compare equal: give them one key
-    uint32_t b = __float_as_uint(s);
-    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-}
-
-__device__ __forceinline__ float combined_value(int visits, float w, int rave_visits, float rw, float rave_k) {
-    if (visits == 0 && rave_visits == 0) return 0.0f;
-    float mcts_value = visits > 0 ? w / (float)visits : 0.0f;
-    float rave_value = rave_visits > 0 ? rw / (float)rave_visits : 0.0f;
-    int three_v = (int)(3u * (uint32_t)visits);
-    float beta = sqrtf(rave_k / ((float)three_v + rave_k));
-    float a = (1.0f - beta) * mcts_value;
-    float b = beta * rave_value;
-    return a + b;
-}
-
-// Keys of the two candidates a child contributes: its score in the first scan of
-// selectChild and its score in the second scan.  The second differs from the first only
-// through the RAVE blend q2 (getCombinedValue: it does not depend on virtual loss, so the
-// caller computes it once per child) or, without RAVE, when 1 + ev is not exact in
-// binary32; a second score equal to the first can never win (strict comparison, first
-// scan comes first), so it is reported as 0.  While |ev| < 2^24 the divisors 1.0f + ev
-// (first scan) and float(1 + ev) (second scan) are the same number, so one division
-// serves both.
-template <bool RAVE>
-__device__ __forceinline__ void child_keys(int n, float w, float p, int vl, float q2, float ep, uint32_t &k1,
-                                           uint32_t &k2) {
-    int ev = (int)((uint32_t)n + (uint32_t)vl);
-    float evalue = w - (float)vl;
-    float q = ev > 0 ? evalue / (float)ev : 0.0f;
-    float prod = p * ep;
-    float u1 = prod / (1.0f + (float)ev);
-    k1 = score_key(q + u1);
-    const bool exact = ev < (1 << 24) && ev > -(1 << 24);
-    if (RAVE) {
-        float u2 = u1;
-        if (!exact) u2 = prod / (float)(int)(1u + (uint32_t)ev);
-        k2 = score_key(q2 + u2);
-    } else if (!exact) {
-        float u2 = prod / (float)(int)(1u + (uint32_t)ev);
-        k2 = score_key(q + u2);
-    } else {
-        k2 = 0u;
-    }
 }
 
 // smallest k >= 1 with k*k >= n

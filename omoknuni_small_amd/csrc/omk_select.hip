@@ -178,6 +178,7 @@ struct TeamCmd {
     int best, btk, bn, bvl;
     float bw, bp, bq2;
     uint32_t hk, hp, sk, spos;
+    int proven;  // kOpRun: the child's keys provably do not increase over the run
     // kOpPartition: the node whose visitors a helper shares out while the owner walks on
     int j_cb, j_off, j_m, j_depth, j_keep, j_run_child;
 };
@@ -885,15 +886,24 @@ __device__ __forceinline__ void batch_emit(const SelectArgs &a, WaveLds<R> &lds,
 // its predecessor (the first one's predecessor is the child's current head (hk, hp), i.e.
 // itself), and the last one must still come before the others' best (sk, spos).  The
 // entries are written whether or not the checks hold; red[2] bit 2 reports a failure.
+// proven: the child's keys provably do not increase over these visits (keys_provably_monotone), so
+// only the run's last entry is evaluated.
 template <int R, bool RAVE, int NT>
 __device__ __forceinline__ void batch_run(const SelectArgs &a, WaveLds<R> &lds, int tid, int L, int goff, int best,
                                           int btk, int bn, float bw, float bp, int bvl, float bq2, float ep,
-                                          uint32_t uvl, uint32_t hk, uint32_t hp, uint32_t sk, uint32_t spos) {
+                                          uint32_t uvl, uint32_t hk, uint32_t hp, uint32_t sk, uint32_t spos,
+                                          bool proven) {
     const int per = (L + NT - 1) / NT;
     const int j0 = tid * per < L ? tid * per : L;
     const int j1 = j0 + per < L ? j0 + per : L;
     bool bad_run = false;
-    if (j0 < j1) {
+    if (proven) {
+        if (tid == 0) {
+            uint32_t kk, p2;
+            entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, btk + L - 1, best, kk, p2);
+            if (kk == 0u || hk == 0u || (sk != 0u && !comes_before(kk, p2, sk, spos))) bad_run = true;
+        }
+    } else if (j0 < j1) {
         uint32_t pk = hk, pp = hp;
         if (j0 > 0) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, btk + j0 - 1, best, pk, pp);
         for (int j = j0; j < j1; j++) {
@@ -1074,7 +1084,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L, best, nk, np2);
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L - 1, best, lk_, lp_);
                 bool bad_run = nk != 0u && comes_before(nk, np2, lk_, lp_);
-                // every entry of the run is checked and written; a long run with the helpers
+                // every entry of the run is checked (unless the order of the child's keys is proven
+                // beforehand) and written; a long run with the helpers
+                const bool proven = keys_provably_monotone<RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L);
                 if (!bad_run) {
                     if (lane == 0) lds.red[2] = 0u;
                     if (L >= 2 * kTeamMin) {
@@ -1098,15 +1110,16 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                             cm.hp = hi_pos;
                             cm.sk = sk;
                             cm.spos = spos;
+                            cm.proven = proven ? 1 : 0;
                         }
                         __syncthreads();
                         batch_run<R, RAVE, kTeam>(a, lds, lane, L, off + done, best, btk, bn, bw, bp, bvl, bq2, c.ep, uvl,
-                                                  hi_key, hi_pos, sk, spos);
+                                                  hi_key, hi_pos, sk, spos, proven);
                         __syncthreads();
                     } else {
                         wave_sync_memory();
                         batch_run<R, RAVE, kWave>(a, lds, lane, L, off + done, best, btk, bn, bw, bp, bvl, bq2, c.ep, uvl,
-                                                  hi_key, hi_pos, sk, spos);
+                                                  hi_key, hi_pos, sk, spos, proven);
                     }
                     bad_run = (lds.red[2] & 4u) != 0u;
                 }
@@ -1724,7 +1737,9 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
     if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) return false;
     bool bad = false;
     uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
-    for (int base = 0; base < m; base += kWave) {
+    // when the order of the child's keys is proven beforehand, the entries in between need no look
+    const bool proven = keys_provably_monotone<RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, m - 1);
+    for (int base = 0; base < m && !proven; base += kWave) {
         const int j = base + lane;
         uint32_t kk = 0u, pp = 0xFFFFFFFFu;
         if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, j, best, kk, pp);
@@ -2628,7 +2643,9 @@ __device__ __forceinline__ void team_help(const ForestDev &f, const SelectArgs &
         const uint32_t hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.hp);
         const uint32_t sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.sk);
         const uint32_t spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)cm.spos);
-        batch_run<R, RAVE, kTeam>(a, lds, tid, total, goff, best, btk, bn, bw, bp, bvl, bq2, ep, uvl, hk, hp, sk, spos);
+        const bool proven = __builtin_amdgcn_readfirstlane(cm.proven) != 0;
+        batch_run<R, RAVE, kTeam>(a, lds, tid, total, goff, best, btk, bn, bw, bp, bvl, bq2, ep, uvl, hk, hp, sk, spos,
+                                  proven);
     }
 }
 

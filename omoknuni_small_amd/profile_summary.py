@@ -99,7 +99,7 @@ def timeline(workload, warmup=8, levels=()):
     print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s  %s" % (
         "level", "node", "visitors", "kind", "start_us", "end_us", "us", "load", "thr", "ord", "emit", "settle", "part",
         "probe", "act", "srch", "cnt", "1win", "work"))
-    names = {0: "node", 1: "slice", 2: "part", 3: "early"}
+    names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
         if len(at) == 0:
@@ -107,6 +107,7 @@ def timeline(workload, warmup=8, levels=()):
         top = at[np.argmax(m[at])]
         same = at[node[at] == node[top]]
         whole = same[(kind[same] == 0) | (kind[same] == 3)]
+        jobs = same[kind[same] == 4]
         first = whole[0] if len(whole) else same[0]
         s0, e1 = start[same].min(), end[same].max()
         n_sl, n_pt = int((kind[same] == 1).sum()), int((kind[same] == 2).sum())
@@ -115,6 +116,10 @@ def timeline(workload, warmup=8, levels=()):
         work = "%d batch(es), %d run(s)" % (batches, runs)
         if n_sl or n_pt:
             work += ", %d slice item(s), %d scatter part(s)" % (n_sl, n_pt)
+        if len(jobs):
+            work += ", order and partition as a job %.1f-%.1f" % (start[jobs].min(), end[jobs].max())
+            same = same[kind[same] != 4]
+            s0, e1 = start[same].min(), end[same].max()
         p = ph[same].sum(axis=0)
         print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
             d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1, e1 - s0, p[4], p[0], p[2], p[3], p[5], p[6],
