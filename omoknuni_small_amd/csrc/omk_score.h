@@ -88,8 +88,9 @@ OMK_HD void child_keys(int n, float w, float p, int vl, float q2, float ep, uint
 //     x_{j+1} > x_j > 0 give E_{j+1} / x_{j+1} <= E_j / x_j, rounded or not.  Where E_j < 0 that
 //     needs E_{j+1} * x_j <= E_j * x_{j+1}; with E_j = w - vl_j + d_j, |d_j| <= 2^-24 |E_j|, it
 //     reduces to uvl * (n + w) >= (d_{j+1} - d_j) * x_j - d_j * uvl, which
-//     uvl * (n + w) >= 2^-23 * max|E| * (x_last + uvl) implies.  (n + w < 0, a value sum below
-//     minus the visit count, makes the real quotient RISE with virtual loss: refused.)
+//     uvl * (n + w) >= 2^-23 * max|E| * (x_last + uvl) implies; when w is integral every E_j is
+//     exact (d_j = 0) and n + w >= 0 suffices.  (n + w < 0, a value sum below minus the visit
+//     count, makes the real quotient RISE with virtual loss: refused.)
 //   * a child with x_0 = 0 scores q = 0 at visit 0 by definition; q_1 = fl(E_1 / x_1) <= 0 needs
 //     w <= vl_1;
 //   * sums of non-increasing terms, rounded, do not increase; score_key keeps order; the entry's key
@@ -109,6 +110,9 @@ OMK_HD bool keys_provably_monotone(int n, float w, float p, int vl0, float q2, f
     const double vl_last = (double)vl0 + (double)j_last * (double)uvl;
     if (n + vl0 == 0 && j_last >= 1 && !(dw <= (double)vl0 + (double)uvl)) return false;
     if (dw >= vl_last) return true;  // the numerator never turns negative
+    // an integral value sum (an unvisited child's 0 above all): w - vl_j is exact, d_j = 0, and
+    // n + w >= 0 is all that is needed
+    if (w == floorf(w) && w > -16777216.0f && w < 16777216.0f) return (double)n + dw >= 0.0;
     const double e0 = fabs(dw - (double)vl0), e1 = fabs(dw - vl_last);
     const double emax = e0 > e1 ? e0 : e1;
     const double lhs = (double)uvl * ((double)n + dw);

@@ -69,8 +69,14 @@ constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-v
 constexpr int kTeam = kTeamWaves * 64;
 constexpr int kTeamMin = 96;              // batch entries from which the helpers are called in
 // a batch of at most this many entries per thread is ordered by counting: a lone wavefront, the block
-constexpr int kCountSortLone = 2, kCountSortTeam = 1;
-constexpr int kSliceEntries = 256;        // visitors per slice of such a node, about
+#ifndef OMK_COUNT_SORT_TEAM
+#define OMK_COUNT_SORT_TEAM 1
+#endif
+constexpr int kCountSortLone = 2, kCountSortTeam = OMK_COUNT_SORT_TEAM;
+#ifndef OMK_SLICE_ENTRIES
+#define OMK_SLICE_ENTRIES 256
+#endif
+constexpr int kSliceEntries = OMK_SLICE_ENTRIES;  // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
@@ -1079,6 +1085,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     hi_l = new_hi < hi_l ? new_hi : hi_l;
                 }
                 const int L = lo_l;
+                OMK_STAMP(13);
                 // the entry after the run must not come before the run's last one
                 uint32_t nk, np2, lk_, lp_;
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L, best, nk, np2);
@@ -1123,6 +1130,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     }
                     bad_run = (lds.red[2] & 4u) != 0u;
                 }
+                OMK_STAMP(14);
 #ifdef OMK_TRACE
                 if (!bad_run && lane == 0) lds.red[3] += 0x100u;  // runs emitted without sorting
 #endif

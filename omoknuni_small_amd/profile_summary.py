@@ -95,10 +95,10 @@ def timeline(workload, warmup=8, levels=()):
           "scored, thr = threshold search and exact counts, ord = entries evaluated and put in order, emit = "
           "emission and checks, settle = all of the settling (includes thr, ord, emit), part = partition or its "
           "hand-over; parts of thr (and of the thresholds a slice derives): probe = run probe, act = bounds and "
-          "active children, srch = threshold search, cnt = exact counts; 1win = the one-winner check")
-    print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s  %s" % (
+          "active children, srch = threshold search, cnt = exact counts; 1win = the one-winner check; runL / runW = length search and emission of runs of one child")
+    print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s %5s %5s  %s" % (
         "level", "node", "visitors", "kind", "start_us", "end_us", "us", "load", "thr", "ord", "emit", "settle", "part",
-        "probe", "act", "srch", "cnt", "1win", "work"))
+        "probe", "act", "srch", "cnt", "1win", "runL", "runW", "work"))
     names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
@@ -121,9 +121,9 @@ def timeline(workload, warmup=8, levels=()):
             same = same[kind[same] != 4]
             s0, e1 = start[same].min(), end[same].max()
         p = ph[same].sum(axis=0)
-        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
+        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
             d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1, e1 - s0, p[4], p[0], p[2], p[3], p[5], p[6],
-            p[8], p[9], p[10], p[11], p[12], work))
+            p[8], p[9], p[10], p[11], p[12], p[13], p[14], work))
     for lv in levels:
         at = np.nonzero(depth == lv)[0]
         top = at[np.argmax(m[at])]
@@ -132,9 +132,9 @@ def timeline(workload, warmup=8, levels=()):
         print("items of node %d at level %d (slice / part number of a heavy node in `work`):" % (node[top], lv))
         for i in same:
             c = int(ctr[i])
-            print("  %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f  %d batch(es), %d run(s), last batch %d entries"
+            print("  %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %d batch(es), %d run(s), last batch %d entries"
                   % (names.get(int(kind[i]), "?"), start[i], end[i], end[i] - start[i], ph[i, 4], ph[i, 0], ph[i, 2], ph[i, 3],
-                     ph[i, 5], ph[i, 6], ph[i, 8], ph[i, 9], ph[i, 10], ph[i, 11], ph[i, 12], c & 0xFF, (c >> 8) & 0xFF, c >> 16))
+                     ph[i, 5], ph[i, 6], ph[i, 8], ph[i, 9], ph[i, 10], ph[i, 11], ph[i, 12], ph[i, 13], ph[i, 14], c & 0xFF, (c >> 8) & 0xFF, c >> 16))
     by_kind = ", ".join("%s %d" % (names[k], int((kind == k).sum())) for k in sorted(names))
     print("items by kind: %s; visitors per item: median %d, largest %d" % (by_kind, int(np.median(m)), int(m.max())))
 

@@ -167,3 +167,21 @@ def test_golden_fixture_is_data_only():
     with open(os.path.join(ROOT, "tests", "golden", "kat_reference.json")) as f:
         g = json.load(f)
     assert {"select", "score_bits", "backup", "virtual_loss_probe"} <= set(g)
+
+
+def test_proof_of_non_increasing_keys_against_brute_force(tmp_path):
+    """keys_provably_monotone (csrc/omk_score.h) lets the kernels skip the entry-by-entry look at a
+    child's successive scores; on the host, with the same arithmetic, every "proven" case is
+    evaluated entry by entry (tests/cpp/lemma_check.cpp), and the test must say yes often enough
+    to be worth having."""
+    import re
+    import subprocess
+    exe = str(tmp_path / "lemma_check")
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-fno-fast-math", "-I",
+                           os.path.join(ROOT, "omoknuni_small_amd", "csrc"),
+                           os.path.join(ROOT, "tests", "cpp", "lemma_check.cpp"), "-o", exe])
+    out = subprocess.run([exe, "200000"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout[-2000:]
+    m = re.search(r"provably monotone: (\d+) without RAVE, (\d+) with; counter-examples 0", out.stdout)
+    assert m, out.stdout[-500:]
+    assert int(m.group(1)) > 100000 and int(m.group(2)) > 100000
