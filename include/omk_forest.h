@@ -222,6 +222,29 @@ int omk_forest_compact_static(omk_forest *f, int32_t new_root, int64_t *h_nodes_
 int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
                      int32_t action_space, int32_t *h_first_child);
 
+/* The same with everything MCTSNode::expand and setPriorProbabilities look at.
+ *   - Progressive widening (expand(use_progressive_widening, cpw, kpw), the MCTSSettings fields of
+ *     include/mcts/mcts_engine.h:98-103, default on, c = 2, k = 0.5): a leaf of N visits that is
+ *     offered L moves gets the first min(L, size_t(max(8.0f, float(cpw * pow(N + 1, kpw))))) of them
+ *     (at least one) as children (src/mcts/mcts_node.cpp:296-341; the reference shuffles first, so
+ *     any L-subset in any order is one of its outcomes).  The branch of expand() that would add
+ *     children to a node that already has some is unreachable in the reference (the compare-exchange
+ *     on is_expanded_ at :264 returns first): here, too, such a node is left alone.
+ *   - One policy vector per simulation, of its own length (h_policy_begin[t] .. h_policy_begin[t+1]
+ *     into h_policy; both NULL = none): empty = setPriorProbabilities is not called and expand's
+ *     uniform 1 / children stays (mcts_engine_batch_tree_simple.cpp:256-258); action_space values =
+ *     clamp(policy[move], 0, 1), 0.01 for a move outside the action space (:537-560); as many values
+ *     as children = clamp(policy[i], 0, 1) by child index (:561-575); any other length = uniform
+ *     1 / children (:576-584). */
+typedef struct omk_expand_params {
+    int32_t action_space;             /* IGameState::getActionSpaceSize() of the leaf states */
+    int32_t use_progressive_widening; /* MCTSSettings::use_progressive_widening */
+    float progressive_widening_c;     /* MCTSSettings::progressive_widening_c */
+    float progressive_widening_k;     /* MCTSSettings::progressive_widening_k */
+} omk_expand_params;
+int omk_expand_batch_ex(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const int32_t *h_policy_begin,
+                        const float *h_policy, const omk_expand_params *params, int32_t *h_first_child);
+
 /* The RAVE statistics of MCTSEngine::backPropagate (src/mcts/mcts_engine_tree.cpp:288-331 with
  * MCTSNode::updateRAVE, src/mcts/mcts_node.cpp:631-643) for the paths of the last selection
  * and the values of omk_batch_set_values: every child of a path node whose action occurs

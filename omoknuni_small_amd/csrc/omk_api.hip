@@ -1002,13 +1002,34 @@ int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_pat
     return OMK_OK;
 }
 
-int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
-                     int32_t action_space, int32_t *h_first_child) {
-    if (!b || !h_move_begin || !h_moves) return fail(OMK_ERR_INVALID, "omk_expand_batch: null argument");
-    if (!b->selected) return fail(OMK_ERR_STATE, "omk_expand_batch: no selected paths");
-    if (int rc = fresh_batch("omk_expand_batch", b)) return rc;
+// How many children MCTSNode::expand creates for a node of `visits` visits that is offered `legal`
+// moves (src/mcts/mcts_node.cpp:296-341): without progressive widening all of them; with it
+// min(legal, size_t(max(8.0f, float(cpw * std::pow(visits + 1, kpw))))), at least 1.  (std::pow of an
+// int and a float is computed in double; the product with the float cpw as well.)  The branch of
+// expand() that adds children to a node that already has some is never reached: the
+// compare-exchange on is_expanded_ at :264 returns first.
+static int32_t widened_children(int32_t legal, int32_t visits, const omk_expand_params *p) {
+    if (!p || !p->use_progressive_widening) return legal;
+    const double grown = (double)p->progressive_widening_c * std::pow((double)(visits + 1), (double)p->progressive_widening_k);
+    const float target_f = std::max(8.0f, static_cast<float>(grown));
+    // a float beyond the range of size_t is undefined in the reference; every such value exceeds `legal`
+    size_t target = target_f >= 1.0e18f ? (size_t)legal : static_cast<size_t>(target_f);
+    if (!(target_f == target_f)) target = 8;  // NaN: std::max(8.0f, NaN) is 8.0f
+    size_t num = std::min((size_t)legal, target);
+    num = std::max(num, (size_t)1);
+    return (int32_t)std::min(num, (size_t)legal);
+}
+
+int omk_expand_batch_ex(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const int32_t *h_policy_begin,
+                        const float *h_policy, const omk_expand_params *params, int32_t *h_first_child) {
+    if (!b || !h_move_begin || !h_moves || !params) return fail(OMK_ERR_INVALID, "omk_expand_batch_ex: null argument");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_expand_batch_ex: no selected paths");
+    if (int rc = fresh_batch("omk_expand_batch_ex", b)) return rc;
+    if ((h_policy != nullptr) != (h_policy_begin != nullptr))
+        return fail(OMK_ERR_INVALID, "omk_expand_batch_ex: policies need both their values and their offsets");
+    const int32_t action_space = params->action_space;
     if (h_policy && action_space <= 0)
-        return fail(OMK_ERR_INVALID, "omk_expand_batch: a policy needs action_space > 0 (got %d)", action_space);
+        return fail(OMK_ERR_INVALID, "omk_expand_batch_ex: a policy needs action_space > 0 (got %d)", action_space);
     omk_forest *f = b->f;
     if (int rc = use_device(f)) return rc;
     hipStream_t s = f->stream;
@@ -1020,12 +1041,13 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
     std::vector<ExpandJob> jobs;
     std::vector<int32_t> job_of((size_t)n, -1), moves;
     std::vector<float> priors;
-    std::vector<int32_t> seen;  // leaves with a job, kept sorted by leaf id via the index below
     {
         std::vector<std::pair<int32_t, int32_t>> order;  // (leaf, traversal) of every offer
         for (int t = 0; t < n; t++) {
             if (h_move_begin[t + 1] < h_move_begin[t])
-                return fail(OMK_ERR_INVALID, "omk_expand_batch: move_begin decreases at traversal %d", t);
+                return fail(OMK_ERR_INVALID, "omk_expand_batch_ex: move_begin decreases at traversal %d", t);
+            if (h_policy_begin && h_policy_begin[t + 1] < h_policy_begin[t])
+                return fail(OMK_ERR_INVALID, "omk_expand_batch_ex: policy_begin decreases at traversal %d", t);
             if (h_move_begin[t + 1] > h_move_begin[t] && leaf[(size_t)t] >= 0) order.emplace_back(leaf[(size_t)t], t);
         }
         std::sort(order.begin(), order.end());
@@ -1033,12 +1055,37 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
         for (size_t i = 0; i < order.size(); i++)
             if (i == 0 || order[i].first != order[i - 1].first) winners.push_back(order[i].second);
         std::sort(winners.begin(), winners.end());  // ids are handed out in traversal order
+        // progressive widening reads the visit count of every leaf that is about to be expanded
+        std::vector<int32_t> visits(winners.size(), 0);
+        if (params->use_progressive_widening && !winners.empty()) {
+            const size_t nw = winners.size();
+            if (nw * 8 > b->exp_bytes) {
+                if (b->exp_buf) HIP_TRY(hipFree(b->exp_buf));
+                b->exp_buf = nullptr;
+                b->exp_bytes = 0;
+                HIP_TRY(hipMalloc(&b->exp_buf, nw * 16));
+                b->exp_bytes = nw * 16;
+            }
+            std::vector<int32_t> ids(nw);
+            for (size_t i = 0; i < nw; i++) ids[i] = leaf[(size_t)winners[i]];
+            int32_t *d_ids = (int32_t *)b->exp_buf, *d_n = d_ids + nw;
+            HIP_TRY(hipMemcpyAsync(d_ids, ids.data(), nw * 4, hipMemcpyHostToDevice, s));
+            HIP_TRY(launch_gather_words((uint32_t *)d_n, (const uint32_t *)f->N, d_ids, (int64_t)nw, s));
+            HIP_TRY(hipMemcpyAsync(visits.data(), d_n, nw * 4, hipMemcpyDeviceToHost, s));
+            HIP_TRY(hipStreamSynchronize(s));
+        }
         int64_t cursor = f->n_nodes;
         bool sorted = true;
         int mf = f->max_fanout;
-        for (int32_t t : winners) {
+        for (size_t wi = 0; wi < winners.size(); wi++) {
+            const int32_t t = winners[wi];
             int32_t cnt = h_move_begin[t + 1] - h_move_begin[t];
             if (cnt > 1000) cnt = 1000;  // MCTSNode::expand: max_reasonable_moves
+            cnt = widened_children(cnt, visits[wi], params);
+            // MCTSNode::setPriorProbabilities (:512-593) is only called with a policy that is not empty
+            // (mcts_engine_batch_tree_simple.cpp:256-258); otherwise expand's uniform prior stays
+            const int32_t psize = h_policy_begin ? h_policy_begin[t + 1] - h_policy_begin[t] : 0;
+            const float *pol = psize > 0 ? h_policy + h_policy_begin[t] : nullptr;
             ExpandJob j;
             j.leaf = leaf[(size_t)t];
             j.begin = (int32_t)cursor;
@@ -1048,14 +1095,20 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
             for (int32_t i = 0; i < cnt; i++) {
                 const int32_t mv = h_moves[h_move_begin[t] + i];
                 float prior;
-                if (!h_policy) {
+                if (!pol) {
                     prior = 1.0f / (float)cnt;  // expand(): uniform prior
-                } else if (mv >= 0 && mv < action_space) {
-                    prior = h_policy[(size_t)t * (size_t)action_space + (size_t)mv];
-                    prior = prior > 0.0f ? prior : 0.0f;  // setPriorProbabilities: clamp to [0, 1]
-                    prior = prior < 1.0f ? prior : 1.0f;
-                } else {
-                    prior = 0.01f;  // move outside the action space
+                } else if (psize == action_space) {  // a policy over the action space (:537-560)
+                    if (mv >= 0 && mv < action_space) {
+                        prior = pol[mv];
+                        prior = std::min(1.0f, std::max(0.0f, prior));  // clamp to [0, 1]
+                    } else {
+                        prior = 0.01f;  // move outside the action space
+                    }
+                } else if (psize == cnt) {  // one value per child, by child index (:561-575)
+                    prior = pol[i];
+                    prior = std::min(1.0f, std::max(0.0f, prior));
+                } else {  // neither size: uniform (:576-584)
+                    prior = 1.0f / (float)cnt;
                 }
                 if (prior > prev) sorted = false;
                 prev = prior;
@@ -1068,9 +1121,9 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
             mf = std::max(mf, (int)cnt);
         }
         if (cursor > f->capacity)
-            return fail(OMK_ERR_CAPACITY, "omk_expand_batch: %lld nodes needed, capacity %lld", (long long)cursor,
+            return fail(OMK_ERR_CAPACITY, "omk_expand_batch_ex: %lld nodes needed, capacity %lld", (long long)cursor,
                         (long long)f->capacity);
-        if (cursor > INT32_MAX) return fail(OMK_ERR_CAPACITY, "omk_expand_batch: node ids exceed 32 bits");
+        if (cursor > INT32_MAX) return fail(OMK_ERR_CAPACITY, "omk_expand_batch_ex: node ids exceed 32 bits");
         if (h_first_child)
             for (int t = 0; t < n; t++) h_first_child[t] = -1;
         if (jobs.empty()) return OMK_OK;
@@ -1105,6 +1158,24 @@ int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h
                 if (job_of[(size_t)t] >= 0) h_first_child[t] = status[(size_t)job_of[(size_t)t]];
     }
     return OMK_OK;
+}
+
+int omk_expand_batch(omk_batch *b, const int32_t *h_move_begin, const int32_t *h_moves, const float *h_policy,
+                     int32_t action_space, int32_t *h_first_child) {
+    if (!b || !h_move_begin || !h_moves) return fail(OMK_ERR_INVALID, "omk_expand_batch: null argument");
+    if (h_policy && action_space <= 0)
+        return fail(OMK_ERR_INVALID, "omk_expand_batch: a policy needs action_space > 0 (got %d)", action_space);
+    omk_expand_params p;
+    p.action_space = action_space;
+    p.use_progressive_widening = 0;
+    p.progressive_widening_c = 0.0f;
+    p.progressive_widening_k = 0.0f;
+    std::vector<int32_t> pb;
+    if (h_policy) {  // one row of action_space values per traversal
+        pb.resize((size_t)b->n + 1);
+        for (int32_t t = 0; t <= b->n; t++) pb[(size_t)t] = t * action_space;
+    }
+    return omk_expand_batch_ex(b, h_move_begin, h_moves, h_policy ? pb.data() : nullptr, h_policy, &p, h_first_child);
 }
 
 int omk_batch_read(omk_batch *b, int32_t *h_paths, int32_t *h_path_len, int32_t *h_leaf, int32_t *h_actions) {

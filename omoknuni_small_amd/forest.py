@@ -23,7 +23,7 @@ u64p = C.POINTER(C.c_uint64)
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
-    "omk_expand_batch", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_reroot_child", "omk_forest_compact", "omk_forest_compact_static",
+    "omk_expand_batch", "omk_expand_batch_ex", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_reroot_child", "omk_forest_compact", "omk_forest_compact_static",
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
@@ -58,6 +58,12 @@ class SelectParams(C.Structure):
 
     def __init__(self, c_puct=1.4, virtual_loss=3, use_rave=False, rave_k=3000.0, pw=False):
         super().__init__(c_puct, int(virtual_loss), int(bool(use_rave)), rave_k, int(bool(pw)))
+
+
+class _ExpandParams(C.Structure):
+    """MCTSSettings fields MCTSNode::expand reads (reference include/mcts/mcts_engine.h:98-103)."""
+    _fields_ = [("action_space", C.c_int32), ("use_progressive_widening", C.c_int32),
+                ("progressive_widening_c", C.c_float), ("progressive_widening_k", C.c_float)]
 
 
 class _BatchDev(C.Structure):
@@ -352,6 +358,25 @@ class Batch:
         first = np.empty(len(mb) - 1, np.int32)
         _check(self._lib.omk_expand_batch(self._h, _ptr(mb, i32p), _ptr(mv, i32p), _ptr(pol, f32p),
                                           C.c_int32(int(action_space)), _ptr(first, i32p)))
+        self.forest.node_count()
+        return first
+
+    def expand_ex(self, move_begin, moves, policy_begin=None, policy=None, action_space=0, widening=None):
+        """expand() with ragged policies (policy_begin [n+1] into policy) and progressive widening
+        (widening = (c, k), None = off): see omk_expand_batch_ex."""
+        mb = np.ascontiguousarray(move_begin, dtype=np.int32)
+        mv = np.ascontiguousarray(moves, dtype=np.int32)
+        if len(mv) == 0:
+            mv = np.zeros(1, np.int32)
+        pb = None if policy_begin is None else np.ascontiguousarray(policy_begin, dtype=np.int32)
+        pol = None if policy is None else np.ascontiguousarray(policy, dtype=np.float32).reshape(-1)
+        if pol is not None and len(pol) == 0:
+            pol = np.zeros(1, np.float32)
+        par = _ExpandParams(int(action_space), 0 if widening is None else 1,
+                            0.0 if widening is None else float(widening[0]), 0.0 if widening is None else float(widening[1]))
+        first = np.empty(len(mb) - 1, np.int32)
+        _check(self._lib.omk_expand_batch_ex(self._h, _ptr(mb, i32p), _ptr(mv, i32p), _ptr(pb, i32p), _ptr(pol, f32p),
+                                             C.byref(par), _ptr(first, i32p)))
         self.forest.node_count()
         return first
 

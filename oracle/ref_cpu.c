@@ -321,10 +321,29 @@ int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_
 
 /* ---- leaf expansion (mcts_node.cpp:238-436, :512-593; call site
  * mcts_engine_batch_tree_simple.cpp:249-259) ---- */
-int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
-                         int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
-                         uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
-                         const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child) {
+/* mcts_node.cpp:296-341: the number of children expand() creates.  The "incremental expansion"
+ * branch (:312-337) needs a node that is already expanded, and such a call has returned at the
+ * compare-exchange of :264 before it gets there: what remains is the first expansion. */
+int32_t ref_widened_children(int32_t legal, int32_t visits, int32_t use_pw, float cpw, float kpw) {
+    size_t num = (size_t)legal;                                   /* :294 */
+    if (use_pw) {
+        /* :305-308; std::pow(int, float) and its product with a float are double arithmetic */
+        double grown = (double)cpw * pow((double)(visits + 1), (double)kpw);
+        float as_float = (float)grown;
+        float at_least = as_float > 8.0f ? as_float : 8.0f;       /* std::max(8.0f, x): 8.0f when x is NaN */
+        size_t target = at_least >= 1.0e18f ? (size_t)legal : (size_t)at_least;
+        if (target > (size_t)legal) target = (size_t)legal;      /* std::min(legal_moves.size(), ...) */
+        num = target > 1 ? target : 1;                            /* :340 */
+    }
+    if (num > (size_t)legal) num = (size_t)legal;                 /* the loop stops at legal_moves.size(), :367 */
+    return (int32_t)num;
+}
+
+int64_t ref_expand_batch_ex(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
+                            int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                            uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
+                            const int32_t *moves, const int32_t *policy_begin, const float *policy,
+                            int32_t action_space, int32_t use_pw, float cpw, float kpw, int32_t *first_child) {
     /* first pass: how many nodes would be added (a leaf counts once: child_count is set below,
      * so a dry run has to remember the leaves it has seen) */
     int64_t need = 0;
@@ -335,7 +354,8 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
         for (int32_t u = 0; u < t && !seen; u++)
             seen = leaf[u] == leaf[t] && move_begin[u + 1] - move_begin[u] > 0;
         if (seen) continue;
-        need += cnt > 1000 ? 1000 : cnt;
+        if (cnt > 1000) cnt = 1000;
+        need += ref_widened_children(cnt, N[leaf[t]], use_pw, cpw, kpw);
     }
     if (n_nodes + need > capacity) return -1;
     for (int32_t t = 0; t < B; t++) {
@@ -345,19 +365,32 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
         int32_t node = leaf[t];
         if (child_count[node] != 0) continue;           /* already expanded: first caller won */
         if (cnt > 1000) cnt = 1000;                     /* max_reasonable_moves */
+        cnt = ref_widened_children(cnt, N[node], use_pw, cpw, kpw);
+        /* setPriorProbabilities is only called with a policy that is not empty
+         * (mcts_engine_batch_tree_simple.cpp:256-258) */
+        const int32_t psize = policy_begin ? policy_begin[t + 1] - policy_begin[t] : 0;
+        const float *pol = psize > 0 ? policy + policy_begin[t] : NULL;
         const int32_t begin = (int32_t)n_nodes;
         for (int32_t i = 0; i < cnt; i++) {
             const int32_t id = begin + i;
             const int32_t mv = moves[move_begin[t] + i];
             float prior;
-            if (!policy) {
-                prior = 1.0f / (float)cnt;              /* expand(): uniform_prior */
-            } else if (mv >= 0 && mv < action_space) {
-                prior = policy[(int64_t)t * action_space + mv];
-                prior = prior > 0.0f ? prior : 0.0f;    /* std::min(1.0f, std::max(0.0f, prob)) */
+            if (!pol) {
+                prior = 1.0f / (float)cnt;              /* expand(): uniform_prior, :426-429 */
+            } else if (psize == action_space) {         /* :537-560 */
+                if (mv >= 0 && mv < action_space) {
+                    prior = pol[mv];
+                    prior = prior > 0.0f ? prior : 0.0f;    /* std::min(1.0f, std::max(0.0f, prob)) */
+                    prior = prior < 1.0f ? prior : 1.0f;
+                } else {
+                    prior = 0.01f;                      /* action out of bounds */
+                }
+            } else if (psize == cnt) {                  /* :561-575: by child index */
+                prior = pol[i];
+                prior = prior > 0.0f ? prior : 0.0f;
                 prior = prior < 1.0f ? prior : 1.0f;
             } else {
-                prior = 0.01f;                          /* action out of bounds */
+                prior = 1.0f / (float)cnt;              /* :576-584: size mismatch, uniform */
             }
             N[id] = 0;
             W[id] = 0.0f;
@@ -376,6 +409,22 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
         if (first_child) first_child[t] = begin;
     }
     return n_nodes;
+}
+
+/* The common case: one policy row of action_space values per traversal (or none), no widening. */
+int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
+                         int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                         uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
+                         const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child) {
+    int32_t *pb = NULL;
+    if (policy) {
+        pb = (int32_t *)malloc(((size_t)B + 1) * sizeof(int32_t));
+        for (int32_t t = 0; t <= B; t++) pb[t] = t * action_space;
+    }
+    int64_t r = ref_expand_batch_ex(n_nodes, capacity, N, W, P, VL, rN, rW, child_begin, child_count, action, legal,
+                                    leaf, B, move_begin, moves, pb, policy, action_space, 0, 0.0f, 0.0f, first_child);
+    free(pb);
+    return r;
 }
 
 /* ---- MCTSEngine::getActionProbabilities (src/mcts/mcts_engine_tree.cpp:388-465) ---- */

@@ -145,6 +145,21 @@ int64_t ref_expand_batch(int64_t n_nodes, int64_t capacity, int32_t *N, float *W
                          uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
                          const int32_t *moves, const float *policy, int32_t action_space, int32_t *first_child);
 
+/* The same with everything expand() and setPriorProbabilities() look at: a policy vector of its own
+ * length per traversal (policy_begin[t] .. policy_begin[t+1]: empty = setPriorProbabilities is not
+ * called, action_space values = by action, as many values as children = by child index, any other
+ * length = uniform, :537-584) and progressive widening (use_pw, cpw, kpw: only the first
+ * ref_widened_children(...) of the offered moves become children, :296-341; the incremental branch
+ * of expand() is unreachable behind the compare-exchange of :264).
+ * Pinned: closed forms of the child count (tests/test_oracle_expand.py), the reference-test facts
+ * (children >= 4 and <= legal moves, tests/mcts/progressive_widening_test.cpp:124-139). */
+int32_t ref_widened_children(int32_t legal, int32_t visits, int32_t use_pw, float cpw, float kpw);
+int64_t ref_expand_batch_ex(int64_t n_nodes, int64_t capacity, int32_t *N, float *W, float *P, int32_t *VL,
+                            int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                            uint32_t *legal, const int32_t *leaf, int32_t B, const int32_t *move_begin,
+                            const int32_t *moves, const int32_t *policy_begin, const float *policy,
+                            int32_t action_space, int32_t use_pw, float cpw, float kpw, int32_t *first_child);
+
 /* Dirichlet noise on the root's priors from caller-drawn gamma samples (see ref_cpu.c). */
 int32_t ref_add_root_noise(ref_tree *t, int32_t root, const float *gamma, int32_t n_gamma, float epsilon);
 

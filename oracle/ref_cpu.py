@@ -48,6 +48,8 @@ def lib():
     global _LIB
     if _LIB is None:
         L = C.CDLL(build())
+        L.ref_widened_children.restype = C.c_int32
+        L.ref_widened_children.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_float]
         L.ref_combined_value.restype = C.c_float
         L.ref_combined_value.argtypes = [C.POINTER(_Tree), C.c_int32, C.c_float]
         L.ref_child_scores.argtypes = [C.POINTER(_Tree), C.c_int32, C.c_int32, C.POINTER(_Params), f32p, f32p]
@@ -194,9 +196,11 @@ class RefTree:
         lib().ref_backup_batch(C.byref(self._c), _ptr(paths, i32p), _ptr(path_len, i32p), _ptr(values, f32p),
                                B, stride, int(amount))
 
-    def expand_batch(self, leaf, move_begin, moves, policy=None, action_space=0):
+    def expand_batch(self, leaf, move_begin, moves, policy=None, action_space=0, policy_begin=None, widening=None):
         """MCTSNode::expand + setPriorProbabilities for the leaves of a batch (see ref_cpu.h).
-        Grows the arrays; returns first_child per traversal (-1 where nothing was added)."""
+        Grows the arrays; returns first_child per traversal (-1 where nothing was added).
+        policy_begin: ragged policies (policy is then their concatenation); widening: (c, k) of
+        progressive widening, None = off."""
         leaf = np.ascontiguousarray(leaf, dtype=np.int32)
         move_begin = np.ascontiguousarray(move_begin, dtype=np.int32)
         moves = np.ascontiguousarray(moves, dtype=np.int32)
@@ -218,15 +222,22 @@ class RefTree:
         self.legal = grow(self.legal, np.uint32, (cap + 31) // 32)
         if self.legal is not None and self.n & 31:
             self.legal[self.n >> 5] &= np.uint32((1 << (self.n & 31)) - 1)  # bits of ids that do not exist yet
-        pol = None if policy is None else np.ascontiguousarray(policy, dtype=np.float32)
+        pol = None if policy is None else np.ascontiguousarray(policy, dtype=np.float32).reshape(-1)
+        if pol is not None and len(pol) == 0:
+            pol = np.zeros(1, np.float32)
+        pb = None
+        if pol is not None:
+            pb = (np.arange(B + 1, dtype=np.int32) * int(action_space) if policy_begin is None
+                  else np.ascontiguousarray(policy_begin, dtype=np.int32))
         first = np.empty(B, dtype=np.int32)
-        fn = lib().ref_expand_batch
+        fn = lib().ref_expand_batch_ex
         fn.restype = C.c_int64
+        use_pw, cpw, kpw = (0, 0.0, 0.0) if widening is None else (1, float(widening[0]), float(widening[1]))
         n_after = fn(C.c_int64(self.n), C.c_int64(cap), _ptr(self.N, i32p), _ptr(self.W, f32p), _ptr(self.P, f32p),
                      _ptr(self.VL, i32p), _ptr(self.rN, i32p), _ptr(self.rW, f32p), _ptr(self.child_begin, i32p),
                      _ptr(self.child_count, i32p), _ptr(self.action, i32p), _ptr(self.legal, u32p), _ptr(leaf, i32p),
-                     B, _ptr(move_begin, i32p), _ptr(moves, i32p), _ptr(pol, f32p), int(action_space),
-                     _ptr(first, i32p))
+                     B, _ptr(move_begin, i32p), _ptr(moves, i32p), _ptr(pb, i32p), _ptr(pol, f32p), int(action_space),
+                     C.c_int32(use_pw), C.c_float(cpw), C.c_float(kpw), _ptr(first, i32p))
         assert n_after >= 0
         self.n = int(n_after)
         for name in ("N", "W", "P", "VL", "rN", "rW", "child_begin", "child_count", "action"):

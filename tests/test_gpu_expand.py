@@ -79,6 +79,56 @@ def test_tree_grows_on_the_device(rave, B):
     assert ref.n > 1000
 
 
+def test_tree_grows_with_progressive_widening_and_ragged_policies():
+    """The reference's default settings (use_progressive_widening, c = 2, k = 0.5): only the first
+    min(legal, max(8, 2 sqrt(N + 1))) offered moves become children; policies of every length
+    setPriorProbabilities distinguishes (action space, number of children, neither, empty)."""
+    import omoknuni_small_amd as omk
+    A, B, D, vl = 120, 400, 10, 3
+    soa = dict(N=np.zeros(1, np.int32), W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=np.zeros(1, np.int32),
+               child_begin=np.zeros(1, np.int32), child_count=np.zeros(1, np.int32), action=np.full(1, -1, np.int32))
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa, capacity=300_000)
+    b = omk.Batch(f, B, D)
+    roots = np.zeros(B, np.int32)
+    b.set_roots(roots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, max_depth=D)
+    rng = np.random.default_rng(8)
+    kinds_seen = set()
+    for step in range(10):
+        rpaths, rlen, rleaf, near = ref.select_batch(roots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths == rpaths).all() and (gleaf == rleaf).all(), "step %d" % step
+        begin, moves, _ = offers(rng, rleaf, A, max_moves=60)
+        # a policy per traversal, its length a function of the leaf (two traversals at one leaf agree)
+        pb, pol = [0], []
+        for t, lf in enumerate(rleaf):
+            legal = int(begin[t + 1] - begin[t])
+            made = R.lib().ref_widened_children(min(legal, 1000), int(ref.N[lf]), 1, 2.0, 0.5) if legal else 0
+            kind = int(lf) % 4
+            size = [A, made, made + 3, 0][kind]
+            kinds_seen.add(kind)
+            pol.extend(np.random.default_rng(int(lf) + 5).uniform(-0.2, 1.2, size).astype(np.float32).tolist())
+            pb.append(len(pol))
+        pol = np.array(pol, np.float32)
+        rfirst = ref.expand_batch(rleaf, begin, moves, policy=pol, action_space=A, policy_begin=pb, widening=(2.0, 0.5))
+        gfirst = b.expand_ex(begin, moves, policy_begin=pb, policy=pol, action_space=A, widening=(2.0, 0.5))
+        assert (gfirst == rfirst).all(), "step %d: new ids differ" % step
+        assert_same_forest(f, ref, "after expansion, step %d" % step)
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, values, vl)
+        b.set_values(values)
+        b.backup(vl)
+        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        ref.W[:] = st["W"]
+    assert kinds_seen == {0, 1, 2, 3} and ref.n > 500
+    # widening at work: no node has more children than its visit count allowed when it was expanded
+    cc = ref.child_count[ref.child_count > 0]
+    assert cc.max() <= 60 and (cc >= 1).all() and (cc[cc < 8] >= 1).all()
+
+
 def test_expand_on_an_uploaded_tree_with_mask_and_shared_leaves():
     import omoknuni_small_amd as omk
     soa, roots = random_tree(77, n_expand=60, fanout=(2, 9), max_depth=5, mask_frac=0.2)

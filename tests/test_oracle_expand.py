@@ -67,6 +67,67 @@ def test_move_list_is_cut_at_the_reference_limit():
     assert t.child_count[0] == 1000 and t.n == 1001 and t.action[1000] == 999
 
 
+def test_widening_child_count_closed_forms():
+    """mcts_node.cpp:305-308: min(legal, size_t(max(8.0f, float(cpw * pow(N + 1, kpw))))), at least one
+    child; off = every legal move.  The reference's own test only fixes >= 4 and <= legal
+    (tests/mcts/progressive_widening_test.cpp:124-139)."""
+    W = R.lib().ref_widened_children
+    assert W(30, 0, 0, 2.0, 0.5) == 30                      # widening off: all legal moves
+    assert W(30, 0, 1, 2.0, 0.5) == 8                       # 2 * 1^0.5 = 2 -> the floor of 8
+    assert W(5, 0, 1, 2.0, 0.5) == 5                        # fewer legal moves than the floor
+    assert W(30, 15, 1, 2.0, 0.5) == 8                      # 2 * sqrt(16) = 8
+    assert W(30, 24, 1, 2.0, 0.5) == 10                     # 2 * sqrt(25) = 10
+    assert W(30, 35, 1, 2.0, 0.5) == 12                     # 2 * 6
+    assert W(30, 3, 1, 2.0, 1.0) == 8 and W(30, 4, 1, 2.0, 1.0) == 10      # k = 1: 2 * (N + 1)
+    assert W(30, 10 ** 6, 1, 2.0, 0.5) == 30                # never more than the legal moves
+    assert W(400, 2 ** 31 - 2, 1, 1e30, 3.0) == 400         # a target beyond any integer: all of them
+    assert W(1, 0, 1, 2.0, 0.5) == 1
+    # the truncation toward zero of the float: 2 * sqrt(20) = 8.94 -> 8, 2 * sqrt(21) = 9.17 -> 9
+    assert W(30, 19, 1, 2.0, 0.5) == 8 and W(30, 20, 1, 2.0, 0.5) == 9
+    for n in range(0, 3000, 7):                             # against the formula in Python doubles / float32
+        want = min(50, int(max(np.float32(8.0), np.float32(2.0 * float(n + 1) ** 0.5))))
+        assert W(50, n, 1, 2.0, 0.5) == want
+        assert 4 <= W(50, n, 1, 2.0, 0.5) <= 50             # the reference-test fact
+
+
+def test_widening_keeps_the_first_moves_offered_and_their_uniform_prior():
+    t = leaf_tree(2)
+    t.N[:] = [24, 0]
+    first = t.expand_batch([0, 1], [0, 20, 40], np.arange(40) % 20, widening=(2.0, 0.5))
+    assert first.tolist() == [2, 12]
+    assert (t.child_begin[0], t.child_count[0]) == (2, 10) and t.action[2:12].tolist() == list(range(10))
+    assert (t.child_begin[1], t.child_count[1]) == (12, 8) and t.action[12:20].tolist() == list(range(8))
+    assert (t.P[2:12] == np.float32(1.0) / np.float32(10.0)).all()      # 1 / children, not 1 / legal moves
+    assert (t.P[12:20] == np.float32(1.0) / np.float32(8.0)).all()
+    assert t.n == 20
+    # an expanded node is left alone, however many visits it has by now (the incremental branch of
+    # expand() sits behind a compare-exchange that returns first)
+    t.N[0] = 10 ** 6
+    assert t.expand_batch([0], [0, 20], np.arange(20), widening=(2.0, 0.5)).tolist() == [-1] and t.n == 20
+
+
+def test_policy_branches_of_set_prior_probabilities():
+    """:537-560 a policy over the action space, :561-575 one value per child, :576-584 any other length
+    -> uniform; an empty policy means setPriorProbabilities is not called at all."""
+    t = leaf_tree(4)
+    A = 6
+    pol = np.array([0.5, 0.1, 0.2, 0.05, 0.1, 0.05,       # traversal 0: the action space
+                    0.7, -0.3, 1.5,                        # traversal 1: as many as children (3), clamped
+                    0.2, 0.8,                              # traversal 2: neither (4 children, 2 values)
+                    ], np.float32)                         # traversal 3: empty
+    pb = [0, 6, 9, 11, 11]
+    t.expand_batch([0, 1, 2, 3], [0, 3, 6, 10, 12], [4, 0, 9, 1, 2, 3, 0, 1, 2, 3, 5, 4], policy=pol, action_space=A,
+                   policy_begin=pb)
+    assert t.P[4:7].tolist() == [np.float32(0.1), 0.5, np.float32(0.01)]           # by action; 9 is outside
+    assert t.P[7:10].tolist() == [np.float32(0.7), 0.0, 1.0]                       # by child index, clamped
+    assert (t.P[10:14] == np.float32(0.25)).all()                                  # mismatch: uniform
+    assert (t.P[14:16] == np.float32(0.5)).all()                                   # no policy: expand's uniform
+    # when the action space has as many entries as the node has children, the action branch wins
+    t2 = leaf_tree()
+    t2.expand_batch([0], [0, 3], [2, 0, 1], policy=np.array([0.1, 0.2, 0.7], np.float32), action_space=3, policy_begin=[0, 3])
+    assert t2.P[1:4].tolist() == [np.float32(0.7), np.float32(0.1), np.float32(0.2)]
+
+
 def test_selection_descends_into_new_children():
     t = leaf_tree()
     t.expand_batch([0], [0, 3], [0, 1, 2], policy=np.array([[0.1, 0.7, 0.2]], np.float32), action_space=3)
