@@ -321,10 +321,47 @@ int omk_tt_destroy(omk_tt *tt);
 int omk_tt_clear(omk_tt *tt);
 /* store(hash, node, depth) for n entries; a key already present keeps its first entry. */
 int omk_tt_insert(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, const int32_t *d_depths, int64_t n);
-/* lookup(hash, min_depth): d_out[i] = node or -1. */
+/* lookup(hash, min_depth): d_out[i] = node or -1; a successful lookup stamps the entry with its time
+ * (phmap_transposition_table.cpp:107; lookup i of the call has the time t + i, see omk_tt_store). */
 int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_depth, int32_t *d_out);
 /* lookup of the position key of every leaf of the last select: d_out[t] = node or -1. */
 int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_out);
+/* PHMapTranspositionTable::store (phmap_transposition_table.cpp:51-84) for n entries: a key that is
+ * not in the table gets a new entry (createEntry :202-216: node, depth as a uint16, the node's visit
+ * count and value as they are now); a key that is there keeps its entry unless the new one's
+ * replacement score exceeds the old one's by the threshold (:64-74, score = recency * importance,
+ * include/mcts/phmap_transposition_table.h:68-72, threshold Config::replacement_threshold = 0.1).
+ * Time: the reference stamps entries with a counter shared by its threads, so its values depend on
+ * the schedule; here entry i of a call has the time t + i and the table's clock t advances by n per
+ * call (lookups likewise).  Among the entries of one call with the same key only the first is
+ * stored: the serial outcome at the reference's two call sites (a node stored from the traversal
+ * has no visits, score 0, and never replaces; the leaves expanded in one step are distinct).
+ * An entry with node < 0 is skipped.  h_counts (NULL or [4]): new entries, replacements, entries
+ * dropped as duplicates within the call, 0.  Waits for the stream. */
+int omk_tt_store(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, const int32_t *d_depths, int64_t n,
+                 int32_t *h_counts);
+int omk_tt_set_replacement_threshold(omk_tt *tt, float threshold);
+/* The transposition-table part of the traversal loop (mcts_engine_batch_tree_simple.cpp:116-162)
+ * for the paths of the last select: at every step the selected child is stored under the key of
+ * the state it stands for when it has no visits yet (:116-128, depth = moves so far), then the key
+ * is looked up, and a node OTHER than the selected one that has visits is a transposition
+ * (:141-142).  The reference then swaps the child pointer of the parent for that node (:143-156),
+ * which turns the tree into a graph; this library reports the transposition and leaves the tree
+ * alone: d_hits (NULL or device memory for n_traversals * max_depth ints, entry t * max_depth + d - 1
+ * for step d of traversal t) receives that node or -1.  Keys: with d_piece_keys the game's Zobrist
+ * tables as in omk_batch_leaf_keys (stone-placing games), with NULL the forest's per-node keys
+ * (omk_soa_view.hash).  h_counts (NULL or [4]): new entries, replacements, duplicates within the
+ * call, transpositions reported.  Waits for the stream. */
+int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
+                    const uint64_t *d_root_keys, const int32_t *d_root_players, int32_t *d_hits, int32_t *h_counts);
+/* What an entry keeps for the replacement policy, slot by slot beside omk_tt_download. */
+typedef struct omk_tt_meta {
+    uint32_t visits;      /* Entry::visits */
+    float value;          /* Entry::value */
+    uint32_t last_access; /* Entry::last_access */
+    int32_t reserved;
+} omk_tt_meta;
+int omk_tt_download_meta(omk_tt *tt, omk_tt_meta *h_meta);
 int omk_tt_upload(omk_tt *tt, const omk_tt_slot *h_slots);
 int omk_tt_download(omk_tt *tt, omk_tt_slot *h_slots);
 

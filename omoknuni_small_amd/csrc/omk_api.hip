@@ -135,8 +135,24 @@ struct omk_tt {
     omk_forest *f = nullptr;
     int log2_slots = 0;
     TTSlot *slots = nullptr;
-    int *d_status = nullptr;
+    TTMeta *meta = nullptr;
+    int *d_status = nullptr;       // 8 counters of the last call
+    uint32_t clock = 0;            // access_counter_ of the reference: entry i of a call has the time clock + i
+    float threshold = 0.1f;        // Config::replacement_threshold
+    void *work = nullptr;          // staging of store / traverse calls
+    size_t work_bytes = 0;
 };
+
+static int tt_work(omk_tt *tt, size_t bytes) {
+    if (bytes <= tt->work_bytes) return OMK_OK;
+    HIP_TRY(hipStreamSynchronize(tt->f->stream));
+    if (tt->work) HIP_TRY(hipFree(tt->work));
+    tt->work = nullptr;
+    tt->work_bytes = 0;
+    HIP_TRY(hipMalloc(&tt->work, bytes));
+    tt->work_bytes = bytes;
+    return OMK_OK;
+}
 
 template <typename T>
 static hipError_t dalloc(T **p, int64_t count) {
@@ -1285,7 +1301,8 @@ int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out) {
     f->children++;
     tt->log2_slots = log2_slots;
     hipError_t e = dalloc(&tt->slots, 1ll << log2_slots);
-    if (e == hipSuccess) e = dalloc(&tt->d_status, 2);
+    if (e == hipSuccess) e = dalloc(&tt->meta, 1ll << log2_slots);
+    if (e == hipSuccess) e = dalloc(&tt->d_status, 8);
     if (e != hipSuccess) {
         int rc = fail(OMK_ERR_HIP, "omk_tt_create: %s", hipGetErrorString(e));
         omk_tt_destroy(tt);
@@ -1300,6 +1317,8 @@ int omk_tt_destroy(omk_tt *tt) {
     (void)hipSetDevice(tt->f->device);
     (void)hipStreamSynchronize(tt->f->stream);
     if (tt->slots) (void)hipFree(tt->slots);
+    if (tt->meta) (void)hipFree(tt->meta);
+    if (tt->work) (void)hipFree(tt->work);
     if (tt->d_status) (void)hipFree(tt->d_status);
     (void)hipGetLastError();
     forest_child_gone(tt->f);
@@ -1310,7 +1329,8 @@ int omk_tt_destroy(omk_tt *tt) {
 int omk_tt_clear(omk_tt *tt) {
     if (!tt) return fail(OMK_ERR_INVALID, "omk_tt_clear: null table");
     if (int rc = use_device(tt->f)) return rc;
-    HIP_TRY(launch_tt_clear(tt->slots, tt->log2_slots, tt->f->stream));
+    HIP_TRY(launch_tt_clear(tt->slots, tt->meta, tt->log2_slots, tt->f->stream));
+    tt->clock = 0;
     return OMK_OK;
 }
 
@@ -1319,7 +1339,7 @@ int omk_tt_insert(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, co
     if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_insert: n %lld", (long long)n);
     if (int rc = use_device(tt->f)) return rc;
     hipStream_t s = tt->f->stream;
-    int status[2] = {0, 0};
+    int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
     HIP_TRY(launch_tt_insert(tt->slots, tt->log2_slots, d_keys, d_nodes, d_depths, n, tt->d_status, s));
     HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
@@ -1333,7 +1353,9 @@ int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_dept
     if (!tt || !d_keys || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe: null argument");
     if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_probe: n %lld", (long long)n);
     if (int rc = use_device(tt->f)) return rc;
-    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, 0, n, min_depth, d_out, tt->f->stream));
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, 0, n, min_depth, d_out, tt->meta,
+                            tt->clock, tt->f->stream));
+    tt->clock += (uint32_t)n;
     return OMK_OK;
 }
 
@@ -1345,7 +1367,98 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
     if (!b->f->has_hash) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: the forest was uploaded without position keys");
     if (int rc = use_device(tt->f)) return rc;
     HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->f->n_nodes, b->n, min_depth, d_out,
-                            tt->f->stream));
+                            tt->meta, tt->clock, tt->f->stream));
+    tt->clock += (uint32_t)b->n;
+    return OMK_OK;
+}
+
+int omk_tt_set_replacement_threshold(omk_tt *tt, float threshold) {
+    if (!tt || !(threshold >= 0.0f)) return fail(OMK_ERR_INVALID, "omk_tt_set_replacement_threshold: bad argument");
+    tt->threshold = threshold;
+    return OMK_OK;
+}
+
+static int tt_report(const char *who, const int *st, int32_t *h_counts) {
+    if (h_counts) {
+        h_counts[0] = st[3];  // new entries
+        h_counts[1] = st[4];  // replacements
+        h_counts[2] = st[2];  // later entries of the call with a key an earlier one carries: dropped
+        h_counts[3] = st[6];  // transpositions reported (traverse)
+    }
+    if (st[1]) return fail(OMK_ERR_INVALID, "%s: %d keys equal the empty marker ~0", who, st[1]);
+    if (st[0]) return fail(OMK_ERR_CAPACITY, "%s: table full, %d entries dropped", who, st[0]);
+    return OMK_OK;
+}
+
+int omk_tt_store(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, const int32_t *d_depths, int64_t n,
+                 int32_t *h_counts) {
+    if (!tt || !d_keys || !d_nodes) return fail(OMK_ERR_INVALID, "omk_tt_store: null argument");
+    if (n < 0 || n > (1ll << 30)) return fail(OMK_ERR_INVALID, "omk_tt_store: n %lld", (long long)n);
+    if (!tt->f->uploaded) return fail(OMK_ERR_STATE, "omk_tt_store: upload the forest first");
+    if (int rc = use_device(tt->f)) return rc;
+    if (int rc = tt_work(tt, (size_t)std::max<int64_t>(n, 1) * 8)) return rc;
+    hipStream_t s = tt->f->stream;
+    int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
+    HIP_TRY(launch_tt_store(tt->f->dev(), tt->slots, tt->meta, tt->log2_slots, d_keys, d_nodes, d_depths, n,
+                            (int64_t *)tt->work, tt->clock, tt->threshold, tt->d_status, s));
+    tt->clock += (uint32_t)n;
+    HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    return tt_report("omk_tt_store", status, h_counts);
+}
+
+int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
+                    const uint64_t *d_root_keys, const int32_t *d_root_players, int32_t *d_hits, int32_t *h_counts) {
+    if (!tt || !b) return fail(OMK_ERR_INVALID, "omk_tt_traverse: null argument");
+    if (tt->f != b->f) return fail(OMK_ERR_INVALID, "omk_tt_traverse: table and batch belong to different forests");
+    if (!b->selected) return fail(OMK_ERR_STATE, "omk_tt_traverse: no selected paths");
+    if (int rc = fresh_batch("omk_tt_traverse", b)) return rc;
+    omk_forest *f = b->f;
+    if (d_piece_keys) {
+        if (!d_player_keys || !d_root_keys || !d_root_players || cells <= 0)
+            return fail(OMK_ERR_INVALID, "omk_tt_traverse: the game's key tables need player keys, root keys, root players "
+                        "and cells > 0");
+    } else if (!f->has_hash) {
+        return fail(OMK_ERR_STATE, "omk_tt_traverse: no key tables given and the forest was uploaded without position keys");
+    }
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    const int64_t n = (int64_t)b->n * b->max_depth;
+    // staging: slot_of [n] i64 | keys [n] u64 | step_nodes, store_nodes, depths, found [n] i32 each
+    if (int rc = tt_work(tt, (size_t)n * 32)) return rc;
+    int64_t *slot_of = (int64_t *)tt->work;
+    uint64_t *keys = (uint64_t *)(slot_of + n);
+    int32_t *step_nodes = (int32_t *)(keys + n), *store_nodes = step_nodes + n, *depths = store_nodes + n;
+    int32_t *found = depths + n;
+    int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
+    HIP_TRY(launch_step_keys(f->dev(), b->paths, b->path_len, b->n, b->stride, b->max_depth, d_piece_keys, cells,
+                             d_player_keys, d_root_keys, d_root_players, keys, step_nodes, store_nodes, depths,
+                             tt->d_status, s));
+    // all stores first, then all lookups: a lookup that the serial loop makes before a later step's
+    // store can only miss a node without visits, and such a node is no transposition (:142)
+    HIP_TRY(launch_tt_store(f->dev(), tt->slots, tt->meta, tt->log2_slots, keys, store_nodes, depths, n, slot_of,
+                            tt->clock, tt->threshold, tt->d_status, s));
+    tt->clock += (uint32_t)n;
+    HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, keys, nullptr, nullptr, 0, n, 0, found, tt->meta, tt->clock, s));
+    tt->clock += (uint32_t)n;
+    if (d_hits) HIP_TRY(launch_tt_hits(f->dev(), step_nodes, found, n, d_hits, tt->d_status, s));
+    HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (status[5])
+        return fail(OMK_ERR_INVALID, "omk_tt_traverse: %d paths hold a node outside the forest or a move outside [0, %d)",
+                    status[5], cells);
+    status[1] = 0;  // steps that do not exist carry the empty marker on purpose
+    return tt_report("omk_tt_traverse", status, h_counts);
+}
+
+int omk_tt_download_meta(omk_tt *tt, omk_tt_meta *h_meta) {
+    if (!tt || !h_meta) return fail(OMK_ERR_INVALID, "omk_tt_download_meta: null argument");
+    if (int rc = use_device(tt->f)) return rc;
+    HIP_TRY(hipStreamSynchronize(tt->f->stream));
+    static_assert(sizeof(omk_tt_meta) == sizeof(TTMeta), "the ABI struct mirrors the device one");
+    HIP_TRY(hipMemcpy(h_meta, tt->meta, sizeof(TTMeta) << tt->log2_slots, hipMemcpyDeviceToHost));
     return OMK_OK;
 }
 

@@ -369,7 +369,7 @@ __device__ __forceinline__ uint64_t tt_home(uint64_t key, int log2_slots) {
     return (key * 0x9E3779B97F4A7C15ull) >> (64 - log2_slots);
 }
 
-__global__ __launch_bounds__(256) void k_tt_clear(TTSlot *slots, int64_t n) {
+__global__ __launch_bounds__(256) void k_tt_clear(TTSlot *slots, TTMeta *meta, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     TTSlot e;
@@ -377,6 +377,201 @@ __global__ __launch_bounds__(256) void k_tt_clear(TTSlot *slots, int64_t n) {
     e.node = -1;
     e.depth = 0;
     slots[i] = e;
+    TTMeta m;
+    m.visits = 0u;
+    m.value = 0.0f;
+    m.last_access = 0u;
+    m.claim = 0x7FFFFFFF;
+    meta[i] = m;
+}
+
+// ---- PHMapTranspositionTable::store (phmap_transposition_table.cpp:51-84) for a batch of entries,
+// in three passes.  Entry i of the call has the time t0 + i.  Among the entries of one call that
+// carry the same key only the first (lowest i) is stored, which is what the serial order gives for
+// the reference's call sites (a node stored from the traversal has no visits, hence replacement
+// score 0, and never replaces; the leaves expanded in one step are distinct).
+
+// Pass 1: every entry finds the slot of its key, or claims an empty one, and bids for it with its index.
+__global__ __launch_bounds__(256) void k_tt_store_claim(TTSlot *slots, TTMeta *meta, int log2_slots,
+                                                        const uint64_t *keys, const int32_t *nodes, int64_t n,
+                                                        int64_t *slot_of, int *d_status) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    slot_of[i] = -1;
+    if (nodes[i] < 0) return;  // nothing to store for this entry (store(): if (!node) return)
+    unsigned long long key = keys[i];
+    if (key == kTTEmpty) {
+        atomicAdd(d_status + 1, 1);
+        return;
+    }
+    uint64_t mask = (1ull << log2_slots) - 1ull;
+    uint64_t s = tt_home(key, log2_slots);
+    for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+        unsigned long long prev = atomicCAS(&slots[s].key, kTTEmpty, key);
+        if (prev == kTTEmpty) slots[s].depth = INT32_MIN;  // claimed just now: no entry behind the key yet
+        if (prev == kTTEmpty || prev == key) {
+            atomicMin(&meta[s].claim, (int)i);
+            slot_of[i] = (int64_t)s;
+            return;
+        }
+    }
+    atomicAdd(d_status, 1);
+}
+
+__device__ __forceinline__ float tt_replacement_score(uint32_t visits, float value, int depth, uint32_t now,
+                                                      uint32_t last_access) {
+    // Entry::getReplacementScore (include/mcts/phmap_transposition_table.h:68-72)
+    float recency = 1.0f / (1.0f + (float)(now - last_access));
+    float importance = (float)visits * (1.0f + value) * (1.0f + (float)depth);
+    return recency * importance;
+}
+
+// Pass 2: the winner of every slot creates the entry (createEntry :202-216: visits and value of the
+// node as they are now) or replaces the one that is there when its score is better by the threshold.
+// d_status[2] duplicates dropped, [3] new entries, [4] replacements.
+__global__ __launch_bounds__(256) void k_tt_store_apply(ForestDev f, TTSlot *slots, TTMeta *meta,
+                                                        const int32_t *nodes, const int32_t *depths, int64_t n,
+                                                        const int64_t *slot_of, uint32_t t0, float threshold,
+                                                        int *d_status) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t s = slot_of[i];
+    if (s < 0) return;
+    if (meta[s].claim != (int)i) {
+        atomicAdd(d_status + 2, 1);
+        return;
+    }
+    const int node = nodes[i];
+    const int depth = (int)(uint16_t)(depths ? depths[i] : 0);  // Entry::depth is a uint16_t
+    uint32_t visits = 0u;
+    float value = 0.0f;
+    if (node < f.n_nodes) {
+        const int nv = f.N[node];
+        visits = (uint32_t)nv;
+        value = nv == 0 ? 0.0f : f.W[node] / (float)nv;  // MCTSNode::getValue, src/mcts/mcts_node.cpp:484-490
+    }
+    bool write = false;
+    if (slots[s].depth == INT32_MIN) {
+        write = true;
+        atomicAdd(d_status + 3, 1);
+    } else {
+        const uint32_t now = t0 + (uint32_t)i;
+        const float existing = tt_replacement_score(meta[s].visits, meta[s].value, slots[s].depth, now, meta[s].last_access);
+        const float fresh = tt_replacement_score(visits, value, depth, now, 0u);
+        if (fresh > existing * (1.0f + threshold)) {
+            write = true;
+            atomicAdd(d_status + 4, 1);
+        }
+    }
+    if (write) {
+        slots[s].node = node;
+        slots[s].depth = depth;
+        meta[s].visits = visits;
+        meta[s].value = value;
+        meta[s].last_access = 0u;  // a new Entry starts with last_access 0
+    }
+}
+
+// Pass 3: the bids are withdrawn.
+__global__ __launch_bounds__(256) void k_tt_store_reset(TTMeta *meta, const int64_t *slot_of, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int64_t s = slot_of[i];
+    if (s >= 0) meta[s].claim = 0x7FFFFFFF;
+}
+
+hipError_t launch_tt_store(const ForestDev &f, TTSlot *slots, TTMeta *meta, int log2_slots, const uint64_t *keys,
+                           const int32_t *nodes, const int32_t *depths, int64_t n, int64_t *slot_of, uint32_t t0,
+                           float threshold, int *d_status, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    hipLaunchKernelGGL(k_tt_store_claim, grid, block, 0, s, slots, meta, log2_slots, keys, nodes, n, slot_of, d_status);
+    hipLaunchKernelGGL(k_tt_store_apply, grid, block, 0, s, f, slots, meta, nodes, depths, n, slot_of, t0, threshold,
+                       d_status);
+    hipLaunchKernelGGL(k_tt_store_reset, grid, block, 0, s, meta, slot_of, n);
+    return hipGetLastError();
+}
+
+// ---- the transposition-table part of the traversal loop (mcts_engine_batch_tree_simple.cpp:116-162)
+// over the paths of a selection ----
+
+// The key of the state after every step of every path, the node selected there and its depth, laid
+// out in the order the serial loop visits them (traversal-major: entry t * max_depth + d - 1 for step
+// d >= 1 of traversal t); node -1 where the path has no such step.  Keys: the forest's per-node
+// position keys, or (piece != nullptr) the root state's key with the piece keys of the path's moves
+// folded in, as in k_leaf_keys.  store_nodes receives the node where the reference stores it
+// (its visit count is 0, :116) and -1 elsewhere.
+__global__ __launch_bounds__(256) void k_step_keys(ForestDev f, const int32_t *paths, const int32_t *path_len, int n,
+                                                   int stride, int max_depth, const uint64_t *piece, int cells,
+                                                   const uint64_t *player, const uint64_t *root_key,
+                                                   const int32_t *root_player, uint64_t *keys, int32_t *step_nodes,
+                                                   int32_t *store_nodes, int32_t *depths, int *d_status) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    const int len = path_len[t];
+    const int p0 = piece ? (root_player[t] & 1) : 0;
+    uint64_t h = piece ? root_key[t] : 0ull;
+    bool bad = false;
+    for (int d = 1; d <= max_depth; d++) {
+        const size_t e = (size_t)t * max_depth + (d - 1);
+        int node = -1;
+        uint64_t key = ~0ull;
+        if (d < len && !bad) {
+            node = paths[(size_t)d * stride + t];
+            if (node < 0 || node >= f.n_nodes) {
+                bad = true;
+                node = -1;
+            } else if (piece) {
+                const int act = f.action ? f.action[node] : node;
+                if (act < 0 || act >= cells) {
+                    bad = true;
+                    node = -1;
+                } else {
+                    h ^= piece[(size_t)((p0 + d - 1) & 1) * cells + act];
+                    key = (d & 1) ? h ^ player[p0] ^ player[p0 ^ 1] : h;
+                }
+            } else {
+                key = f.hash[node];
+            }
+        }
+        keys[e] = key;
+        step_nodes[e] = node;
+        store_nodes[e] = node >= 0 && f.N[node] == 0 ? node : -1;
+        depths[e] = d;
+    }
+    if (bad) atomicAdd(d_status + 5, 1);
+}
+
+// What the loop does with a lookup (:141-156): a node other than the selected one, with visits, is a
+// transposition.  It is reported (hit[e] = that node, else -1), never followed.
+__global__ __launch_bounds__(256) void k_tt_hits(ForestDev f, const int32_t *step_nodes, const int32_t *found, int64_t n,
+                                                 int32_t *hit, int *d_status) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int fn = found[i], node = step_nodes[i];
+    int out = -1;
+    if (node >= 0 && fn >= 0 && fn != node && fn < f.n_nodes && f.N[fn] > 0) out = fn;
+    hit[i] = out;
+    if (out >= 0) atomicAdd(d_status + 6, 1);
+}
+
+hipError_t launch_step_keys(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                            int max_depth, const uint64_t *piece, int cells, const uint64_t *player,
+                            const uint64_t *root_key, const int32_t *root_player, uint64_t *keys, int32_t *step_nodes,
+                            int32_t *store_nodes, int32_t *depths, int *d_status, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_step_keys, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f, paths, path_len, n, stride,
+                       max_depth, piece, cells, player, root_key, root_player, keys, step_nodes, store_nodes, depths,
+                       d_status);
+    return hipGetLastError();
+}
+
+hipError_t launch_tt_hits(const ForestDev &f, const int32_t *step_nodes, const int32_t *found, int64_t n, int32_t *hit,
+                          int *d_status, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_tt_hits, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f, step_nodes, found, n, hit,
+                       d_status);
+    return hipGetLastError();
 }
 
 // d_status[0] counts entries that found no slot, d_status[1] keys equal to the empty marker
@@ -404,9 +599,12 @@ __global__ __launch_bounds__(256) void k_tt_insert(TTSlot *slots, int log2_slots
     atomicAdd(d_status, 1);
 }
 
+// meta / t0: a successful lookup stamps the entry with its time (PHMapTranspositionTable::lookup,
+// phmap_transposition_table.cpp:107: last_access = access_counter++); lookup i of a call has the time
+// t0 + i, the latest wins.
 __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys,
                                                   const int32_t *leaf, const uint64_t *node_hash, int64_t n_nodes,
-                                                  int64_t n, int min_depth, int32_t *out) {
+                                                  int64_t n, int min_depth, int32_t *out, TTMeta *meta, uint32_t t0) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     unsigned long long key = kTTEmpty;
@@ -422,7 +620,10 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
             uint4 raw = *reinterpret_cast<const uint4 *>(slots + s);
             unsigned long long k = ((unsigned long long)raw.y << 32) | raw.x;
             if (k == key) {
-                if ((int)raw.w >= min_depth) found = (int)raw.z;
+                if ((int)raw.w >= min_depth) {
+                    found = (int)raw.z;
+                    if (meta) atomicMax(&meta[s].last_access, t0 + (uint32_t)i);
+                }
                 break;
             }
             if (k == kTTEmpty) break;
@@ -431,18 +632,18 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
     out[i] = found;
 }
 
-hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s) {
+hipError_t launch_tt_clear(TTSlot *slots, TTMeta *meta, int log2_slots, hipStream_t s) {
     int64_t n = 1ll << log2_slots;
-    hipLaunchKernelGGL(k_tt_clear, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, n);
+    hipLaunchKernelGGL(k_tt_clear, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, meta, n);
     return hipGetLastError();
 }
 
 hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
                            const uint64_t *node_hash, int64_t n_nodes, int64_t n, int min_depth, int32_t *out,
-                           hipStream_t s) {
+                           TTMeta *meta, uint32_t t0, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_tt_probe, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, slots, log2_slots, keys, leaf,
-                       node_hash, n_nodes, n, min_depth, out);
+                       node_hash, n_nodes, n, min_depth, out, meta, t0);
     return hipGetLastError();
 }
 

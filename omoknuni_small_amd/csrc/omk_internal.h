@@ -155,13 +155,33 @@ struct TTSlot {
     int32_t node;
     int32_t depth;
 };
-hipError_t launch_tt_clear(TTSlot *slots, int log2_slots, hipStream_t s);
+// What PHMapTranspositionTable::Entry keeps beside key, node and depth for its replacement policy
+// (include/mcts/phmap_transposition_table.h:48-72), in an array beside the slots: a probe reads
+// the 16-byte slot only.
+struct TTMeta {
+    uint32_t visits;
+    float value;
+    uint32_t last_access;
+    int32_t claim;  // lowest index of the entries of a store call that want this slot (0x7FFFFFFF between calls)
+};
+hipError_t launch_tt_clear(TTSlot *slots, TTMeta *meta, int log2_slots, hipStream_t s);
+// d_status: [0] no free slot, [1] key equal to the empty marker, [2] duplicates of a key dropped,
+// [3] new entries, [4] replacements, [5] paths with a step that has no key, [6] transpositions found
+hipError_t launch_tt_store(const ForestDev &f, TTSlot *slots, TTMeta *meta, int log2_slots, const uint64_t *keys,
+                           const int32_t *nodes, const int32_t *depths, int64_t n, int64_t *slot_of, uint32_t t0,
+                           float threshold, int *d_status, hipStream_t s);
+hipError_t launch_step_keys(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                            int max_depth, const uint64_t *piece, int cells, const uint64_t *player,
+                            const uint64_t *root_key, const int32_t *root_player, uint64_t *keys, int32_t *step_nodes,
+                            int32_t *store_nodes, int32_t *depths, int *d_status, hipStream_t s);
+hipError_t launch_tt_hits(const ForestDev &f, const int32_t *step_nodes, const int32_t *found, int64_t n, int32_t *hit,
+                          int *d_status, hipStream_t s);
 // d_status[0] += entries that found no free slot, d_status[1] += keys equal to the empty marker
 hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
                             const int32_t *depths, int64_t n, int *d_status, hipStream_t s);
 // keys == nullptr: the key of entry i is node_hash[leaf[i]] (nothing for a leaf outside [0, n_nodes))
 hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *leaf,
                            const uint64_t *node_hash, int64_t n_nodes, int64_t n, int min_depth, int32_t *out,
-                           hipStream_t s);
+                           TTMeta *meta, uint32_t t0, hipStream_t s);
 
 }  // namespace omk

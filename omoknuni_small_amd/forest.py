@@ -28,11 +28,12 @@ EXPORTS = [
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
-    "omk_tt_probe_leaves", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
+    "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy",
 ]
 
 TT_SLOT = np.dtype([("key", "<u8"), ("node", "<i4"), ("depth", "<i4")])
+TT_META = np.dtype([("visits", "<u4"), ("value", "<f4"), ("last_access", "<u4"), ("reserved", "<i4")])
 
 
 class OmkError(RuntimeError):
@@ -495,6 +496,66 @@ class TranspositionTable:
         finally:
             f.dev_free(do)
         return out
+
+    def store(self, keys, nodes, depths=None):
+        """PHMapTranspositionTable::store for a batch; returns (new entries, replacements, duplicates dropped)."""
+        f = self.forest
+        keys = np.ascontiguousarray(keys, np.uint64)
+        nodes = np.ascontiguousarray(nodes, np.int32)
+        n = len(keys)
+        counts = np.zeros(4, np.int32)
+        dk, dn = f.dev_alloc(n * 8), f.dev_alloc(n * 4)
+        dd = 0
+        try:
+            f.h2d(dk, keys)
+            f.h2d(dn, nodes)
+            if depths is not None:
+                dd = f.dev_alloc(n * 4)
+                f.h2d(dd, np.ascontiguousarray(depths, np.int32))
+            _check(self._lib.omk_tt_store(self._h, C.c_void_p(dk), C.c_void_p(dn), C.c_void_p(dd or 0), C.c_int64(n),
+                                          _ptr(counts, i32p)))
+        finally:
+            for p in (dk, dn, dd):
+                if p:
+                    f.dev_free(p)
+        return tuple(int(x) for x in counts[:3])
+
+    def set_replacement_threshold(self, threshold):
+        _check(self._lib.omk_tt_set_replacement_threshold(self._h, C.c_float(threshold)))
+
+    def traverse(self, batch, zobrist=None):
+        """The table's part of the traversal loop over the paths of batch's last select(): stores the
+        unvisited selected children, looks every step up, reports transpositions.  zobrist: None (the
+        forest's per-node keys) or (piece_keys [2, cells], player_keys [2], root_keys [n], root_players [n]).
+        Returns (hits [n, max_depth] node or -1, (new entries, replacements, duplicates, transpositions))."""
+        f = self.forest
+        n, D = batch.n, batch.max_depth
+        hits = np.empty((n, D), np.int32)
+        counts = np.zeros(4, np.int32)
+        bufs = [f.dev_alloc(hits.nbytes)]
+        args = [0, 0, 0, 0, 0]
+        try:
+            if zobrist is not None:
+                pk = np.ascontiguousarray(zobrist[0], np.uint64)
+                arrs = (pk, np.ascontiguousarray(zobrist[1], np.uint64), np.ascontiguousarray(zobrist[2], np.uint64),
+                        np.ascontiguousarray(zobrist[3], np.int32))
+                for x in arrs:
+                    bufs.append(f.dev_alloc(x.nbytes))
+                    f.h2d(bufs[-1], x)
+                args = [bufs[1], pk.shape[1], bufs[2], bufs[3], bufs[4]]
+            _check(self._lib.omk_tt_traverse(self._h, batch._h, C.c_void_p(args[0]), C.c_int32(int(args[1])),
+                                             C.c_void_p(args[2]), C.c_void_p(args[3]), C.c_void_p(args[4]),
+                                             C.c_void_p(bufs[0]), _ptr(counts, i32p)))
+            f.d2h(hits, bufs[0])
+        finally:
+            for d in bufs:
+                f.dev_free(d)
+        return hits, tuple(int(x) for x in counts)
+
+    def download_meta(self):
+        meta = np.empty(1 << self.log2, dtype=TT_META)
+        _check(self._lib.omk_tt_download_meta(self._h, meta.ctypes.data_as(C.c_void_p)))
+        return meta
 
     def upload(self, slots):
         slots = np.ascontiguousarray(slots, dtype=TT_SLOT)

@@ -319,6 +319,99 @@ int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_
     return hits;
 }
 
+/* ---- PHMapTranspositionTable::store with its replacement policy
+ * (src/mcts/phmap_transposition_table.cpp:51-84, createEntry :202-216, Entry::getReplacementScore
+ * include/mcts/phmap_transposition_table.h:68-72), over the open-addressing table, entries of a call
+ * in index order.  The reference's clock (access_counter_) is shared by its threads and only ticks on
+ * some paths; here entry i of a call has the time t0 + i.  Among the entries of one call that carry
+ * the same key only the first is stored (see ref_cpu.h).  counts: new entries, replacements,
+ * duplicates dropped, -.  Returns 0, -1 when the table is full, -2 on a key equal to the empty marker. */
+static float tt_score(uint32_t visits, float value, int32_t depth, uint32_t now, uint32_t last_access) {
+    float recency = 1.0f / (1.0f + (float)(now - last_access));
+    float importance = (float)visits * (1.0f + value) * (1.0f + (float)depth);
+    return recency * importance;
+}
+
+int ref_tt_store_batch(ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, const ref_tree *t,
+                       const uint64_t *keys, const int32_t *nodes, const int32_t *depths, int64_t n, uint32_t t0,
+                       float threshold, int32_t *counts) {
+    uint64_t mask = ((uint64_t)1 << log2_slots) - 1;
+    int rc = 0;
+    int64_t *touched = (int64_t *)malloc((size_t)(n > 0 ? n : 1) * sizeof(int64_t));
+    int64_t n_touched = 0;
+    counts[0] = counts[1] = counts[2] = counts[3] = 0;
+    for (int64_t i = 0; i < n; i++) {
+        if (nodes[i] < 0) continue;                               /* store(): if (!node) return */
+        if (keys[i] == REF_TT_EMPTY) { rc = -2; continue; }
+        uint64_t s = tt_home(keys[i], log2_slots);
+        int placed = 0;
+        for (uint64_t probe = 0; probe <= mask && !placed; probe++, s = (s + 1) & mask) {
+            if (slots[s].key != keys[i] && slots[s].key != REF_TT_EMPTY) continue;
+            placed = 1;
+            const int fresh = slots[s].key == REF_TT_EMPTY;
+            if (!fresh && meta[s].reserved == 1) { counts[2]++; break; }   /* an earlier entry of this call */
+            const int32_t node = nodes[i];
+            const int32_t depth = (int32_t)(uint16_t)(depths ? depths[i] : 0);  /* Entry::depth is uint16_t */
+            uint32_t visits = 0;
+            float value = 0.0f;
+            if (node < t->n_nodes) {                              /* createEntry :212-213, getValue :484-490 */
+                visits = (uint32_t)t->N[node];
+                value = t->N[node] == 0 ? 0.0f : t->W[node] / (float)t->N[node];
+            }
+            int write = fresh;
+            if (fresh) {
+                counts[0]++;
+            } else {
+                const uint32_t now = t0 + (uint32_t)i;            /* :65 */
+                const float existing = tt_score(meta[s].visits, meta[s].value, slots[s].depth, now, meta[s].last_access);
+                const float incoming = tt_score(visits, value, depth, now, 0u);
+                if (incoming > existing * (1.0f + threshold)) { write = 1; counts[1]++; }   /* :71 */
+            }
+            if (write) {
+                slots[s].key = keys[i];
+                slots[s].node = node;
+                slots[s].depth = depth;
+                meta[s].visits = visits;
+                meta[s].value = value;
+                meta[s].last_access = 0;                          /* a new Entry starts at 0 */
+            }
+            meta[s].reserved = 1;
+            touched[n_touched++] = (int64_t)s;
+        }
+        if (!placed) rc = rc ? rc : -1;
+    }
+    for (int64_t j = 0; j < n_touched; j++) meta[touched[j]].reserved = 0;
+    free(touched);
+    return rc;
+}
+
+/* PHMapTranspositionTable::lookup (:86-117) for a batch: a hit that passes the depth test stamps the
+ * entry with its time (:107), lookup i at t0 + i.  Returns the number of hits. */
+int64_t ref_tt_lookup_batch(const ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, const uint64_t *keys,
+                            int64_t n, int32_t min_depth, uint32_t t0, int32_t *out_node) {
+    uint64_t mask = ((uint64_t)1 << log2_slots) - 1;
+    int64_t hits = 0;
+    for (int64_t i = 0; i < n; i++) {
+        int32_t found = -1;
+        if (keys[i] != REF_TT_EMPTY) {
+            uint64_t s = tt_home(keys[i], log2_slots);
+            for (uint64_t probe = 0; probe <= mask; probe++, s = (s + 1) & mask) {
+                if (slots[s].key == keys[i]) {
+                    if (slots[s].depth >= min_depth) {
+                        found = slots[s].node;
+                        meta[s].last_access = t0 + (uint32_t)i;
+                    }
+                    break;
+                }
+                if (slots[s].key == REF_TT_EMPTY) break;
+            }
+        }
+        out_node[i] = found;
+        if (found >= 0) hits++;
+    }
+    return hits;
+}
+
 /* ---- leaf expansion (mcts_node.cpp:238-436, :512-593; call site
  * mcts_engine_batch_tree_simple.cpp:249-259) ---- */
 /* mcts_node.cpp:296-341: the number of children expand() creates.  The "incremental expansion"

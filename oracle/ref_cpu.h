@@ -209,6 +209,24 @@ typedef struct ref_tt_slot {
 
 void ref_tt_clear(ref_tt_slot *slots, int32_t log2_slots);
 /* 0 stored, 1 key already present (first entry kept), -1 table full, -2 reserved key */
+
+/* What PHMapTranspositionTable::Entry keeps for its replacement policy, beside the slots. */
+typedef struct ref_tt_meta {
+    uint32_t visits;
+    float value;
+    uint32_t last_access;
+    int32_t reserved;
+} ref_tt_meta;
+/* store() with the replacement policy and lookup() with its time stamp, for batches (see ref_cpu.c).
+ * PARITY UNPINNED against the reference (its table is phmap v1.3.8, absent, and its clock depends on
+ * the thread schedule); pinned against a literal Python restatement of store / lookup over a dict
+ * (tests/test_oracle_tt.py), which agrees wherever a key occurs once per call or is stored without
+ * visits, the reference's two call sites. */
+int ref_tt_store_batch(ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, const ref_tree *t,
+                       const uint64_t *keys, const int32_t *nodes, const int32_t *depths, int64_t n, uint32_t t0,
+                       float threshold, int32_t *counts);
+int64_t ref_tt_lookup_batch(const ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, const uint64_t *keys,
+                            int64_t n, int32_t min_depth, uint32_t t0, int32_t *out_node);
 int ref_tt_insert(ref_tt_slot *slots, int32_t log2_slots, uint64_t key, int32_t node, int32_t depth);
 /* out_node[i] = node stored under keys[i] with depth >= min_depth, else -1; returns hits */
 int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_t *keys, int64_t n,

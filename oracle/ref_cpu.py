@@ -308,11 +308,64 @@ class RefTree:
         return out
 
 
+TT_META = np.dtype([("visits", "<u4"), ("value", "<f4"), ("last_access", "<u4"), ("reserved", "<i4")])
+
+
 class RefTT:
     def __init__(self, log2_slots):
         self.log2 = int(log2_slots)
         self.slots = np.empty(1 << self.log2, dtype=TT_SLOT)
+        self.meta = np.zeros(1 << self.log2, dtype=TT_META)
+        self.clock = 0          # entry i of a call has the time clock + i; every call advances it by its length
+        self.threshold = 0.1    # Config::replacement_threshold
         lib().ref_tt_clear(self.slots.ctypes.data, self.log2)
+
+    def store(self, tree, keys, nodes, depths=None):
+        """store() with the replacement policy for a batch; (new entries, replacements, duplicates dropped)."""
+        keys = np.ascontiguousarray(keys, np.uint64)
+        nodes = np.ascontiguousarray(nodes, np.int32)
+        dp = None if depths is None else np.ascontiguousarray(depths, np.int32)
+        counts = np.zeros(4, np.int32)
+        fn = lib().ref_tt_store_batch
+        fn.restype = C.c_int
+        rc = fn(C.c_void_p(self.slots.ctypes.data), C.c_void_p(self.meta.ctypes.data), C.c_int32(self.log2),
+                C.byref(tree._c), _ptr(keys, u64p), _ptr(nodes, i32p), _ptr(dp, i32p), C.c_int64(len(keys)),
+                C.c_uint32(self.clock & 0xFFFFFFFF), C.c_float(self.threshold), _ptr(counts, i32p))
+        self.clock += len(keys)
+        assert rc == 0, rc
+        return tuple(int(x) for x in counts[:3])
+
+    def lookup(self, keys, min_depth=0):
+        """lookup() for a batch, stamping the entries it finds; (nodes, hits)."""
+        keys = np.ascontiguousarray(keys, np.uint64)
+        out = np.empty(len(keys), np.int32)
+        fn = lib().ref_tt_lookup_batch
+        fn.restype = C.c_int64
+        hits = fn(C.c_void_p(self.slots.ctypes.data), C.c_void_p(self.meta.ctypes.data), C.c_int32(self.log2),
+                  _ptr(keys, u64p), C.c_int64(len(keys)), C.c_int32(int(min_depth)), C.c_uint32(self.clock & 0xFFFFFFFF),
+                  _ptr(out, i32p))
+        self.clock += len(keys)
+        return out, int(hits)
+
+    def traverse(self, tree, paths, path_len, step_keys):
+        """The table's part of the traversal loop (mcts_engine_batch_tree_simple.cpp:116-162) over row-major
+        paths: step_keys [B, D] = key of the state after step d + 1 of traversal t.  Stores the selected
+        children without visits, looks every step up; returns (hits [B, D] node or -1, counts)."""
+        B, row = paths.shape
+        D = row - 1
+        d_idx = np.arange(1, row)[None, :]
+        valid = d_idx < path_len[:, None]
+        step_nodes = np.where(valid, paths[:, 1:], -1).astype(np.int32)
+        keys = np.where(valid, step_keys, np.uint64(0xFFFFFFFFFFFFFFFF)).astype(np.uint64)
+        unvisited = valid & (tree.N[np.maximum(step_nodes, 0)] == 0)
+        store_nodes = np.where(unvisited, step_nodes, -1).astype(np.int32)
+        depths = np.broadcast_to(d_idx, (B, D)).astype(np.int32)
+        new, repl, dup = self.store(tree, keys.reshape(-1), store_nodes.reshape(-1), depths.reshape(-1))
+        found, _ = self.lookup(keys.reshape(-1))
+        found = found.reshape(B, D)
+        hit = valid & (found >= 0) & (found != step_nodes) & (tree.N[np.maximum(found, 0)] > 0)
+        hits = np.where(hit, found, -1).astype(np.int32)
+        return hits, (new, repl, dup, int(hit.sum()))
 
     def insert(self, key, node, depth=0):
         return lib().ref_tt_insert(self.slots.ctypes.data, self.log2, int(key), int(node), int(depth))
