@@ -55,7 +55,7 @@ void ForestEngine::selectLeafBatch(const std::vector<int32_t> &roots, std::vecto
     p.virtual_loss = settings_.virtual_loss;
     p.use_rave = (settings_.use_rave && has_rave_) ? 1 : 0;
     p.rave_k = settings_.rave_constant;
-    p.pw = settings_.use_progressive_widening ? 1 : 0;
+    p.pw = settings_.selection_prior_widening ? 1 : 0;
     check(omk_select_batch(batch_, &p), "omk_select_batch");
     const int D = settings_.max_depth;
     h_paths_.resize((size_t)n * (D + 1));
@@ -107,32 +107,31 @@ void ForestEngine::downloadStructure(int64_t n_nodes, int32_t *child_begin, int3
 }
 
 int64_t ForestEngine::expandLeafBatch(const std::vector<std::vector<int>> &legal_moves,
-                                      const std::vector<NetworkOutput> &outputs) {
+                                      const std::vector<NetworkOutput> &outputs, int action_space) {
     if ((int)legal_moves.size() != last_n_) throw std::runtime_error("expandLeafBatch: one move list per simulation");
-    size_t action_space = 0;
-    bool have_policy = outputs.size() == legal_moves.size() && !outputs.empty();
-    if (have_policy) {
-        action_space = outputs[0].policy.size();
-        for (const auto &o : outputs)
-            if (o.policy.size() != action_space) have_policy = false;
-        if (action_space == 0) have_policy = false;
-    }
-    std::vector<int32_t> begin(legal_moves.size() + 1, 0), moves;
+    const bool have_policy = outputs.size() == legal_moves.size();
+    std::vector<int32_t> begin(legal_moves.size() + 1, 0), moves, pbegin(legal_moves.size() + 1, 0);
+    std::vector<float> policy;
     for (size_t i = 0; i < legal_moves.size(); i++) {
         moves.insert(moves.end(), legal_moves[i].begin(), legal_moves[i].end());
         begin[i + 1] = (int32_t)moves.size();
+        if (have_policy) {
+            policy.insert(policy.end(), outputs[i].policy.begin(), outputs[i].policy.end());
+            if (action_space <= 0 && !outputs[i].policy.empty()) action_space = (int)outputs[i].policy.size();
+        }
+        pbegin[i + 1] = (int32_t)policy.size();
     }
     if (moves.empty()) moves.push_back(0);
-    std::vector<float> policy;
-    if (have_policy) {
-        policy.resize(outputs.size() * action_space);
-        for (size_t i = 0; i < outputs.size(); i++)
-            std::copy(outputs[i].policy.begin(), outputs[i].policy.end(), policy.begin() + i * action_space);
-    }
+    const bool with_policy = have_policy && !policy.empty();
+    omk_expand_params p;
+    p.action_space = action_space;
+    p.use_progressive_widening = settings_.use_progressive_widening ? 1 : 0;
+    p.progressive_widening_c = settings_.progressive_widening_c;
+    p.progressive_widening_k = settings_.progressive_widening_k;
     const int64_t before = nodeCount();
-    check(omk_expand_batch(batch_, begin.data(), moves.data(), have_policy ? policy.data() : nullptr,
-                           (int32_t)action_space, nullptr),
-          "omk_expand_batch");
+    check(omk_expand_batch_ex(batch_, begin.data(), moves.data(), with_policy ? pbegin.data() : nullptr,
+                              with_policy ? policy.data() : nullptr, &p, nullptr),
+          "omk_expand_batch_ex");
     return nodeCount() - before;
 }
 

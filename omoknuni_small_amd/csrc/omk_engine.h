@@ -39,8 +39,19 @@ struct MCTSSettings {
     int virtual_loss = 3;
     bool use_rave = true;
     float rave_constant = 3000.0f;
-    bool use_progressive_widening = false;  // selection-time eligibility filter, see omk_select_params::pw
-    int max_depth = 64;                     // longest path the batch buffers hold
+    // MCTSNode::expand's progressive widening, as in the reference (default on, c = 2, k = 0.5): a leaf
+    // of N visits gets min(legal, max(8, c * (N + 1)^k)) children (omk_expand_batch_ex)
+    bool use_progressive_widening = true;
+    float progressive_widening_c = 2.0f;
+    float progressive_widening_k = 0.5f;
+    bool add_dirichlet_noise = true;
+    float dirichlet_alpha = 0.3f;
+    float dirichlet_epsilon = 0.25f;
+    float temperature = 1.0f;
+    // Not in the reference: only the ceil(sqrt(N_parent)) children of highest prior take part in a
+    // selection (omk_select_params::pw; needs children stored by descending prior)
+    bool selection_prior_widening = false;
+    int max_depth = 64;  // longest path the batch buffers hold
 };
 
 // What PendingEvaluation{node, state, path} (reference include/mcts/evaluation_types.h:49-73)
@@ -72,10 +83,14 @@ class ForestEngine {
     // Simulation i starts at roots[i]: independent trees searched side by side.
     void selectLeafBatch(const std::vector<int32_t> &roots, std::vector<LeafItem> &leaves);
     void backPropagateBatch(const std::vector<float> &leaf_values);
-    // Expands the leaves of the last selectLeafBatch on the device: one child per legal move,
-    // priors from the evaluator's policy (uniform when a policy is empty or absent: all
-    // policies of a batch must have the same size).  Returns the nodes added.
-    int64_t expandLeafBatch(const std::vector<std::vector<int>> &legal_moves, const std::vector<NetworkOutput> &outputs);
+    // Expands the leaves of the last selectLeafBatch on the device as MCTSNode::expand +
+    // setPriorProbabilities do (reference src/mcts/mcts_engine_batch_tree_simple.cpp:249-259): children
+    // for the legal moves (the first of them under progressive widening), priors from every
+    // output's own policy (by action when it has action_space entries, by child when it has as
+    // many as children, uniform otherwise or when empty).  action_space <= 0: the size of the
+    // first policy that is not empty.  Returns the nodes added.
+    int64_t expandLeafBatch(const std::vector<std::vector<int>> &legal_moves, const std::vector<NetworkOutput> &outputs,
+                            int action_space = 0);
     void setLegalMovesFunction(LegalMovesFunction fn) { legal_moves_fn_ = std::move(fn); }
     // SearchResult.probabilities (reference MCTSEngine::getActionProbabilities,
     // src/mcts/mcts_engine_tree.cpp:388-465): visit counts of root's children, temperature.

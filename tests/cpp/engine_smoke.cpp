@@ -31,6 +31,7 @@ int main(int argc, char **argv) {
     s.batch_size = atoi(argv[3]);
     s.max_depth = atoi(argv[4]);
     s.use_rave = false;
+    s.use_progressive_widening = false;  // every legal move becomes a child: what the Python side restates
     long leaves_seen = 0;
     auto evaluator = [&](const std::vector<omk::LeafItem> &leaves) {
         std::vector<omk::NetworkOutput> out(leaves.size());

@@ -1,0 +1,170 @@
+"""omk::GPUForestMCTSEngine<State> (csrc/omk_search.h): MCTSEngine::search over the device forest with
+the reference's signatures (search(const State&) -> SearchResult, an InferenceFunction over
+unique_ptr<State> batches, leaf states built by clone + replay), driven by tests/cpp/search_smoke.cpp
+with a mock state, and omk::flattenTree.  The whole search is replayed here through the CPU checker,
+with the mock game and the stand-in evaluator restated in Python: every node of the final tree,
+the move probabilities and the move chosen must come out the same."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "omoknuni_small_amd", "search_smoke")
+CELLS = 12
+
+
+class Ring:
+    """tests/cpp/search_smoke.cpp's RingState."""
+
+    def __init__(self):
+        self.cell = [0] * CELLS
+        self.player, self.winner, self.moves = 1, 0, 0
+
+    def clone(self):
+        c = Ring()
+        c.cell, c.player, c.winner, c.moves = list(self.cell), self.player, self.winner, self.moves
+        return c
+
+    def legal(self):
+        return [i for i in range(CELLS) if self.cell[i] == 0] if self.winner == 0 else []
+
+    def make(self, a):
+        self.cell[a] = self.player
+        if self.cell[(a + 1) % CELLS] == self.player and self.cell[(a - 1) % CELLS] == self.player:
+            self.winner = self.player
+        self.player = 3 - self.player
+        self.moves += 1
+
+    def terminal(self):
+        return self.winner != 0 or self.moves == CELLS
+
+    def hash(self):
+        h = 1469598103934665603
+        for c in self.cell:
+            h = ((h ^ c) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+        return h ^ self.player
+
+
+def evaluate(state):
+    h = state.hash()
+    value = np.float32(np.float32(int(h % 2001) - 1000) / np.float32(1000.0))
+    pol = np.array([np.float32(1 + ((h >> (a * 3)) & 7)) for a in range(CELLS)], np.float32)
+    s = np.float32(0.0)
+    for x in pol:
+        s = np.float32(s + x)
+    return value, (pol / s).astype(np.float32)
+
+
+def replay_search(sims, batch, widening):
+    root_state = Ring()
+    root_state.make(3)
+    z = np.zeros(1, np.int32)
+    ref = R.RefTree(N=z, W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=z, child_begin=z, child_count=z,
+                    action=z - 1)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=16)
+    done, first = 0, True
+    while done < sims:
+        n = 1 if first else min(batch, sims - done)
+        first = False
+        roots = np.zeros(n, np.int32)
+        paths, plen, leaf, _ = ref.select_batch(roots, rp)
+        acts = ref.gather_actions(paths, plen)
+        begin, moves, pb, pol, values = [0], [], [0], [], []
+        for t in range(n):
+            s = root_state.clone()
+            for a in acts[t, :plen[t] - 1]:
+                s.make(int(a))
+            v, p = evaluate(s)
+            values.append(v)
+            if not s.terminal():
+                moves.extend(s.legal())
+            begin.append(len(moves))
+            pol.extend(p.tolist())
+            pb.append(len(pol))
+        ref.expand_batch(leaf, begin, np.array(moves if moves else [0], np.int32), policy=np.array(pol, np.float32),
+                         action_space=CELLS, policy_begin=pb, widening=(2.0, 0.5) if widening else None)
+        ref.backup_batch(paths, plen, np.array(values, np.float32), 3)
+        done += n
+    return ref
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("widening", [0, 1])
+def test_search_with_the_reference_signatures_matches_the_checker(widening):
+    sims, batch = 300, 32
+    r = subprocess.run([EXE, "search", str(sims), str(batch), str(widening), "0", "0"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().split("\n")
+    head = lines[0].split()
+    probs = np.array([float(x) for x in lines[1].split()[1:]], np.float32)
+    nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
+    ref = replay_search(sims, batch, widening)
+    assert int(head[5]) == sims and int(head[7]) == ref.n == len(nodes) and int(head[9]) == sims
+    assert (nodes[:, 0] == ref.N).all() and (nodes[:, 3] == ref.VL).all()
+    assert (nodes[:, 4] == ref.child_begin).all() and (nodes[:, 5] == ref.child_count).all()
+    assert (nodes[:, 6] == ref.action).all()
+    assert np.allclose(nodes[:, 2], ref.P, rtol=0, atol=1e-8)           # printed with 9 digits: exact to the float
+    assert np.abs(nodes[:, 1] - ref.W).max() <= 1e-5 * max(1.0, np.abs(ref.W).max())
+    assert ref.N[0] == sims                                            # every simulation backed up through the root
+    want, children = ref.action_probabilities(0, 0.0, CELLS)
+    assert children == ref.child_count[0] and (probs == want).all()
+    assert int(head[1]) == int(np.argmax(want))                        # temperature 0: the most visited move
+    assert abs(float(head[3]) - float(ref.W[0]) / sims) < 1e-5
+    if widening:
+        assert ref.child_count[0] == 8                                 # root expanded at N = 0: max(8, 2 * 1) of 11 moves
+        assert ref.child_count[ref.child_count > 0].max() <= 11
+    else:
+        assert ref.child_count[0] == 11
+    # a terminal state is answered without a search: the side to move has lost
+    assert lines[-1] == "terminal action -1 value -1 probabilities 12"
+
+
+@pytest.mark.gpu
+def test_search_with_noise_and_temperature_runs_and_is_consistent():
+    r = subprocess.run([EXE, "search", "200", "16", "1", "1", "1.0"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().split("\n")
+    head = lines[0].split()
+    probs = np.array([float(x) for x in lines[1].split()[1:]])
+    nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
+    assert abs(probs.sum() - 1.0) < 1e-4 and probs[int(head[1])] > 0   # the move was drawn from the distribution
+    kids = nodes[int(nodes[0, 4]):int(nodes[0, 4] + nodes[0, 5])]
+    assert nodes[0, 0] == 200 and kids[:, 0].sum() == 199              # the root's own evaluation is the first simulation
+    assert abs(kids[:, 2].sum() - 1.0) < 0.35 and (kids[:, 2] > 0).all()   # priors mixed with noise, still a rough distribution
+    assert (probs[kids[:, 6].astype(int)] > 0).sum() == (kids[:, 0] > 0).sum()
+
+
+@pytest.mark.gpu
+def test_flatten_tree_lays_a_pointer_tree_out_breadth_first_and_searches_on():
+    r = subprocess.run([EXE, "flatten"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    flat = np.array([[float(x) for x in ln.split()[2:]] for ln in r.stdout.split("\n") if ln.startswith("flat ")])
+    # root, its three children in vector order, then the grandchildren in the same order
+    assert flat[:, 0].tolist() == [40, 20, 12, 7, 9, 10, 6]
+    assert flat[:, 6].tolist() == [1, 4, 0, 6, 0, 0, 0] and flat[:, 7].tolist() == [3, 2, 0, 1, 0, 0, 0]
+    assert flat[:, 8].tolist() == [-1, 7, 2, 9, 1, 4, 5]
+    assert flat[:, 1].tolist() == [4.0, 8.0, -3.0, 0.5, 2.25, -5.0, 1.5]        # value sums back from the means
+    assert flat[:, 3].tolist() == [0, 0, 3, 0, 0, 0, 0] and flat[:, 4].tolist() == [0, 10, 6, 3, 4, 5, 3]
+    ref = R.RefTree(N=flat[:, 0], W=flat[:, 1], P=flat[:, 2], VL=flat[:, 3], child_begin=flat[:, 6], child_count=flat[:, 7],
+                    action=flat[:, 8])
+    paths, plen, leaf, _ = ref.select_batch(np.zeros(6, np.int32), R.make_params(c_puct=1.4, virtual_loss=3, max_depth=4))
+    acts = ref.gather_actions(paths, plen)
+    got = [ln for ln in r.stdout.split("\n") if ln.startswith("path")]
+    for t, ln in enumerate(got):
+        ids = [int(x) for x in ln.split(" moves")[0].split()[1:]]
+        mv = [int(x) for x in ln.split(" moves")[1].split()]
+        assert ids == paths[t, :plen[t]].tolist() and mv == acts[t, :plen[t] - 1].tolist()
+
+
+def test_search_driver_reports_errors_without_a_gpu():
+    assert os.path.exists(EXE), "build the adapter first (python -m omoknuni_small_amd.build)"
+    r = subprocess.run([EXE, "flatten"], capture_output=True, text=True, timeout=120)
+    if r.returncode == 1:
+        assert "omk_forest_create" in r.stderr          # no device: an exception with the library's message, no crash
+    else:
+        assert r.returncode == 0
