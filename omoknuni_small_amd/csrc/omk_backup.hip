@@ -606,12 +606,15 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
                                                   const int32_t *leaf, const uint64_t *node_hash, int64_t n_nodes,
                                                   int64_t n, int min_depth, int32_t *out, TTMeta *meta, uint32_t t0) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    const bool valid = i < n;
     unsigned long long key = kTTEmpty;
-    if (keys) key = keys[i];
-    // a traversal without a leaf finds nothing; never index the forest with an id it does not have
-    else if (leaf[i] >= 0 && leaf[i] < n_nodes) key = node_hash[leaf[i]];
+    if (valid) {
+        if (keys) key = keys[i];
+        // a traversal without a leaf finds nothing; never index the forest with an id it does not have
+        else if (leaf[i] >= 0 && leaf[i] < n_nodes) key = node_hash[leaf[i]];
+    }
     int found = -1;
+    unsigned long long hit_slot = ~0ull;
     if (key != kTTEmpty) {
         uint64_t mask = (1ull << log2_slots) - 1ull;
         uint64_t s = tt_home(key, log2_slots);
@@ -622,14 +625,22 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
             if (k == key) {
                 if ((int)raw.w >= min_depth) {
                     found = (int)raw.z;
-                    if (meta) atomicMax(&meta[s].last_access, t0 + (uint32_t)i);
+                    hit_slot = s;
                 }
                 break;
             }
             if (k == kTTEmpty) break;
         }
     }
-    out[i] = found;
+    if (meta) {
+        // Thousands of traversals can end at one leaf (a crowd that follows one child all the way
+        // down), and atomics on one address are served one by one: of neighbouring lookups of a
+        // wavefront that found the same entry only the last, whose time is the latest, stamps it.
+        const unsigned long long next = __shfl_down(hit_slot, 1);
+        const bool last_of_run = (threadIdx.x & 63u) == 63u || next != hit_slot;
+        if (hit_slot != ~0ull && last_of_run) atomicMax(&meta[hit_slot].last_access, t0 + (uint32_t)i);
+    }
+    if (valid) out[i] = found;
 }
 
 hipError_t launch_tt_clear(TTSlot *slots, TTMeta *meta, int log2_slots, hipStream_t s) {

@@ -2,13 +2,18 @@
 
     python -m omoknuni_small_amd.profile_summary stats  <kernel_stats.csv>
     python -m omoknuni_small_amd.profile_summary pmc    <counter_collection.csv> <COUNTER> [copy_bytes]
+    python -m omoknuni_small_amd.profile_summary counters <counter_collection.csv>
+    python -m omoknuni_small_amd.profile_summary traffic <workload> <fetch.csv> <write.csv> <copy_bytes> <out.json> [command]
     OMK_FOREST_LIB=omoknuni_small_amd/libomk_forest_trace.so \
     python -m omoknuni_small_amd.profile_summary timeline <workload> [warmup_steps [level ...]]
 
 `stats` prints calls / total / average duration per kernel.  `pmc` prints, per kernel, the
 sum of a hardware counter over its dispatches; given the bytes the calibration copy kernel
 (k_copy_words) moved each way per launch, it also prints the counter-to-bytes factor that
-copy implies and every kernel's traffic in bytes scaled by it.  `timeline` runs a benchmark
+copy implies and every kernel's traffic in bytes scaled by it.  `counters` prints every counter of
+the file per kernel, averaged over its dispatches.  `traffic` writes the scaled FETCH_SIZE and
+WRITE_SIZE bytes per launch of the two runs into a JSON file under the workload's name (what
+bench.py quotes as roofline.traffic).  `timeline` runs a benchmark
 workload on the GPU through the measurement build of the library (make -C csrc trace), which records
 when every multi-visitor work item of a selection was processed, and prints the chain of crowded
 nodes of one steady-state selection: per tree level the node with most visitors, when its wavefront
@@ -54,6 +59,57 @@ def pmc(path, counter, copy_bytes=None):
         if factor:
             line += " %16.0f" % (tot[k] / calls[k] * factor)
         print(line)
+
+
+def counters(path):
+    rows = list(csv.DictReader(open(path)))
+    tot = defaultdict(lambda: defaultdict(float))
+    calls = defaultdict(lambda: defaultdict(int))
+    names = []
+    for r in rows:
+        k, c = short(r["Kernel_Name"]), r["Counter_Name"]
+        if c not in names:
+            names.append(c)
+        tot[k][c] += float(r["Counter_Value"])
+        calls[k][c] += 1
+    print("per dispatch, averaged over the kernel's dispatches")
+    print("%-44s %8s " % ("kernel", "calls") + " ".join("%20s" % c for c in names))
+    first = names[0]
+    for k in sorted(tot, key=lambda x: -tot[x][first]):
+        print("%-44s %8d " % (k[:44], calls[k][first]) + " ".join("%20.1f" % (tot[k][c] / max(1, calls[k][c])) for c in names))
+
+
+def scaled_bytes(path, counter, copy_bytes):
+    rows = list(csv.DictReader(open(path)))
+    tot = defaultdict(float)
+    calls = defaultdict(int)
+    for r in rows:
+        if r["Counter_Name"] == counter:
+            tot[short(r["Kernel_Name"])] += float(r["Counter_Value"])
+            calls[short(r["Kernel_Name"])] += 1
+    factor = copy_bytes * calls["k_copy_words"] / tot["k_copy_words"]
+    return {k: int(tot[k] / calls[k] * factor) for k in tot if k.startswith("k_") or "k_select" in k}, factor
+
+
+def traffic(workload, fetch_csv, write_csv, copy_bytes, out_json, command=None):
+    import json
+    import os
+    fetch, f_factor = scaled_bytes(fetch_csv, "FETCH_SIZE", copy_bytes)
+    write, w_factor = scaled_bytes(write_csv, "WRITE_SIZE", copy_bytes)
+    for d in (fetch, write):
+        d.pop("k_copy_words", None)
+    sel = sum(v for d in (fetch, write) for k, v in d.items() if "k_select" in k)
+    doc = json.load(open(out_json)) if os.path.exists(out_json) else {}
+    doc[workload] = {
+        "note": "HBM bytes per launch: FETCH_SIZE and WRITE_SIZE of two rocprofv3 --pmc runs, each scaled by what the "
+                "counter reads for the copy kernel k_copy_words of known size; selection = reset + multi-visitor + "
+                "single-visitor kernels of one step",
+        "command": command or "bench.py --workload %s" % workload,
+        "bytes_per_count": {"FETCH_SIZE": round(f_factor, 2), "WRITE_SIZE": round(w_factor, 2)},
+        "fetch_bytes": fetch, "write_bytes": write, "selection_bytes_per_launch": sel}
+    with open(out_json, "w") as fh:
+        json.dump(doc, fh, indent=1, sort_keys=True)
+    print("%s: selection moves %d bytes per launch (fetch + write of its kernels)" % (workload, sel))
 
 
 def timeline(workload, warmup=8, levels=()):
@@ -144,6 +200,10 @@ if __name__ == "__main__":
         stats(sys.argv[2])
     elif len(sys.argv) >= 4 and sys.argv[1] == "pmc":
         pmc(sys.argv[2], sys.argv[3], int(sys.argv[4]) if len(sys.argv) > 4 else None)
+    elif len(sys.argv) >= 3 and sys.argv[1] == "counters":
+        counters(sys.argv[2])
+    elif len(sys.argv) >= 7 and sys.argv[1] == "traffic":
+        traffic(sys.argv[2], sys.argv[3], sys.argv[4], int(sys.argv[5]), sys.argv[6], sys.argv[7] if len(sys.argv) > 7 else None)
     elif len(sys.argv) >= 3 and sys.argv[1] == "timeline":
         timeline(sys.argv[2], int(sys.argv[3]) if len(sys.argv) > 3 else 8, [int(x) for x in sys.argv[4:]])
     else:
