@@ -634,11 +634,18 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
     }
     if (meta) {
         // Thousands of traversals can end at one leaf (a crowd that follows one child all the way
-        // down), and atomics on one address are served one by one: of neighbouring lookups of a
-        // wavefront that found the same entry only the last, whose time is the latest, stamps it.
-        const unsigned long long next = __shfl_down(hit_slot, 1);
-        const bool last_of_run = (threadIdx.x & 63u) == 63u || next != hit_slot;
-        if (hit_slot != ~0ull && last_of_run) atomicMax(&meta[hit_slot].last_access, t0 + (uint32_t)i);
+        // down; a few hundred distinct leaves for 16384 traversals is typical), and atomics on
+        // one address are served one by one: of the lookups of a wavefront that found the same
+        // entry only the last, whose time is the latest, stamps it.
+        const unsigned lane = threadIdx.x & 63u;
+        unsigned long long todo = __ballot(hit_slot != ~0ull);
+        while (todo) {
+            const int lead = __ffsll((long long)todo) - 1;
+            const unsigned long long s0 = __shfl(hit_slot, lead);
+            const unsigned long long same = __ballot(hit_slot == s0);
+            if (lane == 63u - (unsigned)__clzll((long long)same)) atomicMax(&meta[s0].last_access, t0 + (uint32_t)i);
+            todo &= ~same;
+        }
     }
     if (valid) out[i] = found;
 }
