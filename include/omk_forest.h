@@ -265,7 +265,8 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * [1] of these settled by the parallel paths, [2] visitors settled by them, [3] visitors
  * settled one at a time, [4] nodes replayed one visitor at a time because the parallel
  * path's exactness checks did not hold, [5] threshold probes, [6] single-visitor selection
- * steps, [7] unused, [8..14] per-phase cycle counts in measurement builds (else 0),
+ * steps, [7] nodes settled by merging a few entries of other children into the list of the child
+ * that takes nearly every visitor, [8..14] per-phase cycle counts in measurement builds (else 0),
  * [15] nodes cut into slices for several wavefronts. */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
 /* The counters above cost one atomic per processed node (and per single-visitor step), all on
@@ -276,9 +277,11 @@ int omk_batch_set_stats(omk_batch *b, int32_t enabled);
  * of twelve int64 per multi-visitor work item processed: start and end on the GPU's 100 MHz clock,
  * visitors | depth << 32 | item kind << 60, node | (batches | runs << 8 | entries of the last
  * batch << 16) << 32, then eight words holding two 32-bit phase times each (same clock; slots 0-7:
- * threshold phase, -, evaluation and ordering, emission and checks, loading and scoring the
- * children, the whole settling of the visitors, the partition, -; slots 8-15, parts of these: run
- * probe, bounds and active children, threshold search, exact counts, one-winner check, -, -, -).
+ * threshold phase, direct merge: counts and ranks (or 100 x the reason it was refused), evaluation
+ * and ordering, emission and checks, loading and scoring the children, the whole settling of the
+ * visitors, the partition, direct merge: the dominant child's list; slots 8-15, parts of these:
+ * run probe, bounds and active children, threshold search, exact counts, one-winner check, length
+ * search of a run, emission of a run, the direct merge as a whole).
  * h_trace has room for max_entries records.
  * Only a library built with -DOMK_TRACE (csrc/Makefile, target `trace`) records it; any other
  * build returns OMK_ERR_UNSUPPORTED and *h_n = 0. */

@@ -1698,10 +1698,37 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
 // the score it shows to the last visitor still comes before the first score of every
 // other child and its own scores never increase on the way; both are checked on the exact
 // values (m evaluations spread over the lanes).  Returns false when it is not that case.
+// True when entries 0 .. m-1 of a child never come before their predecessor (m evaluations
+// spread over the lanes), or when the arithmetic proves it beforehand.
+template <int R, bool RAVE>
+__device__ __forceinline__ bool entries_in_order(int bn, float bw, float bp, int bvl, float bq2, float ep, uint32_t uvl,
+                                                 int best, int m, int lane) {
+    if (keys_provably_monotone<RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1)) return true;
+    bool bad = false;
+    uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
+    for (int base = 0; base < m; base += kWave) {
+        const int j = base + lane;
+        uint32_t kk = 0u, pp = 0xFFFFFFFFu;
+        if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, j, best, kk, pp);
+        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+        uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+        if (lane == 0) {
+            pk = carry_k;
+            ppos = carry_p;
+        }
+        if (j < m && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad = true;
+        carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+        carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+    }
+    return __ballot(bad) == 0ull;
+}
+
 template <int R, bool RAVE>
 __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
                                            uint32_t bk, uint32_t bpos, int off, int m, bool to_global, int (&cnt)[R],
-                                           int &run_child) {
+                                           int &run_child, bool &contested, int &best0, uint32_t &lk0, uint32_t &lp0) {
+    // contested: the best child's entry for the last visitor, (lk0, lp0), is real but does not come first
+    contested = false;
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     uint32_t hi_key, hi_pos;
@@ -1742,26 +1769,16 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
     // the last visitor's entry decides; then every entry is checked
     uint32_t lk, lp;
     entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, m - 1, best, lk, lp);
-    if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) return false;
-    bool bad = false;
-    uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
-    // when the order of the child's keys is proven beforehand, the entries in between need no look
-    const bool proven = keys_provably_monotone<RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, m - 1);
-    for (int base = 0; base < m && !proven; base += kWave) {
-        const int j = base + lane;
-        uint32_t kk = 0u, pp = 0xFFFFFFFFu;
-        if (j < m) entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, j, best, kk, pp);
-        uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
-        uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
-        if (lane == 0) {
-            pk = carry_k;
-            ppos = carry_p;
-        }
-        if (j < m && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad = true;
-        carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
-        carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+    if (lk == 0u) return false;
+    if (sk != 0u && !comes_before(lk, lp, sk, spos)) {
+        contested = true;  // other children get a look in: the caller may still find that they are few
+        best0 = best;
+        lk0 = lk;
+        lp0 = lp;
+        return false;
     }
-    if (__ballot(bad) != 0ull) return false;
+    // when the order of the child's keys is proven beforehand, the entries in between need no look
+    if (!entries_in_order<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, best, m, lane)) return false;
     if (to_global) {
         for (int j = lane; j < m; j += kWave) {
             a.sc_child[off + j] = best;
@@ -1774,6 +1791,309 @@ __device__ __forceinline__ bool single_run(const SelectArgs &a, const NodeCtx &c
             if (r == (best >> 6)) cnt[r] = m;
     }
     run_child = best;
+    return true;
+}
+
+// How many of a child's entries 0 .. cap-1 come before the entry (tk, tp), given that the child's
+// keys do not increase (the caller checks the entries it then uses): the closed-form estimate,
+// the two entries around it tested with the exact arithmetic, and a gallop away from it plus a
+// bisection when it is further off.  first_known: entry 0 is known to come before (tk, tp).  On
+// return c: entry c-1 was seen to come before (tk, tp) (or c == 0, or c == 1 with first_known),
+// entry c was seen not to (or c == cap).
+template <int R, bool RAVE>
+__device__ __forceinline__ int count_before(int n, float w, float p, int vl, float q2, float ep, uint32_t uvl,
+                                            int child, uint32_t tk, uint32_t tp, int cap, bool first_known) {
+    uint32_t kk, pp;
+    if (!first_known) {
+        entry_key<R, RAVE>(n, w, p, vl, q2, ep, uvl, 0, child, kk, pp);
+        if (!(kk != 0u && comes_before(kk, pp, tk, tp))) return 0;
+    }
+    int lo_c = 1, hi_c = cap;
+    if (hi_c < lo_c) return lo_c;
+    int g = predict_count<RAVE>(n, w, p, vl, q2, ep, uvl, key_score(tk), cap);
+    g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
+    if (g > lo_c) {
+        entry_key<R, RAVE>(n, w, p, vl, q2, ep, uvl, g - 1, child, kk, pp);
+        if (kk != 0u && comes_before(kk, pp, tk, tp)) lo_c = g;
+        else hi_c = g - 1;
+    }
+    if (lo_c == g && g < hi_c) {
+        entry_key<R, RAVE>(n, w, p, vl, q2, ep, uvl, g, child, kk, pp);
+        if (kk != 0u && comes_before(kk, pp, tk, tp)) lo_c = g + 1;
+        else hi_c = g;
+    }
+    if (lo_c < hi_c) {
+        const bool up = lo_c > g;
+        for (int step = 2; lo_c < hi_c; step <<= 1) {
+            int t = up ? lo_c + step : hi_c - step + 1;
+            t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+            entry_key<R, RAVE>(n, w, p, vl, q2, ep, uvl, t - 1, child, kk, pp);
+            const bool before = kk != 0u && comes_before(kk, pp, tk, tp);
+            if (before) lo_c = t;
+            else hi_c = t - 1;
+            if (before != up) break;
+        }
+    }
+    while (lo_c < hi_c) {
+        const int t = (lo_c + hi_c + 1) >> 1;
+        entry_key<R, RAVE>(n, w, p, vl, q2, ep, uvl, t - 1, child, kk, pp);
+        if (kk != 0u && comes_before(kk, pp, tk, tp)) lo_c = t;
+        else hi_c = t - 1;
+    }
+    return lo_c;
+}
+
+constexpr int kSparseMax = 64;  // entries of other children a nearly-one-winner node may hold (one per lane)
+constexpr int kSparseMin = 8;    // visitors from which that direct merge is tried
+static_assert(2 * kHeavyMin <= kBatchCap, "the (key, position) list of the dominant child fits one sort buffer");
+
+#ifdef OMK_TRACE
+// timeline build: why a direct merge was refused (shown in place of a time, in units of 1 us)
+#define OMK_MERGE_FAIL(code)                           \
+    do {                                               \
+        if (lane == 0) lds.tph[1] = 100u * (code);     \
+        return false;                                  \
+    } while (0)
+#else
+#define OMK_MERGE_FAIL(code) return false
+#endif
+
+// A node where one child wins ALMOST every time: the winner order is that child's list with
+// a few entries of other children merged in.  The child, A, is the one that holds out longest,
+// the one with the best entry (lk, lp) for the node's LAST visitor (not always the one with the
+// best next entry: a child whose score is mostly exploration starts high and drops at once).
+// Only a child whose next entry comes before the last-visitor entry (lk0, lp0) of the child
+// with the best next entry can be A or get an entry in (A's last entry is at or before that
+// one), so these few are listed one per lane first.  Every other child's entries that can get
+// in come before (lk, lp); when there are at most 64 of them in all, each finds its place
+// directly: the number of A's entries that come before it (a bisection on A's list, evaluated
+// once into LDS) plus the number of such entries of other children that do.  No threshold
+// search, no sort.  Exactness rests on: A's entries 0 .. m-1 in order (checked one by one);
+// every other child's used entries in order and its first unused one either not before
+// (lk, lp) (count_before brackets the count by two exact evaluations) or looked at and placed
+// behind the m-th winner (checked).  Then the best head at any step is never one of the heads
+// left out, and merging the lists by (key, position) is the serial order.
+// On success: order[q] = (child << 21) | visit number for the m visitors, cnt[] the visits
+// per child.  On failure nothing the caller relies on has changed (order[] is scratch).
+template <int R, bool RAVE>
+__device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
+                                             int best0, uint32_t lk0, uint32_t lp0, int m, WaveLds<R> &lds,
+                                             uint32_t *order, int (&cnt)[R], bool &pending) {
+    constexpr int F = R * kWave;
+    const uint32_t uvl = (uint32_t)a.vl;
+    OMK_S0();
+    // ---- the children that matter, one per lane ----
+    int n0 = 0;
+    bool listed[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        uint32_t hk = k.k1[r], hp = (uint32_t)i;
+        if (k.k2[r] > k.k1[r]) {
+            hk = k.k2[r];
+            hp = (uint32_t)(F + i);
+        }
+        listed[r] = hk != 0u && (i == best0 || comes_before(hk, hp, lk0, lp0));
+        const uint64_t cm = __ballot(listed[r]);
+        if (listed[r]) {
+            const int cl = n0 + __popcll(cm & ((1ull << lane) - 1ull));
+            if (cl < kSparseMax) {
+                lds.st_j0[cl] = i;
+                lds.st_n[cl] = k.n[r];
+                lds.st_w[cl] = k.w[r];
+                lds.st_p[cl] = k.p[r];
+                lds.st_vl[cl] = k.vl[r];
+                lds.st_q2[cl] = k.q2[r];
+            }
+        }
+        n0 += __popcll(cm);
+    }
+    if (n0 < 2 || n0 > kSparseMax) OMK_MERGE_FAIL(1);
+    wave_sync_memory();
+    int ci = -1, cn = 0, cvl = 0;
+    float cw = 0.0f, cp = 0.0f, cq2 = 0.0f;
+    uint32_t hk = 0u, hp = 0xFFFFFFFFu, zk = 0u, zp = 0xFFFFFFFFu;  // the child's next entry and its last-visitor entry
+    if (lane < n0) {
+        ci = lds.st_j0[lane];
+        cn = lds.st_n[lane];
+        cw = lds.st_w[lane];
+        cp = lds.st_p[lane];
+        cvl = lds.st_vl[lane];
+        cq2 = lds.st_q2[lane];
+        entry_key<R, RAVE>(cn, cw, cp, cvl, cq2, c.ep, uvl, 0, ci, hk, hp);
+        entry_key<R, RAVE>(cn, cw, cp, cvl, cq2, c.ep, uvl, m - 1, ci, zk, zp);
+    }
+    // ---- A: the child that holds out longest ----
+    uint32_t lk, lp;
+    wave_best(zk, zp, lk, lp);
+    if (lk == 0u) OMK_MERGE_FAIL(7);
+    const uint64_t am = __ballot(lane < n0 && zk == lk && zp == lp);
+    if (am == 0ull) OMK_MERGE_FAIL(8);
+    const int a_lane = __ffsll((long long)am) - 1;
+    const int a_child = __builtin_amdgcn_readlane(ci, a_lane);
+    const int a_n = __builtin_amdgcn_readlane(cn, a_lane);
+    const int a_vl = __builtin_amdgcn_readlane(cvl, a_lane);
+    const float a_w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cw), a_lane));
+    const float a_p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cp), a_lane));
+    const float a_q2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cq2), a_lane));
+    // ---- the others that can get an entry in: next entry before (lk, lp) ----
+    const bool is_cand = lane < n0 && lane != a_lane && hk != 0u && comes_before(hk, hp, lk, lp);
+    if (__ballot(is_cand) == 0ull) OMK_MERGE_FAIL(9);
+    {
+        // Far too many entries by the estimates: leave before anything exact is paid for.  An entry
+        // of a child gets in only if fewer than m entries come before it; the child's next entry has
+        // r0 of A's entries before it, so its entry number t has at least r0 + t, and no more than
+        // m - r0 of its entries can get in, however many come before (lk, lp) (two children whose
+        // scores hardly move with virtual loss, a RAVE blend that dominates both, can have hundreds
+        // there and still only meet at the very end).
+        int est = 0;
+        if (is_cand) {
+            const int r0 = predict_count<RAVE>(a_n, a_w, a_p, a_vl, a_q2, c.ep, uvl, key_score(hk), m);
+            const int room = m - r0 > 1 ? m - r0 : 1;
+            est = predict_count<RAVE>(cn, cw, cp, cvl, cq2, c.ep, uvl, key_score(lk), kSparseMax + 1);
+            est = est < room ? est : room;
+        }
+        if (wave_sum_i32(est) > kSparseMax + 8) OMK_MERGE_FAIL(2);
+    }
+    // ---- A's entries, all m of them, evaluated once into LDS and checked: none may come before its
+    // predecessor (its head then stays at or before (lk, lp) throughout) ----
+    // as one 64-bit number per entry, smaller = played earlier: inverted key above the position
+    unsigned long long *akp = reinterpret_cast<unsigned long long *>(lds.key[0]);  // m < kHeavyMin = kBatchCap / 2 entries
+    {
+        bool bad_a = false;
+        uint32_t carry_k = 0xFFFFFFFFu, carry_p = 0u;  // entry before the chunk
+        for (int base = 0; base < m; base += kWave) {
+            const int j = base + lane;
+            uint32_t kk = 0u, pp = 0xFFFFFFFFu;
+            if (j < m) {
+                entry_key<R, RAVE>(a_n, a_w, a_p, a_vl, a_q2, c.ep, uvl, j, a_child, kk, pp);
+                akp[j] = ((unsigned long long)~kk << 32) | pp;
+            }
+            uint32_t pk = (uint32_t)__shfl_up((int)kk, 1, kWave);
+            uint32_t ppos = (uint32_t)__shfl_up((int)pp, 1, kWave);
+            if (lane == 0) {
+                pk = carry_k;
+                ppos = carry_p;
+            }
+            if (j < m && (kk == 0u || comes_before(kk, pp, pk, ppos))) bad_a = true;
+            carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
+            carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
+        }
+        if (__ballot(bad_a) != 0ull) OMK_MERGE_FAIL(5);
+    }
+    wave_sync_memory();
+    OMK_STAMP(7);
+    // how many of A's entries come before the entry (tk, tp): the list is in order, so a bisection
+    // on the exact keys
+    auto rank_in_a = [&](uint32_t tk, uint32_t tp) {
+        const unsigned long long t64 = ((unsigned long long)~tk << 32) | tp;
+        int lo = 0, hi = m;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (akp[mid] < t64) lo = mid + 1;
+            else hi = mid;
+        }
+        return lo;
+    };
+    // ---- how many entries each of the others has before (lk, lp), at most m - r0 (see above) ----
+    int cc = 0, cap = 1;
+    if (is_cand) {
+        cap = m - rank_in_a(hk, hp);  // at least 1: A's last entry does not come before this one
+        if (cap > kSparseMax + 1) cap = kSparseMax + 1;
+        if (cap < 1) cap = 1;
+        cc = count_before<R, RAVE>(cn, cw, cp, cvl, cq2, c.ep, uvl, ci, lk, lp, cap, true);
+    }
+    const int inc = wave_inclusive_sum(cc, lane);
+    const int total = __builtin_amdgcn_readlane(inc, 63);
+    if (total > kSparseMax) OMK_MERGE_FAIL(3);
+    const int start = inc - cc;
+    // ---- one lane per entry: (lane of its child, visit number) ----
+    for (int t = 0; t < cc; t++) lds.hist[start + t] = lane | (t << 8);  // start + cc <= total <= 64
+    wave_sync_memory();
+    int bad = 0;  // why the merge is refused (the number only matters to the timeline build)
+    uint32_t ek = 0u, epos = 0xFFFFFFFFu;
+    int e_child = -1, e_t = 0, rank_a = m;
+    if (lane < total) {
+        const uint32_t w0 = (uint32_t)lds.hist[lane];
+        const int e_cl = (int)(w0 & 255u);
+        e_t = (int)(w0 >> 8);
+        e_child = lds.st_j0[e_cl];
+        entry_key<R, RAVE>(lds.st_n[e_cl], lds.st_w[e_cl], lds.st_p[e_cl], lds.st_vl[e_cl], lds.st_q2[e_cl], c.ep, uvl,
+                           e_t, e_child, ek, epos);
+        if (ek == 0u) bad = 1;
+        rank_a = rank_in_a(ek, epos);
+    }
+    {
+        // a child's entries sit in neighbouring lanes, in visit order: none may come before its predecessor
+        const uint32_t pk = (uint32_t)__shfl_up((int)ek, 1, kWave);
+        const uint32_t pp = (uint32_t)__shfl_up((int)epos, 1, kWave);
+        if (lane < total && e_t > 0 && comes_before(ek, epos, pk, pp)) bad = 2;
+    }
+    // ---- the other entries before each of them (equal keys at one position: one child, visit order) ----
+    // as 64-bit numbers again, with the lane below the position: all different, a child's entries in visit order
+    unsigned long long *ekp = reinterpret_cast<unsigned long long *>(lds.key[1]);  // all lanes read all entries: through LDS
+    const unsigned long long e64 =
+        lane < total ? ((unsigned long long)~ek << 32) | ((unsigned long long)epos << 8) | (unsigned)lane : ~0ull;
+    ekp[lane] = e64;
+    wave_sync_memory();
+    int fr = 0;
+    // (eight reads in flight at a time: one wavefront alone waits out every LDS access it depends on)
+    for (int e0 = 0; e0 < total; e0 += 8) {
+        unsigned long long o[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) o[u] = ekp[e0 + u];  // lanes past `total` hold the largest number: before nothing
+#pragma unroll
+        for (int u = 0; u < 8; u++) fr += o[u] < e64 ? 1 : 0;
+    }
+    const int posn = rank_a + fr;
+    const bool valid = lane < total && posn < m;
+    {
+        // of a child's entries the ones that get in are the first ones
+        const int pv = __shfl_up(valid ? 1 : 0, 1, kWave);
+        if (valid && e_t > 0 && pv == 0) bad = 3;
+    }
+    const uint64_t vmask = __ballot(valid);
+    const int nfv = __popcll(vmask);
+    int mine_in = 0;  // entries of this lane's child that get in
+    if (is_cand) {
+        const uint64_t mine = cc >= 64 ? ~0ull : ((1ull << cc) - 1ull);
+        mine_in = __popcll((vmask >> start) & mine);
+        // a child all of whose counted entries get in, counted up to its limit: its next entry was
+        // not looked at
+        if (mine_in == cc && cc == cap) bad = 4;
+    }
+    {
+        const int why = (int)wave_max_u32((uint32_t)bad);
+        if (why != 0) OMK_MERGE_FAIL(40 + why);
+    }
+    OMK_STAMP(1);
+    // ---- the winner order: the others' entries at their places, A's in between ----
+    close_pending(pending);  // the previous node's partition may still read the order buffer
+    for (int q = lane; q < m; q += kWave) order[q] = 0u;
+    wave_sync_memory();
+    if (valid) order[posn] = 0x80000000u | ((uint32_t)e_child << 21) | (uint32_t)e_t;
+    wave_sync_memory();
+    int seen = 0;
+    for (int base = 0; base < m; base += kWave) {
+        const int q = base + lane;
+        const uint32_t v = q < m ? order[q] : 0u;
+        const bool other = (v >> 31) != 0u;
+        const uint64_t om = __ballot(other);
+        const int below = seen + __popcll(om & ((1ull << lane) - 1ull));
+        if (q < m) order[q] = other ? (v & 0x7FFFFFFFu) : (((uint32_t)a_child << 21) | (uint32_t)(q - below));
+        seen += __popcll(om);
+    }
+    if (seen != nfv) OMK_MERGE_FAIL(6);  // two entries at one place: cannot happen when the checks hold
+    // ---- visits per child, back to the lanes that hold the children ----
+    if (lane < n0) lds.hist[kSparseMax + lane] = lane == a_lane ? m - nfv : mine_in;
+    wave_sync_memory();
+    int cl_run = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint64_t cm = __ballot(listed[r]);
+        cnt[r] = listed[r] ? lds.hist[kSparseMax + cl_run + __popcll(cm & ((1ull << lane) - 1ull))] : 0;
+        cl_run += __popcll(cm);
+    }
     return true;
 }
 
@@ -1875,9 +2195,26 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         settled = true;
     }
     OMK_S0();
+    bool contested = false;
+    int best0 = -1;
+    uint32_t lk0 = 0u, lp0 = 0xFFFFFFFFu;
     if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
-        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child);
+        settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child, contested, best0,
+                                      lk0, lp0);
     OMK_STAMP(12);
+    if (!settled && contested && m >= kSparseMin && m < kHeavyMin) {
+        settled = sparse_merge<R, RAVE>(a, c, lane, k, best0, lk0, lp0, m, lds, pl.order, cnt, pending);
+        if (settled) {
+            lds_cur = 0;
+#ifndef OMK_PHASE_TIMERS
+            if (a.stats && lane == 0) atomicAdd(a.stats + 7, 1);
+#endif
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; r++) cnt[r] = 0;
+        }
+        OMK_STAMP(15);
+    }
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first

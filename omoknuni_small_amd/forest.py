@@ -398,7 +398,7 @@ class Batch:
         out = np.zeros(16, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
-                "replayed_nodes", "threshold_probes", "single_visitor_steps", "fail_code", "cyc_threshold",
+                "replayed_nodes", "threshold_probes", "single_visitor_steps", "merged_nodes", "cyc_threshold",
                 "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "sliced_nodes")
         return dict(zip(keys, map(int, out)))
 

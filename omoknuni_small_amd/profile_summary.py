@@ -151,10 +151,11 @@ def timeline(workload, warmup=8, levels=()):
           "scored, thr = threshold search and exact counts, ord = entries evaluated and put in order, emit = "
           "emission and checks, settle = all of the settling (includes thr, ord, emit), part = partition or its "
           "hand-over; parts of thr (and of the thresholds a slice derives): probe = run probe, act = bounds and "
-          "active children, srch = threshold search, cnt = exact counts; 1win = the one-winner check; runL / runW = length search and emission of runs of one child")
-    print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s %5s %5s  %s" % (
+          "active children, srch = threshold search, cnt = exact counts; 1win = the one-winner check; runL / runW = length search and emission of runs of one child; "
+          "mrg = the direct merge of a node where one child wins nearly every time (or the failed attempt at it)")
+    print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s %5s %5s %5s  %s" % (
         "level", "node", "visitors", "kind", "start_us", "end_us", "us", "load", "thr", "ord", "emit", "settle", "part",
-        "probe", "act", "srch", "cnt", "1win", "runL", "runW", "work"))
+        "probe", "act", "srch", "cnt", "1win", "runL", "runW", "mrg", "work"))
     names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
@@ -177,9 +178,9 @@ def timeline(workload, warmup=8, levels=()):
             same = same[kind[same] != 4]
             s0, e1 = start[same].min(), end[same].max()
         p = ph[same].sum(axis=0)
-        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
+        print("%5d %9d %9d %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %s" % (
             d, node[top], m[top], names.get(int(kind[first]), "?"), s0, e1, e1 - s0, p[4], p[0], p[2], p[3], p[5], p[6],
-            p[8], p[9], p[10], p[11], p[12], p[13], p[14], work))
+            p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15], work))
     for lv in levels:
         at = np.nonzero(depth == lv)[0]
         top = at[np.argmax(m[at])]
@@ -188,9 +189,39 @@ def timeline(workload, warmup=8, levels=()):
         print("items of node %d at level %d (slice / part number of a heavy node in `work`):" % (node[top], lv))
         for i in same:
             c = int(ctr[i])
-            print("  %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %d batch(es), %d run(s), last batch %d entries"
+            print("  %7s %9.1f %9.1f %8.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f | %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f %5.1f  %d batch(es), %d run(s), last batch %d entries"
                   % (names.get(int(kind[i]), "?"), start[i], end[i], end[i] - start[i], ph[i, 4], ph[i, 0], ph[i, 2], ph[i, 3],
-                     ph[i, 5], ph[i, 6], ph[i, 8], ph[i, 9], ph[i, 10], ph[i, 11], ph[i, 12], ph[i, 13], ph[i, 14], c & 0xFF, (c >> 8) & 0xFF, c >> 16))
+                     ph[i, 5], ph[i, 6], ph[i, 8], ph[i, 9], ph[i, 10], ph[i, 11], ph[i, 12], ph[i, 13], ph[i, 14], ph[i, 15], c & 0xFF, (c >> 8) & 0xFF, c >> 16))
+    # the critical path: the item that ended last, and the nodes above it up to the root
+    cb, cc = soa["child_begin"].astype(np.int64), soa["child_count"].astype(np.int64)
+    parent = np.full(len(cb), -1, np.int64)
+    has = np.nonzero(cc > 0)[0]
+    parent[np.repeat(cb[has], cc[has]) + (np.arange(int(cc[has].sum())) - np.repeat(np.cumsum(cc[has]) - cc[has], cc[has]))] = \
+        np.repeat(has, cc[has])
+    chain = []
+    n_at = int(node[np.argmax(end)])
+    while n_at >= 0:
+        chain.append(n_at)
+        n_at = int(parent[n_at])
+    print("critical path: the node whose item ended last (%.1f us) and its ancestors" % end.max())
+    print("(mrg = the direct merge or the attempt at it: m.list = the dominant child chosen, its entries evaluated and "
+          "checked; m.rank = counts and ranks of the other children's entries, or, times 1 us, why the merge was "
+          "refused: 1 too many children in question, 2 too many entries by the estimate, 3 too many entries, 5 the "
+          "dominant child's scores rise, 4x / 6-9 a check failed; the rest of mrg is writing the order)")
+    print("%5s %9s %9s %9s %9s %8s %9s | %6s %6s %6s %6s %6s %6s %6s %6s %6s %6s" % (
+        "level", "node", "visitors", "start_us", "end_us", "us", "gap_us", "load", "1win", "mrg", "m.list", "m.rank",
+        "thr", "ord", "emit", "settle", "part"))
+    prev_end = 0.0
+    for n_at in reversed(chain):
+        same = np.nonzero(node == n_at)[0]
+        if len(same) == 0:
+            continue
+        s0, e1 = start[same].min(), end[same].max()
+        p = ph[same].sum(axis=0)
+        print("%5d %9d %9d %9.1f %9.1f %8.1f %9.1f | %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f %6.1f" % (
+            depth[same[0]], n_at, m[same].max(), s0, e1, e1 - s0, s0 - prev_end, p[4], p[12], p[15], p[7], p[1],
+            p[0], p[2], p[3], p[5], p[6]))
+        prev_end = e1
     by_kind = ", ".join("%s %d" % (names[k], int((kind == k).sum())) for k in sorted(names))
     print("items by kind: %s; visitors per item: median %d, largest %d" % (by_kind, int(np.median(m)), int(m.max())))
 

@@ -185,3 +185,20 @@ def test_proof_of_non_increasing_keys_against_brute_force(tmp_path):
     m = re.search(r"provably monotone: (\d+) without RAVE, (\d+) with; counter-examples 0", out.stdout)
     assert m, out.stdout[-500:]
     assert int(m.group(1)) > 100000 and int(m.group(2)) > 100000
+
+
+def test_direct_merge_rule_against_the_serial_loop(tmp_path):
+    """The rule by which the selection kernel settles a node where one child takes nearly every
+    visitor (merge the few entries of the others into that child's list by rank: no threshold search,
+    no sort), restated step by step on the host with the kernel's own score arithmetic
+    (tests/cpp/merge_check.cpp): every node it accepts must come out as the serial loop plays it."""
+    import re
+    import subprocess
+    exe = str(tmp_path / "merge_check")
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-fno-fast-math", "-I",
+                           os.path.join(ROOT, "omoknuni_small_amd", "csrc"),
+                           os.path.join(ROOT, "tests", "cpp", "merge_check.cpp"), "-o", exe])
+    out = subprocess.run([exe, "60000", "7"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stdout[-2000:]
+    m = re.search(r"merged: (\d+); wrong 0;", out.stdout)
+    assert m and int(m.group(1)) > 30000, out.stdout[-500:]

@@ -45,7 +45,7 @@ def test_random_forests_and_crowds(seed):
             tr = np.sort(rng.integers(0, len(roots), B)).astype(np.int32)
             st = select_both(soa, roots[tr], 3, steps=2)
         if st["replayed_nodes"]:
-            replayed.append((case, kind, st["replayed_nodes"], st["group_nodes"], st.get("fail_code")))
+            replayed.append((case, kind, st["replayed_nodes"], st["group_nodes"], st.get("merged_nodes")))
     # a node whose checks fail is replayed one visitor at a time: allowed (the results above are
     # exact either way), but it must stay the exception
     print("replayed:", replayed)

@@ -79,7 +79,8 @@ def select_both(soa, troots, D, vl=3, rave=False, rave_k=1000.0, steps=2):
         assert len(bad) == 0, "step %d: %d paths differ, first traversal %d (near ties flagged: %d)" % (
             step, len(bad), bad[0], int((near >= 0).sum()))
         assert (f.download()["VL"] == ref.VL).all()
-        stats = b.stats()
+        step_stats = b.stats()
+        stats = step_stats if stats is None else {k: stats[k] + v for k, v in step_stats.items()}  # over all steps
         values = rng.uniform(-1, 1, len(troots)).astype(np.float32)
         ref.backup_batch(rpaths, rlen, values, vl)
         b.set_values(values)
@@ -219,3 +220,74 @@ def test_long_chains_of_crowded_nodes(dominate, fan, B):
     soa = chain_forest(11, 40, fan, dominate)
     st = select_both(soa, np.zeros(B, np.int32), 50, steps=3)
     assert st["replayed_nodes"] == 0, st
+
+
+def dominated_forest(seed, fan, depth, rave, kind, visitors):
+    """A chain of nodes in each of which ONE child takes nearly every visitor and a few others get a
+    visit or two in between.  The dominant child scores 0.9 and loses about 1.1e-4 per visit; the
+    rivals' first scores are placed in the band it sweeps with `visitors` visits.  kind "few" =
+    rivals with few visits (one entry each gets in), "some" = rivals that hold out for several
+    entries, "late" = a child whose score is mostly exploration shows the best first score of all
+    and drops at once, "plateau" (RAVE) = rivals whose blended score hardly moves with virtual loss
+    and that meet the dominant child near the end."""
+    rng = np.random.default_rng(seed)
+    N, W, P, cb, cc, act, rN, rW = ([] for _ in range(8))
+
+    def add(n, w, p, a, rn=0, rw=0.0):
+        N.append(int(n)); W.append(float(w)); P.append(float(p)); cb.append(0); cc.append(0); act.append(a)
+        rN.append(int(rn)); rW.append(float(rw))
+        return len(N) - 1
+
+    node = add(60_000, 0.0, 0.0, -1)
+    for level in range(depth):
+        ep = 1.4 * np.sqrt(N[node])
+        cb[node] = len(N)
+        cc[node] = fan
+        dom = int(rng.integers(fan))
+        kids = []
+        for i in range(fan):
+            n = int(rng.integers(5, 60))
+            q = rng.uniform(-0.2, 0.5)
+            rn = int(rng.integers(0, 30))
+            kids.append(add(n, q * n, rng.uniform(1e-5, 2e-4), i, rn, rng.uniform(-0.5, 0.3) * rn))
+        c = kids[dom]
+        N[c] = 50_000; W[c] = 0.9 * 50_000; P[c] = 0.01; rN[c] = 600; rW[c] = 0.5 * 600
+        swept = 1.1e-4 * visitors  # what the dominant child's score loses over the visits
+        rivals = [k for k in rng.permutation(fan) if k != dom][:4]
+        for j, k in enumerate(rivals):
+            r = kids[k]
+            target = 0.9 - swept * rng.uniform(0.1, 0.95)  # first score inside the band
+            if kind == "late" and j == 0:
+                N[r] = 3; W[r] = 1.0; P[r] = (0.97 - 1.0 / 3) * 4 / ep
+            elif kind == "plateau" and j < 2:
+                n, rn, rave_value = 40_000, 500, 0.45
+                beta = np.sqrt(1000.0 / (3 * n + 1000.0))
+                N[r] = n; W[r] = (target - beta * rave_value) / (1 - beta) * n; P[r] = 1e-6; rN[r] = rn; rW[r] = rave_value * rn
+            elif kind == "some":
+                N[r] = 3000; W[r] = 0.85 * 3000; P[r] = (target - 0.85) * 3001 / ep
+            else:
+                N[r] = 30; W[r] = 0.6 * 30; P[r] = (target - 0.6) * 31 / ep
+        node = c
+    soa = dict(N=np.array(N, np.int32), W=np.array(W, np.float32), P=np.array(P, np.float32),
+               VL=np.zeros(len(N), np.int32), child_begin=np.array(cb, np.int32), child_count=np.array(cc, np.int32),
+               action=np.array(act, np.int32))
+    if rave:
+        soa["rN"] = np.array(rN, np.int32)
+        soa["rW"] = np.array(rW, np.float32)
+    return soa
+
+
+@pytest.mark.parametrize("visitors", [9, 40, 200, 900])
+@pytest.mark.parametrize("fan,rave,kind", [(40, False, "few"), (40, False, "some"), (40, False, "late"),
+                                           (362, True, "few"), (362, True, "late"), (362, True, "plateau"),
+                                           (150, True, "plateau"), (150, True, "some")])
+def test_one_child_takes_nearly_every_visitor(visitors, fan, rave, kind):
+    """Nodes settled by merging the few entries of other children into the dominant child's list
+    (no threshold search, no sort) give the serial order, for every way such a node comes about."""
+    soa = dominated_forest(100 + visitors + fan, fan, 6, rave, kind, visitors)
+    st = select_both(soa, np.zeros(visitors, np.int32), 8, rave=rave, steps=3)
+    assert st["replayed_nodes"] == 0, st
+    # (with plateau rivals the child that holds out longest takes over for good near the end, and
+    # everything before that is "other children's entries": merged only while those are few)
+    if kind != "plateau" or visitors <= 40:
+        assert st["merged_nodes"] >= 1, st
