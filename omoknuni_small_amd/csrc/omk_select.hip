@@ -1953,7 +1953,9 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
             est = predict_count<RAVE>(cn, cw, cp, cvl, cq2, c.ep, uvl, key_score(lk), kSparseMax + 1);
             est = est < room ? est : room;
         }
-        if (wave_sum_i32(est) > kSparseMax + 8) OMK_MERGE_FAIL(2);
+        // (a little below the capacity: the exact counts tend to come out above the estimates, and
+        // a refusal after them costs three times what one here does)
+        if (wave_sum_i32(est) > kSparseMax - 4) OMK_MERGE_FAIL(2);
     }
     // ---- A's entries, all m of them, evaluated once into LDS and checked: none may come before its
     // predecessor (its head then stays at or before (lk, lp) throughout) ----

@@ -152,7 +152,7 @@ static bool sparse_merge(const std::vector<Kid> &k, float ep, uint32_t uvl, int 
             const int room = m - r0 > 1 ? m - r0 : 1;
             est_sum += std::min(predict_count(k[L[l]], ep, uvl, key_score(lk), kSparseMax + 1), room);
         }
-    if (est_sum > kSparseMax + 8) return refusal = 2, false;
+    if (est_sum > kSparseMax - 4) return refusal = 2, false;
     std::vector<unsigned long long> akp(m);
     {
         uint32_t pk = 0xFFFFFFFFu, ppos = 0;
