@@ -319,6 +319,15 @@ typedef struct omk_tt_slot {
 int omk_batch_leaf_keys(omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
                         const uint64_t *d_root_keys, const int32_t *d_root_players, uint64_t *d_out);
 
+/* Position keys of single nodes: hash[h_nodes[i]] = h_keys[i] (host arrays).  For a game whose keys cannot
+ * be folded from the move list (captures: Go), the keys are the game's own: the caller has the state of
+ * every leaf it evaluates (the clone with the moves replayed, mcts_engine_batch_tree_simple.cpp:170-178)
+ * and passes state->getHash() (include/core/igamestate.h) for the leaf's node.  A forest uploaded without
+ * keys gets the array on the first call; a node that has no key yet (all of them then, and every node that
+ * omk_expand_batch* adds) carries the key ~0, which the table neither stores nor finds.  Waits for the
+ * stream. */
+int omk_forest_set_keys(omk_forest *f, const int32_t *h_nodes, const uint64_t *h_keys, int64_t n);
+
 int omk_tt_create(omk_forest *f, int32_t log2_slots, omk_tt **out);
 int omk_tt_destroy(omk_tt *tt);
 int omk_tt_clear(omk_tt *tt);
@@ -350,7 +359,7 @@ int omk_tt_set_replacement_threshold(omk_tt *tt, float threshold);
  * is looked up, and a node OTHER than the selected one that has visits is a transposition
  * (:141-142).  The reference then swaps the child pointer of the parent for that node (:143-156),
  * which turns the tree into a graph; this library reports the transposition and leaves the tree
- * alone: d_hits (NULL or device memory for n_traversals * max_depth ints, entry t * max_depth + d - 1
+ * alone: d_hits (NULL when only the counts are wanted, or device memory for n_traversals * max_depth ints, entry t * max_depth + d - 1
  * for step d of traversal t) receives that node or -1.  Keys: with d_piece_keys the game's Zobrist
  * tables as in omk_batch_leaf_keys (stone-placing games), with NULL the forest's per-node keys
  * (omk_soa_view.hash).  h_counts (NULL or [4]): new entries, replacements, duplicates within the

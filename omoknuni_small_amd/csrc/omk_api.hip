@@ -400,6 +400,40 @@ int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_chi
     return OMK_OK;
 }
 
+int omk_forest_set_keys(omk_forest *f, const int32_t *h_nodes, const uint64_t *h_keys, int64_t n) {
+    if (!f || (n > 0 && (!h_nodes || !h_keys))) return fail(OMK_ERR_INVALID, "omk_forest_set_keys: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_set_keys: nothing uploaded");
+    if (n < 0) return fail(OMK_ERR_INVALID, "omk_forest_set_keys: n = %lld", (long long)n);
+    if (int rc = use_device(f)) return rc;
+    hipStream_t s = f->stream;
+    if (!f->has_hash) {
+        // a forest that came without position keys: every node starts with "no key"
+        if (!f->hash) HIP_TRY(dalloc(&f->hash, f->capacity));
+        HIP_TRY(launch_fill_words(f->hash, 0xFFFFFFFFu, f->capacity * 2, s));
+        f->has_hash = true;
+    }
+    if (n == 0) return OMK_OK;
+    int32_t *d_nodes = nullptr;
+    uint64_t *d_keys = nullptr;
+    int *d_bad = nullptr;
+    hipError_t e = dalloc(&d_nodes, n);
+    if (e == hipSuccess) e = dalloc(&d_keys, n);
+    if (e == hipSuccess) e = dalloc(&d_bad, 1);
+    int bad = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(d_nodes, h_nodes, (size_t)n * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_keys, h_keys, (size_t)n * 8, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(d_bad, &bad, 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = launch_set_keys(f->hash, d_nodes, d_keys, n, f->n_nodes, d_bad, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(&bad, d_bad, 4, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (d_nodes) (void)hipFree(d_nodes);
+    if (d_keys) (void)hipFree(d_keys);
+    if (d_bad) (void)hipFree(d_bad);
+    if (e != hipSuccess) return fail(OMK_ERR_HIP, "omk_forest_set_keys: %s", hipGetErrorString(e));
+    if (bad) return fail(OMK_ERR_INVALID, "omk_forest_set_keys: %d node ids outside the forest (skipped)", bad);
+    return OMK_OK;
+}
+
 int omk_forest_add_root_noise(omk_forest *f, int32_t root, const float *h_gamma, int32_t n_gamma, float epsilon) {
     if (!f || !h_gamma) return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: null argument");
     if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_add_root_noise: nothing uploaded");
@@ -1443,7 +1477,7 @@ int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int3
     tt->clock += (uint32_t)n;
     HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, keys, nullptr, nullptr, 0, n, 0, found, tt->meta, tt->clock, s));
     tt->clock += (uint32_t)n;
-    if (d_hits) HIP_TRY(launch_tt_hits(f->dev(), step_nodes, found, n, d_hits, tt->d_status, s));
+    HIP_TRY(launch_tt_hits(f->dev(), step_nodes, found, n, d_hits, tt->d_status, s));
     HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     if (status[5])

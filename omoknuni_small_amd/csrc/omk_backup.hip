@@ -202,7 +202,7 @@ __global__ __launch_bounds__(64) void k_expand(ForestMut f, const ExpandJob *job
         if (f.rW) f.rW[id] = 0.0f;
         f.span[id] = int2{0, 0};
         if (f.action) f.action[id] = moves[job.off + i];
-        if (f.hash) f.hash[id] = 0ull;
+        if (f.hash) f.hash[id] = ~0ull;  // no position key yet (omk_forest_set_keys)
         if (f.legal && fresh) atomicOr(f.legal + ((uint32_t)id >> 5), 1u << ((uint32_t)id & 31u));
     }
     __syncthreads();
@@ -551,7 +551,7 @@ __global__ __launch_bounds__(256) void k_tt_hits(ForestDev f, const int32_t *ste
     const int fn = found[i], node = step_nodes[i];
     int out = -1;
     if (node >= 0 && fn >= 0 && fn != node && fn < f.n_nodes && f.N[fn] > 0) out = fn;
-    hit[i] = out;
+    if (hit) hit[i] = out;  // a caller that only wants the count passes no array
     if (out >= 0) atomicAdd(d_status + 6, 1);
 }
 
@@ -648,6 +648,27 @@ __global__ __launch_bounds__(256) void k_tt_probe(const TTSlot *slots, int log2_
         }
     }
     if (valid) out[i] = found;
+}
+
+// Position keys of single nodes, from the host's game states (IGameState::getHash of the state a
+// node stands for).  An id outside the forest is counted, not written.
+__global__ __launch_bounds__(256) void k_set_keys(uint64_t *hash, const int32_t *nodes, const uint64_t *keys, int64_t n,
+                                                  int64_t n_nodes, int *d_bad) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int node = nodes[i];
+    if (node < 0 || node >= n_nodes) {
+        atomicAdd(d_bad, 1);
+        return;
+    }
+    hash[node] = keys[i];
+}
+
+hipError_t launch_set_keys(uint64_t *hash, const int32_t *nodes, const uint64_t *keys, int64_t n, int64_t n_nodes,
+                           int *d_bad, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_set_keys, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, hash, nodes, keys, n, n_nodes, d_bad);
+    return hipGetLastError();
 }
 
 hipError_t launch_tt_clear(TTSlot *slots, TTMeta *meta, int log2_slots, hipStream_t s) {

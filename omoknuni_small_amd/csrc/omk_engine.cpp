@@ -16,6 +16,7 @@ ForestEngine::ForestEngine(InferenceFunction inference_fn, const MCTSSettings &s
 }
 
 ForestEngine::~ForestEngine() {
+    if (table_) omk_tt_destroy(table_);
     if (batch_) omk_batch_destroy(batch_);
     if (forest_) omk_forest_destroy(forest_);
 }
@@ -93,6 +94,23 @@ std::vector<float> ForestEngine::getActionProbabilities(int32_t root, float temp
 void ForestEngine::addDirichletNoise(int32_t root, const std::vector<float> &gamma_samples, float epsilon) {
     check(omk_forest_add_root_noise(forest_, root, gamma_samples.data(), (int32_t)gamma_samples.size(), epsilon),
           "omk_forest_add_root_noise");
+}
+
+void ForestEngine::setPositionKeys(const std::vector<int32_t> &nodes, const std::vector<uint64_t> &keys) {
+    if (nodes.size() != keys.size()) throw std::invalid_argument("setPositionKeys: one key per node");
+    check(omk_forest_set_keys(forest_, nodes.data(), keys.data(), (int64_t)nodes.size()), "omk_forest_set_keys");
+}
+
+std::array<int32_t, 4> ForestEngine::traverseTranspositionTable() {
+    if (!table_) {
+        // 32 bytes per slot; the largest power of two that fits the configured size, 2^10 .. 2^26 slots
+        int log2 = 10;
+        while (log2 < 26 && (size_t(64) << log2) <= settings_.transposition_table_size_mb * (size_t(1) << 20)) log2++;
+        check(omk_tt_create(forest_, log2, &table_), "omk_tt_create");
+    }
+    std::array<int32_t, 4> counts{0, 0, 0, 0};
+    check(omk_tt_traverse(table_, batch_, nullptr, 0, nullptr, nullptr, nullptr, nullptr, counts.data()), "omk_tt_traverse");
+    return counts;
 }
 
 int64_t ForestEngine::nodeCount() const {

@@ -17,6 +17,7 @@
 
 #include <cstdint>
 #include <functional>
+#include <array>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -48,6 +49,9 @@ struct MCTSSettings {
     float dirichlet_alpha = 0.3f;
     float dirichlet_epsilon = 0.25f;
     float temperature = 1.0f;
+    // the table of positions (reference :97-98; the slots here are 32 bytes with their policy fields)
+    bool use_transposition_table = true;
+    size_t transposition_table_size_mb = 128;
     // Not in the reference: only the ceil(sqrt(N_parent)) children of highest prior take part in a
     // selection (omk_select_params::pw; needs children stored by descending prior)
     bool selection_prior_widening = false;
@@ -99,6 +103,15 @@ class ForestEngine {
     // src/mcts/mcts_engine_eval.cpp:78-110): one gamma(alpha, 1) sample per child, drawn by
     // the caller's generator as the reference draws them from its own.
     void addDirichletNoise(int32_t root, const std::vector<float> &gamma_samples, float epsilon);
+    // Position keys of nodes from the game's own states (IGameState::getHash of the state a node stands
+    // for): what the traversal loop gets by cloning and replaying (reference
+    // src/mcts/mcts_engine_batch_tree_simple.cpp:119-124,133-137), for any game.
+    void setPositionKeys(const std::vector<int32_t> &nodes, const std::vector<uint64_t> &keys);
+    // The table's part of the traversal loop (reference :116-162) over the paths of the last
+    // selectLeafBatch, keyed by the nodes' position keys: unvisited children stored, every step looked
+    // up, transpositions counted (never followed).  The table is created on first use with about
+    // settings.transposition_table_size_mb.  Returns {new entries, replacements, duplicates, transpositions}.
+    std::array<int32_t, 4> traverseTranspositionTable();
     int64_t nodeCount() const;
     void downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action);
 
@@ -118,6 +131,7 @@ class ForestEngine {
     MCTSSettings settings_;
     omk_forest *forest_ = nullptr;
     omk_batch *batch_ = nullptr;
+    omk_tt *table_ = nullptr;
     int batch_capacity_ = 0;
     int last_n_ = 0;
     bool has_rave_ = false;

@@ -107,6 +107,8 @@ hipError_t launch_leaf_keys(const ForestDev &f, const int32_t *paths, const int3
                             const int32_t *root_player, uint64_t *out, int *d_status, hipStream_t s);
 hipError_t launch_copy_words(void *dst, const void *src, int64_t n_words, hipStream_t s);
 hipError_t launch_fill_words(void *dst, uint32_t value, int64_t n_words, hipStream_t s);
+hipError_t launch_set_keys(uint64_t *hash, const int32_t *nodes, const uint64_t *keys, int64_t n, int64_t n_nodes,
+                           int *d_bad, hipStream_t s);
 
 // The same arrays for the one operation that writes the structure (leaf expansion).
 struct ForestMut {

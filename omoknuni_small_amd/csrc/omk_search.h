@@ -27,19 +27,42 @@
 #include <memory>
 #include <numeric>
 #include <random>
+#include <type_traits>
+#include <utility>
 
 #include "omk_engine.h"
 
 namespace omk {
 
-// reference include/mcts/mcts_engine.h:199-211 (without the statistics block)
+// reference include/mcts/mcts_engine.h:199-211 (of the statistics block: what this path counts)
 struct SearchResult {
     int action = -1;
     std::vector<float> probabilities;
     float value = 0.0f;
     int simulations = 0;
     int64_t nodes = 0;
+    // the table of positions over the whole search (settings.use_transposition_table): entries stored,
+    // and lookups that found ANOTHER visited node for the position reached: what the reference would
+    // redirect to (src/mcts/mcts_engine_batch_tree_simple.cpp:141-157); counted, never followed
+    int64_t table_entries = 0, transpositions = 0;
 };
+
+// reference include/mcts/evaluation_types.h:49-73: a leaf waiting for the network, with the tree on the
+// device: the node is an id, the path a list of ids
+template <class State>
+struct PendingEvaluation {
+    int32_t node = -1;
+    std::unique_ptr<State> state;
+    std::vector<int32_t> path;
+};
+
+namespace detail {
+// a state type that reports a position key (IGameState::getHash, include/core/igamestate.h)
+template <class S, class = void>
+struct has_hash : std::false_type {};
+template <class S>
+struct has_hash<S, std::void_t<decltype(std::declval<const S &>().getHash())>> : std::true_type {};
+}  // namespace detail
 
 // The arrays of a flattened tree, owning their memory; view() is what omk_forest_upload takes.
 struct FlatTree {
@@ -96,12 +119,15 @@ FlatTree flattenTree(Node &root, std::vector<Node *> *node_of_id = nullptr) {
     return t;
 }
 
-template <class State>
+// Output: what the inference function returns per state, anything with `policy` (std::vector<float>)
+// and `value` (float) members: the reference's mcts::NetworkOutput passes through unchanged.
+template <class State, class Output = NetworkOutput>
 class GPUForestMCTSEngine {
    public:
     using StatePtr = std::unique_ptr<State>;
     // the reference's InferenceFunction (include/mcts/mcts_engine.h:230-231) with State = core::IGameState
-    using InferenceFunction = std::function<std::vector<NetworkOutput>(const std::vector<StatePtr> &)>;
+    // and Output = mcts::NetworkOutput
+    using InferenceFunction = std::function<std::vector<Output>(const std::vector<StatePtr> &)>;
 
     GPUForestMCTSEngine(InferenceFunction inference_fn, const MCTSSettings &settings, int64_t capacity_nodes,
                         int device = 0, uint64_t seed = 5489u)
@@ -146,7 +172,6 @@ class GPUForestMCTSEngine {
         v.hash = nullptr;
         engine_.uploadTree(v);
 
-        std::vector<LeafItem> leaves;
         std::vector<StatePtr> states;
         std::vector<float> values;
         int completed = 0;
@@ -155,18 +180,35 @@ class GPUForestMCTSEngine {
             // the first batch is the root alone: it is expanded and evaluated before anything else
             // (runSearch: expandNonTerminalLeaf(root_)), and gets its Dirichlet noise
             const int n = root_expanded ? std::min(st.batch_size, st.num_simulations - completed) : 1;
-            engine_.selectLeafBatch(0, n, leaves);
-            // the leaf states: a clone of the root state, the path's moves replayed
-            // (mcts_engine_batch_tree_simple.cpp:170-178)
+            // phase 1 and the leaf gather: the leaf states are a clone of the root state with the path's
+            // moves replayed (mcts_engine_batch_tree_simple.cpp:170-178)
+            std::vector<PendingEvaluation<State>> pending = collectLeafBatch(state, n);
             states.clear();
-            states.reserve(leaves.size());
-            for (const LeafItem &lf : leaves) {
-                StatePtr s = state.clone();
-                for (int move : lf.move_sequence) s->makeMove(move);
-                states.push_back(std::move(s));
+            states.reserve(pending.size());
+            for (auto &pe : pending) states.push_back(std::move(pe.state));
+            if constexpr (detail::has_hash<State>::value) {
+                if (st.use_transposition_table) {
+                    // the keys of the positions reached, from the game itself, then the table's part of the
+                    // traversal (:116-162) over the paths just selected
+                    key_nodes_.clear();
+                    key_values_.clear();
+                    for (size_t i = 0; i < pending.size(); i++) {
+                        key_nodes_.push_back(pending[i].node);
+                        key_values_.push_back((uint64_t)states[i]->getHash());
+                    }
+                    engine_.setPositionKeys(key_nodes_, key_values_);
+                    const std::array<int32_t, 4> c = engine_.traverseTranspositionTable();
+                    result.table_entries += c[0];
+                    result.transpositions += c[3];
+                }
             }
-            std::vector<NetworkOutput> out = inference_fn_(states);  // phase 2 (:212-236)
-            if (out.size() != states.size()) throw std::runtime_error("inference function returned a short batch");
+            std::vector<Output> raw = inference_fn_(states);  // phase 2 (:212-236)
+            if (raw.size() != states.size()) throw std::runtime_error("inference function returned a short batch");
+            std::vector<NetworkOutput> out(raw.size());
+            for (size_t i = 0; i < raw.size(); i++) {
+                out[i].policy = std::move(raw[i].policy);
+                out[i].value = raw[i].value;
+            }
             std::vector<std::vector<int>> legal(states.size());
             values.resize(out.size());
             for (size_t i = 0; i < states.size(); i++) {
@@ -216,6 +258,21 @@ class GPUForestMCTSEngine {
         return result;
     }
 
+    // Phase 1 and the leaf gather of one batch of n simulations from the root of the tree on the device:
+    // what the reference's collectors hand to the evaluator (PendingEvaluation: node, state, path).
+    std::vector<PendingEvaluation<State>> collectLeafBatch(const State &root_state, int n) {
+        engine_.selectLeafBatch(0, n, leaves_);
+        std::vector<PendingEvaluation<State>> pending(leaves_.size());
+        for (size_t i = 0; i < leaves_.size(); i++) {
+            StatePtr s = root_state.clone();
+            for (int move : leaves_[i].move_sequence) s->makeMove(move);
+            pending[i].node = leaves_[i].node;
+            pending[i].state = std::move(s);
+            pending[i].path = leaves_[i].path;
+        }
+        return pending;
+    }
+
    private:
     // MCTSEngine::addDirichletNoise (src/mcts/mcts_engine_eval.cpp:78-110): gamma(alpha, 1) samples from
     // the engine's own generator, one per child of the root
@@ -253,6 +310,9 @@ class GPUForestMCTSEngine {
     InferenceFunction inference_fn_;
     ForestEngine engine_;
     std::mt19937 random_engine_;
+    std::vector<LeafItem> leaves_;
+    std::vector<int32_t> key_nodes_;
+    std::vector<uint64_t> key_values_;
 };
 
 }  // namespace omk

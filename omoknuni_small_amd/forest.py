@@ -23,7 +23,7 @@ u64p = C.POINTER(C.c_uint64)
 EXPORTS = [
     "omk_last_error", "omk_version", "omk_forest_create", "omk_forest_destroy", "omk_forest_set_stream", "omk_forest_get_stream",
     "omk_forest_upload", "omk_forest_download", "omk_forest_node_count", "omk_forest_download_structure",
-    "omk_expand_batch", "omk_expand_batch_ex", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_reroot_child", "omk_forest_compact", "omk_forest_compact_static",
+    "omk_expand_batch", "omk_expand_batch_ex", "omk_forest_action_probabilities", "omk_forest_add_root_noise", "omk_forest_set_keys", "omk_forest_reroot_child", "omk_forest_compact", "omk_forest_compact_static",
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
@@ -207,6 +207,14 @@ class Forest:
         gamma = np.ascontiguousarray(gamma, dtype=np.float32)
         _check(self._lib.omk_forest_add_root_noise(self._h, C.c_int32(int(root)), _ptr(gamma, f32p),
                                                    C.c_int32(len(gamma)), C.c_float(epsilon)))
+
+    def set_keys(self, nodes, keys):
+        """Position keys of single nodes (the game's own getHash() of the states they stand for)."""
+        nodes = np.ascontiguousarray(nodes, dtype=np.int32)
+        keys = np.ascontiguousarray(keys, dtype=np.uint64)
+        assert len(nodes) == len(keys)
+        _check(self._lib.omk_forest_set_keys(self._h, _ptr(nodes, i32p), _ptr(keys, C.POINTER(C.c_uint64)),
+                                             C.c_int64(len(nodes))))
 
     def download_structure(self):
         """Returns dict(child_begin, child_count, action) of the current nodes."""

@@ -68,6 +68,13 @@ struct PtrNode {
     float getRAVEValue() const { return rave_n ? rave_sum / rave_n : 0.0f; }
 };
 
+// stands for the reference's own mcts::NetworkOutput (include/mcts/evaluation_types.h:14-17): the search
+// takes the evaluator's output type as it is
+struct RefNetworkOutput {
+    std::vector<float> policy;
+    float value = 0.0f;
+};
+
 static int run_search(int sims, int batch, bool widening, bool noise, float temperature) {
     omk::MCTSSettings s;
     s.num_simulations = sims;
@@ -77,10 +84,11 @@ static int run_search(int sims, int batch, bool widening, bool noise, float temp
     s.add_dirichlet_noise = noise;
     s.temperature = temperature;
     s.max_depth = 16;
-    using Engine = omk::GPUForestMCTSEngine<RingState>;
+    s.transposition_table_size_mb = 1;  // 2^15 slots
+    using Engine = omk::GPUForestMCTSEngine<RingState, RefNetworkOutput>;
     long evaluated = 0;
     Engine::InferenceFunction evaluator = [&](const std::vector<std::unique_ptr<RingState>> &states) {
-        std::vector<omk::NetworkOutput> out(states.size());
+        std::vector<RefNetworkOutput> out(states.size());
         for (size_t i = 0; i < states.size(); i++) {
             const uint64_t h = states[i]->getHash();
             out[i].value = (float)((int)(h % 2001ull) - 1000) / 1000.0f;
@@ -101,6 +109,7 @@ static int run_search(int sims, int batch, bool widening, bool noise, float temp
     omk::SearchResult r = engine.search(root);
     printf("action %d value %.9g simulations %d nodes %lld evaluated %ld\n", r.action, r.value, r.simulations,
            (long long)r.nodes, evaluated);
+    printf("table entries %lld transpositions %lld\n", (long long)r.table_entries, (long long)r.transpositions);
     printf("probabilities");
     for (float p : r.probabilities) printf(" %.9g", p);
     printf("\n");

@@ -122,3 +122,57 @@ def test_traversal_part_of_the_table(mode):
     assert stored > 50
     if mode == "node_keys":
         assert reported > 0, "no transposition was ever reported: nothing tested"
+
+
+def test_keys_set_node_by_node_from_the_game():
+    """omk_forest_set_keys: a forest uploaded without position keys gets them node by node, as the host
+    learns them from the states it replays (IGameState::getHash); nodes without a key are neither stored
+    nor found, nodes added by an expansion start without one, an id outside the forest is refused."""
+    import omoknuni_small_amd as omk
+    soa, roots, boards, players = board_forest(41, cells=81, root_stones=6, n_expand=200, fanout=(2, 8), max_depth=6,
+                                               n_roots=2, n_max=30, zero_frac=0.5)
+    n = len(soa["N"])
+    assert "hash" not in soa
+    rng = np.random.default_rng(8)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa, capacity=n + 64)
+    B, D, vl = 400, 7, 3
+    b = omk.Batch(f, B, D)
+    troots = roots[np.arange(B) % len(roots)].astype(np.int32)
+    b.set_roots(troots)
+    sp, rp = omk.SelectParams(virtual_loss=vl), R.make_params(virtual_loss=vl, max_depth=D)
+    tt, ref_tt = omk.TranspositionTable(f, 13), R.RefTT(13)
+    no_key = np.uint64(0xFFFFFFFFFFFFFFFF)
+    keys = np.full(n + 64, no_key, np.uint64)
+    pool = rng.integers(1, 2**63, 150, dtype=np.uint64)    # fewer keys than nodes: some positions are shared
+    stored = reported = 0
+    for step in range(5):
+        rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths == rpaths).all()
+        # the host has just replayed the states of these leaves: it knows their keys now
+        leaves = np.unique(rleaf)
+        new = leaves[keys[leaves] == no_key]
+        keys[new] = pool[rng.integers(0, len(pool), len(new))]
+        f.set_keys(new, keys[new])
+        step_keys = keys[np.maximum(rpaths[:, 1:], 0)]
+        ghits, gcounts = tt.traverse(b)
+        rhits, rcounts = ref_tt.traverse(ref, rpaths, rlen, step_keys)
+        assert gcounts == rcounts and (ghits == rhits).all(), "step %d" % step
+        same_tables(tt, ref_tt, "step %d" % step)
+        stored += gcounts[0]
+        reported += gcounts[3]
+        vals = rng.uniform(-1, 1, B).astype(np.float32)
+        b.set_values(vals)
+        b.backup(vl)
+        ref.backup_batch(rpaths, rlen, vals, vl)
+        ref.W[:] = f.download()["W"]
+    assert stored > 20 and reported > 0, (stored, reported)
+    # the leaves' own lookups go by the same keys
+    got = tt.probe_leaves(b)
+    want, _ = ref_tt.lookup(keys[rleaf])
+    assert (got == want).all()
+    with pytest.raises(omk.OmkError) as e:
+        f.set_keys(np.array([0, n + 1000], np.int32), np.array([5, 6], np.uint64))
+    assert e.value.code == -1, e.value       # OMK_ERR_INVALID: the id outside the forest was skipped, the other one set

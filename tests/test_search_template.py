@@ -66,6 +66,11 @@ def replay_search(sims, batch, widening):
     ref = R.RefTree(N=z, W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=z, child_begin=z, child_count=z,
                     action=z - 1)
     rp = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=16)
+    # the table of positions: keys of the nodes from the game's own hash of the states they stand for,
+    # known once a node has been a leaf; a node without a key is neither stored nor found
+    table, key_of = R.RefTT(15), {}
+    no_key = np.uint64(0xFFFFFFFFFFFFFFFF)
+    entries = transpositions = 0
     done, first = 0, True
     while done < sims:
         n = 1 if first else min(batch, sims - done)
@@ -74,10 +79,20 @@ def replay_search(sims, batch, widening):
         paths, plen, leaf, _ = ref.select_batch(roots, rp)
         acts = ref.gather_actions(paths, plen)
         begin, moves, pb, pol, values = [0], [], [0], [], []
+        states = []
         for t in range(n):
             s = root_state.clone()
             for a in acts[t, :plen[t] - 1]:
                 s.make(int(a))
+            states.append(s)
+            key_of[int(leaf[t])] = np.uint64(s.hash())
+        step_keys = np.array([[key_of.get(int(paths[t, d]), no_key) if d < plen[t] else no_key
+                               for d in range(1, paths.shape[1])] for t in range(n)], np.uint64).reshape(n, -1)
+        _, counts = table.traverse(ref, paths, plen, step_keys)
+        entries += counts[0]
+        transpositions += counts[3]
+        for t in range(n):
+            s = states[t]
             v, p = evaluate(s)
             values.append(v)
             if not s.terminal():
@@ -89,6 +104,7 @@ def replay_search(sims, batch, widening):
                          action_space=CELLS, policy_begin=pb, widening=(2.0, 0.5) if widening else None)
         ref.backup_batch(paths, plen, np.array(values, np.float32), 3)
         done += n
+    ref.table_counts = (entries, transpositions)
     return ref
 
 
@@ -101,9 +117,14 @@ def test_search_with_the_reference_signatures_matches_the_checker(widening):
     assert r.returncode == 0, r.stderr
     lines = r.stdout.strip().split("\n")
     head = lines[0].split()
-    probs = np.array([float(x) for x in lines[1].split()[1:]], np.float32)
+    probs = np.array([float(x) for x in next(ln for ln in lines if ln.startswith("probabilities")).split()[1:]], np.float32)
+    table = next(ln for ln in lines if ln.startswith("table entries")).split()
     nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
     ref = replay_search(sims, batch, widening)
+    # the table of positions, keyed by the mock game's own getHash(): entries stored for unvisited children
+    # and positions reached by another order of moves, as the checker counts them
+    assert (int(table[2]), int(table[4])) == ref.table_counts, (table, ref.table_counts)
+    assert ref.table_counts[0] > 0
     assert int(head[5]) == sims and int(head[7]) == ref.n == len(nodes) and int(head[9]) == sims
     assert (nodes[:, 0] == ref.N).all() and (nodes[:, 3] == ref.VL).all()
     assert (nodes[:, 4] == ref.child_begin).all() and (nodes[:, 5] == ref.child_count).all()
@@ -130,7 +151,7 @@ def test_search_with_noise_and_temperature_runs_and_is_consistent():
     assert r.returncode == 0, r.stderr
     lines = r.stdout.strip().split("\n")
     head = lines[0].split()
-    probs = np.array([float(x) for x in lines[1].split()[1:]])
+    probs = np.array([float(x) for x in next(ln for ln in lines if ln.startswith("probabilities")).split()[1:]])
     nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
     assert abs(probs.sum() - 1.0) < 1e-4 and probs[int(head[1])] > 0   # the move was drawn from the distribution
     kids = nodes[int(nodes[0, 4]):int(nodes[0, 4] + nodes[0, 5])]
