@@ -929,6 +929,130 @@ __device__ __forceinline__ void batch_run(const SelectArgs &a, WaveLds<R> &lds, 
     team_sync<NT>();
 }
 
+// The children of a node that can contribute entries at or above a lower bound, listed
+// densely (one per lane and round) so that work on them costs one round per 64 ACTIVE
+// children instead of one per 64 children.
+template <int R>
+struct ActiveSet {
+    int rounds;
+    int c[R];  // child index, -1 = none
+    int n[R];
+    int vl[R];
+    float w[R], p[R], q2[R];
+    uint32_t head[R];
+};
+
+// Exact number of entries of every active child at or above threshold T (at most m each):
+// the closed-form estimate, then the two entries around it are tested with the exact
+// arithmetic; if the estimate is further off, gallop away from it and bisect the rest.
+// A child whose key hardly moves with virtual loss (a RAVE blend that dominates) defeats the
+// estimate by thousands of entries at a threshold near its plateau: a few such children
+// left after three gallop steps are counted by the whole wavefront instead, one child at a
+// time, 64 candidate counts per round (two or three rounds where the lane alone takes
+// twenty-odd evaluations while the other 63 wait).
+constexpr int kCoopCountMax = 4;  // children counted that way per round of the active set, at most
+template <int R, bool RAVE>
+__device__ __forceinline__ void active_counts(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t T, int m,
+                                              int (&out)[R], int lane) {
+    const float tau = key_score(T);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        out[r] = 0;
+        if (r >= s.rounds) continue;  // uniform
+        // invariant: lo_c entries are known to be at or above T, the entry number hi_c is known
+        // not to be (or hi_c is the cap)
+        int lo_c = 0, hi_c = 0;
+        bool up = false, galloping = false;  // the gallop away from the estimate: direction, still under way
+        int step = 2;
+        if (s.c[r] >= 0 && s.head[r] >= T) {
+            lo_c = 1;  // the first entry itself is at or above T
+            hi_c = m;
+            int g = predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, tau, m);
+            g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
+            uint32_t kk, pp;
+            if (g > lo_c) {
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g - 1, s.c[r], kk, pp);
+                if (kk >= T) lo_c = g;
+                else hi_c = g - 1;
+            }
+            if (lo_c == g && g < hi_c) {
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g, s.c[r], kk, pp);
+                if (kk >= T) lo_c = g + 1;
+                else hi_c = g;
+            }
+            if (lo_c < hi_c) {
+                up = lo_c > g;
+                galloping = true;
+                for (; lo_c < hi_c && step <= 8; step <<= 1) {
+                    int t = up ? lo_c + step : hi_c - step + 1;
+                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+                    entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
+                    const bool ge = kk >= T;
+                    if (ge) lo_c = t;
+                    else hi_c = t - 1;
+                    if (ge != up) {
+                        galloping = false;
+                        break;
+                    }
+                }
+            }
+        }
+        // still far open: the whole wavefront on one child at a time
+        uint64_t open = __ballot(hi_c - lo_c > kWave);
+        if (__popcll(open) <= kCoopCountMax) {
+            while (open != 0ull) {
+                const int src = __ffsll((long long)open) - 1;
+                open &= open - 1ull;
+                const int cn = __builtin_amdgcn_readlane(s.n[r], src), cvl = __builtin_amdgcn_readlane(s.vl[r], src);
+                const int cc = __builtin_amdgcn_readlane(s.c[r], src);
+                const float cw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s.w[r]), src));
+                const float cp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s.p[r]), src));
+                const float cq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s.q2[r]), src));
+                int lo0 = __builtin_amdgcn_readlane(lo_c, src), hi0 = __builtin_amdgcn_readlane(hi_c, src);
+                while (lo0 < hi0) {
+                    const int step = (hi0 - lo0 + kWave - 1) / kWave;
+                    const int cand = lo0 + (lane + 1) * step;  // a count: its last entry is number cand - 1
+                    bool ge = false;
+                    if (cand <= hi0) {
+                        uint32_t kk, pp;
+                        entry_key<R, RAVE>(cn, cw, cp, cvl, cq2, ep, uvl, cand - 1, cc, kk, pp);
+                        ge = kk >= T;
+                    }
+                    const uint64_t gm = __ballot(ge);
+                    const int n_ge = gm == ~0ull ? kWave : __builtin_ctzll(~gm);  // leading run of successes
+                    const int new_lo = lo0 + n_ge * step;
+                    const int new_hi = lo0 + (n_ge + 1) * step - 1;
+                    lo0 = new_lo < hi0 ? new_lo : hi0;
+                    hi0 = new_hi < hi0 ? new_hi : hi0;
+                }
+                if (lane == src) lo_c = hi_c = lo0;
+            }
+        }
+        if (lo_c < hi_c) {
+            // gallop on from where the three steps above left off, then bisect
+            uint32_t kk, pp;
+            if (galloping) {
+                for (; lo_c < hi_c; step <<= 1) {
+                    int t = up ? lo_c + step : hi_c - step + 1;
+                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
+                    entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
+                    const bool ge = kk >= T;
+                    if (ge) lo_c = t;
+                    else hi_c = t - 1;
+                    if (ge != up) break;
+                }
+            }
+            while (lo_c < hi_c) {
+                int t = (lo_c + hi_c + 1) >> 1;
+                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
+                if (kk >= T) lo_c = t;
+                else hi_c = t - 1;
+            }
+        }
+        out[r] = lo_c;
+    }
+}
+
 // The visitors of a crowded node in batches (see the file header).  On success cnt[r]
 // holds the visitors of every child and sc_child / sc_occ hold (child, visit number) of
 // every visitor; returns false when the node has to be replayed one visitor at a time
@@ -1486,67 +1610,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
     return true;
 }
 
-// The children of a node that can contribute entries at or above a lower bound, listed
-// densely (one per lane and round) so that work on them costs one round per 64 ACTIVE
-// children instead of one per 64 children.
-template <int R>
-struct ActiveSet {
-    int rounds;
-    int c[R];  // child index, -1 = none
-    int n[R];
-    int vl[R];
-    float w[R], p[R], q2[R];
-    uint32_t head[R];
-};
-
-// Exact number of entries of every active child at or above threshold T (at most m each):
-// the closed-form estimate, then the two entries around it are tested with the exact
-// arithmetic; if the estimate is further off, gallop away from it and bisect the rest.
-template <int R, bool RAVE>
-__device__ __forceinline__ void active_counts(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t T, int m,
-                                              int (&out)[R]) {
-    const float tau = key_score(T);
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        out[r] = 0;
-        if (r < s.rounds && s.c[r] >= 0 && s.head[r] >= T) {
-            int lo_c = 1, hi_c = m;  // the first entry itself is at or above T
-            int g = predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, tau, m);
-            g = g < lo_c ? lo_c : (g > hi_c ? hi_c : g);
-            uint32_t kk, pp;
-            if (g > lo_c) {
-                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g - 1, s.c[r], kk, pp);
-                if (kk >= T) lo_c = g;
-                else hi_c = g - 1;
-            }
-            if (lo_c == g && g < hi_c) {
-                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, g, s.c[r], kk, pp);
-                if (kk >= T) lo_c = g + 1;
-                else hi_c = g;
-            }
-            if (lo_c < hi_c) {
-                const bool up = lo_c > g;
-                for (int step = 2; lo_c < hi_c; step <<= 1) {
-                    int t = up ? lo_c + step : hi_c - step + 1;
-                    t = t > hi_c ? hi_c : (t <= lo_c ? lo_c + 1 : t);
-                    entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
-                    const bool ge = kk >= T;
-                    if (ge) lo_c = t;
-                    else hi_c = t - 1;
-                    if (ge != up) break;
-                }
-            }
-            while (lo_c < hi_c) {
-                int t = (lo_c + hi_c + 1) >> 1;
-                entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, t - 1, s.c[r], kk, pp);
-                if (kk >= T) lo_c = t;
-                else hi_c = t - 1;
-            }
-            out[r] = lo_c;
-        }
-    }
-}
-
 // A threshold at or above which about `target` of the node's entries lie, found on ESTIMATED
 // counts (search_threshold).  The thresholds of a node's targets come out ordered like the
 // targets: a search either stops with its count inside [target, target + window], and the windows
@@ -1667,7 +1730,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     if (target_hi > 0) {
         T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m);
         OMK_STAMP(10);
-        active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta);
+        active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta, lane);
         OMK_STAMP(11);
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -1680,7 +1743,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     if (target_lo > 0) {
         T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m);
         OMK_STAMP(10);
-        active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta);
+        active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta, lane);
         OMK_STAMP(11);
 #pragma unroll
         for (int r = 0; r < R; r++)
