@@ -549,9 +549,11 @@ __device__ __forceinline__ bool wait_list(const SelectArgs &a, int off, int dept
 // bracket straddles score zero, where the keys are densest.  Deterministic: the same arguments
 // give the same key on every wavefront.  Only efficiency depends on the result: whatever key comes
 // out, the caller counts exactly.
-template <typename Est>
+// plateau(klo, khi), asked now and then once six steps have not brought the count into the window: a key
+// to return at once, or 0.
+template <typename Est, typename Plateau>
 __device__ __forceinline__ uint32_t search_threshold(uint32_t lo_key, uint32_t hi_key, int target, int acc_hi,
-                                                     int acc_below, int &evals, Est est) {
+                                                     int acc_below, int &evals, Est est, Plateau plateau) {
     uint32_t klo = lo_key, khi = hi_key;
     auto y_of = [](uint32_t k) {
         float d = key_score(k) + 1.0f;
@@ -589,8 +591,19 @@ __device__ __forceinline__ uint32_t search_threshold(uint32_t lo_key, uint32_t h
             if (last < 0) flo *= 0.5f;
             last = -1;
         }
+        if (it >= 5 && (it - 5) % 3 == 0 && it <= 17 && khi - klo > 1u) {
+            const uint32_t kp = plateau(klo, khi);
+            if (kp >= lo_key && kp <= hi_key && kp != 0u) return kp;
+        }
     }
     return klo;
+}
+
+template <typename Est>
+__device__ __forceinline__ uint32_t search_threshold(uint32_t lo_key, uint32_t hi_key, int target, int acc_hi,
+                                                     int acc_below, int &evals, Est est) {
+    return search_threshold(lo_key, hi_key, target, acc_hi, acc_below, evals, est,
+                            [](uint32_t, uint32_t) { return 0u; });
 }
 
 template <int NT>
@@ -1617,19 +1630,83 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
 // still reaches the target; the counts do not increase with the key, so in every combination the
 // larger target gets the lower key.  (The estimate's fast arithmetic may break that monotonicity
 // by a hair; the caller checks the order of the thresholds and of the exact counts.)
+//
+// A target whose rank falls inside the run of ONE child whose key hardly moves with virtual loss (a RAVE
+// blend that dominates: thousands of its entries within a few hundred keys, or on one key) cannot be met by
+// looking at estimated counts: they jump from far below to far above the target between neighbouring
+// keys, and the estimate for that child is the ill-conditioned one.  When six steps have not met the
+// window and one child accounts for most of the difference between the counts at the two ends of the
+// bracket, the threshold is taken from that child's own list instead: the EXACT key of its entry number
+// target - (what the others have at the upper end), which puts about `target` entries at or above it
+// whatever the estimate said about the child itself.  Still a function of the node and the target only,
+// and decreasing in the target (the child's keys do not increase), so neighbouring slices agree and the
+// order of the thresholds holds; the callers check both anyway.
 template <int R, bool RAVE>
 __device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, float ep, uint32_t uvl, uint32_t lo_key,
-                                                     uint32_t hi_key, int target, int window, int m) {
+                                                     uint32_t hi_key, int target, int window, int m, int lane) {
     int n_evals = 0;
-    return search_threshold(lo_key, hi_key, target, target + window, target, n_evals, [&](uint32_t kmid) {
-        const float mid = key_score(kmid);
-        int est = 0;
+    return search_threshold(
+        lo_key, hi_key, target, target + window, target, n_evals,
+        [&](uint32_t kmid) {
+            const float mid = key_score(kmid);
+            int est = 0;
 #pragma unroll
-        for (int r = 0; r < R; r++)
-            if (r < s.rounds && s.c[r] >= 0)
-                est += predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, mid, m);
-        return wave_sum_i32(est);
-    });
+            for (int r = 0; r < R; r++)
+                if (r < s.rounds && s.c[r] >= 0)
+                    est += predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, mid, m);
+            return wave_sum_i32(est);
+        },
+        [&](uint32_t klo, uint32_t khi) {
+            const float tlo = key_score(klo), thi = key_score(khi);
+            // the child whose estimated count differs most between the two ends (lowest child on ties)
+            uint32_t best = 0u;  // (difference << 10) | (1023 - slot in the active set): the largest wins
+            int my_hi[R];
+            int sum_lo = 0, sum_hi = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                my_hi[r] = 0;
+                if (r < s.rounds && s.c[r] >= 0) {
+                    const int a = predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, tlo, m);
+                    my_hi[r] = predict_count<RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], ep, uvl, thi, m);
+                    sum_lo += a;
+                    sum_hi += my_hi[r];
+                    const int d = a - my_hi[r] > 0 ? a - my_hi[r] : 0;
+                    const uint32_t v = ((uint32_t)(d > 0x1FFFFF ? 0x1FFFFF : d) << 10) | (uint32_t)(1023 - (r * kWave + lane));
+                    best = best > v ? best : v;
+                }
+            }
+            const int e_lo = wave_sum_i32(sum_lo), e_hi = wave_sum_i32(sum_hi);
+            const uint32_t top = wave_max_u32(best);
+            const int d_top = (int)(top >> 10), slot = 1023 - (int)(top & 1023u);
+            // no single child behind the jump, or the target is not between the ends
+            if (top == 0u || e_lo < target || e_hi >= target || (long long)d_top * 10 < (long long)(e_lo - e_hi) * 6) return 0u;
+            const int src = slot & 63;
+            int an = 0, avl = 0, ac = 0, ah = 0;
+            float aw = 0.0f, ap = 0.0f, aq2 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (r == (slot >> 6)) {
+                    an = s.n[r];
+                    avl = s.vl[r];
+                    ac = s.c[r];
+                    ah = my_hi[r];
+                    aw = s.w[r];
+                    ap = s.p[r];
+                    aq2 = s.q2[r];
+                }
+            an = __builtin_amdgcn_readlane(an, src);
+            avl = __builtin_amdgcn_readlane(avl, src);
+            ac = __builtin_amdgcn_readlane(ac, src);
+            ah = __builtin_amdgcn_readlane(ah, src);
+            aw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aw), src));
+            ap = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ap), src));
+            aq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aq2), src));
+            const int ja = target - (e_hi - ah);  // entries of that child wanted at or above the threshold
+            if (ac < 0 || ja < 1 || ja > m) return 0u;
+            uint32_t kk, pp;
+            entry_key<R, RAVE>(an, aw, ap, avl, aq2, ep, uvl, ja - 1, ac, kk, pp);
+            return kk;
+        });
 }
 
 // For a slice of a heavy node: the thresholds of the cumulative targets target_hi and
@@ -1728,7 +1805,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
 #pragma unroll
     for (int r = 0; r < R; r++) ct_hi[r] = ct_lo[r] = 0;
     if (target_hi > 0) {
-        T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m);
+        T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m, lane);
         OMK_STAMP(10);
         active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta, lane);
         OMK_STAMP(11);
@@ -1741,7 +1818,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
         wave_sync_memory();
     }
     if (target_lo > 0) {
-        T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m);
+        T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m, lane);
         OMK_STAMP(10);
         active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta, lane);
         OMK_STAMP(11);
