@@ -170,7 +170,7 @@ struct Kids {
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
 // so that it sits at the same place for every fan-out class.
-enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3, kOpPartition = 4 };
+enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3, kOpPartition = 4, kOpLoad = 5 };
 struct TeamCmd {
     int op;
     int rounds;  // R of the node's fan-out class: 1, or the kernel's RMAX
@@ -187,6 +187,11 @@ struct TeamCmd {
     int proven;  // kOpRun: the child's keys provably do not increase over the run
     // kOpPartition: the node whose visitors a helper shares out while the owner walks on
     int j_cb, j_off, j_m, j_depth, j_keep, j_run_child;
+    // kOpPartition: the node the owner walks on into (-1: none) and its N_parent: the two helpers that
+    // do not partition load and score their share of that node's children meanwhile (load_ahead).
+    // kOpLoad: the same for the node the owner has just taken from the queue, whose child range it
+    // knows (pre_cb, pre_cc; pre_cc < 0: not known, the helpers fetch it)
+    int pre_node, pre_np, pre_cb, pre_cc;
 };
 
 // What that helper reads, at the same place for every fan-out class: the owner's next node
@@ -297,6 +302,61 @@ __device__ __forceinline__ void score_round(Kids<R, RAVE> &k, int r, float ep) {
     k.k2[r] = b;
 }
 
+// Rounds R0 .. R1-1 of load_kids (look-ahead variant) and score_round; the other rounds of k are
+// left alone.
+template <int R, bool RAVE, int R0, int R1>
+__device__ __forceinline__ void load_score_rounds(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
+                                                  float ep, Kids<R, RAVE> &k) {
+    int rn[R];
+    float rw[R];
+    uint32_t word[R];
+#pragma unroll
+    for (int r = R0; r < R1; r++) {
+        const int i = r * kWave + lane;
+        const bool in = i < nelig;
+        const int id = cb + i;
+        word[r] = in && f.legal ? f.legal[(uint32_t)id >> 5] : 0xFFFFFFFFu;
+        k.n[r] = in ? f.N[id] : 0;
+        k.w[r] = in ? f.W[id] : 0.0f;
+        k.p[r] = in ? f.P[id] : 0.0f;
+        k.vl[r] = in ? f.VL[id] : 0;
+        rn[r] = RAVE && in ? f.rN[id] : 0;
+        rw[r] = RAVE && in ? f.rW[id] : 0.0f;
+    }
+#pragma unroll
+    for (int r = R0; r < R1; r++) {
+        const int i = r * kWave + lane;
+        const int id = cb + i;
+        const bool in = i < nelig && ((word[r] >> ((uint32_t)id & 31u)) & 1u);
+        k.part[r] = in;
+        if (!in) {
+            k.n[r] = 0;
+            k.w[r] = 0.0f;
+            k.p[r] = 0.0f;
+            k.vl[r] = 0;
+            rn[r] = 0;
+            rw[r] = 0.0f;
+        }
+        k.q2[r] = RAVE ? combined_value(k.n[r], k.w[r], rn[r], rw[r], rave_k) : 0.0f;
+        score_round<R, RAVE>(k, r, ep);
+    }
+}
+
+// A wide node that its owner walks on into (fan-out class R > 1) is loaded by three wavefronts of the
+// block: while one helper shares out the visitors of the node before it, the owner takes the first
+// kAheadShare rounds of the children and the other two helpers the rest, which they leave in LDS
+// (statistics, blend, keys); the owner collects them at the barrier that ends the partition request.
+// One wavefront issues an instruction every few cycles at best, and six rounds of divisions and square
+// roots (two scans, RAVE blend) are a few microseconds of that on every node of the chain.
+template <int R>
+struct AheadShare {
+    static constexpr int kRounds = (R + 2) / 3;
+};
+
+template <int R, bool RAVE>
+__device__ __forceinline__ void load_ahead(const ForestDev &f, const SelectArgs &a, WaveLds<R> &lds, int node, int np,
+                                           int cb, int cc, int wave, int lane);
+
 // Best candidate of this lane in the order (key descending, position ascending); the
 // candidates of the second scan sit at positions R*64 + i, after all of the first scan.
 template <int R, bool RAVE>
@@ -383,6 +443,32 @@ __device__ __forceinline__ NodeCtx node_ctx(const ForestDev &f, const SelectArgs
     }
     c.ep = a.c_puct * sqrtf((float)np);
     return c;
+}
+
+template <int R, bool RAVE>
+__device__ __forceinline__ void load_ahead(const ForestDev &f, const SelectArgs &a, WaveLds<R> &lds, int node, int np,
+                                           int cb, int cc, int wave, int lane) {
+    constexpr int S = AheadShare<R>::kRounds;
+    const NodeCtx c = node_ctx(f, a, node, np, cc >= 0, int2{cb, cc});
+    if (c.cc <= kWave) return;  // a leaf, or a node of the narrow class: its owner loads it alone
+    Kids<R, RAVE> k;
+    if (wave == 2) load_score_rounds<R, RAVE, (S < R ? S : R), (2 * S < R ? 2 * S : R)>(f, c.cb, c.nelig, lane, a.rave_k, c.ep, k);
+    else load_score_rounds<R, RAVE, (2 * S < R ? 2 * S : R), R>(f, c.cb, c.nelig, lane, a.rave_k, c.ep, k);
+    const int r0 = wave == 2 ? S : 2 * S, r1 = wave == 2 ? 2 * S : R;
+#pragma unroll
+    for (int r = S; r < R; r++) {
+        if (r >= r0 && r < r1) {
+            const int i = r * kWave + lane;
+            lds.st_n[i] = k.n[r];
+            lds.st_w[i] = k.w[r];
+            lds.st_p[i] = k.p[r];
+            lds.st_vl[i] = k.vl[r];
+            lds.st_q2[i] = k.q2[r];
+            lds.key[0][i] = k.k1[r];
+            lds.key[1][i] = k.k2[r];
+            lds.pay[i] = k.part[r] ? 1u : 0u;
+        }
+    }
 }
 
 // One selection for a single visitor.  Returns the child index or -1; np_child receives
@@ -2246,6 +2332,7 @@ struct Continuation {
     int m;
     int np;
     int2 span;  // (child_begin, child_count) of that node, loaded ahead of time
+    bool ahead;  // two helpers load their share of that node's children (load_ahead), if it is a wide one
 };
 
 // All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
@@ -2268,7 +2355,8 @@ struct Continuation {
 template <int R, bool RAVE, int RMAX>
 __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                             const Item &item, const int32_t *seg_in, int32_t *seg_out,
-                                            WaveLds<R> &lds, PartLds<RMAX> &pl, bool &pending, Continuation &next) {
+                                            WaveLds<R> &lds, PartLds<RMAX> &pl, bool &pending, Continuation &next,
+                                            bool ahead) {
     OMK_T0();
     const int off = item.off, m = item.m, depth = item.depth;
     // a heavy node is settled and shared out by several wavefronts, which read its visitor
@@ -2297,11 +2385,49 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             cnt[r] = 0;
         }
     } else {
-        load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
+        if (R > 1 && R == RMAX && !ahead) {
+            // a wide node from the queue: the helpers are idle (or finish the partition of the node this
+            // wavefront settled last), two of them take their share of the children
+            close_pending(pending);
+            if (lane == 0) {
+                TeamCmd &cm = lds.cmd;
+                cm.op = kOpLoad;
+                cm.rounds = R;
+                cm.pre_node = item.node;
+                cm.pre_np = item.np;
+                cm.pre_cb = c.cb;
+                cm.pre_cc = c.cc;
+            }
+            __syncthreads();  // the request is open until close_pending
+            pending = true;
+            ahead = true;
+        }
+        if (R > 1 && R == RMAX && ahead) {
+            // this wavefront's share of the children; the rest is in LDS once the request is closed
+            constexpr int S = AheadShare<R>::kRounds;
+            load_score_rounds<R, RAVE, 0, (S < R ? S : R)>(f, c.cb, c.nelig, lane, a.rave_k, c.ep, k);
+            close_pending(pending);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            score_round<R, RAVE>(k, r, c.ep);
-            cnt[r] = 0;
+            for (int r = S; r < R; r++) {
+                const int i = r * kWave + lane;
+                k.n[r] = lds.st_n[i];
+                k.w[r] = lds.st_w[i];
+                k.p[r] = lds.st_p[i];
+                k.vl[r] = lds.st_vl[i];
+                k.q2[r] = lds.st_q2[i];
+                k.k1[r] = lds.key[0][i];
+                k.k2[r] = lds.key[1][i];
+                k.part[r] = lds.pay[i] != 0u;
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) cnt[r] = 0;
+        } else {
+            load_kids<R, RAVE, true>(f, c.cb, c.nelig, lane, a.rave_k, k);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                score_round<R, RAVE>(k, r, c.ep);
+                cnt[r] = 0;
+            }
         }
         if (RAVE) {
             // no real score in the first scan: the reference never runs the second one
@@ -2588,6 +2714,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             }
             carry += __builtin_amdgcn_readlane(inc, 63);
         }
+        const int np_next = keep >= 0 ? __builtin_amdgcn_readlane(np_keep, keep & 63) : 0;
+        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth;
         if (lane == 0) {
             TeamCmd &cm = lds.cmd;
             cm.op = kOpPartition;
@@ -2598,16 +2726,21 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             cm.j_depth = depth;
             cm.j_keep = keep;
             cm.j_run_child = run_child;
+            cm.pre_node = ahead_next ? c.cb + keep : -1;
+            cm.pre_np = np_next;
+            cm.pre_cc = -1;
         }
         __syncthreads();  // the request is open until close_pending
         pending = true;
         next.node = -1;
+        next.ahead = false;
         if (keep >= 0) {
             next.node = c.cb + keep;
             next.off = off + __builtin_amdgcn_readlane(ex_keep, keep & 63);
             next.m = (int)gmax;
-            next.np = __builtin_amdgcn_readlane(np_keep, keep & 63);
+            next.np = np_next;
             next.span = keep_span;
+            next.ahead = ahead_next;
         }
         OMK_TICK(14);
         return kStepDescended;
@@ -2940,7 +3073,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = f.N[it.node];
             for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
-        bool have_span = false;
+        bool have_span = false, ahead = false;
         int2 pre_span = int2{0, 0};
         for (;;) {
             const int depth = it.depth;
@@ -2955,13 +3088,15 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             int status = kStepLeaf;
             Continuation next;
             next.node = -1;
+            next.ahead = false;
             if (c.cc > 0 && depth < a.max_depth) {
                 if (c.cc <= kWave)
                     status = select_group<1, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out,
-                                                         reinterpret_cast<WaveLds<1> &>(s_lds), s_part, pending, next);
+                                                         reinterpret_cast<WaveLds<1> &>(s_lds), s_part, pending, next,
+                                                         false);
                 else
                     status = select_group<RMAX, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out, s_lds, s_part, pending,
-                                                            next);
+                                                            next, ahead);
             }
 #ifdef OMK_TRACE
             if (lane == 0) {
@@ -3000,6 +3135,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.pad[0] = it.pad[1] = it.pad[2] = 0;
             have_span = true;
             pre_span = next.span;
+            ahead = next.ahead;
         }
     }
 }
@@ -3168,6 +3304,14 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const int cur = __builtin_amdgcn_readfirstlane(s_lds.cmd.cur);
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
+        if (RMAX > 1 && (op == kOpPartition || op == kOpLoad) && (tid >> 6) >= 2) {
+            const int pn = __builtin_amdgcn_readfirstlane(s_lds.cmd.pre_node);
+            if (pn >= 0)
+                load_ahead<RMAX, RAVE>(f, a, s_lds, pn, __builtin_amdgcn_readfirstlane(s_lds.cmd.pre_np),
+                                       __builtin_amdgcn_readfirstlane(s_lds.cmd.pre_cb),
+                                       op == kOpLoad ? __builtin_amdgcn_readfirstlane(s_lds.cmd.pre_cc) : -1, tid >> 6,
+                                       tid & 63);
+        }
         if (rounds == 1)
             team_help<1, RAVE, RMAX>(f, a, reinterpret_cast<WaveLds<1> &>(s_lds), s_part, tid, op, total, keep, goff, cur,
                                      ep, uvl);
