@@ -282,13 +282,19 @@ def traffic_of(workload):
         "kernel; not measured in this run" % tj[workload].get("command", "bench.py --workload %s" % workload))
 
 
-def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parity=True):
-    """Everything bench.py reports about one workload."""
+def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parity=True, relaid=False):
+    """Everything bench.py reports about one workload.  relaid: the same forest without the empty
+    slots of its board layout (omk_soa_compact_legal), the layout of the reference's own children_
+    vectors; everything (byte model, parity, CPU baseline) is then taken on that forest."""
     kw = {}
     if scale != 1.0:
         kw["nodes_per_tree"] = max(1000, int(synth.CONFIGS[name]["nodes_per_tree"] * scale))
     t0 = time.time()
     soa, roots, meta = synth.generate(name, seed=seed, **kw)
+    if relaid:
+        soa, old_to_new, _ = omk.compact_legal(soa)
+        roots = old_to_new[np.asarray(roots)]
+        meta = dict(meta, n_nodes=len(soa["N"]))
     gen_s = time.time() - t0
     n_nodes = len(soa["N"])
     B = int(meta["n_traversals"])
@@ -389,10 +395,11 @@ def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parit
     sel_ms_step = sel_ms / K
     bak_ms_step = bak_ms / K
     achieved = sel_bytes / (sel_ms * 1e-3) / 1e9
-    traffic, traffic_source = traffic_of(name) if scale == 1.0 else (None, None)
+    traffic, traffic_source = traffic_of(name) if scale == 1.0 and not relaid else (None, None)
     res = {
-        "workload": "%s: %d tree(s) x %d nodes, %d traversals per step, depth <= %d, c_puct %.2f, virtual loss %d%s%s%s"
-                    % (name, meta["n_trees"], meta["nodes_per_tree"], B, D, meta["c_puct"], vl,
+        "workload": "%s%s: %d tree(s) x %d nodes, %d traversals per step, depth <= %d, c_puct %.2f, virtual loss %d%s%s%s"
+                    % (name, " re-laid without its empty slots (%d nodes kept)" % n_nodes if relaid else "",
+                       meta["n_trees"], meta["nodes_per_tree"], B, D, meta["c_puct"], vl,
                        ", RAVE k=%g" % meta["rave_k"] if meta.get("has_rave") else "",
                        ", progressive widening" if meta.get("pw") else "",
                        ", 2^%d-slot table probes" % meta["tt_log2"] if meta.get("tt_log2") else ""),
@@ -453,6 +460,11 @@ def main():
     ap.add_argument("--workload", default="c3", choices=BENCH_CONFIGS + ["wide"])
     ap.add_argument("--configs", default=",".join(BENCH_CONFIGS),
                     help="comma-separated workloads measured beside --workload into per_config ('none': only --workload)")
+    ap.add_argument("--relaid", default="c2,c4,wide",
+                    help="comma-separated board workloads also measured on the forest re-laid without its empty "
+                         "slots, into per_config_relaid ('none': skip)")
+    ap.add_argument("--head-relaid", action="store_true",
+                    help="measure --workload itself on the re-laid forest (for profiler runs of that layout)")
     ap.add_argument("--seed", type=int, default=2025)
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget of the CPU baseline leg of --workload (0 = skip); the other configurations get a third")
@@ -482,7 +494,7 @@ def main():
         return
 
     head = measure(omk, synth, args.workload, args.steps, args.warmup, args.seed, args.cpu_seconds, args.scale,
-                   parity=not args.no_parity)
+                   parity=not args.no_parity, relaid=args.head_relaid)
 
     # outside every timed region: three plain copies of 64 MiB, the known-size kernel that a
     # profiler run of this command scales its traffic counters by
@@ -534,7 +546,7 @@ def main():
         if name not in BENCH_CONFIGS + ["wide"]:
             print("bench.py: unknown configuration %r in --configs" % name, file=sys.stderr)
             sys.exit(2)
-        if name == args.workload:
+        if name == args.workload and not args.head_relaid:
             r = head
         else:
             r = measure(omk, synth, name, args.steps, args.warmup, args.seed, args.cpu_seconds / 3.0, args.scale,
@@ -560,6 +572,33 @@ def main():
                     per[name]["cpu_baseline"][k] = cb[k]
     if per:
         out["per_config"] = per
+
+    def short(r):
+        d = {
+            "workload": r["workload"],
+            "select_ms": r["select_ms"],
+            "backup_ms": r["backup_ms"],
+            "ms_per_step": r["ms_per_step"],
+            "traversals_per_s": r["traversals_per_s"],
+            "select_traversals_per_s": r["select_traversals_per_s"],
+            "backups_per_s": r["backups_per_s"],
+            "select_ms_first_last": r["select_ms_first_last"],
+            "roofline": {k: r["roofline"][k] for k in ("kernel", "achieved", "frac", "algorithmic_bytes",
+                                                        "backup_algorithmic_bytes", "backup_achieved", "traffic")},
+            "parity": r["parity"],
+        }
+        return d
+
+    relaid = [] if args.relaid.strip().lower() in ("", "none") else [c.strip() for c in args.relaid.split(",")]
+    rel = {}
+    for name in relaid:
+        if name not in BENCH_CONFIGS + ["wide"] or not synth.CONFIGS[name].get("dense"):
+            print("bench.py: %r in --relaid is not a board workload" % name, file=sys.stderr)
+            sys.exit(2)
+        rel[name] = short(measure(omk, synth, name, args.steps, args.warmup, args.seed, 0.0, args.scale,
+                                  parity=not args.no_parity, relaid=True))
+    if rel:
+        out["per_config_relaid"] = rel
     print(json.dumps(out))
 
 

@@ -120,6 +120,26 @@ int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_chi
                                   int32_t *h_action);
 int omk_sync(omk_forest *f);
 
+/* Host-side re-layout of a forest whose nodes keep one slot per action and a legal mask (a board
+ * layout: 362 slots per expanded Go node, a bit per slot) into the layout of the reference itself,
+ * whose children_ vector holds the legal moves only (MCTSNode::expand, src/mcts/mcts_node.cpp:238-436):
+ * the nodes whose bit is set, in their old order, renumbered 0 .. count-1, child ranges shrunk to
+ * match, the slot index kept as the node's action.  A selection on the result visits the same
+ * children in the same order (ties still go to the lowest child), reads half the cache lines and
+ * takes four rounds of 64 lanes where a 362-slot node takes six; node ids in paths and leaves are
+ * the new ones, new_to_old maps them back.  No GPU call; omk_forest_upload takes the result
+ * (legal = NULL).
+ * omk_soa_count_legal: how many nodes the result has (n_nodes when the view has no mask).
+ * omk_soa_compact_legal: fills the caller's arrays of that many elements (rN, rW, hash: NULL when
+ * the view has none or they are not wanted) and the two id maps (old_to_new: n_nodes entries, -1 for
+ * an empty slot; new_to_old: count entries; either may be NULL).  action receives the view's action
+ * of every kept node or, when the view has none, the node's slot in its parent's range (-1 for a
+ * node that is nobody's child). */
+int64_t omk_soa_count_legal(const omk_soa_view *h_view);
+int omk_soa_compact_legal(const omk_soa_view *h_view, int64_t count, int32_t *N, float *W, float *P, int32_t *VL,
+                          int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                          uint64_t *hash, int32_t *old_to_new, int32_t *new_to_old);
+
 /* ---- batch: the per-search buffers of executeBatchedTreeSearch
  *      (leaf_nodes / paths / leaf_states, mcts_engine_batch_tree_simple.cpp:41-57) ---- */
 int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, omk_batch **out);

@@ -373,6 +373,71 @@ int omk_forest_download(omk_forest *f, omk_soa_view *v) {
     return OMK_OK;
 }
 
+static inline bool view_legal(const omk_soa_view *v, int64_t i) {
+    return !v->legal || ((v->legal[i >> 5] >> (i & 31)) & 1u);
+}
+
+int64_t omk_soa_count_legal(const omk_soa_view *v) {
+    if (!v || v->n_nodes < 0) return fail(OMK_ERR_INVALID, "omk_soa_count_legal: null view");
+    if (!v->legal) return v->n_nodes;
+    int64_t c = 0;
+    const int64_t words = v->n_nodes >> 5;
+    for (int64_t w = 0; w < words; w++) c += __builtin_popcount(v->legal[w]);
+    for (int64_t i = words << 5; i < v->n_nodes; i++) c += view_legal(v, i);
+    return c;
+}
+
+int omk_soa_compact_legal(const omk_soa_view *v, int64_t count, int32_t *N, float *W, float *P, int32_t *VL,
+                          int32_t *rN, float *rW, int32_t *child_begin, int32_t *child_count, int32_t *action,
+                          uint64_t *hash, int32_t *old_to_new, int32_t *new_to_old) {
+    if (!v || !N || !W || !P || !VL || !child_begin || !child_count)
+        return fail(OMK_ERR_INVALID, "omk_soa_compact_legal: N, W, P, VL, child_begin, child_count are required");
+    const int64_t n = v->n_nodes;
+    if (n <= 0 || !v->N || !v->W || !v->P || !v->VL || !v->child_begin || !v->child_count)
+        return fail(OMK_ERR_INVALID, "omk_soa_compact_legal: the view has no nodes or lacks a required array");
+    if ((rN && !v->rN) || (rW && !v->rW) || (hash && !v->hash))
+        return fail(OMK_ERR_INVALID, "omk_soa_compact_legal: rN, rW or hash asked for, the view has none");
+    // rank[i]: kept nodes before node i
+    std::vector<int32_t> rank((size_t)n + 1);
+    int64_t c = 0;
+    for (int64_t i = 0; i < n; i++) {
+        rank[(size_t)i] = (int32_t)c;
+        c += view_legal(v, i);
+    }
+    rank[(size_t)n] = (int32_t)c;
+    if (c != count)
+        return fail(OMK_ERR_INVALID, "omk_soa_compact_legal: the view keeps %lld nodes, room for %lld was announced",
+                    (long long)c, (long long)count);
+    if (action && !v->action)
+        for (int64_t j = 0; j < c; j++) action[j] = -1;
+    for (int64_t i = 0; i < n; i++) {
+        if (old_to_new) old_to_new[i] = view_legal(v, i) ? rank[(size_t)i] : -1;
+        if (!view_legal(v, i)) continue;
+        const int64_t j = rank[(size_t)i];
+        N[j] = v->N[i];
+        W[j] = v->W[i];
+        P[j] = v->P[i];
+        VL[j] = v->VL[i];
+        if (rN) rN[j] = v->rN[i];
+        if (rW) rW[j] = v->rW[i];
+        if (hash) hash[j] = v->hash[i];
+        if (new_to_old) new_to_old[j] = (int32_t)i;
+        const int64_t cb = v->child_begin[i], cc = v->child_count[i];
+        if (cc < 0 || cb < 0 || cb + cc > n)
+            return fail(OMK_ERR_INVALID, "omk_soa_compact_legal: node %lld has the child range [%lld, +%lld)", (long long)i,
+                        (long long)cb, (long long)cc);
+        child_count[j] = cc > 0 ? rank[(size_t)(cb + cc)] - rank[(size_t)cb] : 0;
+        child_begin[j] = child_count[j] > 0 ? rank[(size_t)cb] : 0;
+        if (action) {
+            if (v->action) action[j] = v->action[i];
+            else
+                for (int64_t q = cb; q < cb + cc; q++)
+                    if (view_legal(v, q)) action[rank[(size_t)q]] = (int32_t)(q - cb);
+        }
+    }
+    return OMK_OK;
+}
+
 int omk_forest_download_structure(omk_forest *f, int64_t n_nodes, int32_t *h_child_begin, int32_t *h_child_count,
                                   int32_t *h_action) {
     if (!f) return fail(OMK_ERR_INVALID, "omk_forest_download_structure: null forest");

@@ -29,7 +29,7 @@ EXPORTS = [
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
-    "omk_dev_d2h", "omk_dev_copy",
+    "omk_dev_d2h", "omk_dev_copy", "omk_soa_count_legal", "omk_soa_compact_legal",
 ]
 
 TT_SLOT = np.dtype([("key", "<u8"), ("node", "<i4"), ("depth", "<i4")])
@@ -93,6 +93,7 @@ def load_library():
     for name in EXPORTS:
         if name != "omk_last_error":
             getattr(L, name).restype = C.c_int
+    L.omk_soa_count_legal.restype = C.c_int64
     _LIB = L
     return L
 
@@ -108,6 +109,43 @@ def _ptr(a, ty):
 
 def _arr(x, dtype):
     return None if x is None else np.ascontiguousarray(x, dtype=dtype)
+
+
+def _view_of(keep):
+    return _SoaView(len(keep["N"]), _ptr(keep["N"], i32p), _ptr(keep["W"], f32p), _ptr(keep["P"], f32p),
+                    _ptr(keep["VL"], i32p), _ptr(keep["rN"], i32p), _ptr(keep["rW"], f32p),
+                    _ptr(keep["child_begin"], i32p), _ptr(keep["child_count"], i32p), _ptr(keep["action"], i32p),
+                    _ptr(keep["legal"], u32p), _ptr(keep["hash"], u64p))
+
+
+def compact_legal(soa):
+    """A forest with one slot per action and a legal mask, re-laid without its empty slots
+    (omk_soa_compact_legal; host only).  Returns (soa without a mask, old_to_new, new_to_old)."""
+    lib = load_library()
+    keep = dict(N=_arr(soa["N"], np.int32), W=_arr(soa["W"], np.float32), P=_arr(soa["P"], np.float32),
+                VL=_arr(soa["VL"], np.int32), rN=_arr(soa.get("rN"), np.int32), rW=_arr(soa.get("rW"), np.float32),
+                child_begin=_arr(soa["child_begin"], np.int32), child_count=_arr(soa["child_count"], np.int32),
+                action=_arr(soa.get("action"), np.int32), legal=_arr(soa.get("legal"), np.uint32),
+                hash=_arr(soa.get("hash"), np.uint64))
+    n = len(keep["N"])
+    if keep["legal"] is not None and len(keep["legal"]) * 32 < n:
+        raise ValueError("legal mask shorter than the node count")
+    v = _view_of(keep)
+    cnt = int(lib.omk_soa_count_legal(C.byref(v)))
+    if cnt < 0:
+        _check(cnt)
+    out = dict(N=np.empty(cnt, np.int32), W=np.empty(cnt, np.float32), P=np.empty(cnt, np.float32),
+               VL=np.empty(cnt, np.int32), child_begin=np.empty(cnt, np.int32), child_count=np.empty(cnt, np.int32),
+               action=np.empty(cnt, np.int32))
+    for k, dt in (("rN", np.int32), ("rW", np.float32), ("hash", np.uint64)):
+        out[k] = np.empty(cnt, dt) if keep[k] is not None else None
+    old_to_new, new_to_old = np.empty(n, np.int32), np.empty(cnt, np.int32)
+    _check(lib.omk_soa_compact_legal(C.byref(v), C.c_int64(cnt), _ptr(out["N"], i32p), _ptr(out["W"], f32p),
+                                     _ptr(out["P"], f32p), _ptr(out["VL"], i32p), _ptr(out["rN"], i32p),
+                                     _ptr(out["rW"], f32p), _ptr(out["child_begin"], i32p),
+                                     _ptr(out["child_count"], i32p), _ptr(out["action"], i32p),
+                                     _ptr(out["hash"], u64p), _ptr(old_to_new, i32p), _ptr(new_to_old, i32p)))
+    return {k: a for k, a in out.items() if a is not None}, old_to_new, new_to_old
 
 
 class Forest:
