@@ -62,7 +62,7 @@ constexpr int kRunMin = 4;                // visitors from which the one-winner 
 constexpr int kWaterLevelMin = 24;        // visitors from which the parallel path is tried
 constexpr int kWaterLevelMaxJ = 1 << 21;  // entries per child representable in the sort payload
 constexpr int kBatchCap = 2048;           // entries put in winner order at a time (LDS resident)
-constexpr int kSortBits = 6;              // widest radix digit of that sort (one lane per digit value)
+constexpr int kSortBits = 8;              // widest radix digit of that sort
 constexpr int kSortBins = 1 << kSortBits;
 constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-visitor kernel: one owner that
                                           // takes the items, three helpers for the batch work of its node
@@ -897,9 +897,9 @@ __device__ __forceinline__ int batch_order(WaveLds<R> &lds, int tid, int total, 
                 dig[r] = (int)d;
                 rank[r] = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32),
                                                          __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
-                if (lane < ndig) {
-                    lds.hist[lane * nb1 + blk] = 0;
-                    if (blk == 0 && nb1 != nblocks) lds.hist[lane * nb1 + nblocks] = 0;  // the pad column
+                for (int dv = lane; dv < ndig; dv += kWave) {
+                    lds.hist[dv * nb1 + blk] = 0;
+                    if (blk == 0 && nb1 != nblocks) lds.hist[dv * nb1 + nblocks] = 0;  // the pad column
                 }
                 wave_sync_memory();
                 if (valid && rank[r] == 0) lds.hist[(int)d * nb1 + blk] = __popcll(same);
