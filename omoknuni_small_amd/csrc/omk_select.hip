@@ -82,7 +82,7 @@ constexpr int kRunShortcutMin = 128;      // entries from which a run of one chi
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
 constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
-constexpr int kMaxWalkerBlocks = 32;         // blocks of walkers of the persistent launch, at most
+constexpr int kMaxWalkerBlocks = 16;         // blocks of walkers of the persistent launch, at most
 constexpr int kFastSinglesMax = 16384;    // traversals up to which the single-visitor kernel trades bytes for latency
 constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
                                           // is shared out like a heavy node's instead of left to one helper
@@ -3490,15 +3490,14 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
     // mask: three trips per level become one), not on a compact one (two become one).
     const bool fast = f.legal && n_traversals <= kFastSinglesMax;
     if (n_items0 > 0) {
-        // One persistent launch: teams for the multi-visitor items (as many as can be resident,
-        // but no more than there can be items at once: an item has at least two visitors) and,
-        // behind them, blocks of walkers for the lone visitors the teams create.
-        int per_cu = 1;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_select_groups<RMAX, RAVE>, kTeam, 0) !=
-                hipSuccess ||
-            per_cu < 1)
-            per_cu = 1;
-        int capacity = n_cus * per_cu;
+        // One persistent launch: teams for the multi-visitor items (no more than there can be items
+        // at once: an item has at least two visitors) and, behind them, blocks of walkers for the lone
+        // visitors the teams create.  ONE block per compute unit, although two or three would fit: a
+        // selection takes as long as its longest chain of crowded nodes, the wavefront that works on that
+        // chain issues an instruction every few cycles at best, and every other block on its compute
+        // unit (waiting for work, polling) takes issue slots, cache and LDS bandwidth from it.  Measured
+        // on the 4 M-node chess-like tree: 0.247 ms a selection with two blocks per unit, 0.222 with one.
+        int capacity = n_cus;
 #ifdef OMK_TRACE
         if (a0.dbg_grid > 0 && capacity > a0.dbg_grid) capacity = a0.dbg_grid;
 #endif
