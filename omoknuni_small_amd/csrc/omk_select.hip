@@ -74,7 +74,7 @@ constexpr int kTeamMin = 96;              // batch entries from which the helper
 #endif
 constexpr int kCountSortLone = 2, kCountSortTeam = OMK_COUNT_SORT_TEAM;
 #ifndef OMK_SLICE_ENTRIES
-#define OMK_SLICE_ENTRIES 256
+#define OMK_SLICE_ENTRIES 192
 #endif
 constexpr int kSliceEntries = OMK_SLICE_ENTRIES;  // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
