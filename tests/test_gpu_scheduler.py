@@ -238,8 +238,10 @@ def dominated_forest(seed, fan, depth, rave, kind, visitors):
         rN.append(int(rn)); rW.append(float(rw))
         return len(N) - 1
 
+    fans = fan if isinstance(fan, (list, tuple)) else [fan]
     node = add(60_000, 0.0, 0.0, -1)
     for level in range(depth):
+        fan = fans[level % len(fans)]
         ep = 1.4 * np.sqrt(N[node])
         cb[node] = len(N)
         cc[node] = fan
@@ -291,3 +293,15 @@ def test_one_child_takes_nearly_every_visitor(visitors, fan, rave, kind):
     # everything before that is "other children's entries": merged only while those are few)
     if kind != "plateau" or visitors <= 40:
         assert st["merged_nodes"] >= 1, st
+
+
+@pytest.mark.parametrize("visitors", [40, 900])
+@pytest.mark.parametrize("rave,kind", [(False, "few"), (True, "few"), (True, "plateau"), (False, "some")])
+def test_chain_through_narrow_and_wide_nodes(rave, kind, visitors):
+    """The crowd walks down a chain whose nodes change between the narrow class (at most 64 children, one
+    wavefront loads them) and the wide one (three wavefronts share the children of the node the owner
+    walks on into), in every order: narrow to wide, wide to narrow, wide to wider."""
+    soa = dominated_forest(31, [40, 200, 64, 65, 362, 10, 130, 300, 300, 7], 20, rave, kind, visitors)
+    st = select_both(soa, np.zeros(visitors, np.int32), 22, rave=rave, steps=3)
+    assert st["replayed_nodes"] == 0, st
+
