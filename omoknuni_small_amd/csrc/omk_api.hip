@@ -55,6 +55,8 @@ struct omk_forest {
     uint32_t *legal = nullptr;
     uint64_t *hash = nullptr;
     bool has_legal = false, has_action = false, has_hash = false;
+    void *key_stage = nullptr;  // staging of omk_forest_set_keys: keys, node ids, one status word
+    size_t key_stage_bytes = 0;
     int children = 0;       // live batches and tables created on this forest
     bool released = false;  // omk_forest_destroy was called while children were alive
 
@@ -141,7 +143,22 @@ struct omk_tt {
     float threshold = 0.1f;        // Config::replacement_threshold
     void *work = nullptr;          // staging of store / traverse calls
     size_t work_bytes = 0;
+    int64_t generation = -1;       // the forest's generation the stored node ids belong to (-1: nothing stored yet)
 };
+
+// The entries hold node ids.  They are the reference's weak_ptr entries, which die with the tree they
+// point into (PHMapTranspositionTable::lookup erases an entry whose node is gone,
+// src/mcts/phmap_transposition_table.cpp:100-108): once the forest's node ids have taken a new meaning
+// (a compaction, an upload of another tree), every entry stored before is such a dead entry, and the
+// table is emptied before anything else is done with it.  The access counter runs on, as the
+// reference's does.
+static int tt_same_tree(omk_tt *tt) {
+    omk_forest *f = tt->f;
+    if (tt->generation == f->generation) return OMK_OK;
+    if (tt->generation >= 0) HIP_TRY(launch_tt_clear(tt->slots, tt->meta, tt->log2_slots, f->stream));
+    tt->generation = f->generation;
+    return OMK_OK;
+}
 
 static int tt_work(omk_tt *tt, size_t bytes) {
     if (bytes <= tt->work_bytes) return OMK_OK;
@@ -217,7 +234,7 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
 static void forest_free(omk_forest *f) {
     (void)hipSetDevice(f->device);
     if (f->own_stream) (void)hipStreamSynchronize(f->own_stream);
-    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->action, f->legal, f->hash};
+    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->action, f->legal, f->hash, f->key_stage};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     if (f->own_stream) (void)hipStreamDestroy(f->own_stream);
@@ -478,22 +495,27 @@ int omk_forest_set_keys(omk_forest *f, const int32_t *h_nodes, const uint64_t *h
         f->has_hash = true;
     }
     if (n == 0) return OMK_OK;
-    int32_t *d_nodes = nullptr;
-    uint64_t *d_keys = nullptr;
-    int *d_bad = nullptr;
-    hipError_t e = dalloc(&d_nodes, n);
-    if (e == hipSuccess) e = dalloc(&d_keys, n);
-    if (e == hipSuccess) e = dalloc(&d_bad, 1);
+    // staging kept with the forest (a search calls this every batch): keys | node ids | status word
+    const size_t need = (size_t)n * 12 + 8;
+    if (need > f->key_stage_bytes) {
+        HIP_TRY(hipStreamSynchronize(s));
+        if (f->key_stage) HIP_TRY(hipFree(f->key_stage));
+        f->key_stage = nullptr;
+        f->key_stage_bytes = 0;
+        const size_t room = need + need / 2;
+        HIP_TRY(hipMalloc(&f->key_stage, room));
+        f->key_stage_bytes = room;
+    }
+    uint64_t *d_keys = (uint64_t *)f->key_stage;
+    int32_t *d_nodes = (int32_t *)(d_keys + n);
+    int *d_bad = (int *)(d_nodes + n + (n & 1));
     int bad = 0;
-    if (e == hipSuccess) e = hipMemcpyAsync(d_nodes, h_nodes, (size_t)n * 4, hipMemcpyHostToDevice, s);
+    hipError_t e = hipMemcpyAsync(d_nodes, h_nodes, (size_t)n * 4, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(d_keys, h_keys, (size_t)n * 8, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(d_bad, &bad, 4, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = launch_set_keys(f->hash, d_nodes, d_keys, n, f->n_nodes, d_bad, s);
     if (e == hipSuccess) e = hipMemcpyAsync(&bad, d_bad, 4, hipMemcpyDeviceToHost, s);
     if (e == hipSuccess) e = hipStreamSynchronize(s);
-    if (d_nodes) (void)hipFree(d_nodes);
-    if (d_keys) (void)hipFree(d_keys);
-    if (d_bad) (void)hipFree(d_bad);
     if (e != hipSuccess) return fail(OMK_ERR_HIP, "omk_forest_set_keys: %s", hipGetErrorString(e));
     if (bad) return fail(OMK_ERR_INVALID, "omk_forest_set_keys: %d node ids outside the forest (skipped)", bad);
     return OMK_OK;
@@ -1430,6 +1452,7 @@ int omk_tt_clear(omk_tt *tt) {
     if (int rc = use_device(tt->f)) return rc;
     HIP_TRY(launch_tt_clear(tt->slots, tt->meta, tt->log2_slots, tt->f->stream));
     tt->clock = 0;
+    tt->generation = -1;
     return OMK_OK;
 }
 
@@ -1437,6 +1460,7 @@ int omk_tt_insert(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, co
     if (!tt || !d_keys || !d_nodes) return fail(OMK_ERR_INVALID, "omk_tt_insert: null argument");
     if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_insert: n %lld", (long long)n);
     if (int rc = use_device(tt->f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
     hipStream_t s = tt->f->stream;
     int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
@@ -1452,6 +1476,7 @@ int omk_tt_probe(omk_tt *tt, const uint64_t *d_keys, int64_t n, int32_t min_dept
     if (!tt || !d_keys || !d_out) return fail(OMK_ERR_INVALID, "omk_tt_probe: null argument");
     if (n < 0) return fail(OMK_ERR_INVALID, "omk_tt_probe: n %lld", (long long)n);
     if (int rc = use_device(tt->f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
     HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, d_keys, nullptr, nullptr, 0, n, min_depth, d_out, tt->meta,
                             tt->clock, tt->f->stream));
     tt->clock += (uint32_t)n;
@@ -1465,6 +1490,7 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
     if (int rc = fresh_batch("omk_tt_probe_leaves", b)) return rc;
     if (!b->f->has_hash) return fail(OMK_ERR_STATE, "omk_tt_probe_leaves: the forest was uploaded without position keys");
     if (int rc = use_device(tt->f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
     HIP_TRY(launch_tt_probe(tt->slots, tt->log2_slots, nullptr, b->leaf, b->f->hash, b->f->n_nodes, b->n, min_depth, d_out,
                             tt->meta, tt->clock, tt->f->stream));
     tt->clock += (uint32_t)b->n;
@@ -1495,6 +1521,7 @@ int omk_tt_store(omk_tt *tt, const uint64_t *d_keys, const int32_t *d_nodes, con
     if (n < 0 || n > (1ll << 30)) return fail(OMK_ERR_INVALID, "omk_tt_store: n %lld", (long long)n);
     if (!tt->f->uploaded) return fail(OMK_ERR_STATE, "omk_tt_store: upload the forest first");
     if (int rc = use_device(tt->f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
     if (int rc = tt_work(tt, (size_t)std::max<int64_t>(n, 1) * 8)) return rc;
     hipStream_t s = tt->f->stream;
     int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1522,6 +1549,7 @@ int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int3
         return fail(OMK_ERR_STATE, "omk_tt_traverse: no key tables given and the forest was uploaded without position keys");
     }
     if (int rc = use_device(f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
     hipStream_t s = f->stream;
     const int64_t n = (int64_t)b->n * b->max_depth;
     // staging: slot_of [n] i64 | keys [n] u64 | step_nodes, store_nodes, depths, found [n] i32 each
@@ -1589,6 +1617,7 @@ int omk_tt_upload(omk_tt *tt, const omk_tt_slot *h_slots) {
     if (int rc = use_device(tt->f)) return rc;
     HIP_TRY(hipStreamSynchronize(tt->f->stream));
     HIP_TRY(hipMemcpy(tt->slots, h_slots, sizeof(TTSlot) << tt->log2_slots, hipMemcpyHostToDevice));
+    tt->generation = tt->f->generation;  // the caller's node ids are ids of the forest as it is now
     return OMK_OK;
 }
 

@@ -45,6 +45,10 @@ struct MCTSSettings {
     bool use_progressive_widening = true;
     float progressive_widening_c = 2.0f;
     float progressive_widening_k = 0.5f;
+    // MCTSNode::expand shuffles a node's legal moves before it creates the children (reference
+    // src/mcts/mcts_node.cpp:357-364); omk_expand_batch_ex keeps the order it is given, so the search
+    // (omk_search.h) shuffles on the host.  Off: children in the game's own move order.
+    bool shuffle_moves = true;
     bool add_dirichlet_noise = true;
     float dirichlet_alpha = 0.3f;
     float dirichlet_epsilon = 0.25f;

@@ -134,7 +134,8 @@ class GPUForestMCTSEngine {
         : inference_fn_(std::move(inference_fn)),
           engine_([](const std::vector<LeafItem> &) { return std::vector<NetworkOutput>(); }, settings, capacity_nodes,
                   device, false),
-          random_engine_(seed) {}
+          random_engine_(seed),
+          shuffle_engine_(seed + 1u) {}
 
     const MCTSSettings &getSettings() const { return engine_.settings(); }
     ForestEngine &forest() { return engine_; }
@@ -213,6 +214,10 @@ class GPUForestMCTSEngine {
             values.resize(out.size());
             for (size_t i = 0; i < states.size(); i++) {
                 if (!states[i]->isTerminal()) legal[i] = states[i]->getLegalMoves();  // a terminal node stays a leaf
+                // MCTSNode::expand shuffles the legal moves before it creates the children (reference
+                // src/mcts/mcts_node.cpp:357-364), so that the children kept under progressive widening are
+                // a random subset and not the moves of lowest index at every node of the tree
+                if (st.shuffle_moves) shuffleMoves(legal[i]);
                 values[i] = out[i].value;
             }
             engine_.expandLeafBatch(legal, out, action_space);  // phase 3, first half (:249-259)
@@ -274,6 +279,16 @@ class GPUForestMCTSEngine {
     }
 
    private:
+    // Fisher-Yates from the last place down, one raw 32-bit output of the generator per place
+    // (j = output mod (k + 1)): spelled out rather than std::shuffle, whose use of the generator is
+    // the standard library's own, so that a test can restate it
+    void shuffleMoves(std::vector<int> &moves) {
+        for (size_t k = moves.size(); k-- > 1;) {
+            const size_t j = (size_t)(shuffle_engine_() % (uint32_t)(k + 1));
+            std::swap(moves[k], moves[j]);
+        }
+    }
+
     // MCTSEngine::addDirichletNoise (src/mcts/mcts_engine_eval.cpp:78-110): gamma(alpha, 1) samples from
     // the engine's own generator, one per child of the root
     void addDirichletNoise() {
@@ -310,6 +325,7 @@ class GPUForestMCTSEngine {
     InferenceFunction inference_fn_;
     ForestEngine engine_;
     std::mt19937 random_engine_;
+    std::mt19937 shuffle_engine_;  // its own stream: noise and the move drawn do not depend on the tree's size
     std::vector<LeafItem> leaves_;
     std::vector<int32_t> key_nodes_;
     std::vector<uint64_t> key_values_;

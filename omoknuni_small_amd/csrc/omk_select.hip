@@ -170,7 +170,7 @@ struct Kids {
 
 // What the owner wavefront of a block asks of its helpers; first member of the LDS scratch,
 // so that it sits at the same place for every fan-out class.
-enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3, kOpPartition = 4, kOpLoad = 5 };
+enum { kOpExit = 0, kOpOrder = 1, kOpEmit = 2, kOpRun = 3, kOpPartition = 4, kOpLoad = 5, kOpChain = 6 };
 struct TeamCmd {
     int op;
     int rounds;  // R of the node's fan-out class: 1, or the kernel's RMAX
@@ -192,6 +192,8 @@ struct TeamCmd {
     // kOpLoad: the same for the node the owner has just taken from the queue, whose child range it
     // knows (pre_cb, pre_cc; pre_cc < 0: not known, the helpers fetch it)
     int pre_node, pre_np, pre_cb, pre_cc;
+    // kOpChain: the node a chain walk starts at (chain_walk), its N, child range, depth, and its visitors
+    int c_node, c_np, c_cb, c_cc, c_depth, c_off, c_m;
 };
 
 // What that helper reads, at the same place for every fan-out class: the owner's next node
@@ -2325,6 +2327,273 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     return true;
 }
 
+
+// ---- Chains of nodes whose visitors all follow one child ----
+// Most crowded nodes below the top of a tree are of that kind, often a dozen in a row (a whole
+// selection of the Go workload with 16 visitors per tree is a chain of 21), and on such a node nothing
+// is decided: the visitors stay together, in the same order.  The walk below does these nodes and
+// nothing else, by all wavefronts of the block in lockstep instead of one owner directing helpers: every
+// wavefront loads and scores its rounds of the children (statistics, legality bits and the child ranges
+// of all children in range in ONE trip to memory), leaves its best candidate, the best candidate of its
+// other children and the best child's statistics in LDS; after one block barrier every wavefront knows
+// the node's best child and the best candidate of all others, makes the one-winner test of single_run
+// (the entry the best child shows the LAST visitor still comes first, and its entries are in order),
+// and on success writes its share of the visitors' next path entry and moves on into the child: one
+// barrier and one dependent trip to memory per level, no partition (the visitor list does not change;
+// it is kept in registers and written once, where the walk ends, into the buffer the next node reads).
+// The walk ends at a leaf (or the depth cap) or at the first node that fails the test, which is
+// then settled the general way (select_group) from scratch.
+constexpr int kChainMin = 2;  // visitors from which a node is tried that way
+
+struct ChainSlot {
+    uint32_t bk, bpos;  // best candidate among the children this wavefront loaded (key 0 = none)
+    uint32_t sk, spos;  // best candidate of its children other than that one's child
+    int n, vl;          // that child's statistics and child range
+    float w, p, q2;
+    int sx, sy;
+    uint32_t any1;      // one of its children has a real first-scan key
+};
+
+struct ChainEnd {
+    int node, np, cb, cc, depth;  // where the walk stands: a node that has not been settled
+};
+
+template <int RMAX, bool RAVE, int NW>
+__device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave, int lane, int node, int np, int cb,
+                                            int cc, int depth, int off, int m) {
+    constexpr int F = RMAX * kWave;
+    constexpr int Q = (RMAX + NW - 1) / NW;       // rounds of children per wavefront
+    constexpr int NT = NW * kWave;
+    constexpr int U = (kHeavyMin + NT - 1) / NT;  // visitors per thread, at most
+    __shared__ ChainSlot slots[2][NW];
+    const int tid = wave * kWave + lane;
+    const uint32_t uvl = (uint32_t)a.vl;
+    const int d0 = depth;
+    const int32_t *src = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
+    int tt[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int j = tid + u * NT;
+        tt[u] = j < m ? src[off + j] : -1;
+    }
+    int par = 0;
+    for (;;) {
+        if (cc <= 0 || depth >= a.max_depth) break;
+#ifdef OMK_TRACE
+        const long long tr0 = wall_clock64();
+#endif
+        int nelig = cc;
+        if (a.pw) {
+            const int kk = ceil_sqrt_i32(np);
+            nelig = kk < cc ? kk : cc;
+        }
+        const float ep = a.c_puct * sqrtf((float)np);
+        // ---- this wavefront's rounds of the children ----
+        int kn[Q], kvl[Q];
+        float kw[Q], kp[Q], kq2[Q];
+        uint32_t k1[Q], k2[Q];
+        int2 ksp[Q];
+        {
+            int rn[Q];
+            float rw[Q];
+            uint32_t word[Q];
+#pragma unroll
+            for (int q = 0; q < Q; q++) {
+                const int r = wave + q * NW;
+                const int i = r * kWave + lane;
+                const bool in = r < RMAX && i < nelig;
+                const int id = cb + i;
+                word[q] = in && f.legal ? f.legal[(uint32_t)id >> 5] : 0xFFFFFFFFu;
+                kn[q] = in ? f.N[id] : 0;
+                kw[q] = in ? f.W[id] : 0.0f;
+                kp[q] = in ? f.P[id] : 0.0f;
+                kvl[q] = in ? f.VL[id] : 0;
+                rn[q] = RAVE && in ? f.rN[id] : 0;
+                rw[q] = RAVE && in ? f.rW[id] : 0.0f;
+                ksp[q] = in ? f.span[id] : int2{0, 0};
+            }
+#pragma unroll
+            for (int q = 0; q < Q; q++) {
+                const int r = wave + q * NW;
+                const int i = r * kWave + lane;
+                const int id = cb + i;
+                const bool in = r < RMAX && i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
+                k1[q] = k2[q] = 0u;
+                kq2[q] = 0.0f;
+                if (in) {
+                    if (RAVE) kq2[q] = combined_value(kn[q], kw[q], rn[q], rw[q], a.rave_k);
+                    child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
+                }
+            }
+        }
+        // ---- its best candidate, and the best candidate of its other children ----
+        uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
+        bool has1 = false;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            has1 |= k1[q] != 0u;
+            if (k1[q] > bk) { bk = k1[q]; bpos = i; }
+        }
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            if (k2[q] > bk) { bk = k2[q]; bpos = (uint32_t)F + i; }
+        }
+        uint32_t mk, mpos;
+        wave_best(bk, bpos, mk, mpos);
+        const uint32_t mine = mk == 0u ? 0xFFFFFFFFu : (mpos >= (uint32_t)F ? mpos - (uint32_t)F : mpos);
+        uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            if (i != mine && k1[q] > ok_) { ok_ = k1[q]; opos = i; }
+        }
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            if (i != mine && k2[q] > ok_) { ok_ = k2[q]; opos = (uint32_t)F + i; }
+        }
+        uint32_t sk, spos;
+        wave_best(ok_, opos, sk, spos);
+        int tn = 0, tvl = 0, tsx = 0, tsy = 0;
+        float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            if ((uint32_t)(wave + q * NW) == (mine >> 6)) {
+                tn = kn[q];
+                tw = kw[q];
+                tp = kp[q];
+                tvl = kvl[q];
+                tq2 = kq2[q];
+                tsx = ksp[q].x;
+                tsy = ksp[q].y;
+            }
+        }
+        const int ml = (int)(mine & 63u);
+        int bn = __builtin_amdgcn_readlane(tn, ml), bvl = __builtin_amdgcn_readlane(tvl, ml);
+        int bsx = __builtin_amdgcn_readlane(tsx, ml), bsy = __builtin_amdgcn_readlane(tsy, ml);
+        float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), ml));
+        float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ml));
+        float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), ml));
+        bool any1 = __ballot(has1) != 0ull;
+        uint32_t hk = mk, hp = mpos;
+        if (NW > 1) {
+            // ---- the same over the wavefronts of the block ----
+            if (lane == 0) {
+                ChainSlot &sl = slots[par][wave];
+                sl.bk = mk;
+                sl.bpos = mpos;
+                sl.sk = sk;
+                sl.spos = spos;
+                sl.n = bn;
+                sl.vl = bvl;
+                sl.w = bw;
+                sl.p = bp;
+                sl.q2 = bq2;
+                sl.sx = bsx;
+                sl.sy = bsy;
+                sl.any1 = any1 ? 1u : 0u;
+            }
+            __syncthreads();
+            hk = 0u;
+            hp = 0xFFFFFFFFu;
+            int won = 0;
+            uint32_t a1 = 0u;
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const uint32_t k_ = slots[par][w].bk, p_ = slots[par][w].bpos;
+                a1 |= slots[par][w].any1;
+                if (k_ != 0u && comes_before(k_, p_, hk, hp)) {
+                    hk = k_;
+                    hp = p_;
+                    won = w;
+                }
+            }
+            won = __builtin_amdgcn_readfirstlane(won);
+            sk = 0u;
+            spos = 0xFFFFFFFFu;
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const uint32_t k_ = w == won ? slots[par][w].sk : slots[par][w].bk;
+                const uint32_t p_ = w == won ? slots[par][w].spos : slots[par][w].bpos;
+                if (k_ != 0u && comes_before(k_, p_, sk, spos)) {
+                    sk = k_;
+                    spos = p_;
+                }
+            }
+            const ChainSlot &ws = slots[par][won];
+            bn = __builtin_amdgcn_readfirstlane(ws.n);
+            bvl = __builtin_amdgcn_readfirstlane(ws.vl);
+            bsx = __builtin_amdgcn_readfirstlane(ws.sx);
+            bsy = __builtin_amdgcn_readfirstlane(ws.sy);
+            bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.w)));
+            bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.p)));
+            bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.q2)));
+            hk = (uint32_t)__builtin_amdgcn_readfirstlane((int)hk);
+            hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)hp);
+            sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)sk);
+            spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)spos);
+            any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
+        }
+        // ---- the one-winner test (single_run) ----
+        // (with RAVE and no real first-scan score at all the reference never runs its second scan: such a
+        // node goes the general way, which knows)
+        if (hk == 0u || (RAVE && !any1)) break;
+        const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
+        uint32_t lk, lp;
+        entry_key<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1, best, lk, lp);
+        if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) break;
+        if (!entries_in_order<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, best, m, lane)) break;
+        // ---- every visitor takes that child ----
+        const int child = cb + best;
+        int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (tt[u] >= 0) path_next[tt[u]] = child;
+        if (tid == 0) {
+            atomicAdd(f.VL + child, (int)(uvl * (uint32_t)m));
+            if (a.stats) {
+                atomicAdd(a.stats + 0, 1);
+                atomicAdd(a.stats + 1, 1);
+                atomicAdd(a.stats + 2, m);
+            }
+#ifdef OMK_TRACE
+            const int ti = atomicAdd(a.trace_n, 1);
+            if (ti < a.trace_cap) {
+                a.trace[12 * ti + 0] = tr0;
+                a.trace[12 * ti + 1] = wall_clock64();
+                a.trace[12 * ti + 2] = (long long)m | ((long long)depth << 32) | (5ll << 60);
+                a.trace[12 * ti + 3] = (long long)node;
+                for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+            }
+#endif
+        }
+        node = child;
+        np = bn;
+        cb = bsx;
+        cc = bsy;
+        depth++;
+        par ^= 1;
+    }
+    // the visitor list, where the node the walk stands at reads it
+    if (depth > d0) {
+        int32_t *dst = a.seg[(depth - 1) & 1];
+        if (dst != src) {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+                if (tt[u] >= 0) dst[off + tid + u * NT] = tt[u];
+        }
+    }
+    ChainEnd e;
+    e.node = node;
+    e.np = np;
+    e.cb = cb;
+    e.cc = cc;
+    e.depth = depth;
+    return e;
+}
+
 // Where the walk goes on after a multi-visitor node whose visitors all chose one child.
 struct Continuation {
     int node;
@@ -2715,7 +2984,8 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             carry += __builtin_amdgcn_readlane(inc, 63);
         }
         const int np_next = keep >= 0 ? __builtin_amdgcn_readlane(np_keep, keep & 63) : 0;
-        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth;
+        // (a kept child of ordinary size is tried by chain_walk first, which loads it with the whole block)
+        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth && (int)gmax >= kHeavyMin;
         if (lane == 0) {
             TeamCmd &cm = lds.cmd;
             cm.op = kOpPartition;
@@ -3073,7 +3343,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = f.N[it.node];
             for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
-        bool have_span = false, ahead = false;
+        bool have_span = false, ahead = false, chain_tried = false;
         int2 pre_span = int2{0, 0};
         for (;;) {
             const int depth = it.depth;
@@ -3085,6 +3355,42 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             if (lane < 16) s_lds.tph[lane] = 0u;
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
+            if (!chain_tried && it.pad[0] == 0 && it.m >= kChainMin && it.m < kHeavyMin && a.vl > 0 && c.cc > 0 &&
+                depth < a.max_depth) {
+                // a plain node of ordinary size: first the walk down the nodes whose visitors all follow
+                // one child (chain_walk), by the whole block on a wide layout.  Its visitor list comes from
+                // the previous node's partition, and the helpers are needed.
+                close_pending(pending);
+                ChainEnd e;
+                if (RMAX > 1) {
+                    if (lane == 0) {
+                        TeamCmd &cm = s_lds.cmd;
+                        cm.op = kOpChain;
+                        cm.c_node = it.node;
+                        cm.c_np = it.np;
+                        cm.c_cb = c.cb;
+                        cm.c_cc = c.cc;
+                        cm.c_depth = depth;
+                        cm.c_off = it.off;
+                        cm.c_m = it.m;
+                    }
+                    __syncthreads();
+                    e = chain_walk<RMAX, RAVE, kTeamWaves>(f, a, 0, lane, it.node, it.np, c.cb, c.cc, depth, it.off, it.m);
+                    __syncthreads();
+                } else {
+                    e = chain_walk<RMAX, RAVE, 1>(f, a, 0, lane, it.node, it.np, c.cb, c.cc, depth, it.off, it.m);
+                    wave_sync_memory();
+                }
+                it.node = __builtin_amdgcn_readfirstlane(e.node);
+                it.np = __builtin_amdgcn_readfirstlane(e.np);
+                it.depth = __builtin_amdgcn_readfirstlane(e.depth);
+                have_span = true;
+                pre_span = int2{__builtin_amdgcn_readfirstlane(e.cb), __builtin_amdgcn_readfirstlane(e.cc)};
+                ahead = false;
+                chain_tried = true;  // the node the walk stopped at is settled the general way
+                continue;
+            }
+            chain_tried = false;
             int status = kStepLeaf;
             Continuation next;
             next.node = -1;
@@ -3304,6 +3610,18 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const int cur = __builtin_amdgcn_readfirstlane(s_lds.cmd.cur);
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
+        if (RMAX > 1 && op == kOpChain) {
+            const TeamCmd &cm = s_lds.cmd;
+            chain_walk<RMAX, RAVE, kTeamWaves>(f, a, tid >> 6, tid & 63, __builtin_amdgcn_readfirstlane(cm.c_node),
+                                               __builtin_amdgcn_readfirstlane(cm.c_np),
+                                               __builtin_amdgcn_readfirstlane(cm.c_cb),
+                                               __builtin_amdgcn_readfirstlane(cm.c_cc),
+                                               __builtin_amdgcn_readfirstlane(cm.c_depth),
+                                               __builtin_amdgcn_readfirstlane(cm.c_off),
+                                               __builtin_amdgcn_readfirstlane(cm.c_m));
+            __syncthreads();  // the request is done
+            continue;
+        }
         if (RMAX > 1 && (op == kOpPartition || op == kOpLoad) && (tid >> 6) >= 2) {
             const int pn = __builtin_amdgcn_readfirstlane(s_lds.cmd.pre_node);
             if (pn >= 0)

@@ -143,7 +143,7 @@ def timeline(workload, warmup=8, levels=()):
     ctr = (tr[:, 3] >> 32) & 0xFFFFFFFF
     print("workload %s, selection number %d: %d multi-visitor items traced, span %.1f us (100 MHz clock)"
           % (workload, int(warmup) + 1, len(tr), end.max()))
-    print("chain of crowded nodes: per level the node with most visitors (kinds: node = taken as a whole, "
+    print("chain of crowded nodes: per level the node with most visitors (kinds: node = taken as a whole, chain = a node whose visitors all follow one child, taken by the walk down such nodes, "
           "early = published before its visitor list was complete; a node cut into slices / scatter parts shows "
           "their number and the span from the first start to the last end)")
     ph = np.stack([(tr[:, 4 + q // 2] >> (32 * (q % 2))) & 0xFFFFFFFF for q in range(16)], axis=1) / 100.0
@@ -156,14 +156,14 @@ def timeline(workload, warmup=8, levels=()):
     print("%5s %9s %9s %7s %9s %9s %8s %6s %6s %6s %6s %6s %6s | %5s %5s %5s %5s %5s %5s %5s %5s  %s" % (
         "level", "node", "visitors", "kind", "start_us", "end_us", "us", "load", "thr", "ord", "emit", "settle", "part",
         "probe", "act", "srch", "cnt", "1win", "runL", "runW", "mrg", "work"))
-    names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job"}
+    names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job", 5: "chain"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
         if len(at) == 0:
             continue
         top = at[np.argmax(m[at])]
         same = at[node[at] == node[top]]
-        whole = same[(kind[same] == 0) | (kind[same] == 3)]
+        whole = same[(kind[same] == 0) | (kind[same] == 3) | (kind[same] == 5)]
         jobs = same[kind[same] == 4]
         first = whole[0] if len(whole) else same[0]
         s0, e1 = start[same].min(), end[same].max()

@@ -1,7 +1,8 @@
 // Drives omk::GPUForestMCTSEngine<State> (csrc/omk_search.h) with a mock game state that has
 // core::IGameState's method names, and omk::flattenTree with a mock node that has MCTSNode's
 // accessors.  Prints what the Python test compares with the CPU checker.
-//   search_smoke search <num_simulations> <batch_size> <widening 0|1> <noise 0|1> <temperature>
+//   search_smoke search <num_simulations> <batch_size> <widening 0|1> <noise 0|1> <temperature> [searches]
+//     (searches > 1: that many searches one after the other on ONE engine, the last one printed)
 //   search_smoke flatten
 //
 // The game: players 1 and 2 alternately take one of 12 cells; a player who takes a cell whose
@@ -75,7 +76,7 @@ struct RefNetworkOutput {
     float value = 0.0f;
 };
 
-static int run_search(int sims, int batch, bool widening, bool noise, float temperature) {
+static int run_search(int sims, int batch, bool widening, bool noise, float temperature, int searches) {
     omk::MCTSSettings s;
     s.num_simulations = sims;
     s.batch_size = batch;
@@ -106,7 +107,11 @@ static int run_search(int sims, int batch, bool widening, bool noise, float temp
     Engine engine(evaluator, s, 200000);
     RingState root;
     root.makeMove(3);  // not the empty board: the root state has a history the leaves replay on top of
-    omk::SearchResult r = engine.search(root);
+    omk::SearchResult r;
+    for (int k = 0; k < searches; k++) {
+        evaluated = 0;
+        r = engine.search(root);  // every search starts a new tree: the table's entries for the old one are gone
+    }
     printf("action %d value %.9g simulations %d nodes %lld evaluated %ld\n", r.action, r.value, r.simulations,
            (long long)r.nodes, evaluated);
     printf("table entries %lld transpositions %lld\n", (long long)r.table_entries, (long long)r.transpositions);
@@ -186,7 +191,8 @@ static int run_flatten() {
 int main(int argc, char **argv) {
     try {
         if (argc >= 7 && !strcmp(argv[1], "search"))
-            return run_search(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]) != 0, atoi(argv[5]) != 0, (float)atof(argv[6]));
+            return run_search(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]) != 0, atoi(argv[5]) != 0, (float)atof(argv[6]),
+                              argc >= 8 ? atoi(argv[7]) : 1);
         if (argc >= 2 && !strcmp(argv[1], "flatten")) return run_flatten();
     } catch (const std::exception &e) {
         fprintf(stderr, "search_smoke: %s\n", e.what());

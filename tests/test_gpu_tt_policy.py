@@ -176,3 +176,45 @@ def test_keys_set_node_by_node_from_the_game():
     with pytest.raises(omk.OmkError) as e:
         f.set_keys(np.array([0, n + 1000], np.int32), np.array([5, 6], np.uint64))
     assert e.value.code == -1, e.value       # OMK_ERR_INVALID: the id outside the forest was skipped, the other one set
+
+
+def test_entries_die_with_the_tree_they_point_into():
+    """Entries hold node ids.  A compaction renumbers the nodes and an upload of another tree replaces
+    them: whatever was stored before is then what an expired weak pointer is in the reference's table
+    (PHMapTranspositionTable::lookup erases it, src/mcts/phmap_transposition_table.cpp:100-108) and must
+    neither be found nor stand in the way of a new entry under the same key."""
+    import omoknuni_small_amd as omk
+    soa, roots = random_tree(91, n_expand=200, fanout=(2, 10), max_depth=6, n_max=40, zero_frac=0.2)
+    n = len(soa["N"])
+    f = omk.Forest.from_soa(soa, capacity=n)
+    tt = omk.TranspositionTable(f, 10)
+    rng = np.random.default_rng(5)
+    keys = rng.integers(1, 2**63, 300, dtype=np.uint64)
+    nodes = rng.integers(0, n, 300).astype(np.int32)
+    depths = rng.integers(0, 9, 300).astype(np.int32)
+    assert tt.store(keys, nodes, depths)[0] == 300
+    assert (tt.probe(keys, 0) == nodes).all()
+    # the same statistics again: ids keep their meaning, the entries stay
+    f.upload(soa)
+    assert (tt.probe(keys, 0) == nodes).all()
+    # a compaction below a child of the root renumbers the nodes
+    child = int(soa["child_begin"][0])
+    n_after = len(f.compact(child))
+    assert n_after < n
+    assert (tt.probe(keys, 0) == -1).all()
+    new_nodes = rng.integers(0, n_after, 300).astype(np.int32)
+    got = tt.store(keys, new_nodes, depths)
+    assert got[0] == 300 and got[1] == 0, got          # all new: nothing old to replace
+    assert (tt.probe(keys, 0) == new_nodes).all()
+    # another tree in the same forest: again nothing is left
+    f.upload(tiny_tree(50))
+    assert (tt.probe(keys, 0) == -1).all()
+
+
+def tiny_tree(n):
+    """A root with n - 1 leaf children."""
+    z = np.zeros(n, np.int32)
+    cb, cc = z.copy(), z.copy()
+    cb[0], cc[0] = 1, n - 1
+    return dict(N=z.copy(), W=np.zeros(n, np.float32), P=np.full(n, 1.0 / n, np.float32), VL=z.copy(),
+                child_begin=cb, child_count=cc)

@@ -59,7 +59,36 @@ def evaluate(state):
     return value, (pol / s).astype(np.float32)
 
 
-def replay_search(sims, batch, widening):
+class Mt19937:
+    """Raw 32-bit outputs of std::mt19937(seed): numpy's legacy generator is the same engine with the same
+    seeding, and a full-range draw returns its outputs one by one (5489 -> 3499211612 first)."""
+
+    def __init__(self, seed):
+        self.rs = np.random.RandomState(seed)
+
+    def __call__(self):
+        return int(self.rs.randint(0, 2 ** 32, dtype=np.uint64))
+
+
+def shuffle_moves(moves, gen):
+    """GPUForestMCTSEngine::shuffleMoves: Fisher-Yates from the last place down, j = output mod (k + 1)."""
+    for k in range(len(moves) - 1, 0, -1):
+        j = gen() % (k + 1)
+        moves[k], moves[j] = moves[j], moves[k]
+    return moves
+
+
+def replay_search(sims, batch, widening, seed=5489, searches=1):
+    """`searches` searches one after the other on one engine (the generator of the shuffles runs on, the
+    tree and the table of positions start empty every time: a table entry dies with the tree its node
+    belongs to); the last one is returned."""
+    gen = Mt19937(seed + 1)
+    for _ in range(searches):
+        ref = replay_one_search(sims, batch, widening, gen)
+    return ref
+
+
+def replay_one_search(sims, batch, widening, gen):
     root_state = Ring()
     root_state.make(3)
     z = np.zeros(1, np.int32)
@@ -96,7 +125,7 @@ def replay_search(sims, batch, widening):
             v, p = evaluate(s)
             values.append(v)
             if not s.terminal():
-                moves.extend(s.legal())
+                moves.extend(shuffle_moves(s.legal(), gen))   # the search shuffles as MCTSNode::expand does
             begin.append(len(moves))
             pol.extend(p.tolist())
             pb.append(len(pol))
@@ -139,10 +168,30 @@ def test_search_with_the_reference_signatures_matches_the_checker(widening):
     if widening:
         assert ref.child_count[0] == 8                                 # root expanded at N = 0: max(8, 2 * 1) of 11 moves
         assert ref.child_count[ref.child_count > 0].max() <= 11
+        # the children kept are a random subset of the legal moves, not the moves of lowest index at every node
+        kept = [tuple(sorted(nodes[int(b):int(b + c), 6].astype(int))) for b, c in zip(nodes[:, 4], nodes[:, 5]) if c == 8]
+        assert any(k != tuple(range(k[0], k[0] + 8)) and k[-1] > 8 for k in kept)
+        assert len({k for k in kept}) > 1
     else:
         assert ref.child_count[0] == 11
     # a terminal state is answered without a search: the side to move has lost
     assert lines[-1] == "terminal action -1 value -1 probabilities 12"
+
+
+@pytest.mark.gpu
+def test_second_search_on_one_engine_starts_from_an_empty_table():
+    """Node ids start again at 0 with every search's new tree; entries of the table that point into the old
+    tree must not be found (the reference's entries are weak pointers that die with it)."""
+    sims, batch = 150, 16
+    r = subprocess.run([EXE, "search", str(sims), str(batch), "1", "0", "0", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().split("\n")
+    table = next(ln for ln in lines if ln.startswith("table entries")).split()
+    nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
+    ref = replay_search(sims, batch, 1, searches=2)
+    assert (int(table[2]), int(table[4])) == ref.table_counts, (table, ref.table_counts)
+    assert len(nodes) == ref.n and (nodes[:, 0] == ref.N).all() and (nodes[:, 6] == ref.action).all()
 
 
 @pytest.mark.gpu
