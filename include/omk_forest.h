@@ -286,26 +286,36 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * settled one at a time, [4] nodes replayed one visitor at a time because the parallel
  * path's exactness checks did not hold, [5] threshold probes, [6] single-visitor selection
  * steps, [7] nodes settled by merging a few entries of other children into the list of the child
- * that takes nearly every visitor, [8..14] per-phase cycle counts in measurement builds (else 0),
- * [15] nodes cut into slices for several wavefronts. */
+ * that takes nearly every visitor, [8] when the first block of the persistent launch started,
+ * [9] when its last team of wavefronts left, [10] when its last walker left (low 31 bits of the
+ * device's 100 MHz clock; these three are kept whether or not the counters are on), [11] the number
+ * of walks of lone visitors inside that launch, [12..14] per-phase cycle counts in measurement builds (else 0), [15] nodes cut into
+ * slices for several wavefronts.  (Nodes taken by the walk down one-winner nodes count in [0]..[2].) */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
 /* The counters above cost one atomic per processed node (and per single-visitor step), all on
  * the same few addresses, so they are off unless switched on here (enabled != 0); with
  * them off omk_batch_stats returns zeros.  Diagnostics only; no counterpart in the reference. */
 int omk_batch_set_stats(omk_batch *b, int32_t enabled);
-/* Measurement aid, no counterpart in the reference: the timeline of the last select, one record
- * of twelve int64 per multi-visitor work item processed: start and end on the GPU's 100 MHz clock,
- * visitors | depth << 32 | item kind << 60, node | (batches | runs << 8 | entries of the last
- * batch << 16) << 32, then eight words holding two 32-bit phase times each (same clock; slots 0-7:
- * threshold phase, direct merge: counts and ranks (or 100 x the reason it was refused), evaluation
- * and ordering, emission and checks, loading and scoring the children, the whole settling of the
- * visitors, the partition, direct merge: the dominant child's list; slots 8-15, parts of these:
- * run probe, bounds and active children, threshold search, exact counts, one-winner check, length
- * search of a run, emission of a run, the direct merge as a whole).
- * h_trace has room for max_entries records.
- * Only a library built with -DOMK_TRACE (csrc/Makefile, target `trace`) records it; any other
- * build returns OMK_ERR_UNSUPPORTED and *h_n = 0. */
+/* Measurement aid, no counterpart in the reference: the timeline of the last select, switched on
+ * with omk_batch_set_trace before that select.  One record of twelve int64 per piece of work: start
+ * and end on the GPU's 100 MHz clock, visitors | depth << 32 | kind << 60 (0 a node settled as a
+ * whole, 1 a slice of a heavy node, 2 a part of its partition, 3 a node published before its visitor
+ * list was complete, 5 a node whose visitors all follow one child, taken by the walk down such nodes,
+ * 6 the walk of a lone visitor inside the persistent launch), node | (batches | runs << 8 | entries of
+ * the last batch << 16) << 32, then eight words holding two 32-bit phase times each.  The phase
+ * times and the counters beside the node are filled by a library built with -DOMK_TRACE only
+ * (csrc/Makefile, target `trace`; 0 otherwise): slots 0-7 threshold phase, direct merge: counts and
+ * ranks (or 100 x the reason it was refused), evaluation and ordering, emission and checks, loading
+ * and scoring the children, the whole settling of the visitors, the partition, direct merge: the
+ * dominant child's list; slots 8-15, parts of these: run probe, bounds and active children,
+ * threshold search, exact counts, one-winner check, length search of a run, emission of a run, the
+ * direct merge as a whole.
+ * h_trace has room for max_entries records; the records live in the staging memory of
+ * omk_batch_read until the next call of it. */
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n);
+/* Switches the recording of that timeline on or off for the selects that follow (off by default: a
+ * record costs one atomic and twelve stores per work item). */
+int omk_batch_set_trace(omk_batch *b, int32_t enabled);
 /* The multi-visitor selection kernel is persistent: its wavefronts wait for work items that
  * other wavefronts publish.  Every wait is bounded; a wavefront that polls `polls` times in
  * vain raises an abort flag, all wavefronts leave, and omk_batch_read reports OMK_ERR_STATE

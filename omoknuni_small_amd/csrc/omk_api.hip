@@ -118,6 +118,7 @@ struct omk_batch {
     int32_t *counters = nullptr;
     int32_t poll_sleep = 1;
     bool stats_on = false;
+    bool trace_on = false;  // the selection records its timeline (omk_batch_set_trace)
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
     int32_t *single_ready = nullptr;  // the same per entry of the single-visitor queue
     int32_t *hctx = nullptr;     // contexts of heavy nodes
@@ -125,10 +126,11 @@ struct omk_batch {
     int32_t hctx_cap = 0;
     int32_t q_cap = 0;
     int32_t epoch = 0;           // select calls so far
-    int32_t spin_limit = 1 << 22;
+    int32_t spin_limit = 1 << 18;  // polls of about a microsecond: a quarter of a second, a selection takes a millisecond
     int32_t n_cus = 0;
     int32_t n_items0 = 0;
     int32_t *out_paths = nullptr, *out_actions = nullptr;  // row-major staging for the host
+    int64_t out_ints = 0;  // int32 words of out_paths
     void *exp_buf = nullptr;  // staging of an expansion: jobs, moves, priors, status
     size_t exp_bytes = 0;
 };
@@ -906,7 +908,9 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->single_ready, max_traversals);
     if (e == hipSuccess) e = hipMemset(b->single_ready, 0, (size_t)std::max(max_traversals, 1) * 4);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&b->n_cus, hipDeviceAttributeMultiprocessorCount, f->device);
-    if (e == hipSuccess) e = dalloc(&b->out_paths, B * (max_depth + 1));
+    // (also the staging of the timeline records, omk_debug_trace: room for 16384 of them at least)
+    b->out_ints = std::max<int64_t>(B * (max_depth + 1), 24 * 16384);
+    if (e == hipSuccess) e = dalloc(&b->out_paths, b->out_ints);
     if (e == hipSuccess) e = dalloc(&b->out_actions, B * max_depth);
     if (e == hipSuccess) e = hipMemset(b->values, 0, (size_t)B * 4);
     if (e != hipSuccess) {
@@ -1052,10 +1056,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.hctx_cap = b->hctx_cap;
     a.list_flag = b->list_flag;
     static_assert(kHeavyCtxInts >= 16 + OMK_MAX_FANOUT, "context too small");
-#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
-    a.trace = (long long *)b->out_paths;  // staging that only omk_batch_read uses
+    a.times = b->counters + 26;
+    a.trace = b->trace_on ? (long long *)b->out_paths : nullptr;  // staging that only omk_batch_read uses
     a.trace_n = b->counters + 24;
-    a.trace_cap = (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 24);
+    a.trace_cap = (int32_t)(b->out_ints / 24);
+#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
     a.dbg_grid = getenv("OMK_DBG_GRID") ? atoi(getenv("OMK_DBG_GRID")) : 0;
 #endif
     a.singles0 = b->singles0;
@@ -1387,7 +1392,11 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_batch_stats: no selected paths");
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipMemcpyAsync(h_stats8, b->counters + 1, 64, hipMemcpyDeviceToHost, b->f->stream));
+    int32_t times[3] = {0, 0, 0};
+    HIP_TRY(hipMemcpyAsync(times, b->counters + 26, sizeof(times), hipMemcpyDeviceToHost, b->f->stream));
     HIP_TRY(hipStreamSynchronize(b->f->stream));
+    // the three time stamps are kept whether or not the counters are on
+    for (int i = 0; i < 3; i++) h_stats8[8 + i] = times[i];
     return OMK_OK;
 }
 
@@ -1395,19 +1404,22 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
 // only a build with -DOMK_TRACE records.
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
     if (!b || !h_trace || !h_n || max_entries < 0) return fail(OMK_ERR_INVALID, "omk_debug_trace: bad argument");
-#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
+    *h_n = 0;
+    if (!b->trace_on) return fail(OMK_ERR_STATE, "omk_debug_trace: switch the timeline on first (omk_batch_set_trace)");
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_debug_trace: no selected paths");
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(hipStreamSynchronize(b->f->stream));
     HIP_TRY(hipMemcpy(h_n, b->counters + 24, 4, hipMemcpyDeviceToHost));
-    int32_t n = std::min(std::min(*h_n, max_entries), (int32_t)((int64_t)b->stride * (b->max_depth + 1) / 24));
+    int32_t n = std::min(std::min(*h_n, max_entries), (int32_t)(b->out_ints / 24));
     if (n > 0) HIP_TRY(hipMemcpy(h_trace, b->out_paths, (size_t)n * 96, hipMemcpyDeviceToHost));
     *h_n = n;
     return OMK_OK;
-#else
-    *h_n = 0;
-    return fail(OMK_ERR_UNSUPPORTED, "omk_debug_trace: this library was built without -DOMK_TRACE (make trace)");
-#endif
+}
+
+int omk_batch_set_trace(omk_batch *b, int32_t enabled) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_batch_set_trace: null batch");
+    b->trace_on = enabled != 0;
+    return OMK_OK;
 }
 
 // ---------------------------------------------------------------- transposition table

@@ -60,12 +60,13 @@ struct SelectArgs {
     int32_t poll_sleep;    // s_sleep(32) units between two polls of a waiting wavefront
     int32_t q_cap;
     int32_t epoch;         // number of this select call on the batch, > 0
-#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
-    long long *trace;      // per processed node: start, end (100 MHz clock), visitors | depth << 32, node
+    long long *trace;      // nullptr, or per processed node: start, end (100 MHz clock), visitors | depth << 32 |
+                           // kind << 60, node, and eight words of phase times (measurement builds only, else 0)
     int32_t *trace_n;
     int32_t trace_cap;
-    int32_t dbg_grid;      // cap on the blocks of the multi-visitor kernel (0 = none)
-#endif
+    int32_t dbg_grid;      // cap on the blocks of the multi-visitor kernel (0 = none; measurement builds)
+    int32_t *times;        // [0] when the first block of the persistent launch started, [1] when the last team
+                           // left, [2] when the last walker left (100 MHz clock, low 31 bits)
     int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag
     int32_t *single_ready;  // per entry of the single-visitor queue: number of the select call that wrote it
     int32_t *singles_head;  // tickets of the walkers of the persistent launch

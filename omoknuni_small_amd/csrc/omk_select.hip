@@ -582,13 +582,73 @@ __device__ __forceinline__ int predict_count(int n, float w, float p, int vl, fl
     return cnt >= (float)cap ? cap : (int)cnt;
 }
 
+constexpr int kChainMin = 2;         // visitors from which a node is tried that way
+constexpr int kChainMaxLevels = 64;  // levels one walk records; a longer chain goes on as another walk
+constexpr int kChainLoaders = 3;
+
+struct ChainSlot {
+    uint32_t bk, bpos;  // best candidate among the children this wavefront loaded (key 0 = none)
+    uint32_t sk, spos;  // best candidate of its children other than that one's child
+    int n, vl;          // that child's statistics and child range
+    float w, p, q2;
+    int sx, sy;
+    uint32_t any1;      // one of its children has a real first-scan key
+};
+
+struct ChainLds {
+    ChainSlot slot[2][kChainLoaders];
+    int arrive;                  // slots written, counted over the levels of one walk
+    int levels;                  // levels walked
+    int nodes[kChainMaxLevels];  // the child taken at every one of them
+    int e_node, e_np, e_cb, e_cc, e_depth;  // where the walk stands: a node that has not been settled
+    int e_kids;       // that node's children are in the LDS scratch (it failed the one-winner test), with:
+    int e_contested;  // single_run's verdict: the best child's entry for the last visitor is real but not first,
+    int e_best0;      // that child,
+    uint32_t e_lk0;   // that entry's key,
+    int e_second;     // and whether it is a candidate of the second scan
+    // the path entries of the last walk are still to be written (chain_finish): it started at depth d_depth with
+    // the d_m visitors listed from d_off on
+    int debt, d_depth, d_off, d_m;
+};
+typedef __attribute__((address_space(3))) unsigned char *LdsBytesP;
+// one per block of the multi-visitor kernel
+__shared__ ChainLds g_chain;
+
+
+// After a walk down one-winner nodes (chain_walk): the path entries of its visitors for every level walked,
+// and their list where the node the walk stopped at reads it.  By the owner, once the list the walk started
+// from is complete: the partition that writes it ran beside the walk, and the block barrier that ends that
+// request has been passed.
+__device__ __noinline__ void chain_finish(const int32_t *seg0, int32_t *seg_a, int32_t *seg_b, int32_t *paths, int stride,
+                                          int lane) {
+    const int k = __builtin_amdgcn_readfirstlane(g_chain.levels);
+    const int d0 = __builtin_amdgcn_readfirstlane(g_chain.d_depth), off = __builtin_amdgcn_readfirstlane(g_chain.d_off);
+    const int m = __builtin_amdgcn_readfirstlane(g_chain.d_m);
+    const int32_t *src = d0 == 0 ? seg0 : (((d0 - 1) & 1) ? seg_b : seg_a);
+    int32_t *dst = ((d0 + k - 1) & 1) ? seg_b : seg_a;
+    for (int j = lane; j < m; j += kWave) {
+        const int t = src[off + j];
+        for (int i = 0; i < k; i++) paths[(size_t)(d0 + 1 + i) * stride + t] = g_chain.nodes[i];
+        if (dst != src) dst[off + j] = t;
+    }
+}
+
 // The owner may have left the partition of its previous node with a helper: the block
 // barrier that ends that request is still open.  Everything that needs the helpers, the
-// visitor lists that partition writes, or the LDS it reads, closes it first.
-__device__ __forceinline__ void close_pending(bool &pending) {
+// visitor lists that partition writes, or the LDS it reads, closes it first.  A walk down
+// one-winner nodes that ran beside that partition has its path entries written here.
+__device__ __forceinline__ void close_pending(const SelectArgs &a, bool &pending, int lane) {
     if (pending) {
         __syncthreads();
         pending = false;
+        if (__builtin_amdgcn_readfirstlane(g_chain.debt)) {
+            chain_finish(a.seg0, a.seg[0], a.seg[1], a.paths, a.stride, lane);
+            if (lane == 0) g_chain.debt = 0;
+            // what follows may read the list just written, and the debt word
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        }
     }
 }
 
@@ -1322,7 +1382,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 if (!bad_run) {
                     if (lane == 0) lds.red[2] = 0u;
                     if (L >= 2 * kTeamMin) {
-                        close_pending(pending);
+                        close_pending(a, pending, lane);
                         if (lane == 0) {
                             TeamCmd &cm = lds.cmd;
                             cm.op = kOpRun;
@@ -1614,7 +1674,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const bool team = total >= kTeamMin;
         int cur;
         if (team) {
-            close_pending(pending);
+            close_pending(a, pending, lane);
             if (lane == 0) {
                 lds.cmd.op = kOpOrder;
                 lds.cmd.rounds = R;
@@ -1648,7 +1708,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         // a node that this one batch settles keeps its winner order in LDS for the partition
         const bool only_batch = allow_lds && done == 0 && keep == m;
         if (team) {
-            close_pending(pending);
+            close_pending(a, pending, lane);
             if (lane == 0) {
                 lds.cmd.op = kOpEmit;
                 lds.cmd.rounds = R;
@@ -1661,7 +1721,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             batch_emit<R, kTeam>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
             __syncthreads();
         } else {
-            if (only_batch) close_pending(pending);  // the previous node's partition may still read the order
+            if (only_batch) close_pending(a, pending, lane);  // the previous node's partition may still read the order
             batch_emit<R, kWave>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
         }
         if (only_batch) lds_cur = 0;
@@ -2298,7 +2358,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     }
     OMK_STAMP(1);
     // ---- the winner order: the others' entries at their places, A's in between ----
-    close_pending(pending);  // the previous node's partition may still read the order buffer
+    close_pending(a, pending, lane);  // the previous node's partition may still read the order buffer
     for (int q = lane; q < m; q += kWave) order[q] = 0u;
     wave_sync_memory();
     if (valid) order[posn] = 0x80000000u | ((uint32_t)e_child << 21) | (uint32_t)e_t;
@@ -2331,67 +2391,61 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
 // ---- Chains of nodes whose visitors all follow one child ----
 // Most crowded nodes below the top of a tree are of that kind, often a dozen in a row (a whole
 // selection of the Go workload with 16 visitors per tree is a chain of 21), and on such a node nothing
-// is decided: the visitors stay together, in the same order.  The walk below does these nodes and
-// nothing else, by all wavefronts of the block in lockstep instead of one owner directing helpers: every
-// wavefront loads and scores its rounds of the children (statistics, legality bits and the child ranges
-// of all children in range in ONE trip to memory), leaves its best candidate, the best candidate of its
-// other children and the best child's statistics in LDS; after one block barrier every wavefront knows
-// the node's best child and the best candidate of all others, makes the one-winner test of single_run
-// (the entry the best child shows the LAST visitor still comes first, and its entries are in order),
-// and on success writes its share of the visitors' next path entry and moves on into the child: one
-// barrier and one dependent trip to memory per level, no partition (the visitor list does not change;
-// it is kept in registers and written once, where the walk ends, into the buffer the next node reads).
-// The walk ends at a leaf (or the depth cap) or at the first node that fails the test, which is
-// then settled the general way (select_group) from scratch.
-constexpr int kChainMin = 2;  // visitors from which a node is tried that way
+// is decided: the visitors stay together, in the same order.  chain_walk does these nodes and nothing
+// else.  On a wide layout three wavefronts of the block walk in lockstep (the owner and two helpers;
+// the third helper meanwhile shares out the visitors of the node settled before, if there is one):
+// each loads and scores its rounds of the children (statistics, legality bits and the child ranges of
+// all children in range in ONE trip to memory), leaves its best candidate, the best candidate of its
+// other children and the best child's statistics in LDS, and waits for the other two on a counter in
+// LDS (no block barrier: the fourth wavefront is busy); then each of them knows the node's best child
+// and the best candidate of all others, makes the one-winner test of single_run (the entry the best
+// child shows the LAST visitor still comes first, and its entries are in order) and moves on into the
+// child.  One dependent trip to memory per level, no partition: the visitor list does not change, so
+// the walk does not even read it; it records the children it took, and when it has stopped the whole
+// block writes the visitors' path entries for all its levels at once (chain_finish) and the list into
+// the buffer the next node reads.  The walk stops at a leaf (or the depth cap), or at the first node
+// that fails the test: that node's children, loaded and scored, are left in the LDS scratch together
+// with the verdict, and select_group settles it from there.
+// One round of a node's children, as select_group collects them from the LDS scratch of fan-out class R.
+template <int R>
+__device__ __forceinline__ void chain_dump(LdsBytesP base, int i, int n, float w, float p, int vl, float q2,
+                                           uint32_t k1, uint32_t k2, bool part) {
+    typedef __attribute__((address_space(3))) WaveLds<R> *P;
+    P l = (P)base;
+    l->st_n[i] = n;
+    l->st_w[i] = w;
+    l->st_p[i] = p;
+    l->st_vl[i] = vl;
+    l->st_q2[i] = q2;
+    l->key[0][i] = k1;
+    l->key[1][i] = k2;
+    l->pay[i] = part ? 1u : 0u;
+}
 
-struct ChainSlot {
-    uint32_t bk, bpos;  // best candidate among the children this wavefront loaded (key 0 = none)
-    uint32_t sk, spos;  // best candidate of its children other than that one's child
-    int n, vl;          // that child's statistics and child range
-    float w, p, q2;
-    int sx, sy;
-    uint32_t any1;      // one of its children has a real first-scan key
-};
-
-struct ChainEnd {
-    int node, np, cb, cc, depth;  // where the walk stands: a node that has not been settled
-};
-
-template <int RMAX, bool RAVE, int NW>
-__device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave, int lane, int node, int np, int cb,
-                                            int cc, int depth, int off, int m) {
+// li: which of the NL loaders this wavefront is (0 = the owner).
+template <int RMAX, bool RAVE, int NL>
+__device__ __noinline__ void chain_walk(ForestDev f, SelectArgs a, LdsBytesP scratch, int li, int lane, int node, int np,
+                                        int cb, int cc, int depth, int m) {
     constexpr int F = RMAX * kWave;
-    constexpr int Q = (RMAX + NW - 1) / NW;       // rounds of children per wavefront
-    constexpr int NT = NW * kWave;
-    constexpr int U = (kHeavyMin + NT - 1) / NT;  // visitors per thread, at most
-    __shared__ ChainSlot slots[2][NW];
-    const int tid = wave * kWave + lane;
+    constexpr int Q = (RMAX + NL - 1) / NL;  // rounds of children per loader: li takes rounds li*Q .. li*Q + Q - 1
     const uint32_t uvl = (uint32_t)a.vl;
-    const int d0 = depth;
-    const int32_t *src = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
-    int tt[U];
-#pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int j = tid + u * NT;
-        tt[u] = j < m ? src[off + j] : -1;
-    }
-    int par = 0;
+    int level = 0, kids = 0, contested = 0, best0 = -1, second = 0;
+    uint32_t lk0 = 0u;
     for (;;) {
-        if (cc <= 0 || depth >= a.max_depth) break;
-#ifdef OMK_TRACE
-        const long long tr0 = wall_clock64();
-#endif
+        if (cc <= 0 || depth >= a.max_depth || level >= kChainMaxLevels) break;
+        const long long tr0 = a.trace && li == 0 ? wall_clock64() : 0ll;
         int nelig = cc;
         if (a.pw) {
             const int kk = ceil_sqrt_i32(np);
             nelig = kk < cc ? kk : cc;
         }
         const float ep = a.c_puct * sqrtf((float)np);
+        const int par = level & 1;
         // ---- this wavefront's rounds of the children ----
         int kn[Q], kvl[Q];
         float kw[Q], kp[Q], kq2[Q];
         uint32_t k1[Q], k2[Q];
+        bool kin[Q];
         int2 ksp[Q];
         {
             int rn[Q];
@@ -2399,7 +2453,7 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
             uint32_t word[Q];
 #pragma unroll
             for (int q = 0; q < Q; q++) {
-                const int r = wave + q * NW;
+                const int r = li * Q + q;
                 const int i = r * kWave + lane;
                 const bool in = r < RMAX && i < nelig;
                 const int id = cb + i;
@@ -2414,15 +2468,20 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
             }
 #pragma unroll
             for (int q = 0; q < Q; q++) {
-                const int r = wave + q * NW;
+                const int r = li * Q + q;
                 const int i = r * kWave + lane;
                 const int id = cb + i;
-                const bool in = r < RMAX && i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
+                kin[q] = r < RMAX && i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
                 k1[q] = k2[q] = 0u;
                 kq2[q] = 0.0f;
-                if (in) {
+                if (kin[q]) {
                     if (RAVE) kq2[q] = combined_value(kn[q], kw[q], rn[q], rw[q], a.rave_k);
                     child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
+                } else {
+                    kn[q] = 0;
+                    kw[q] = 0.0f;
+                    kp[q] = 0.0f;
+                    kvl[q] = 0;
                 }
             }
         }
@@ -2431,27 +2490,27 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
         bool has1 = false;
 #pragma unroll
         for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
             has1 |= k1[q] != 0u;
             if (k1[q] > bk) { bk = k1[q]; bpos = i; }
         }
 #pragma unroll
         for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
             if (k2[q] > bk) { bk = k2[q]; bpos = (uint32_t)F + i; }
         }
-        uint32_t mk, mpos;
-        wave_best(bk, bpos, mk, mpos);
-        const uint32_t mine = mk == 0u ? 0xFFFFFFFFu : (mpos >= (uint32_t)F ? mpos - (uint32_t)F : mpos);
+        uint32_t hk, hp;
+        wave_best(bk, bpos, hk, hp);
+        const uint32_t mine = hk == 0u ? 0xFFFFFFFFu : (hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
         uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
 #pragma unroll
         for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
             if (i != mine && k1[q] > ok_) { ok_ = k1[q]; opos = i; }
         }
 #pragma unroll
         for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((wave + q * NW) * kWave + lane);
+            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
             if (i != mine && k2[q] > ok_) { ok_ = k2[q]; opos = (uint32_t)F + i; }
         }
         uint32_t sk, spos;
@@ -2460,7 +2519,7 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
         float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
 #pragma unroll
         for (int q = 0; q < Q; q++) {
-            if ((uint32_t)(wave + q * NW) == (mine >> 6)) {
+            if ((uint32_t)(li * Q + q) == (mine >> 6)) {
                 tn = kn[q];
                 tw = kw[q];
                 tp = kp[q];
@@ -2477,33 +2536,48 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
         float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ml));
         float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), ml));
         bool any1 = __ballot(has1) != 0ull;
-        uint32_t hk = mk, hp = mpos;
-        if (NW > 1) {
-            // ---- the same over the wavefronts of the block ----
+        bool gave_up = false;
+        if (NL > 1) {
+            // ---- the same over the loaders ----
             if (lane == 0) {
-                ChainSlot &sl = slots[par][wave];
-                sl.bk = mk;
-                sl.bpos = mpos;
-                sl.sk = sk;
-                sl.spos = spos;
-                sl.n = bn;
-                sl.vl = bvl;
-                sl.w = bw;
-                sl.p = bp;
-                sl.q2 = bq2;
-                sl.sx = bsx;
-                sl.sy = bsy;
-                sl.any1 = any1 ? 1u : 0u;
+                g_chain.slot[par][li].bk = hk;
+                g_chain.slot[par][li].bpos = hp;
+                g_chain.slot[par][li].sk = sk;
+                g_chain.slot[par][li].spos = spos;
+                g_chain.slot[par][li].n = bn;
+                g_chain.slot[par][li].vl = bvl;
+                g_chain.slot[par][li].w = bw;
+                g_chain.slot[par][li].p = bp;
+                g_chain.slot[par][li].q2 = bq2;
+                g_chain.slot[par][li].sx = bsx;
+                g_chain.slot[par][li].sy = bsy;
+                g_chain.slot[par][li].any1 = any1 ? 1u : 0u;
             }
-            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (lane == 0) __hip_atomic_fetch_add(&g_chain.arrive, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const int target = NL * (level + 1);
+            for (int spins = 0;; spins++) {
+                int v = 0;
+                if (lane == 0) v = __hip_atomic_load(&g_chain.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                v = __builtin_amdgcn_readfirstlane(v);
+                if (v >= target) break;
+                if (spins >= a.spin_limit) {  // cannot happen: the loaders take the same steps; bounded like every wait
+                    if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 5);
+                    gave_up = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            if (gave_up) break;
             hk = 0u;
             hp = 0xFFFFFFFFu;
             int won = 0;
             uint32_t a1 = 0u;
 #pragma unroll
-            for (int w = 0; w < NW; w++) {
-                const uint32_t k_ = slots[par][w].bk, p_ = slots[par][w].bpos;
-                a1 |= slots[par][w].any1;
+            for (int w = 0; w < NL; w++) {
+                const uint32_t k_ = g_chain.slot[par][w].bk, p_ = g_chain.slot[par][w].bpos;
+                a1 |= g_chain.slot[par][w].any1;
                 if (k_ != 0u && comes_before(k_, p_, hk, hp)) {
                     hk = k_;
                     hp = p_;
@@ -2514,22 +2588,21 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
             sk = 0u;
             spos = 0xFFFFFFFFu;
 #pragma unroll
-            for (int w = 0; w < NW; w++) {
-                const uint32_t k_ = w == won ? slots[par][w].sk : slots[par][w].bk;
-                const uint32_t p_ = w == won ? slots[par][w].spos : slots[par][w].bpos;
+            for (int w = 0; w < NL; w++) {
+                const uint32_t k_ = w == won ? g_chain.slot[par][w].sk : g_chain.slot[par][w].bk;
+                const uint32_t p_ = w == won ? g_chain.slot[par][w].spos : g_chain.slot[par][w].bpos;
                 if (k_ != 0u && comes_before(k_, p_, sk, spos)) {
                     sk = k_;
                     spos = p_;
                 }
             }
-            const ChainSlot &ws = slots[par][won];
-            bn = __builtin_amdgcn_readfirstlane(ws.n);
-            bvl = __builtin_amdgcn_readfirstlane(ws.vl);
-            bsx = __builtin_amdgcn_readfirstlane(ws.sx);
-            bsy = __builtin_amdgcn_readfirstlane(ws.sy);
-            bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.w)));
-            bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.p)));
-            bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.q2)));
+            bn = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].n);
+            bvl = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].vl);
+            bsx = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].sx);
+            bsy = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].sy);
+            bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].w)));
+            bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].p)));
+            bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].q2)));
             hk = (uint32_t)__builtin_amdgcn_readfirstlane((int)hk);
             hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)hp);
             sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)sk);
@@ -2537,61 +2610,106 @@ __device__ __noinline__ ChainEnd chain_walk(ForestDev f, SelectArgs a, int wave,
             any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
         }
         // ---- the one-winner test (single_run) ----
-        // (with RAVE and no real first-scan score at all the reference never runs its second scan: such a
-        // node goes the general way, which knows)
-        if (hk == 0u || (RAVE && !any1)) break;
+        bool one = hk != 0u && (!RAVE || any1);
+        // (with RAVE and no real first-scan score at all the reference never runs its second scan;
+        // select_group knows, and gets no verdict)
         const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
-        uint32_t lk, lp;
-        entry_key<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1, best, lk, lp);
-        if (lk == 0u || (sk != 0u && !comes_before(lk, lp, sk, spos))) break;
-        if (!entries_in_order<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, best, m, lane)) break;
+        if (one) {
+            uint32_t lk, lp;
+            entry_key<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1, best, lk, lp);
+            if (lk == 0u) {
+                one = false;
+            } else if (sk != 0u && !comes_before(lk, lp, sk, spos)) {
+                one = false;
+                contested = 1;
+                best0 = best;
+                lk0 = lk;
+                second = lp >= (uint32_t)F ? 1 : 0;
+            } else if (!entries_in_order<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, best, m, lane)) {
+                one = false;
+            }
+        }
+        if (!one) {
+            // the node's children, where select_group collects them (its own fan-out class)
+            kids = 1;
+            if (gave_up) kids = 0;
+            else if (cc <= kWave) {
+#pragma unroll
+                for (int q = 0; q < Q; q++)
+                    if (li * Q + q < 1)
+                        chain_dump<1>(scratch, (li * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q], k2[q],
+                                      kin[q]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < Q; q++)
+                    if (li * Q + q < RMAX)
+                        chain_dump<RMAX>(scratch, (li * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q],
+                                         k2[q], kin[q]);
+            }
+            if (NL > 1 && kids) {
+                // the owner goes on with these children at once: it waits here until all of them are there
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                if (lane == 0) __hip_atomic_fetch_add(&g_chain.arrive, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (li == 0) {
+                    const int target = NL * (level + 2);
+                    for (int spins = 0;; spins++) {
+                        int v = 0;
+                        if (lane == 0) v = __hip_atomic_load(&g_chain.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        v = __builtin_amdgcn_readfirstlane(v);
+                        if (v >= target) break;
+                        if (spins >= a.spin_limit) {
+                            if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 5);
+                            kids = 0;
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                }
+            }
+            break;
+        }
         // ---- every visitor takes that child ----
         const int child = cb + best;
-        int *path_next = a.paths + (size_t)(depth + 1) * a.stride;
-#pragma unroll
-        for (int u = 0; u < U; u++)
-            if (tt[u] >= 0) path_next[tt[u]] = child;
-        if (tid == 0) {
+        if (li == 0 && lane == 0) {
+            g_chain.nodes[level] = child;
             atomicAdd(f.VL + child, (int)(uvl * (uint32_t)m));
             if (a.stats) {
                 atomicAdd(a.stats + 0, 1);
                 atomicAdd(a.stats + 1, 1);
                 atomicAdd(a.stats + 2, m);
             }
-#ifdef OMK_TRACE
-            const int ti = atomicAdd(a.trace_n, 1);
-            if (ti < a.trace_cap) {
-                a.trace[12 * ti + 0] = tr0;
-                a.trace[12 * ti + 1] = wall_clock64();
-                a.trace[12 * ti + 2] = (long long)m | ((long long)depth << 32) | (5ll << 60);
-                a.trace[12 * ti + 3] = (long long)node;
-                for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+            if (a.trace) {
+                const int ti = atomicAdd(a.trace_n, 1);
+                if (ti < a.trace_cap) {
+                    a.trace[12 * ti + 0] = tr0;
+                    a.trace[12 * ti + 1] = wall_clock64();
+                    a.trace[12 * ti + 2] = (long long)m | ((long long)depth << 32) | (5ll << 60);
+                    a.trace[12 * ti + 3] = (long long)node;
+                    for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+                }
             }
-#endif
         }
         node = child;
         np = bn;
         cb = bsx;
         cc = bsy;
         depth++;
-        par ^= 1;
+        level++;
     }
-    // the visitor list, where the node the walk stands at reads it
-    if (depth > d0) {
-        int32_t *dst = a.seg[(depth - 1) & 1];
-        if (dst != src) {
-#pragma unroll
-            for (int u = 0; u < U; u++)
-                if (tt[u] >= 0) dst[off + tid + u * NT] = tt[u];
-        }
+    if (li == 0 && lane == 0) {
+        g_chain.levels = level;
+        g_chain.e_node = node;
+        g_chain.e_np = np;
+        g_chain.e_cb = cb;
+        g_chain.e_cc = cc;
+        g_chain.e_depth = depth;
+        g_chain.e_kids = kids;
+        g_chain.e_contested = contested;
+        g_chain.e_best0 = best0;
+        g_chain.e_lk0 = lk0;
+        g_chain.e_second = second;
     }
-    ChainEnd e;
-    e.node = node;
-    e.np = np;
-    e.cb = cb;
-    e.cc = cc;
-    e.depth = depth;
-    return e;
 }
 
 // Where the walk goes on after a multi-visitor node whose visitors all chose one child.
@@ -2602,6 +2720,7 @@ struct Continuation {
     int np;
     int2 span;  // (child_begin, child_count) of that node, loaded ahead of time
     bool ahead;  // two helpers load their share of that node's children (load_ahead), if it is a wide one
+    bool chain_open;  // the request that shares out this node's visitors also starts the walk at that node (chain_walk)
 };
 
 // All visitors of a multi-visitor item.  Records the chosen child of every visitor, bumps
@@ -2625,7 +2744,10 @@ template <int R, bool RAVE, int RMAX>
 __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
                                             const Item &item, const int32_t *seg_in, int32_t *seg_out,
                                             WaveLds<R> &lds, PartLds<RMAX> &pl, bool &pending, Continuation &next,
-                                            bool ahead) {
+                                            int preload) {
+    // preload: 0 the children are loaded here; 1 two helpers are loading their share (load_ahead); 2 a walk down
+    // one-winner nodes stopped at this node and left its children, scored, in the LDS scratch, with the verdict
+    bool ahead = preload == 1;
     OMK_T0();
     const int off = item.off, m = item.m, depth = item.depth;
     // a heavy node is settled and shared out by several wavefronts, which read its visitor
@@ -2637,7 +2759,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // the visitor list of an item of kind 3, and of the slices of one, may not be there yet:
     // whoever shares out the visitors waits for it (below), settling them does not need it
     bool list_ok = !(item.pad[0] == 3 || (item.pad[0] == 1 && ((item.pad[2] >> 30) & 1)));
-    if (m >= kHeavyMin) close_pending(pending);
+    if (m >= kHeavyMin) close_pending(a, pending, lane);
     Kids<R, RAVE> k;
     int cnt[R];
     uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
@@ -2654,10 +2776,24 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             cnt[r] = 0;
         }
     } else {
-        if (R > 1 && R == RMAX && !ahead) {
+        if (preload == 2) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int i = r * kWave + lane;
+                k.n[r] = lds.st_n[i];
+                k.w[r] = lds.st_w[i];
+                k.p[r] = lds.st_p[i];
+                k.vl[r] = lds.st_vl[i];
+                k.q2[r] = lds.st_q2[i];
+                k.k1[r] = lds.key[0][i];
+                k.k2[r] = lds.key[1][i];
+                k.part[r] = lds.pay[i] != 0u;
+                cnt[r] = 0;
+            }
+        } else if (R > 1 && R == RMAX && !ahead) {
             // a wide node from the queue: the helpers are idle (or finish the partition of the node this
             // wavefront settled last), two of them take their share of the children
-            close_pending(pending);
+            close_pending(a, pending, lane);
             if (lane == 0) {
                 TeamCmd &cm = lds.cmd;
                 cm.op = kOpLoad;
@@ -2671,11 +2807,12 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             pending = true;
             ahead = true;
         }
-        if (R > 1 && R == RMAX && ahead) {
+        if (preload == 2) {
+        } else if (R > 1 && R == RMAX && ahead) {
             // this wavefront's share of the children; the rest is in LDS once the request is closed
             constexpr int S = AheadShare<R>::kRounds;
             load_score_rounds<R, RAVE, 0, (S < R ? S : R)>(f, c.cb, c.nelig, lane, a.rave_k, c.ep, k);
-            close_pending(pending);
+            close_pending(a, pending, lane);
 #pragma unroll
             for (int r = S; r < R; r++) {
                 const int i = r * kWave + lane;
@@ -2735,7 +2872,13 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     bool contested = false;
     int best0 = -1;
     uint32_t lk0 = 0u, lp0 = 0xFFFFFFFFu;
-    if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
+    if (preload == 2) {
+        // the walk has made the one-winner test on these very children, and it failed
+        contested = __builtin_amdgcn_readfirstlane(g_chain.e_contested) != 0;
+        best0 = __builtin_amdgcn_readfirstlane(g_chain.e_best0);
+        lk0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)g_chain.e_lk0);
+        lp0 = (uint32_t)(__builtin_amdgcn_readfirstlane(g_chain.e_second) ? R * kWave + best0 : best0);
+    } else if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
         settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child, contested, best0,
                                       lk0, lp0);
     OMK_STAMP(12);
@@ -2889,7 +3032,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         run_child = -1;
         lds_cur = -1;
         const bool seq_lds = m < kHeavyMin;  // few enough visitors to keep their order in LDS
-        if (seq_lds) close_pending(pending);  // the previous node's partition may still read that buffer
+        if (seq_lds) close_pending(a, pending, lane);  // the previous node's partition may still read that buffer
         for (int done = 0; done < m; done++) {
             int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
             if (i < 0) return kStepLeaf;  // no child takes part: uniform, and then for every visitor
@@ -2943,7 +3086,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 
     // ---- partition of the visitors by chosen child ----
     // this node's visitor list is written by the previous node's partition
-    close_pending(pending);
+    close_pending(a, pending, lane);
     if (!list_ok) {
         if (!wait_list(a, off, depth, lane)) return kStepParked;
         list_ok = true;
@@ -2984,11 +3127,14 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             carry += __builtin_amdgcn_readlane(inc, 63);
         }
         const int np_next = keep >= 0 ? __builtin_amdgcn_readlane(np_keep, keep & 63) : 0;
-        // (a kept child of ordinary size is tried by chain_walk first, which loads it with the whole block)
-        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth && (int)gmax >= kHeavyMin;
+        const int off_next = keep >= 0 ? off + __builtin_amdgcn_readlane(ex_keep, keep & 63) : 0;
+        // a kept child of ordinary size: the same request starts the walk down one-winner nodes at it
+        // (chain_walk), so that the owner does not wait for this partition
+        const bool chain_next = keep >= 0 && (int)gmax < kHeavyMin && a.vl > 0;
+        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth && !chain_next;
         if (lane == 0) {
             TeamCmd &cm = lds.cmd;
-            cm.op = kOpPartition;
+            cm.op = chain_next ? kOpChain : kOpPartition;
             cm.rounds = R;
             cm.j_cb = c.cb;
             cm.j_off = off;
@@ -2999,14 +3145,25 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             cm.pre_node = ahead_next ? c.cb + keep : -1;
             cm.pre_np = np_next;
             cm.pre_cc = -1;
+            if (chain_next) {
+                cm.c_node = c.cb + keep;
+                cm.c_np = np_next;
+                cm.c_cb = keep_span.x;
+                cm.c_cc = keep_span.y;
+                cm.c_depth = depth + 1;
+                cm.c_off = off_next;
+                cm.c_m = (int)gmax;
+                g_chain.arrive = 0;
+            }
         }
-        __syncthreads();  // the request is open until close_pending
-        pending = true;
+        __syncthreads();  // the request is open until close_pending (the owner runs its part of the walk first)
+        pending = !chain_next;
         next.node = -1;
         next.ahead = false;
+        next.chain_open = chain_next;
         if (keep >= 0) {
             next.node = c.cb + keep;
-            next.off = off + __builtin_amdgcn_readlane(ex_keep, keep & 63);
+            next.off = off_next;
             next.m = (int)gmax;
             next.np = np_next;
             next.span = keep_span;
@@ -3343,29 +3500,30 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = f.N[it.node];
             for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
-        bool have_span = false, ahead = false, chain_tried = false;
+        bool have_span = false, chain_tried = false, chain_open = false;
+        int preload = 0;  // what select_group finds of the node's children (its argument of that name)
         int2 pre_span = int2{0, 0};
         for (;;) {
             const int depth = it.depth;
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
             int32_t *seg_out = a.seg[depth & 1];
+            const long long tr0 = a.trace ? wall_clock64() : 0ll;  // the timeline, when it is switched on
 #ifdef OMK_TRACE
-            const long long tr0 = wall_clock64();
             if (lane == 0) s_lds.red[3] = 0u;
             if (lane < 16) s_lds.tph[lane] = 0u;
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
-            if (!chain_tried && it.pad[0] == 0 && it.m >= kChainMin && it.m < kHeavyMin && a.vl > 0 && c.cc > 0 &&
-                depth < a.max_depth) {
-                // a plain node of ordinary size: first the walk down the nodes whose visitors all follow
-                // one child (chain_walk), by the whole block on a wide layout.  Its visitor list comes from
-                // the previous node's partition, and the helpers are needed.
-                close_pending(pending);
-                ChainEnd e;
-                if (RMAX > 1) {
+            if (chain_open || (!chain_tried && it.pad[0] == 0 && it.m >= kChainMin && it.m < kHeavyMin && a.vl > 0 &&
+                               c.cc > 0 && depth < a.max_depth)) {
+                // A plain node of ordinary size: first the walk down the nodes whose visitors all follow one
+                // child (chain_walk).  The request is open already when the partition of the node settled
+                // before carries it (select_group); otherwise it is opened here, with no partition to do.
+                if (!chain_open) {
+                    close_pending(a, pending, lane);
                     if (lane == 0) {
                         TeamCmd &cm = s_lds.cmd;
                         cm.op = kOpChain;
+                        cm.j_m = 0;
                         cm.c_node = it.node;
                         cm.c_np = it.np;
                         cm.c_cb = c.cb;
@@ -3373,53 +3531,69 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                         cm.c_depth = depth;
                         cm.c_off = it.off;
                         cm.c_m = it.m;
+                        g_chain.arrive = 0;
                     }
                     __syncthreads();
-                    e = chain_walk<RMAX, RAVE, kTeamWaves>(f, a, 0, lane, it.node, it.np, c.cb, c.cc, depth, it.off, it.m);
-                    __syncthreads();
-                } else {
-                    e = chain_walk<RMAX, RAVE, 1>(f, a, 0, lane, it.node, it.np, c.cb, c.cc, depth, it.off, it.m);
-                    wave_sync_memory();
                 }
-                it.node = __builtin_amdgcn_readfirstlane(e.node);
-                it.np = __builtin_amdgcn_readfirstlane(e.np);
-                it.depth = __builtin_amdgcn_readfirstlane(e.depth);
+                chain_open = false;
+                chain_walk<RMAX, RAVE, (RMAX > 1 ? kChainLoaders : 1)>(f, a, (LdsBytesP)&s_lds, 0, lane, it.node, it.np, c.cb,
+                                                                       c.cc, depth, it.m);
+                // The request stays open (the helper that shares out the previous node's visitors may still be
+                // at it); the walk's path entries need the list that helper writes, and are written when the
+                // request is closed (close_pending).
+                pending = true;
+                if (lane == 0) {
+                    g_chain.debt = g_chain.levels > 0 ? 1 : 0;
+                    g_chain.d_depth = depth;
+                    g_chain.d_off = it.off;
+                    g_chain.d_m = it.m;
+                }
+                wave_sync_memory();
+                it.node = __builtin_amdgcn_readfirstlane(g_chain.e_node);
+                it.np = __builtin_amdgcn_readfirstlane(g_chain.e_np);
+                it.depth = __builtin_amdgcn_readfirstlane(g_chain.e_depth);
                 have_span = true;
-                pre_span = int2{__builtin_amdgcn_readfirstlane(e.cb), __builtin_amdgcn_readfirstlane(e.cc)};
-                ahead = false;
+                pre_span = int2{__builtin_amdgcn_readfirstlane(g_chain.e_cb), __builtin_amdgcn_readfirstlane(g_chain.e_cc)};
+                preload = __builtin_amdgcn_readfirstlane(g_chain.e_kids) ? 2 : 0;
                 chain_tried = true;  // the node the walk stopped at is settled the general way
                 continue;
             }
             chain_tried = false;
+            const int preload_now = preload;
+            preload = 0;
             int status = kStepLeaf;
             Continuation next;
             next.node = -1;
             next.ahead = false;
+            next.chain_open = false;
             if (c.cc > 0 && depth < a.max_depth) {
                 if (c.cc <= kWave)
                     status = select_group<1, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out,
-                                                         reinterpret_cast<WaveLds<1> &>(s_lds), s_part, pending, next,
-                                                         false);
+                                                         reinterpret_cast<WaveLds<1> &>(s_lds), s_part, pending,
+                                                         next, preload_now == 2 ? 2 : 0);
                 else
                     status = select_group<RMAX, RAVE, RMAX>(f, a, c, lane, it, seg_in, seg_out, s_lds, s_part, pending,
-                                                            next, ahead);
+                                                            next, preload_now);
             }
-#ifdef OMK_TRACE
-            if (lane == 0) {
-                int ti = atomicAdd(a.trace_n, 1);
+            if (a.trace && lane == 0) {
+                const int ti = atomicAdd(a.trace_n, 1);
                 if (ti < a.trace_cap) {
                     a.trace[12 * ti + 0] = tr0;
                     a.trace[12 * ti + 1] = wall_clock64();
                     a.trace[12 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
+#ifdef OMK_TRACE
                     a.trace[12 * ti + 3] = (long long)it.node | ((long long)s_lds.red[3] << 32);
                     for (int q = 0; q < 8; q++)
                         a.trace[12 * ti + 4 + q] = (long long)s_lds.tph[2 * q] | ((long long)s_lds.tph[2 * q + 1] << 32);
+#else
+                    a.trace[12 * ti + 3] = (long long)it.node;
+                    for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+#endif
                 }
             }
-#endif
             if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
             if (status == kStepLeaf) {
-                close_pending(pending);  // the visitor list comes from the previous node's partition
+                close_pending(a, pending, lane);  // the visitor list comes from the previous node's partition
                 if (it.pad[0] == 3 && !wait_list(a, it.off, depth, lane)) break;
                 for (int j = lane; j < it.m; j += kWave) {
                     int t = seg_in[it.off + j];
@@ -3441,7 +3615,8 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.pad[0] = it.pad[1] = it.pad[2] = 0;
             have_span = true;
             pre_span = next.span;
-            ahead = next.ahead;
+            preload = next.ahead ? 1 : 0;
+            chain_open = next.chain_open;
         }
     }
 }
@@ -3586,15 +3761,22 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
     __shared__ WaveLds<RMAX> s_lds;
     __shared__ PartLds<RMAX> s_part;
     const int tid = threadIdx.x;
+    // three time stamps of the launch (100 MHz clock, low 31 bits): when its first block started, when the
+    // last team left, when the last walker left
+    if (blockIdx.x == 0 && tid == 0) a.times[0] = (int)(wall_clock64() & 0x7FFFFFFF);
     if ((int)blockIdx.x >= a.n_team_blocks) {
         walkers_loop<RMAX, RAVE>(f, a, tid & 63);
+        if ((tid & 63) == 0) atomicMax(a.times + 2, (int)(wall_clock64() & 0x7FFFFFFF));
         return;
     }
     if (tid < kWave) {
         // every path out of the owner's loop comes back here: the helpers are always released
         bool pending = false;
+        if (tid == 0) g_chain.debt = 0;
+        wave_sync_memory();
         owner_loop<RMAX, RAVE>(f, a, s_lds, s_part, pending, tid);
-        close_pending(pending);
+        close_pending(a, pending, tid);
+        if (tid == 0) atomicMax(a.times + 1, (int)(wall_clock64() & 0x7FFFFFFF));
         if (tid == 0) s_lds.cmd.op = kOpExit;
         __syncthreads();
         return;
@@ -3610,15 +3792,26 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const int cur = __builtin_amdgcn_readfirstlane(s_lds.cmd.cur);
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
-        if (RMAX > 1 && op == kOpChain) {
+        if (op == kOpChain) {
+            // a walk down one-winner nodes by the owner and, on a wide layout, two helpers, while the
+            // remaining helper shares out the visitors of the node settled before (if the request
+            // carries one)
             const TeamCmd &cm = s_lds.cmd;
-            chain_walk<RMAX, RAVE, kTeamWaves>(f, a, tid >> 6, tid & 63, __builtin_amdgcn_readfirstlane(cm.c_node),
-                                               __builtin_amdgcn_readfirstlane(cm.c_np),
-                                               __builtin_amdgcn_readfirstlane(cm.c_cb),
-                                               __builtin_amdgcn_readfirstlane(cm.c_cc),
-                                               __builtin_amdgcn_readfirstlane(cm.c_depth),
-                                               __builtin_amdgcn_readfirstlane(cm.c_off),
-                                               __builtin_amdgcn_readfirstlane(cm.c_m));
+            const int wv = tid >> 6;
+            if (wv == 1) {
+                if (__builtin_amdgcn_readfirstlane(cm.j_m) > 0) {
+                    if (rounds == 1) partition_async<1, RMAX>(f, a, cm, s_part, tid & 63);
+                    else partition_async<RMAX, RMAX>(f, a, cm, s_part, tid & 63);
+                }
+            } else if (RMAX > 1) {
+                chain_walk<RMAX, RAVE, kChainLoaders>(f, a, (LdsBytesP)&s_lds, wv - 1, tid & 63,
+                                                      __builtin_amdgcn_readfirstlane(cm.c_node),
+                                                      __builtin_amdgcn_readfirstlane(cm.c_np),
+                                                      __builtin_amdgcn_readfirstlane(cm.c_cb),
+                                                      __builtin_amdgcn_readfirstlane(cm.c_cc),
+                                                      __builtin_amdgcn_readfirstlane(cm.c_depth),
+                                                      __builtin_amdgcn_readfirstlane(cm.c_m));
+            }
             __syncthreads();  // the request is done
             continue;
         }
@@ -3758,8 +3951,20 @@ __device__ __noinline__ void walkers_loop(ForestDev f, SelectArgs a, int lane) {
         if (!got) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         const Item it = a.singles_q[ticket];
+        const long long tr0 = a.trace ? wall_clock64() : 0ll;
         if (a.fast_singles) walk_single<RMAX, RAVE, 2>(f, a, it, lane);
         else walk_single<RMAX, RAVE, 0>(f, a, it, lane);
+        if (a.stats && lane == 0) atomicAdd(a.stats + 11, 1);
+        if (a.trace && lane == 0) {  // the timeline: a lone visitor's walk, kind 6
+            const int ti = atomicAdd(a.trace_n, 1);
+            if (ti < a.trace_cap) {
+                a.trace[12 * ti + 0] = tr0;
+                a.trace[12 * ti + 1] = wall_clock64();
+                a.trace[12 * ti + 2] = 1ll | ((long long)it.depth << 32) | (6ll << 60);
+                a.trace[12 * ti + 3] = (long long)it.node;
+                for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+            }
+        }
     }
 }
 
@@ -3778,11 +3983,10 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         a.sched_wait[0] = open0;
         a.sched_wait[1] = 0;
         *a.hctx_n = 0;
-#ifdef OMK_TRACE
         *a.trace_n = 0;
-#endif
     }
     if (a.stats && gid < 16) a.stats[gid] = 0;
+    if (gid < 3) a.times[gid] = 0;
     for (int i = gid; i < n_items0; i += step) {
         a.items_q[i] = a.items0[i];
         a.q_ready[i] = a.epoch;

@@ -27,7 +27,7 @@ EXPORTS = [
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_set_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy", "omk_soa_count_legal", "omk_soa_compact_legal",
 ]
@@ -444,12 +444,17 @@ class Batch:
         out = np.zeros(16, np.int32)
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
-                "replayed_nodes", "threshold_probes", "single_visitor_steps", "merged_nodes", "cyc_threshold",
-                "cyc_evaluate", "cyc_sort", "cyc_emit", "cyc_load", "cyc_settle", "cyc_partition", "sliced_nodes")
+                "replayed_nodes", "threshold_probes", "single_visitor_steps", "merged_nodes", "t_first_block",
+                "t_last_team", "t_last_walker", "walks_in_launch", "cyc_load", "cyc_settle", "cyc_partition",
+                "sliced_nodes")
         return dict(zip(keys, map(int, out)))
 
+    def enable_trace(self, on=True):
+        """The selects that follow record their timeline (see debug_trace())."""
+        _check(self._lib.omk_batch_set_trace(self._h, C.c_int32(1 if on else 0)))
+
     def debug_trace(self, max_entries=1 << 16):
-        """Timeline of the last select() from a library built with -DOMK_TRACE: int64 array [n, 12] of
+        """Timeline of the last select() after enable_trace(): int64 array [n, 12] of
         (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | counters << 32 and
         eight words of two 32-bit phase times each (see omk_debug_trace in the header)."""
         buf = np.zeros((int(max_entries), 12), np.int64)

@@ -130,8 +130,11 @@ def timeline(workload, warmup=8, levels=()):
     for _ in range(int(warmup)):
         batch.select(sp)
         batch.backup(vl)
+    batch.enable_trace()
     batch.select(sp)
     tr = batch.debug_trace()
+    batch.enable_trace(False)
+    batch.read()  # reports a selection that was given up (and reuses the staging memory the records were in)
     batch.backup(vl)
     t0 = tr[:, 0].min()
     start = (tr[:, 0] - t0) / 100.0  # microseconds
@@ -141,8 +144,18 @@ def timeline(workload, warmup=8, levels=()):
     kind = ((tr[:, 2] >> 60) & 7).astype(np.int64)
     node = (tr[:, 3] & 0xFFFFFFFF).astype(np.int64)
     ctr = (tr[:, 3] >> 32) & 0xFFFFFFFF
+    walks = kind == 6  # lone visitors walked by the walker blocks of the persistent launch
+    w_start, w_end, w_depth = start[walks], end[walks], depth[walks]
+    span_all = end.max()
+    keep = ~walks
+    tr, start, end, m, depth, kind, node, ctr = tr[keep], start[keep], end[keep], m[keep], depth[keep], kind[keep], node[keep], ctr[keep]
     print("workload %s, selection number %d: %d multi-visitor items traced, span %.1f us (100 MHz clock)"
           % (workload, int(warmup) + 1, len(tr), end.max()))
+    if len(w_end):
+        dur = w_end - w_start
+        print("lone visitors walked inside the persistent launch: %d walks, first start %.1f us, last end %.1f us "
+              "(median walk %.1f us, longest %.1f us, median start depth %d); everything ended at %.1f us"
+              % (len(w_end), w_start.min(), w_end.max(), float(np.median(dur)), dur.max(), int(np.median(w_depth)), span_all))
     print("chain of crowded nodes: per level the node with most visitors (kinds: node = taken as a whole, chain = a node whose visitors all follow one child, taken by the walk down such nodes, "
           "early = published before its visitor list was complete; a node cut into slices / scatter parts shows "
           "their number and the span from the first start to the last end)")
