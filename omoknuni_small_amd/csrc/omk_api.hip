@@ -52,6 +52,11 @@ struct omk_forest {
     int2 *span = nullptr;
     int32_t *N = nullptr, *VL = nullptr, *rN = nullptr, *action = nullptr;
     float *W = nullptr, *P = nullptr, *rW = nullptr;
+    // RAVE blend per node (ForestDev::q2): valid for the RAVE constant blend_k while blend_valid; whatever
+    // changes N, W, rN or rW of nodes refreshes it or clears the flag
+    float *Q2 = nullptr;
+    bool blend_valid = false, blend_k_known = false;
+    float blend_k = 0.0f;
     uint32_t *legal = nullptr;
     uint64_t *hash = nullptr;
     bool has_legal = false, has_action = false, has_hash = false;
@@ -69,6 +74,7 @@ struct omk_forest {
         m.VL = VL;
         m.rN = has_rave ? rN : nullptr;
         m.rW = has_rave ? rW : nullptr;
+        m.q2 = has_rave ? Q2 : nullptr;
         m.legal = has_legal ? legal : nullptr;
         m.action = has_action ? action : nullptr;
         m.hash = has_hash ? hash : nullptr;
@@ -84,6 +90,7 @@ struct omk_forest {
         d.VL = VL;
         d.rN = has_rave ? rN : nullptr;
         d.rW = has_rave ? rW : nullptr;
+        d.q2 = has_rave ? Q2 : nullptr;
         d.legal = has_legal ? legal : nullptr;
         d.action = has_action ? action : nullptr;
         d.hash = has_hash ? hash : nullptr;
@@ -223,6 +230,7 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
     if (e == hipSuccess) e = dalloc(&f->VL, n);
     if (e == hipSuccess && f->has_rave) e = dalloc(&f->rN, n);
     if (e == hipSuccess && f->has_rave) e = dalloc(&f->rW, n);
+    if (e == hipSuccess && f->has_rave) e = dalloc(&f->Q2, n);
     if (e != hipSuccess) {
         int rc = fail(OMK_ERR_HIP, "omk_forest_create: %s", hipGetErrorString(e));
         omk_forest_destroy(f);
@@ -236,7 +244,7 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
 static void forest_free(omk_forest *f) {
     (void)hipSetDevice(f->device);
     if (f->own_stream) (void)hipStreamSynchronize(f->own_stream);
-    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->action, f->legal, f->hash, f->key_stage};
+    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->Q2, f->action, f->legal, f->hash, f->key_stage};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     if (f->own_stream) (void)hipStreamDestroy(f->own_stream);
@@ -371,6 +379,13 @@ int omk_forest_upload(omk_forest *f, const omk_soa_view *v) {
     f->max_fanout = mf;
     f->prior_sorted = sorted;
     f->uploaded = true;
+    // the RAVE blend of every node from the new statistics, for the constant the selections have been using
+    // (a first selection, or one with another constant, computes it itself)
+    f->blend_valid = false;
+    if (f->has_rave && f->blend_k_known) {
+        HIP_TRY(launch_blend_all(f->dev(), f->blend_k, s));
+        f->blend_valid = true;
+    }
     return OMK_OK;
 }
 
@@ -733,6 +748,7 @@ static int compact_in(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, i
     if (f->has_rave) {
         move_words(f->rN);
         move_words(f->rW);
+        move_words(f->Q2);  // the nodes keep their statistics, hence their RAVE blend
     }
     if (f->has_action) move_words(f->action);
     if (e == hipSuccess && f->has_hash) {
@@ -1019,6 +1035,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
                     "omk_select_batch: progressive widening needs children stored in prior-descending order "
                     "and no legal mask");
     if (int rc = use_device(f)) return rc;
+    if (p->use_rave && (!f->blend_valid || !f->blend_k_known || f->blend_k != p->rave_k)) {
+        HIP_TRY(launch_blend_all(f->dev(), p->rave_k, f->stream));
+        f->blend_valid = f->blend_k_known = true;
+        f->blend_k = p->rave_k;
+    }
     SelectArgs a;
     memset(&a, 0, sizeof(a));
     a.items0 = b->items0;
@@ -1089,6 +1110,10 @@ int omk_backup_batch(omk_batch *b, int32_t virtual_loss) {
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_backup(b->f->dev(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
                           virtual_loss, b->f->stream));
+    // N and W of the nodes on the paths have changed: their RAVE blend with them
+    if (b->f->has_rave && b->f->blend_valid)
+        HIP_TRY(launch_blend_paths(b->f->dev(), b->paths, b->path_len, b->n, b->stride, b->max_depth + 1, b->f->blend_k,
+                                   b->f->stream));
     return OMK_OK;
 }
 
@@ -1100,6 +1125,7 @@ int omk_backup_rave_batch(omk_batch *b) {
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_rave_backup(b->f->mut(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
                                b->f->stream));
+    b->f->blend_valid = false;  // rN and rW of children of path nodes have changed: the next selection starts over
     return OMK_OK;
 }
 
@@ -1141,6 +1167,8 @@ int omk_backup_paths(omk_forest *f, const int32_t *d_paths, const int32_t *d_pat
     if (int rc = check_paths_args("omk_backup_paths", f, d_paths, d_path_len, n, stride, max_len)) return rc;
     if (!d_values) return fail(OMK_ERR_INVALID, "omk_backup_paths: null values");
     HIP_TRY(launch_backup(f->dev(), d_paths, d_path_len, d_values, n, stride, max_len, virtual_loss, f->stream));
+    if (f->has_rave && f->blend_valid)
+        HIP_TRY(launch_blend_paths(f->dev(), d_paths, d_path_len, n, stride, max_len, f->blend_k, f->stream));
     return OMK_OK;
 }
 

@@ -17,6 +17,8 @@
 // too small" reaches it without a lock (after the first clamp fires the value never
 // rises above 0 again, and the last operation on the address is always a clamp or a
 // subtract that stayed non-negative).
+#include <algorithm>
+
 #include "omk_internal.h"
 
 namespace omk {
@@ -200,6 +202,7 @@ __global__ __launch_bounds__(64) void k_expand(ForestMut f, const ExpandJob *job
         f.VL[id] = 0;
         if (f.rN) f.rN[id] = 0;
         if (f.rW) f.rW[id] = 0.0f;
+        if (f.q2) f.q2[id] = 0.0f;  // getCombinedValue of a node without visits of either kind
         f.span[id] = int2{0, 0};
         if (f.action) f.action[id] = moves[job.off + i];
         if (f.hash) f.hash[id] = ~0ull;  // no position key yet (omk_forest_set_keys)
@@ -340,6 +343,42 @@ hipError_t launch_backup(const ForestDev &f, const int32_t *paths, const int32_t
     if (n <= 0 || max_len <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_backup, dim3((n + 255) / 256, max_len), dim3(256), 0, s, f, paths, path_len, values, n,
                        stride, vl);
+    return hipGetLastError();
+}
+
+// ---- the RAVE blend kept per node ----
+// MCTSNode::getCombinedValue (reference src/mcts/mcts_node.cpp:657-678) is a function of the node's own N, W,
+// rN, rW and the RAVE constant; virtual loss does not enter.  A selection reads it for every child of every
+// node visited (three divisions and a square root each), and between two backups it does not change: it is
+// kept in f.q2, computed by the same function from the same binary32 inputs as the selection would, by
+// whatever changes one of the four (upload, backup; a node created by an expansion starts at 0).
+__global__ void k_blend_all(ForestDev f, float rave_k) {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < f.n_nodes; i += (int64_t)gridDim.x * blockDim.x)
+        f.q2[i] = combined_value(f.N[i], f.W[i], f.rN[i], f.rW[i], rave_k);
+}
+
+__global__ void k_blend_paths(ForestDev f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                              float rave_k) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int d = blockIdx.y;
+    if (t >= n || d >= path_len[t]) return;
+    const int node = paths[(size_t)d * stride + t];
+    if (node < 0 || node >= f.n_nodes) return;
+    f.q2[node] = combined_value(f.N[node], f.W[node], f.rN[node], f.rW[node], rave_k);
+}
+
+hipError_t launch_blend_all(const ForestDev &f, float rave_k, hipStream_t s) {
+    if (!f.q2 || f.n_nodes <= 0) return hipSuccess;
+    const int64_t blocks = std::min<int64_t>((f.n_nodes + 255) / 256, 1 << 16);
+    hipLaunchKernelGGL(k_blend_all, dim3((unsigned)blocks), dim3(256), 0, s, f, rave_k);
+    return hipGetLastError();
+}
+
+hipError_t launch_blend_paths(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                              int max_len, float rave_k, hipStream_t s) {
+    if (!f.q2 || n <= 0 || max_len <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_blend_paths, dim3((n + 255) / 256, max_len), dim3(256), 0, s, f, paths, path_len, n, stride,
+                       rave_k);
     return hipGetLastError();
 }
 

@@ -17,6 +17,9 @@ struct ForestDev {
     int32_t *VL;
     const int32_t *rN;
     const float *rW;
+    // RAVE blend of every node (MCTSNode::getCombinedValue: a function of the node's own N, W, rN, rW and the
+    // RAVE constant, not of virtual loss), kept by whatever changes these four; nullptr without RAVE arrays
+    float *q2;
     const uint32_t *legal;  // nullptr = every slot holds a child
     const int32_t *action;  // nullptr = node id
     const uint64_t *hash;   // nullptr = none
@@ -99,6 +102,11 @@ hipError_t launch_revert_vl(const ForestDev &f, const int32_t *paths, const int3
                             int max_len, int vl, hipStream_t s);
 hipError_t launch_backup(const ForestDev &f, const int32_t *paths, const int32_t *path_len, const float *values,
                          int n, int stride, int max_len, int vl, hipStream_t s);
+// The per-node RAVE blend f.q2 from the node's statistics as they are: of every node, or of the nodes on the
+// paths given (after a backup has changed their N and W).
+hipError_t launch_blend_all(const ForestDev &f, float rave_k, hipStream_t s);
+hipError_t launch_blend_paths(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
+                              int max_len, float rave_k, hipStream_t s);
 // row-major copies for the host: paths [n][max_depth+1], actions [n][max_depth], -1 padded
 hipError_t launch_export(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                          int max_depth, int32_t *out_paths, int32_t *out_actions, hipStream_t s);
@@ -120,6 +128,7 @@ struct ForestMut {
     int32_t *VL;
     int32_t *rN;
     float *rW;
+    float *q2;
     uint32_t *legal;
     int32_t *action;
     uint64_t *hash;

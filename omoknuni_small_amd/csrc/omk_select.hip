@@ -53,6 +53,7 @@
 // create them (one wavefront per walk, no LDS); a batch whose traversals are all alone at
 // their roots is one launch of the single-visitor kernel instead.
 #include <algorithm>
+#include <cstddef>
 
 #include "omk_internal.h"
 
@@ -241,8 +242,6 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
                                           Kids<R, RAVE> &k, int2 *sp = nullptr) {
     static_assert(AHEAD || !SPAN, "the child ranges are only fetched by the look-ahead variant");
     if (AHEAD) {
-        int rn[R];
-        float rw[R];
         uint32_t word[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -254,8 +253,7 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
             k.w[r] = in ? f.W[id] : 0.0f;
             k.p[r] = in ? f.P[id] : 0.0f;
             k.vl[r] = in ? f.VL[id] : 0;
-            rn[r] = RAVE && in ? f.rN[id] : 0;
-            rw[r] = RAVE && in ? f.rW[id] : 0.0f;
+            k.q2[r] = RAVE && in ? f.q2[id] : 0.0f;  // the RAVE blend, kept per node (k_blend_all, k_blend_paths)
             if (SPAN) sp[r] = in ? f.span[id] : int2{0, 0};
         }
 #pragma unroll
@@ -269,10 +267,8 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
                 k.w[r] = 0.0f;
                 k.p[r] = 0.0f;
                 k.vl[r] = 0;
-                rn[r] = 0;
-                rw[r] = 0.0f;
+                k.q2[r] = 0.0f;
             }
-            k.q2[r] = RAVE ? combined_value(k.n[r], k.w[r], rn[r], rw[r], rave_k) : 0.0f;
         }
         return;
     }
@@ -287,12 +283,7 @@ __device__ __forceinline__ void load_kids(const ForestDev &f, int cb, int nelig,
         k.w[r] = in ? f.W[id] : 0.0f;
         k.p[r] = in ? f.P[id] : 0.0f;
         k.vl[r] = in ? f.VL[id] : 0;
-        k.q2[r] = 0.0f;
-        if (RAVE) {
-            int rn = in ? f.rN[id] : 0;
-            float rw = in ? f.rW[id] : 0.0f;
-            k.q2[r] = combined_value(k.n[r], k.w[r], rn, rw, rave_k);
-        }
+        k.q2[r] = RAVE && in ? f.q2[id] : 0.0f;
     }
 }
 
@@ -309,8 +300,6 @@ __device__ __forceinline__ void score_round(Kids<R, RAVE> &k, int r, float ep) {
 template <int R, bool RAVE, int R0, int R1>
 __device__ __forceinline__ void load_score_rounds(const ForestDev &f, int cb, int nelig, int lane, float rave_k,
                                                   float ep, Kids<R, RAVE> &k) {
-    int rn[R];
-    float rw[R];
     uint32_t word[R];
 #pragma unroll
     for (int r = R0; r < R1; r++) {
@@ -322,8 +311,7 @@ __device__ __forceinline__ void load_score_rounds(const ForestDev &f, int cb, in
         k.w[r] = in ? f.W[id] : 0.0f;
         k.p[r] = in ? f.P[id] : 0.0f;
         k.vl[r] = in ? f.VL[id] : 0;
-        rn[r] = RAVE && in ? f.rN[id] : 0;
-        rw[r] = RAVE && in ? f.rW[id] : 0.0f;
+        k.q2[r] = RAVE && in ? f.q2[id] : 0.0f;
     }
 #pragma unroll
     for (int r = R0; r < R1; r++) {
@@ -336,10 +324,8 @@ __device__ __forceinline__ void load_score_rounds(const ForestDev &f, int cb, in
             k.w[r] = 0.0f;
             k.p[r] = 0.0f;
             k.vl[r] = 0;
-            rn[r] = 0;
-            rw[r] = 0.0f;
+            k.q2[r] = 0.0f;
         }
-        k.q2[r] = RAVE ? combined_value(k.n[r], k.w[r], rn[r], rw[r], rave_k) : 0.0f;
         score_round<R, RAVE>(k, r, ep);
     }
 }
@@ -582,22 +568,9 @@ __device__ __forceinline__ int predict_count(int n, float w, float p, int vl, fl
     return cnt >= (float)cap ? cap : (int)cnt;
 }
 
-constexpr int kChainMin = 2;         // visitors from which a node is tried that way
 constexpr int kChainMaxLevels = 64;  // levels one walk records; a longer chain goes on as another walk
-constexpr int kChainLoaders = 3;
-
-struct ChainSlot {
-    uint32_t bk, bpos;  // best candidate among the children this wavefront loaded (key 0 = none)
-    uint32_t sk, spos;  // best candidate of its children other than that one's child
-    int n, vl;          // that child's statistics and child range
-    float w, p, q2;
-    int sx, sy;
-    uint32_t any1;      // one of its children has a real first-scan key
-};
 
 struct ChainLds {
-    ChainSlot slot[2][kChainLoaders];
-    int arrive;                  // slots written, counted over the levels of one walk
     int levels;                  // levels walked
     int nodes[kChainMaxLevels];  // the child taken at every one of them
     int e_node, e_np, e_cb, e_cc, e_depth;  // where the walk stands: a node that has not been settled
@@ -606,49 +579,21 @@ struct ChainLds {
     int e_best0;      // that child,
     uint32_t e_lk0;   // that entry's key,
     int e_second;     // and whether it is a candidate of the second scan
-    // the path entries of the last walk are still to be written (chain_finish): it started at depth d_depth with
-    // the d_m visitors listed from d_off on
-    int debt, d_depth, d_off, d_m;
+    int part_done;    // the helper that shares out the visitors of the node settled before has finished: the list the
+                      // walk started from is complete
 };
 typedef __attribute__((address_space(3))) unsigned char *LdsBytesP;
 // one per block of the multi-visitor kernel
 __shared__ ChainLds g_chain;
 
 
-// After a walk down one-winner nodes (chain_walk): the path entries of its visitors for every level walked,
-// and their list where the node the walk stopped at reads it.  By the owner, once the list the walk started
-// from is complete: the partition that writes it ran beside the walk, and the block barrier that ends that
-// request has been passed.
-__device__ __noinline__ void chain_finish(const int32_t *seg0, int32_t *seg_a, int32_t *seg_b, int32_t *paths, int stride,
-                                          int lane) {
-    const int k = __builtin_amdgcn_readfirstlane(g_chain.levels);
-    const int d0 = __builtin_amdgcn_readfirstlane(g_chain.d_depth), off = __builtin_amdgcn_readfirstlane(g_chain.d_off);
-    const int m = __builtin_amdgcn_readfirstlane(g_chain.d_m);
-    const int32_t *src = d0 == 0 ? seg0 : (((d0 - 1) & 1) ? seg_b : seg_a);
-    int32_t *dst = ((d0 + k - 1) & 1) ? seg_b : seg_a;
-    for (int j = lane; j < m; j += kWave) {
-        const int t = src[off + j];
-        for (int i = 0; i < k; i++) paths[(size_t)(d0 + 1 + i) * stride + t] = g_chain.nodes[i];
-        if (dst != src) dst[off + j] = t;
-    }
-}
-
 // The owner may have left the partition of its previous node with a helper: the block
 // barrier that ends that request is still open.  Everything that needs the helpers, the
-// visitor lists that partition writes, or the LDS it reads, closes it first.  A walk down
-// one-winner nodes that ran beside that partition has its path entries written here.
-__device__ __forceinline__ void close_pending(const SelectArgs &a, bool &pending, int lane) {
+// visitor lists that partition writes, or the LDS it reads, closes it first.
+__device__ __forceinline__ void close_pending(bool &pending) {
     if (pending) {
         __syncthreads();
         pending = false;
-        if (__builtin_amdgcn_readfirstlane(g_chain.debt)) {
-            chain_finish(a.seg0, a.seg[0], a.seg[1], a.paths, a.stride, lane);
-            if (lane == 0) g_chain.debt = 0;
-            // what follows may read the list just written, and the debt word
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        }
     }
 }
 
@@ -1382,7 +1327,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 if (!bad_run) {
                     if (lane == 0) lds.red[2] = 0u;
                     if (L >= 2 * kTeamMin) {
-                        close_pending(a, pending, lane);
+                        close_pending(pending);
                         if (lane == 0) {
                             TeamCmd &cm = lds.cmd;
                             cm.op = kOpRun;
@@ -1674,7 +1619,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const bool team = total >= kTeamMin;
         int cur;
         if (team) {
-            close_pending(a, pending, lane);
+            close_pending(pending);
             if (lane == 0) {
                 lds.cmd.op = kOpOrder;
                 lds.cmd.rounds = R;
@@ -1708,7 +1653,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         // a node that this one batch settles keeps its winner order in LDS for the partition
         const bool only_batch = allow_lds && done == 0 && keep == m;
         if (team) {
-            close_pending(a, pending, lane);
+            close_pending(pending);
             if (lane == 0) {
                 lds.cmd.op = kOpEmit;
                 lds.cmd.rounds = R;
@@ -1721,7 +1666,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             batch_emit<R, kTeam>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
             __syncthreads();
         } else {
-            if (only_batch) close_pending(a, pending, lane);  // the previous node's partition may still read the order
+            if (only_batch) close_pending(pending);  // the previous node's partition may still read the order
             batch_emit<R, kWave>(a, lds, order, lane, total, keep, only_batch ? -1 : off + done, cur);
         }
         if (only_batch) lds_cur = 0;
@@ -2358,7 +2303,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     }
     OMK_STAMP(1);
     // ---- the winner order: the others' entries at their places, A's in between ----
-    close_pending(a, pending, lane);  // the previous node's partition may still read the order buffer
+    close_pending(pending);  // the previous node's partition may still read the order buffer
     for (int q = lane; q < m; q += kWave) order[q] = 0u;
     wave_sync_memory();
     if (valid) order[posn] = 0x80000000u | ((uint32_t)e_child << 21) | (uint32_t)e_t;
@@ -2390,22 +2335,19 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
 
 // ---- Chains of nodes whose visitors all follow one child ----
 // Most crowded nodes below the top of a tree are of that kind, often a dozen in a row (a whole
-// selection of the Go workload with 16 visitors per tree is a chain of 21), and on such a node nothing
-// is decided: the visitors stay together, in the same order.  chain_walk does these nodes and nothing
-// else.  On a wide layout three wavefronts of the block walk in lockstep (the owner and two helpers;
-// the third helper meanwhile shares out the visitors of the node settled before, if there is one):
-// each loads and scores its rounds of the children (statistics, legality bits and the child ranges of
-// all children in range in ONE trip to memory), leaves its best candidate, the best candidate of its
-// other children and the best child's statistics in LDS, and waits for the other two on a counter in
-// LDS (no block barrier: the fourth wavefront is busy); then each of them knows the node's best child
-// and the best candidate of all others, makes the one-winner test of single_run (the entry the best
-// child shows the LAST visitor still comes first, and its entries are in order) and moves on into the
-// child.  One dependent trip to memory per level, no partition: the visitor list does not change, so
-// the walk does not even read it; it records the children it took, and when it has stopped the whole
-// block writes the visitors' path entries for all its levels at once (chain_finish) and the list into
-// the buffer the next node reads.  The walk stops at a leaf (or the depth cap), or at the first node
-// that fails the test: that node's children, loaded and scored, are left in the LDS scratch together
-// with the verdict, and select_group settles it from there.
+// selection of the Go workload with 16 visitors per tree starts with a chain of them), and on such a
+// node nothing is decided: the visitors stay together, in the same order.  chain_walk does these nodes
+// and nothing else, by the owner wavefront alone, while a helper shares out the visitors of the node
+// settled before (if there is one): it loads and scores the children (statistics, legality bits and
+// the child ranges of all children in range in ONE trip to memory), makes the one-winner test of
+// single_run (the entry the best child shows the LAST visitor still comes first, and its entries are in
+// order) and moves on into the child.  One dependent trip to memory per level, no block barrier, no
+// partition: the visitor list does not change, so the walk does not even read it; it records the children
+// it took, and the visitors' path entries for all its levels are written at once when the request that
+// runs beside it is closed (close_pending: chain_finish), together with the list in the buffer the next
+// node reads.  The walk stops at a leaf (or the depth cap), or at the first node that fails the test:
+// that node's children, loaded and scored, are left in the LDS scratch together with the verdict, and
+// select_group settles it from there.
 // One round of a node's children, as select_group collects them from the LDS scratch of fan-out class R.
 template <int R>
 __device__ __forceinline__ void chain_dump(LdsBytesP base, int i, int n, float w, float p, int vl, float q2,
@@ -2422,199 +2364,143 @@ __device__ __forceinline__ void chain_dump(LdsBytesP base, int i, int n, float w
     l->pay[i] = part ? 1u : 0u;
 }
 
-// li: which of the NL loaders this wavefront is (0 = the owner).
-template <int RMAX, bool RAVE, int NL>
-__device__ __noinline__ void chain_walk(ForestDev f, SelectArgs a, LdsBytesP scratch, int li, int lane, int node, int np,
-                                        int cb, int cc, int depth, int m) {
+// The kernel's arguments where the hardware put them: a function that is not inlined reads what it needs
+// from there (scalar loads through the constant cache) instead of receiving copies through the stack,
+// which cost a round trip to memory at every call.
+struct SelectKernArgs {
+    ForestDev f;
+    SelectArgs a;
+};
+typedef const __attribute__((address_space(4))) SelectKernArgs *KernArgsP;
+static_assert(offsetof(SelectKernArgs, a) == sizeof(ForestDev),
+              "k_select_groups(ForestDev, SelectArgs): the second argument follows the first");
+
+template <int RMAX, bool RAVE>
+__device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lane, int node, int np, int cb, int cc,
+                                        int depth, int m) {
     constexpr int F = RMAX * kWave;
-    constexpr int Q = (RMAX + NL - 1) / NL;  // rounds of children per loader: li takes rounds li*Q .. li*Q + Q - 1
-    const uint32_t uvl = (uint32_t)a.vl;
+    const int32_t *const fN = ka->f.N, *const fVL = ka->f.VL;
+    const float *const fW = ka->f.W, *const fP = ka->f.P, *const fq2 = ka->f.q2;
+    const uint32_t *const flegal = ka->f.legal;
+    const int2 *const fspan = ka->f.span;
+    const int max_depth = ka->a.max_depth, pw = ka->a.pw;
+    const float c_puct = ka->a.c_puct;
+    const uint32_t uvl = (uint32_t)ka->a.vl;
+    long long *const trace = ka->a.trace;
     int level = 0, kids = 0, contested = 0, best0 = -1, second = 0;
     uint32_t lk0 = 0u;
     for (;;) {
-        if (cc <= 0 || depth >= a.max_depth || level >= kChainMaxLevels) break;
-        const long long tr0 = a.trace && li == 0 ? wall_clock64() : 0ll;
+        if (cc <= 0 || depth >= max_depth || level >= kChainMaxLevels) break;
+        const long long tr0 = trace ? wall_clock64() : 0ll;
         int nelig = cc;
-        if (a.pw) {
+        if (pw) {
             const int kk = ceil_sqrt_i32(np);
             nelig = kk < cc ? kk : cc;
         }
-        const float ep = a.c_puct * sqrtf((float)np);
-        const int par = level & 1;
-        // ---- this wavefront's rounds of the children ----
-        int kn[Q], kvl[Q];
-        float kw[Q], kp[Q], kq2[Q];
-        uint32_t k1[Q], k2[Q];
-        bool kin[Q];
-        int2 ksp[Q];
+        const float ep = c_puct * sqrtf((float)np);
+        // ---- the children ----
+        int kn[RMAX], kvl[RMAX];
+        float kw[RMAX], kp[RMAX], kq2[RMAX];
+        uint32_t k1[RMAX], k2[RMAX];
+        bool kin[RMAX];
+        int2 ksp[RMAX];
         {
-            int rn[Q];
-            float rw[Q];
-            uint32_t word[Q];
+            uint32_t word[RMAX];
 #pragma unroll
-            for (int q = 0; q < Q; q++) {
-                const int r = li * Q + q;
+            for (int r = 0; r < RMAX; r++) {
                 const int i = r * kWave + lane;
-                const bool in = r < RMAX && i < nelig;
+                const bool in = i < nelig;
                 const int id = cb + i;
-                word[q] = in && f.legal ? f.legal[(uint32_t)id >> 5] : 0xFFFFFFFFu;
-                kn[q] = in ? f.N[id] : 0;
-                kw[q] = in ? f.W[id] : 0.0f;
-                kp[q] = in ? f.P[id] : 0.0f;
-                kvl[q] = in ? f.VL[id] : 0;
-                rn[q] = RAVE && in ? f.rN[id] : 0;
-                rw[q] = RAVE && in ? f.rW[id] : 0.0f;
-                ksp[q] = in ? f.span[id] : int2{0, 0};
+                word[r] = 0xFFFFFFFFu;
+                kn[r] = 0;
+                kw[r] = 0.0f;
+                kp[r] = 0.0f;
+                kvl[r] = 0;
+                kq2[r] = 0.0f;
+                ksp[r] = int2{0, 0};
+                if (r * kWave < nelig) {  // uniform: a node narrower than the layout's widest skips the rounds it lacks
+                    if (in && flegal) word[r] = flegal[(uint32_t)id >> 5];
+                    if (in) {
+                        kn[r] = fN[id];
+                        kw[r] = fW[id];
+                        kp[r] = fP[id];
+                        kvl[r] = fVL[id];
+                        if (RAVE) kq2[r] = fq2[id];
+                        ksp[r] = fspan[id];
+                    }
+                }
             }
 #pragma unroll
-            for (int q = 0; q < Q; q++) {
-                const int r = li * Q + q;
+            for (int r = 0; r < RMAX; r++) {
                 const int i = r * kWave + lane;
                 const int id = cb + i;
-                kin[q] = r < RMAX && i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
-                k1[q] = k2[q] = 0u;
-                kq2[q] = 0.0f;
-                if (kin[q]) {
-                    if (RAVE) kq2[q] = combined_value(kn[q], kw[q], rn[q], rw[q], a.rave_k);
-                    child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
-                } else {
-                    kn[q] = 0;
-                    kw[q] = 0.0f;
-                    kp[q] = 0.0f;
-                    kvl[q] = 0;
+                kin[r] = i < nelig && ((word[r] >> ((uint32_t)id & 31u)) & 1u);
+                k1[r] = k2[r] = 0u;
+                if (r * kWave < nelig) {
+                    if (kin[r]) {
+                        child_keys<RAVE>(kn[r], kw[r], kp[r], kvl[r], kq2[r], ep, k1[r], k2[r]);
+                    } else {
+                        kn[r] = 0;
+                        kw[r] = 0.0f;
+                        kp[r] = 0.0f;
+                        kvl[r] = 0;
+                        kq2[r] = 0.0f;
+                    }
                 }
             }
         }
-        // ---- its best candidate, and the best candidate of its other children ----
+        // ---- the best candidate, and the best candidate of the other children ----
         uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
         bool has1 = false;
 #pragma unroll
-        for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
-            has1 |= k1[q] != 0u;
-            if (k1[q] > bk) { bk = k1[q]; bpos = i; }
+        for (int r = 0; r < RMAX; r++) {
+            has1 |= k1[r] != 0u;
+            if (k1[r] > bk) { bk = k1[r]; bpos = (uint32_t)(r * kWave + lane); }
         }
 #pragma unroll
-        for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
-            if (k2[q] > bk) { bk = k2[q]; bpos = (uint32_t)F + i; }
-        }
+        for (int r = 0; r < RMAX; r++)
+            if (k2[r] > bk) { bk = k2[r]; bpos = (uint32_t)(F + r * kWave + lane); }
         uint32_t hk, hp;
         wave_best(bk, bpos, hk, hp);
-        const uint32_t mine = hk == 0u ? 0xFFFFFFFFu : (hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
-        uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
-#pragma unroll
-        for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
-            if (i != mine && k1[q] > ok_) { ok_ = k1[q]; opos = i; }
-        }
-#pragma unroll
-        for (int q = 0; q < Q; q++) {
-            const uint32_t i = (uint32_t)((li * Q + q) * kWave + lane);
-            if (i != mine && k2[q] > ok_) { ok_ = k2[q]; opos = (uint32_t)F + i; }
-        }
-        uint32_t sk, spos;
-        wave_best(ok_, opos, sk, spos);
-        int tn = 0, tvl = 0, tsx = 0, tsy = 0;
-        float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
-#pragma unroll
-        for (int q = 0; q < Q; q++) {
-            if ((uint32_t)(li * Q + q) == (mine >> 6)) {
-                tn = kn[q];
-                tw = kw[q];
-                tp = kp[q];
-                tvl = kvl[q];
-                tq2 = kq2[q];
-                tsx = ksp[q].x;
-                tsy = ksp[q].y;
-            }
-        }
-        const int ml = (int)(mine & 63u);
-        int bn = __builtin_amdgcn_readlane(tn, ml), bvl = __builtin_amdgcn_readlane(tvl, ml);
-        int bsx = __builtin_amdgcn_readlane(tsx, ml), bsy = __builtin_amdgcn_readlane(tsy, ml);
-        float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), ml));
-        float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ml));
-        float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), ml));
-        bool any1 = __ballot(has1) != 0ull;
-        bool gave_up = false;
-        if (NL > 1) {
-            // ---- the same over the loaders ----
-            if (lane == 0) {
-                g_chain.slot[par][li].bk = hk;
-                g_chain.slot[par][li].bpos = hp;
-                g_chain.slot[par][li].sk = sk;
-                g_chain.slot[par][li].spos = spos;
-                g_chain.slot[par][li].n = bn;
-                g_chain.slot[par][li].vl = bvl;
-                g_chain.slot[par][li].w = bw;
-                g_chain.slot[par][li].p = bp;
-                g_chain.slot[par][li].q2 = bq2;
-                g_chain.slot[par][li].sx = bsx;
-                g_chain.slot[par][li].sy = bsy;
-                g_chain.slot[par][li].any1 = any1 ? 1u : 0u;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            if (lane == 0) __hip_atomic_fetch_add(&g_chain.arrive, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            const int target = NL * (level + 1);
-            for (int spins = 0;; spins++) {
-                int v = 0;
-                if (lane == 0) v = __hip_atomic_load(&g_chain.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                v = __builtin_amdgcn_readfirstlane(v);
-                if (v >= target) break;
-                if (spins >= a.spin_limit) {  // cannot happen: the loaders take the same steps; bounded like every wait
-                    if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 5);
-                    gave_up = true;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            if (gave_up) break;
-            hk = 0u;
-            hp = 0xFFFFFFFFu;
-            int won = 0;
-            uint32_t a1 = 0u;
-#pragma unroll
-            for (int w = 0; w < NL; w++) {
-                const uint32_t k_ = g_chain.slot[par][w].bk, p_ = g_chain.slot[par][w].bpos;
-                a1 |= g_chain.slot[par][w].any1;
-                if (k_ != 0u && comes_before(k_, p_, hk, hp)) {
-                    hk = k_;
-                    hp = p_;
-                    won = w;
-                }
-            }
-            won = __builtin_amdgcn_readfirstlane(won);
-            sk = 0u;
-            spos = 0xFFFFFFFFu;
-#pragma unroll
-            for (int w = 0; w < NL; w++) {
-                const uint32_t k_ = w == won ? g_chain.slot[par][w].sk : g_chain.slot[par][w].bk;
-                const uint32_t p_ = w == won ? g_chain.slot[par][w].spos : g_chain.slot[par][w].bpos;
-                if (k_ != 0u && comes_before(k_, p_, sk, spos)) {
-                    sk = k_;
-                    spos = p_;
-                }
-            }
-            bn = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].n);
-            bvl = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].vl);
-            bsx = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].sx);
-            bsy = __builtin_amdgcn_readfirstlane(g_chain.slot[par][won].sy);
-            bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].w)));
-            bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].p)));
-            bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(g_chain.slot[par][won].q2)));
-            hk = (uint32_t)__builtin_amdgcn_readfirstlane((int)hk);
-            hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)hp);
-            sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)sk);
-            spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)spos);
-            any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
-        }
-        // ---- the one-winner test (single_run) ----
-        bool one = hk != 0u && (!RAVE || any1);
         // (with RAVE and no real first-scan score at all the reference never runs its second scan;
         // select_group knows, and gets no verdict)
+        const bool any1 = __ballot(has1) != 0ull;
+        bool one = hk != 0u && (!RAVE || any1);
         const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
+        int bn = 0, bsx = 0, bsy = 0;
         if (one) {
+            uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
+#pragma unroll
+            for (int r = 0; r < RMAX; r++)
+                if (r * kWave + lane != best && k1[r] > ok_) { ok_ = k1[r]; opos = (uint32_t)(r * kWave + lane); }
+#pragma unroll
+            for (int r = 0; r < RMAX; r++)
+                if (r * kWave + lane != best && k2[r] > ok_) { ok_ = k2[r]; opos = (uint32_t)(F + r * kWave + lane); }
+            uint32_t sk, spos;
+            wave_best(ok_, opos, sk, spos);
+            int tn = 0, tvl = 0, tsx = 0, tsy = 0;
+            float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < RMAX; r++) {
+                if (r == (best >> 6)) {
+                    tn = kn[r];
+                    tw = kw[r];
+                    tp = kp[r];
+                    tvl = kvl[r];
+                    tq2 = kq2[r];
+                    tsx = ksp[r].x;
+                    tsy = ksp[r].y;
+                }
+            }
+            const int bl = best & 63;
+            bn = __builtin_amdgcn_readlane(tn, bl);
+            bsx = __builtin_amdgcn_readlane(tsx, bl);
+            bsy = __builtin_amdgcn_readlane(tsy, bl);
+            const int bvl = __builtin_amdgcn_readlane(tvl, bl);
+            const float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), bl));
+            const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), bl));
+            const float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), bl));
+            // ---- the one-winner test (single_run) ----
             uint32_t lk, lp;
             entry_key<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1, best, lk, lp);
             if (lk == 0u) {
@@ -2632,61 +2518,34 @@ __device__ __noinline__ void chain_walk(ForestDev f, SelectArgs a, LdsBytesP scr
         if (!one) {
             // the node's children, where select_group collects them (its own fan-out class)
             kids = 1;
-            if (gave_up) kids = 0;
-            else if (cc <= kWave) {
-#pragma unroll
-                for (int q = 0; q < Q; q++)
-                    if (li * Q + q < 1)
-                        chain_dump<1>(scratch, (li * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q], k2[q],
-                                      kin[q]);
+            if (cc <= kWave) {
+                chain_dump<1>(scratch, lane, kn[0], kw[0], kp[0], kvl[0], kq2[0], k1[0], k2[0], kin[0]);
             } else {
 #pragma unroll
-                for (int q = 0; q < Q; q++)
-                    if (li * Q + q < RMAX)
-                        chain_dump<RMAX>(scratch, (li * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q],
-                                         k2[q], kin[q]);
-            }
-            if (NL > 1 && kids) {
-                // the owner goes on with these children at once: it waits here until all of them are there
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                if (lane == 0) __hip_atomic_fetch_add(&g_chain.arrive, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                if (li == 0) {
-                    const int target = NL * (level + 2);
-                    for (int spins = 0;; spins++) {
-                        int v = 0;
-                        if (lane == 0) v = __hip_atomic_load(&g_chain.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        v = __builtin_amdgcn_readfirstlane(v);
-                        if (v >= target) break;
-                        if (spins >= a.spin_limit) {
-                            if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 5);
-                            kids = 0;
-                            break;
-                        }
-                        __builtin_amdgcn_s_sleep(1);
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                }
+                for (int r = 0; r < RMAX; r++)
+                    chain_dump<RMAX>(scratch, r * kWave + lane, kn[r], kw[r], kp[r], kvl[r], kq2[r], k1[r], k2[r], kin[r]);
             }
             break;
         }
         // ---- every visitor takes that child ----
         const int child = cb + best;
-        if (li == 0 && lane == 0) {
+        if (lane == 0) {
             g_chain.nodes[level] = child;
-            atomicAdd(f.VL + child, (int)(uvl * (uint32_t)m));
-            if (a.stats) {
-                atomicAdd(a.stats + 0, 1);
-                atomicAdd(a.stats + 1, 1);
-                atomicAdd(a.stats + 2, m);
+            atomicAdd(ka->f.VL + child, (int)(uvl * (uint32_t)m));
+            int32_t *const stats = ka->a.stats;
+            if (stats) {
+                atomicAdd(stats + 0, 1);
+                atomicAdd(stats + 1, 1);
+                atomicAdd(stats + 2, m);
             }
-            if (a.trace) {
-                const int ti = atomicAdd(a.trace_n, 1);
-                if (ti < a.trace_cap) {
-                    a.trace[12 * ti + 0] = tr0;
-                    a.trace[12 * ti + 1] = wall_clock64();
-                    a.trace[12 * ti + 2] = (long long)m | ((long long)depth << 32) | (5ll << 60);
-                    a.trace[12 * ti + 3] = (long long)node;
-                    for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+            if (trace) {
+                const int ti = atomicAdd(ka->a.trace_n, 1);
+                if (ti < ka->a.trace_cap) {
+                    trace[12 * ti + 0] = tr0;
+                    trace[12 * ti + 1] = wall_clock64();
+                    trace[12 * ti + 2] = (long long)m | ((long long)depth << 32) | (5ll << 60);
+                    trace[12 * ti + 3] = (long long)node;
+                    for (int q = 0; q < 8; q++) trace[12 * ti + 4 + q] = 0;
                 }
             }
         }
@@ -2697,7 +2556,7 @@ __device__ __noinline__ void chain_walk(ForestDev f, SelectArgs a, LdsBytesP scr
         depth++;
         level++;
     }
-    if (li == 0 && lane == 0) {
+    if (lane == 0) {
         g_chain.levels = level;
         g_chain.e_node = node;
         g_chain.e_np = np;
@@ -2709,6 +2568,35 @@ __device__ __noinline__ void chain_walk(ForestDev f, SelectArgs a, LdsBytesP scr
         g_chain.e_best0 = best0;
         g_chain.e_lk0 = lk0;
         g_chain.e_second = second;
+    }
+}
+
+// After a walk: the path entries of its visitors for every level walked, and their list where the node the
+// walk stopped at reads it.  By the wavefront that walked, once the list the walk started from is complete (the
+// helper that writes it says so in LDS; bounded wait).
+__device__ __noinline__ void chain_finish(KernArgsP ka, int lane, int d0, int off, int m) {
+    const int k = __builtin_amdgcn_readfirstlane(g_chain.levels);
+    if (k <= 0) return;
+    const int spin_limit = ka->a.spin_limit;
+    for (int spins = 0;; spins++) {
+        int v = 0;
+        if (lane == 0) v = __hip_atomic_load(&g_chain.part_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (__builtin_amdgcn_readfirstlane(v)) break;
+        if (spins >= spin_limit) {  // the other helper never finished: cannot happen; give the selection up
+            if (lane == 0) atomicCAS(ka->a.sched_wait + 1, 0, 5);
+            return;
+        }
+        __builtin_amdgcn_s_sleep(2);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const int32_t *src = d0 == 0 ? ka->a.seg0 : ka->a.seg[(d0 - 1) & 1];
+    int32_t *dst = ka->a.seg[(d0 + k - 1) & 1];
+    int32_t *paths = ka->a.paths;
+    const int stride = ka->a.stride;
+    for (int j = lane; j < m; j += kWave) {
+        const int t = src[off + j];
+        for (int i = 0; i < k; i++) paths[(size_t)(d0 + 1 + i) * stride + t] = g_chain.nodes[i];
+        if (dst != src) dst[off + j] = t;
     }
 }
 
@@ -2759,7 +2647,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // the visitor list of an item of kind 3, and of the slices of one, may not be there yet:
     // whoever shares out the visitors waits for it (below), settling them does not need it
     bool list_ok = !(item.pad[0] == 3 || (item.pad[0] == 1 && ((item.pad[2] >> 30) & 1)));
-    if (m >= kHeavyMin) close_pending(a, pending, lane);
+    if (m >= kHeavyMin) close_pending(pending);
     Kids<R, RAVE> k;
     int cnt[R];
     uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
@@ -2793,7 +2681,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         } else if (R > 1 && R == RMAX && !ahead) {
             // a wide node from the queue: the helpers are idle (or finish the partition of the node this
             // wavefront settled last), two of them take their share of the children
-            close_pending(a, pending, lane);
+            close_pending(pending);
             if (lane == 0) {
                 TeamCmd &cm = lds.cmd;
                 cm.op = kOpLoad;
@@ -2812,7 +2700,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             // this wavefront's share of the children; the rest is in LDS once the request is closed
             constexpr int S = AheadShare<R>::kRounds;
             load_score_rounds<R, RAVE, 0, (S < R ? S : R)>(f, c.cb, c.nelig, lane, a.rave_k, c.ep, k);
-            close_pending(a, pending, lane);
+            close_pending(pending);
 #pragma unroll
             for (int r = S; r < R; r++) {
                 const int i = r * kWave + lane;
@@ -3032,7 +2920,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         run_child = -1;
         lds_cur = -1;
         const bool seq_lds = m < kHeavyMin;  // few enough visitors to keep their order in LDS
-        if (seq_lds) close_pending(a, pending, lane);  // the previous node's partition may still read that buffer
+        if (seq_lds) close_pending(pending);  // the previous node's partition may still read that buffer
         for (int done = 0; done < m; done++) {
             int i = wave_pick<R, RAVE>(k, lane, bk, bpos);
             if (i < 0) return kStepLeaf;  // no child takes part: uniform, and then for every visitor
@@ -3086,7 +2974,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 
     // ---- partition of the visitors by chosen child ----
     // this node's visitor list is written by the previous node's partition
-    close_pending(a, pending, lane);
+    close_pending(pending);
     if (!list_ok) {
         if (!wait_list(a, off, depth, lane)) return kStepParked;
         list_ok = true;
@@ -3130,7 +3018,9 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         const int off_next = keep >= 0 ? off + __builtin_amdgcn_readlane(ex_keep, keep & 63) : 0;
         // a kept child of ordinary size: the same request starts the walk down one-winner nodes at it
         // (chain_walk), so that the owner does not wait for this partition
-        const bool chain_next = keep >= 0 && (int)gmax < kHeavyMin && a.vl > 0;
+        // (only below a node that was itself of that kind: chains are long, and at a node that splits its visitors
+        // the attempt would cost what it saves: the children would be loaded by one wavefront instead of three)
+        const bool chain_next = keep >= 0 && (int)gmax < kHeavyMin && a.vl > 0 && run_child >= 0;
         const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth && !chain_next;
         if (lane == 0) {
             TeamCmd &cm = lds.cmd;
@@ -3153,11 +3043,11 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 cm.c_depth = depth + 1;
                 cm.c_off = off_next;
                 cm.c_m = (int)gmax;
-                g_chain.arrive = 0;
+                g_chain.part_done = 0;
             }
         }
-        __syncthreads();  // the request is open until close_pending (the owner runs its part of the walk first)
-        pending = !chain_next;
+        __syncthreads();  // the request is open until close_pending
+        pending = true;
         next.node = -1;
         next.ahead = false;
         next.chain_open = chain_next;
@@ -3500,7 +3390,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             it.np = f.N[it.node];
             for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
         }
-        bool have_span = false, chain_tried = false, chain_open = false;
+        bool have_span = false, chain_open = false;
         int preload = 0;  // what select_group finds of the node's children (its argument of that name)
         int2 pre_span = int2{0, 0};
         for (;;) {
@@ -3513,52 +3403,20 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             if (lane < 16) s_lds.tph[lane] = 0u;
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
-            if (chain_open || (!chain_tried && it.pad[0] == 0 && it.m >= kChainMin && it.m < kHeavyMin && a.vl > 0 &&
-                               c.cc > 0 && depth < a.max_depth)) {
-                // A plain node of ordinary size: first the walk down the nodes whose visitors all follow one
-                // child (chain_walk).  The request is open already when the partition of the node settled
-                // before carries it (select_group); otherwise it is opened here, with no partition to do.
-                if (!chain_open) {
-                    close_pending(a, pending, lane);
-                    if (lane == 0) {
-                        TeamCmd &cm = s_lds.cmd;
-                        cm.op = kOpChain;
-                        cm.j_m = 0;
-                        cm.c_node = it.node;
-                        cm.c_np = it.np;
-                        cm.c_cb = c.cb;
-                        cm.c_cc = c.cc;
-                        cm.c_depth = depth;
-                        cm.c_off = it.off;
-                        cm.c_m = it.m;
-                        g_chain.arrive = 0;
-                    }
-                    __syncthreads();
-                }
+            if (chain_open) {
+                // The node settled before sent all its visitors here, and the request that shares them out also
+                // has a helper walk down from this node for as long as the visitors stay together (chain_walk,
+                // chain_finish): wait for both, and go on where that walk stopped.
                 chain_open = false;
-                chain_walk<RMAX, RAVE, (RMAX > 1 ? kChainLoaders : 1)>(f, a, (LdsBytesP)&s_lds, 0, lane, it.node, it.np, c.cb,
-                                                                       c.cc, depth, it.m);
-                // The request stays open (the helper that shares out the previous node's visitors may still be
-                // at it); the walk's path entries need the list that helper writes, and are written when the
-                // request is closed (close_pending).
-                pending = true;
-                if (lane == 0) {
-                    g_chain.debt = g_chain.levels > 0 ? 1 : 0;
-                    g_chain.d_depth = depth;
-                    g_chain.d_off = it.off;
-                    g_chain.d_m = it.m;
-                }
-                wave_sync_memory();
+                close_pending(pending);
                 it.node = __builtin_amdgcn_readfirstlane(g_chain.e_node);
                 it.np = __builtin_amdgcn_readfirstlane(g_chain.e_np);
                 it.depth = __builtin_amdgcn_readfirstlane(g_chain.e_depth);
                 have_span = true;
                 pre_span = int2{__builtin_amdgcn_readfirstlane(g_chain.e_cb), __builtin_amdgcn_readfirstlane(g_chain.e_cc)};
                 preload = __builtin_amdgcn_readfirstlane(g_chain.e_kids) ? 2 : 0;
-                chain_tried = true;  // the node the walk stopped at is settled the general way
                 continue;
             }
-            chain_tried = false;
             const int preload_now = preload;
             preload = 0;
             int status = kStepLeaf;
@@ -3593,7 +3451,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             }
             if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
             if (status == kStepLeaf) {
-                close_pending(a, pending, lane);  // the visitor list comes from the previous node's partition
+                close_pending(pending);  // the visitor list comes from the previous node's partition
                 if (it.pad[0] == 3 && !wait_list(a, it.off, depth, lane)) break;
                 for (int j = lane; j < it.m; j += kWave) {
                     int t = seg_in[it.off + j];
@@ -3772,10 +3630,8 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
     if (tid < kWave) {
         // every path out of the owner's loop comes back here: the helpers are always released
         bool pending = false;
-        if (tid == 0) g_chain.debt = 0;
-        wave_sync_memory();
         owner_loop<RMAX, RAVE>(f, a, s_lds, s_part, pending, tid);
-        close_pending(a, pending, tid);
+        close_pending(pending);
         if (tid == 0) atomicMax(a.times + 1, (int)(wall_clock64() & 0x7FFFFFFF));
         if (tid == 0) s_lds.cmd.op = kOpExit;
         __syncthreads();
@@ -3793,24 +3649,24 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
         if (op == kOpChain) {
-            // a walk down one-winner nodes by the owner and, on a wide layout, two helpers, while the
-            // remaining helper shares out the visitors of the node settled before (if the request
-            // carries one)
+            // one helper shares out the visitors of the node just settled, all of which follow one child; another
+            // walks down from that child for as long as they stay together, and then writes their path entries
             const TeamCmd &cm = s_lds.cmd;
             const int wv = tid >> 6;
             if (wv == 1) {
-                if (__builtin_amdgcn_readfirstlane(cm.j_m) > 0) {
-                    if (rounds == 1) partition_async<1, RMAX>(f, a, cm, s_part, tid & 63);
-                    else partition_async<RMAX, RMAX>(f, a, cm, s_part, tid & 63);
-                }
-            } else if (RMAX > 1) {
-                chain_walk<RMAX, RAVE, kChainLoaders>(f, a, (LdsBytesP)&s_lds, wv - 1, tid & 63,
-                                                      __builtin_amdgcn_readfirstlane(cm.c_node),
-                                                      __builtin_amdgcn_readfirstlane(cm.c_np),
-                                                      __builtin_amdgcn_readfirstlane(cm.c_cb),
-                                                      __builtin_amdgcn_readfirstlane(cm.c_cc),
-                                                      __builtin_amdgcn_readfirstlane(cm.c_depth),
-                                                      __builtin_amdgcn_readfirstlane(cm.c_m));
+                if (rounds == 1) partition_async<1, RMAX>(f, a, cm, s_part, tid & 63);
+                else partition_async<RMAX, RMAX>(f, a, cm, s_part, tid & 63);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the kept child's list is written
+                if ((tid & 63) == 0)
+                    __hip_atomic_store(&g_chain.part_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else if (wv == 2) {
+                const KernArgsP ka = (KernArgsP)__builtin_amdgcn_kernarg_segment_ptr();
+                const int c_depth = __builtin_amdgcn_readfirstlane(cm.c_depth), c_m = __builtin_amdgcn_readfirstlane(cm.c_m);
+                const int c_off = __builtin_amdgcn_readfirstlane(cm.c_off);
+                chain_walk<RMAX, RAVE>(ka, (LdsBytesP)&s_lds, tid & 63, __builtin_amdgcn_readfirstlane(cm.c_node),
+                                       __builtin_amdgcn_readfirstlane(cm.c_np), __builtin_amdgcn_readfirstlane(cm.c_cb),
+                                       __builtin_amdgcn_readfirstlane(cm.c_cc), c_depth, c_m);
+                chain_finish(ka, tid & 63, c_depth, c_off, c_m);
             }
             __syncthreads();  // the request is done
             continue;

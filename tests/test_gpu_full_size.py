@@ -1,8 +1,12 @@
 """GPU parity on the five benchmark workloads at their FULL size (the trees and batches the benchmark
 times: 200 k nodes / 64 traversals, 256 x 50 k / 256, 64 x 1 M / 1024, 4 M / 4096 with progressive
 widening, 16 M with RAVE / 16384 and the 2^24-slot table), two search steps each, against the CPU
-checker after every phase: paths, lengths, leaves, move lists, N and virtual loss bit-exact, W within
-1e-5 relative, table probes of the leaves' keys identical."""
+checker after every phase: paths, lengths, leaves, move lists, N and virtual loss bit-exact, table
+probes of the leaves' keys identical.  W: device, serial binary32 checker and exact double sums are
+held against each other at 1e-5 relative to max(|W|, 1, sqrt(k)), k the values a node takes in the step;
+the strict figure |W_device - W_checker| / max(|W_checker|, 1) is printed beside it with the number of
+nodes above 1e-5 (a root that takes 16384 values of either sign is where the serial binary32 sum
+itself is 3e-6 away from the exact one)."""
 import numpy as np
 import pytest
 
@@ -58,6 +62,7 @@ def test_full_size_workload(name):
     rng = np.random.default_rng(9)
     near_total = 0
     worst = (0.0, 0.0, 0.0)
+    strict_worst, strict_above = 0.0, 0
     for step in range(2):
         rpaths, rlen, rleaf, near = ref.select_batch(troots, rp)
         near_total += int((near >= 0).sum())
@@ -102,6 +107,11 @@ def test_full_size_workload(name):
         assert err_gpu <= W_RTOL, "W after backup against the exact sums: %g" % err_gpu
         assert err_both <= W_RTOL + 1.01 * err_ref, (err_both, err_ref)
         worst = max(worst, (err_gpu, err_ref, err_both))
+        strict = np.abs(gw - ref.W) / np.maximum(np.abs(ref.W.astype(np.float64)), 1.0)
+        strict_worst = max(strict_worst, float(strict.max()))
+        strict_above += int((strict > W_RTOL).sum())
         ref.W[:] = st["W"]
     print("%s: near-tie traversals flagged by the checker over 2 steps: %d; W max rel err: device vs exact %.2e, "
-          "serial binary32 checker vs exact %.2e, device vs checker %.2e" % ((name, near_total) + worst))
+          "serial binary32 checker vs exact %.2e, device vs checker %.2e; strict |dW| / max(|W|, 1) device vs "
+          "checker %.3e, nodes above 1e-5 under that definition: %d"
+          % ((name, near_total) + worst + (strict_worst, strict_above)))
