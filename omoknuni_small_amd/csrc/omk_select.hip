@@ -579,8 +579,7 @@ struct ChainLds {
     int e_best0;      // that child,
     uint32_t e_lk0;   // that entry's key,
     int e_second;     // and whether it is a candidate of the second scan
-    int part_done;    // the helper that shares out the visitors of the node settled before has finished: the list the
-                      // walk started from is complete
+    int n_barriers;   // -1 while a walk is under way, then the number of block barriers it took
 };
 typedef __attribute__((address_space(3))) unsigned char *LdsBytesP;
 // one per block of the multi-visitor kernel
@@ -2336,18 +2335,23 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
 // ---- Chains of nodes whose visitors all follow one child ----
 // Most crowded nodes below the top of a tree are of that kind, often a dozen in a row (a whole
 // selection of the Go workload with 16 visitors per tree starts with a chain of them), and on such a
-// node nothing is decided: the visitors stay together, in the same order.  chain_walk does these nodes
-// and nothing else, by the owner wavefront alone, while a helper shares out the visitors of the node
-// settled before (if there is one): it loads and scores the children (statistics, legality bits and
-// the child ranges of all children in range in ONE trip to memory), makes the one-winner test of
-// single_run (the entry the best child shows the LAST visitor still comes first, and its entries are in
-// order) and moves on into the child.  One dependent trip to memory per level, no block barrier, no
-// partition: the visitor list does not change, so the walk does not even read it; it records the children
-// it took, and the visitors' path entries for all its levels are written at once when the request that
-// runs beside it is closed (close_pending: chain_finish), together with the list in the buffer the next
-// node reads.  The walk stops at a leaf (or the depth cap), or at the first node that fails the test:
-// that node's children, loaded and scored, are left in the LDS scratch together with the verdict, and
-// select_group settles it from there.
+// node nothing is decided: the visitors stay together, in the same order.  When the owner finds such a
+// node (single_run), it does not share out its visitors: it hands the node's child to its three helpers,
+// which walk down from there in lockstep for as long as the visitors stay together (chain_walk): each
+// loads and scores its rounds of the children (statistics, legality bits and the child ranges of all
+// children in range in ONE trip to memory), leaves its best candidate, the best candidate of its other
+// children and the best child's statistics in LDS; after one block barrier each of them knows the
+// node's best child and the best candidate of all others, makes the one-winner test of single_run
+// (the entry the best child shows the LAST visitor still comes first, and its entries are in order)
+// and moves on into the child.  One barrier and one dependent trip to memory per level, no partition:
+// the visitor list does not change, so the walk does not even read it; it records the children it
+// took, and when it has stopped the three write the visitors' path entries for all its levels at
+// once, the level of the owner's node included, and the list into the buffer the next node reads
+// (chain_finish).  The walk stops at a leaf (or the depth cap), or at the first node that fails the
+// test: that node's children, loaded and scored, are left in the LDS scratch together with the
+// verdict, and select_group settles it from there.  The owner takes the walk's barriers with it
+// (a block barrier counts every wavefront) and does nothing else meanwhile: the code of the walk
+// stays out of the owner's own, whose registers are its scarcest resource.
 // One round of a node's children, as select_group collects them from the LDS scratch of fan-out class R.
 template <int R>
 __device__ __forceinline__ void chain_dump(LdsBytesP base, int i, int n, float w, float p, int vl, float q2,
@@ -2375,10 +2379,27 @@ typedef const __attribute__((address_space(4))) SelectKernArgs *KernArgsP;
 static_assert(offsetof(SelectKernArgs, a) == sizeof(ForestDev),
               "k_select_groups(ForestDev, SelectArgs): the second argument follows the first");
 
+// What one of the walking wavefronts found among the children it loaded, one level.
+struct ChainSlot {
+    uint32_t bk, bpos;  // its best candidate (key 0 = none)
+    uint32_t sk, spos;  // the best candidate of its children other than that one's child
+    int n, vl;          // that child's statistics and child range
+    float w, p, q2;
+    int sx, sy;
+    uint32_t any1;      // one of its children has a real first-scan key
+};
+constexpr int kChainWalkers = 3;
+__shared__ ChainSlot g_chain_slot[2][kChainWalkers];
+
+// wi: which of the three walking wavefronts this is.  Every block barrier in here is also taken by the owner,
+// which waits the walk out (owner_loop).
 template <int RMAX, bool RAVE>
-__device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lane, int node, int np, int cb, int cc,
-                                        int depth, int m) {
+__device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, int lane, int node, int np, int cb,
+                                       int cc, int depth, int m) {
     constexpr int F = RMAX * kWave;
+    // a layout without wide nodes: one wavefront walks alone (no exchange, no barrier per level)
+    constexpr bool SOLO = RMAX == 1;
+    constexpr int Q = SOLO ? 1 : (RMAX + kChainWalkers - 1) / kChainWalkers;  // rounds of children per wavefront: wi*Q .. wi*Q+Q-1
     const int32_t *const fN = ka->f.N, *const fVL = ka->f.VL;
     const float *const fW = ka->f.W, *const fP = ka->f.P, *const fq2 = ka->f.q2;
     const uint32_t *const flegal = ka->f.legal;
@@ -2387,120 +2408,198 @@ __device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lan
     const float c_puct = ka->a.c_puct;
     const uint32_t uvl = (uint32_t)ka->a.vl;
     long long *const trace = ka->a.trace;
-    int level = 0, kids = 0, contested = 0, best0 = -1, second = 0;
+    int level = 1;  // level 0 is the node settled before, whose child this walk starts at
+    int bars = 0;   // block barriers taken
+    int kids = 0, contested = 0, best0 = -1, second = 0;
     uint32_t lk0 = 0u;
     for (;;) {
         if (cc <= 0 || depth >= max_depth || level >= kChainMaxLevels) break;
-        const long long tr0 = trace ? wall_clock64() : 0ll;
+        const long long tr0 = trace && wi == 0 ? wall_clock64() : 0ll;
         int nelig = cc;
         if (pw) {
             const int kk = ceil_sqrt_i32(np);
             nelig = kk < cc ? kk : cc;
         }
         const float ep = c_puct * sqrtf((float)np);
-        // ---- the children ----
-        int kn[RMAX], kvl[RMAX];
-        float kw[RMAX], kp[RMAX], kq2[RMAX];
-        uint32_t k1[RMAX], k2[RMAX];
-        bool kin[RMAX];
-        int2 ksp[RMAX];
+        const int par = level & 1;
+        // ---- this wavefront's rounds of the children ----
+        int kn[Q], kvl[Q];
+        float kw[Q], kp[Q], kq2[Q];
+        uint32_t k1[Q], k2[Q];
+        bool kin[Q];
+        int2 ksp[Q];
         {
-            uint32_t word[RMAX];
+            uint32_t word[Q];
 #pragma unroll
-            for (int r = 0; r < RMAX; r++) {
+            for (int q = 0; q < Q; q++) {
+                const int r = wi * Q + q;
                 const int i = r * kWave + lane;
                 const bool in = i < nelig;
                 const int id = cb + i;
-                word[r] = 0xFFFFFFFFu;
-                kn[r] = 0;
-                kw[r] = 0.0f;
-                kp[r] = 0.0f;
-                kvl[r] = 0;
-                kq2[r] = 0.0f;
-                ksp[r] = int2{0, 0};
-                if (r * kWave < nelig) {  // uniform: a node narrower than the layout's widest skips the rounds it lacks
-                    if (in && flegal) word[r] = flegal[(uint32_t)id >> 5];
+                word[q] = 0xFFFFFFFFu;
+                kn[q] = 0;
+                kw[q] = 0.0f;
+                kp[q] = 0.0f;
+                kvl[q] = 0;
+                kq2[q] = 0.0f;
+                ksp[q] = int2{0, 0};
+                if (r * kWave < nelig) {  // uniform: rounds the node lacks are skipped
+                    if (in && flegal) word[q] = flegal[(uint32_t)id >> 5];
                     if (in) {
-                        kn[r] = fN[id];
-                        kw[r] = fW[id];
-                        kp[r] = fP[id];
-                        kvl[r] = fVL[id];
-                        if (RAVE) kq2[r] = fq2[id];
-                        ksp[r] = fspan[id];
+                        kn[q] = fN[id];
+                        kw[q] = fW[id];
+                        kp[q] = fP[id];
+                        kvl[q] = fVL[id];
+                        if (RAVE) kq2[q] = fq2[id];
+                        ksp[q] = fspan[id];
                     }
                 }
             }
 #pragma unroll
-            for (int r = 0; r < RMAX; r++) {
+            for (int q = 0; q < Q; q++) {
+                const int r = wi * Q + q;
                 const int i = r * kWave + lane;
                 const int id = cb + i;
-                kin[r] = i < nelig && ((word[r] >> ((uint32_t)id & 31u)) & 1u);
-                k1[r] = k2[r] = 0u;
+                kin[q] = i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
+                k1[q] = k2[q] = 0u;
                 if (r * kWave < nelig) {
-                    if (kin[r]) {
-                        child_keys<RAVE>(kn[r], kw[r], kp[r], kvl[r], kq2[r], ep, k1[r], k2[r]);
+                    if (kin[q]) {
+                        child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
                     } else {
-                        kn[r] = 0;
-                        kw[r] = 0.0f;
-                        kp[r] = 0.0f;
-                        kvl[r] = 0;
-                        kq2[r] = 0.0f;
+                        kn[q] = 0;
+                        kw[q] = 0.0f;
+                        kp[q] = 0.0f;
+                        kvl[q] = 0;
+                        kq2[q] = 0.0f;
                     }
                 }
             }
         }
-        // ---- the best candidate, and the best candidate of the other children ----
+        // ---- its best candidate, and the best candidate of its other children ----
         uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
         bool has1 = false;
 #pragma unroll
-        for (int r = 0; r < RMAX; r++) {
-            has1 |= k1[r] != 0u;
-            if (k1[r] > bk) { bk = k1[r]; bpos = (uint32_t)(r * kWave + lane); }
+        for (int q = 0; q < Q; q++) {
+            has1 |= k1[q] != 0u;
+            if (k1[q] > bk) { bk = k1[q]; bpos = (uint32_t)((wi * Q + q) * kWave + lane); }
         }
 #pragma unroll
-        for (int r = 0; r < RMAX; r++)
-            if (k2[r] > bk) { bk = k2[r]; bpos = (uint32_t)(F + r * kWave + lane); }
+        for (int q = 0; q < Q; q++)
+            if (k2[q] > bk) { bk = k2[q]; bpos = (uint32_t)(F + (wi * Q + q) * kWave + lane); }
         uint32_t hk, hp;
         wave_best(bk, bpos, hk, hp);
-        // (with RAVE and no real first-scan score at all the reference never runs its second scan;
-        // select_group knows, and gets no verdict)
-        const bool any1 = __ballot(has1) != 0ull;
-        bool one = hk != 0u && (!RAVE || any1);
-        const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
-        int bn = 0, bsx = 0, bsy = 0;
-        if (one) {
-            uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
+        const uint32_t mine = hk == 0u ? 0xFFFFFFFFu : (hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
+        uint32_t ok_ = 0u, opos = 0xFFFFFFFFu;
 #pragma unroll
-            for (int r = 0; r < RMAX; r++)
-                if (r * kWave + lane != best && k1[r] > ok_) { ok_ = k1[r]; opos = (uint32_t)(r * kWave + lane); }
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wi * Q + q) * kWave + lane);
+            if (i != mine && k1[q] > ok_) { ok_ = k1[q]; opos = i; }
+        }
 #pragma unroll
-            for (int r = 0; r < RMAX; r++)
-                if (r * kWave + lane != best && k2[r] > ok_) { ok_ = k2[r]; opos = (uint32_t)(F + r * kWave + lane); }
-            uint32_t sk, spos;
-            wave_best(ok_, opos, sk, spos);
+        for (int q = 0; q < Q; q++) {
+            const uint32_t i = (uint32_t)((wi * Q + q) * kWave + lane);
+            if (i != mine && k2[q] > ok_) { ok_ = k2[q]; opos = (uint32_t)F + i; }
+        }
+        uint32_t sk, spos;
+        wave_best(ok_, opos, sk, spos);
+        int bn, bvl, bsx, bsy;
+        float bw, bp, bq2;
+        bool any1;
+        if (SOLO) {
+            int tn = kn[0], tvl = kvl[0], tsx = ksp[0].x, tsy = ksp[0].y;
+            float tw = kw[0], tp = kp[0], tq2 = kq2[0];
+            const int ml = (int)(mine & 63u);
+            bn = __builtin_amdgcn_readlane(tn, ml);
+            bvl = __builtin_amdgcn_readlane(tvl, ml);
+            bsx = __builtin_amdgcn_readlane(tsx, ml);
+            bsy = __builtin_amdgcn_readlane(tsy, ml);
+            bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), ml));
+            bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ml));
+            bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), ml));
+            any1 = __ballot(has1) != 0ull;
+        } else {
+        {
             int tn = 0, tvl = 0, tsx = 0, tsy = 0;
             float tw = 0.0f, tp = 0.0f, tq2 = 0.0f;
 #pragma unroll
-            for (int r = 0; r < RMAX; r++) {
-                if (r == (best >> 6)) {
-                    tn = kn[r];
-                    tw = kw[r];
-                    tp = kp[r];
-                    tvl = kvl[r];
-                    tq2 = kq2[r];
-                    tsx = ksp[r].x;
-                    tsy = ksp[r].y;
+            for (int q = 0; q < Q; q++) {
+                if ((uint32_t)(wi * Q + q) == (mine >> 6)) {
+                    tn = kn[q];
+                    tw = kw[q];
+                    tp = kp[q];
+                    tvl = kvl[q];
+                    tq2 = kq2[q];
+                    tsx = ksp[q].x;
+                    tsy = ksp[q].y;
                 }
             }
-            const int bl = best & 63;
-            bn = __builtin_amdgcn_readlane(tn, bl);
-            bsx = __builtin_amdgcn_readlane(tsx, bl);
-            bsy = __builtin_amdgcn_readlane(tsy, bl);
-            const int bvl = __builtin_amdgcn_readlane(tvl, bl);
-            const float bw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tw), bl));
-            const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), bl));
-            const float bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), bl));
-            // ---- the one-winner test (single_run) ----
+            // the lane that holds the wavefront's best child writes the slot (one lane, one pass)
+            const bool any1w = __ballot(has1) != 0ull;
+            if (lane == (int)(mine == 0xFFFFFFFFu ? 0u : (mine & 63u))) {
+                ChainSlot &sl = g_chain_slot[par][wi];
+                sl.bk = hk;
+                sl.bpos = hp;
+                sl.sk = sk;
+                sl.spos = spos;
+                sl.n = tn;
+                sl.vl = tvl;
+                sl.w = tw;
+                sl.p = tp;
+                sl.q2 = tq2;
+                sl.sx = tsx;
+                sl.sy = tsy;
+                sl.any1 = any1w ? 1u : 0u;
+            }
+        }
+        __syncthreads();
+        bars++;
+        // ---- the same over the three wavefronts ----
+        hk = 0u;
+        hp = 0xFFFFFFFFu;
+        int won = 0;
+        uint32_t a1 = 0u;
+#pragma unroll
+        for (int w = 0; w < kChainWalkers; w++) {
+            const uint32_t k_ = g_chain_slot[par][w].bk, p_ = g_chain_slot[par][w].bpos;
+            a1 |= g_chain_slot[par][w].any1;
+            if (k_ != 0u && comes_before(k_, p_, hk, hp)) {
+                hk = k_;
+                hp = p_;
+                won = w;
+            }
+        }
+        won = __builtin_amdgcn_readfirstlane(won);
+        sk = 0u;
+        spos = 0xFFFFFFFFu;
+#pragma unroll
+        for (int w = 0; w < kChainWalkers; w++) {
+            const uint32_t k_ = w == won ? g_chain_slot[par][w].sk : g_chain_slot[par][w].bk;
+            const uint32_t p_ = w == won ? g_chain_slot[par][w].spos : g_chain_slot[par][w].bpos;
+            if (k_ != 0u && comes_before(k_, p_, sk, spos)) {
+                sk = k_;
+                spos = p_;
+            }
+        }
+        const ChainSlot &ws = g_chain_slot[par][won];
+        bn = __builtin_amdgcn_readfirstlane(ws.n);
+        bvl = __builtin_amdgcn_readfirstlane(ws.vl);
+        bsx = __builtin_amdgcn_readfirstlane(ws.sx);
+        bsy = __builtin_amdgcn_readfirstlane(ws.sy);
+        bw = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.w)));
+        bp = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.p)));
+        bq2 = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(ws.q2)));
+        hk = (uint32_t)__builtin_amdgcn_readfirstlane((int)hk);
+        hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)hp);
+        sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)sk);
+        spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)spos);
+        any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
+        }  // !SOLO
+        // ---- the one-winner test (single_run) ----
+        // (with RAVE and no real first-scan score at all the reference never runs its second scan;
+        // select_group knows, and gets no verdict)
+        bool one = hk != 0u && (!RAVE || any1);
+        const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
+        if (one) {
             uint32_t lk, lp;
             entry_key<RMAX, RAVE>(bn, bw, bp, bvl, bq2, ep, uvl, m - 1, best, lk, lp);
             if (lk == 0u) {
@@ -2519,18 +2618,23 @@ __device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lan
             // the node's children, where select_group collects them (its own fan-out class)
             kids = 1;
             if (cc <= kWave) {
-                chain_dump<1>(scratch, lane, kn[0], kw[0], kp[0], kvl[0], kq2[0], k1[0], k2[0], kin[0]);
+#pragma unroll
+                for (int q = 0; q < Q; q++)
+                    if (wi * Q + q < 1)
+                        chain_dump<1>(scratch, lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q], k2[q], kin[q]);
             } else {
 #pragma unroll
-                for (int r = 0; r < RMAX; r++)
-                    chain_dump<RMAX>(scratch, r * kWave + lane, kn[r], kw[r], kp[r], kvl[r], kq2[r], k1[r], k2[r], kin[r]);
+                for (int q = 0; q < Q; q++)
+                    if (wi * Q + q < RMAX)
+                        chain_dump<RMAX>(scratch, (wi * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q],
+                                         k2[q], kin[q]);
             }
             break;
         }
         // ---- every visitor takes that child ----
         const int child = cb + best;
-        if (lane == 0) {
-            g_chain.nodes[level] = child;
+        if (lane == 0) g_chain.nodes[level] = child;  // every walker for itself: chain_finish reads them without a barrier
+        if (wi == 0 && lane == 0) {
             atomicAdd(ka->f.VL + child, (int)(uvl * (uint32_t)m));
             int32_t *const stats = ka->a.stats;
             if (stats) {
@@ -2556,7 +2660,7 @@ __device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lan
         depth++;
         level++;
     }
-    if (lane == 0) {
+    if (wi == 0 && lane == 0) {
         g_chain.levels = level;
         g_chain.e_node = node;
         g_chain.e_np = np;
@@ -2568,32 +2672,21 @@ __device__ __noinline__ void chain_walk(KernArgsP ka, LdsBytesP scratch, int lan
         g_chain.e_best0 = best0;
         g_chain.e_lk0 = lk0;
         g_chain.e_second = second;
+        // the owner counts the block barriers it takes with the walk: it leaves after the one that follows these
+        g_chain.n_barriers = bars;
     }
+    return level;
 }
 
-// After a walk: the path entries of its visitors for every level walked, and their list where the node the
-// walk stopped at reads it.  By the wavefront that walked, once the list the walk started from is complete (the
-// helper that writes it says so in LDS; bounded wait).
-__device__ __noinline__ void chain_finish(KernArgsP ka, int lane, int d0, int off, int m) {
-    const int k = __builtin_amdgcn_readfirstlane(g_chain.levels);
-    if (k <= 0) return;
-    const int spin_limit = ka->a.spin_limit;
-    for (int spins = 0;; spins++) {
-        int v = 0;
-        if (lane == 0) v = __hip_atomic_load(&g_chain.part_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (__builtin_amdgcn_readfirstlane(v)) break;
-        if (spins >= spin_limit) {  // the other helper never finished: cannot happen; give the selection up
-            if (lane == 0) atomicCAS(ka->a.sched_wait + 1, 0, 5);
-            return;
-        }
-        __builtin_amdgcn_s_sleep(2);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+// After a walk: the path entries of its visitors for every level, the first of which is the node settled
+// before the walk (all of whose visitors went into the child the walk started at, in their order), and
+// their list where the node the walk stopped at reads it.  Shared by the three wavefronts.
+__device__ __noinline__ void chain_finish(KernArgsP ka, int tid3, int n_threads, int k, int d0, int off, int m) {
     const int32_t *src = d0 == 0 ? ka->a.seg0 : ka->a.seg[(d0 - 1) & 1];
     int32_t *dst = ka->a.seg[(d0 + k - 1) & 1];
     int32_t *paths = ka->a.paths;
     const int stride = ka->a.stride;
-    for (int j = lane; j < m; j += kWave) {
+    for (int j = tid3; j < m; j += n_threads) {
         const int t = src[off + j];
         for (int i = 0; i < k; i++) paths[(size_t)(d0 + 1 + i) * stride + t] = g_chain.nodes[i];
         if (dst != src) dst[off + j] = t;
@@ -2979,6 +3072,42 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         if (!wait_list(a, off, depth, lane)) return kStepParked;
         list_ok = true;
     }
+    if (run_child >= 0 && !as_scatter && !as_slice && m < kHeavyMin && a.vl > 0) {
+        // Every visitor follows one child: nothing to share out.  The helpers walk down from that child for as
+        // long as the visitors stay together, and write the path entries of all those levels, this node's
+        // included (chain_walk, chain_finish); the owner takes the walk's barriers with them (owner_loop).
+        int tn = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (r == (run_child >> 6)) tn = k.n[r];
+        const int np_next = __builtin_amdgcn_readlane(tn, run_child & 63);
+        const int child = c.cb + run_child;
+        const int2 child_span = f.span[child];
+        if (lane == 0) {
+            TeamCmd &cm = lds.cmd;
+            cm.op = kOpChain;
+            cm.c_node = child;
+            cm.c_np = np_next;
+            cm.c_cb = child_span.x;
+            cm.c_cc = child_span.y;
+            cm.c_depth = depth + 1;
+            cm.c_off = off;
+            cm.c_m = m;
+            g_chain.nodes[0] = child;
+            g_chain.n_barriers = -1;
+            atomicAdd(f.VL + child, (int)((uint32_t)a.vl * (uint32_t)m));
+        }
+        __syncthreads();  // the request is open; the owner takes part in its barriers
+        next.node = child;
+        next.off = off;
+        next.m = m;
+        next.np = np_next;
+        next.span = child_span;
+        next.ahead = false;
+        next.chain_open = true;
+        OMK_TICK(14);
+        return kStepDescended;
+    }
     // (1) from the visits per child: the segment of every child, in LDS for all lanes
     uint32_t lmax = 0u;
 #pragma unroll
@@ -3016,15 +3145,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         }
         const int np_next = keep >= 0 ? __builtin_amdgcn_readlane(np_keep, keep & 63) : 0;
         const int off_next = keep >= 0 ? off + __builtin_amdgcn_readlane(ex_keep, keep & 63) : 0;
-        // a kept child of ordinary size: the same request starts the walk down one-winner nodes at it
-        // (chain_walk), so that the owner does not wait for this partition
-        // (only below a node that was itself of that kind: chains are long, and at a node that splits its visitors
-        // the attempt would cost what it saves: the children would be loaded by one wavefront instead of three)
-        const bool chain_next = keep >= 0 && (int)gmax < kHeavyMin && a.vl > 0 && run_child >= 0;
-        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth && !chain_next;
+        const bool ahead_next = RMAX > 1 && keep >= 0 && depth + 1 < a.max_depth;
         if (lane == 0) {
             TeamCmd &cm = lds.cmd;
-            cm.op = chain_next ? kOpChain : kOpPartition;
+            cm.op = kOpPartition;
             cm.rounds = R;
             cm.j_cb = c.cb;
             cm.j_off = off;
@@ -3035,22 +3159,12 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             cm.pre_node = ahead_next ? c.cb + keep : -1;
             cm.pre_np = np_next;
             cm.pre_cc = -1;
-            if (chain_next) {
-                cm.c_node = c.cb + keep;
-                cm.c_np = np_next;
-                cm.c_cb = keep_span.x;
-                cm.c_cc = keep_span.y;
-                cm.c_depth = depth + 1;
-                cm.c_off = off_next;
-                cm.c_m = (int)gmax;
-                g_chain.part_done = 0;
-            }
         }
         __syncthreads();  // the request is open until close_pending
         pending = true;
         next.node = -1;
         next.ahead = false;
-        next.chain_open = chain_next;
+        next.chain_open = false;
         if (keep >= 0) {
             next.node = c.cb + keep;
             next.off = off_next;
@@ -3404,11 +3518,19 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
 #endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
             if (chain_open) {
-                // The node settled before sent all its visitors here, and the request that shares them out also
-                // has a helper walk down from this node for as long as the visitors stay together (chain_walk,
-                // chain_finish): wait for both, and go on where that walk stopped.
+                // The node settled before sent all its visitors here, and the helpers walk down from this node for
+                // as long as the visitors stay together (chain_walk, chain_finish).  Their block barriers count
+                // this wavefront too: it takes them, one per level and the one that ends the request, and goes
+                // on where the walk stopped.
                 chain_open = false;
-                close_pending(pending);
+                for (int taken = 1;; taken++) {
+                    __syncthreads();
+                    int nb = -1;
+                    if (lane == 0) nb = __hip_atomic_load(&g_chain.n_barriers, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    nb = __builtin_amdgcn_readfirstlane(nb);
+                    if (nb >= 0 && taken == nb + 1) break;
+                }
+                pending = true;  // the helpers are writing the path entries: the barrier that ends the request is open
                 it.node = __builtin_amdgcn_readfirstlane(g_chain.e_node);
                 it.np = __builtin_amdgcn_readfirstlane(g_chain.e_np);
                 it.depth = __builtin_amdgcn_readfirstlane(g_chain.e_depth);
@@ -3649,25 +3771,24 @@ __global__ __launch_bounds__(kTeam) void k_select_groups(ForestDev f, SelectArgs
         const float ep = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_lds.cmd.ep)));
         const uint32_t uvl = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_lds.cmd.uvl);
         if (op == kOpChain) {
-            // one helper shares out the visitors of the node just settled, all of which follow one child; another
-            // walks down from that child for as long as they stay together, and then writes their path entries
+            // the helpers walk down from the child that all visitors of the owner's node follow, for as long as
+            // they stay together (three of them in lockstep on a layout with wide nodes, one alone otherwise);
+            // the owner goes on at the barrier that follows the walk, the path entries are written after it
+            // (the request stays open until the owner needs what they write: close_pending)
             const TeamCmd &cm = s_lds.cmd;
-            const int wv = tid >> 6;
-            if (wv == 1) {
-                if (rounds == 1) partition_async<1, RMAX>(f, a, cm, s_part, tid & 63);
-                else partition_async<RMAX, RMAX>(f, a, cm, s_part, tid & 63);
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the kept child's list is written
-                if ((tid & 63) == 0)
-                    __hip_atomic_store(&g_chain.part_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else if (wv == 2) {
-                const KernArgsP ka = (KernArgsP)__builtin_amdgcn_kernarg_segment_ptr();
-                const int c_depth = __builtin_amdgcn_readfirstlane(cm.c_depth), c_m = __builtin_amdgcn_readfirstlane(cm.c_m);
-                const int c_off = __builtin_amdgcn_readfirstlane(cm.c_off);
-                chain_walk<RMAX, RAVE>(ka, (LdsBytesP)&s_lds, tid & 63, __builtin_amdgcn_readfirstlane(cm.c_node),
-                                       __builtin_amdgcn_readfirstlane(cm.c_np), __builtin_amdgcn_readfirstlane(cm.c_cb),
-                                       __builtin_amdgcn_readfirstlane(cm.c_cc), c_depth, c_m);
-                chain_finish(ka, tid & 63, c_depth, c_off, c_m);
-            }
+            const KernArgsP ka = (KernArgsP)__builtin_amdgcn_kernarg_segment_ptr();
+            const int wi = (tid >> 6) - 1;
+            const int c_depth = __builtin_amdgcn_readfirstlane(cm.c_depth), c_m = __builtin_amdgcn_readfirstlane(cm.c_m);
+            const int c_off = __builtin_amdgcn_readfirstlane(cm.c_off);
+            int levels = 0;
+            if (RMAX > 1 || wi == 0)
+                levels = chain_walk<RMAX, RAVE>(ka, (LdsBytesP)&s_lds, wi, tid & 63, __builtin_amdgcn_readfirstlane(cm.c_node),
+                                                __builtin_amdgcn_readfirstlane(cm.c_np),
+                                                __builtin_amdgcn_readfirstlane(cm.c_cb),
+                                                __builtin_amdgcn_readfirstlane(cm.c_cc), c_depth, c_m);
+            __syncthreads();  // the walk has stopped
+            if (RMAX > 1) chain_finish(ka, tid - kWave, kChainWalkers * kWave, levels, c_depth - 1, c_off, c_m);
+            else if (wi == 0) chain_finish(ka, tid & 63, kWave, levels, c_depth - 1, c_off, c_m);
             __syncthreads();  // the request is done
             continue;
         }
