@@ -62,6 +62,16 @@ template <class S, class = void>
 struct has_hash : std::false_type {};
 template <class S>
 struct has_hash<S, std::void_t<decltype(std::declval<const S &>().getHash())>> : std::true_type {};
+// a node type that reports its value sum and its RAVE value sum as they are stored (the reference's MCTSNode
+// exposes the means only, include/mcts/mcts_node.h:93,163: one-line accessors a maintainer adds)
+template <class N, class = void>
+struct has_value_sum : std::false_type {};
+template <class N>
+struct has_value_sum<N, std::void_t<decltype(std::declval<const N &>().getValueSum())>> : std::true_type {};
+template <class N, class = void>
+struct has_rave_value_sum : std::false_type {};
+template <class N>
+struct has_rave_value_sum<N, std::void_t<decltype(std::declval<const N &>().getRAVEValueSum())>> : std::true_type {};
 }  // namespace detail
 
 // The arrays of a flattened tree, owning their memory; view() is what omk_forest_upload takes.
@@ -89,9 +99,13 @@ struct FlatTree {
 // Breadth-first flattening of a pointer tree: the root becomes node 0, the children of a node take
 // consecutive ids in the order of its children vector (so "lowest child index wins a tie" keeps its
 // meaning).  Node is anything with MCTSNode's accessors: getChildren() (a container of pointers to
-// Node), getAction(), getVisitCount(), getValue() (the mean: the value sum is mean * visits, exact
-// whenever the sum is what the mean was divided from), getPriorProbability(), getVirtualLoss(),
-// getRAVECount(), getRAVEValue().  node_of_id (optional) receives the node behind every id.
+// Node), getAction(), getVisitCount(), getValue(), getPriorProbability(), getVirtualLoss(),
+// getRAVECount(), getRAVEValue().  The value sums: getValueSum() / getRAVEValueSum() when the node type
+// has them (the stored sums: a search that goes on from the arrays is then bit for bit the one that
+// would have gone on from the pointer tree); otherwise mean * visits, which in binary32 is NOT in
+// general the sum the mean was divided from ((W / N) * N can differ from W in the last place), so
+// statistics and near-tie selections of the continued search can differ from the pointer tree's.
+// node_of_id (optional) receives the node behind every id.
 template <class Node>
 FlatTree flattenTree(Node &root, std::vector<Node *> *node_of_id = nullptr) {
     FlatTree t;
@@ -107,12 +121,14 @@ FlatTree flattenTree(Node &root, std::vector<Node *> *node_of_id = nullptr) {
     for (Node *node : order) {
         const int visits = node->getVisitCount();
         t.N.push_back(visits);
-        t.W.push_back(node->getValue() * (float)visits);
+        if constexpr (detail::has_value_sum<Node>::value) t.W.push_back(node->getValueSum());
+        else t.W.push_back(node->getValue() * (float)visits);
         t.P.push_back(node->getPriorProbability());
         t.VL.push_back(node->getVirtualLoss());
         const int rave_visits = node->getRAVECount();
         t.rN.push_back(rave_visits);
-        t.rW.push_back(node->getRAVEValue() * (float)rave_visits);
+        if constexpr (detail::has_rave_value_sum<Node>::value) t.rW.push_back(node->getRAVEValueSum());
+        else t.rW.push_back(node->getRAVEValue() * (float)rave_visits);
         t.action.push_back(node->getAction());
     }
     if (node_of_id) *node_of_id = order;

@@ -70,14 +70,8 @@ constexpr int kTeamWaves = 4;             // wavefronts per block of the multi-v
 constexpr int kTeam = kTeamWaves * 64;
 constexpr int kTeamMin = 96;              // batch entries from which the helpers are called in
 // a batch of at most this many entries per thread is ordered by counting: a lone wavefront, the block
-#ifndef OMK_COUNT_SORT_TEAM
-#define OMK_COUNT_SORT_TEAM 1
-#endif
-constexpr int kCountSortLone = 2, kCountSortTeam = OMK_COUNT_SORT_TEAM;
-#ifndef OMK_SLICE_ENTRIES
-#define OMK_SLICE_ENTRIES 192
-#endif
-constexpr int kSliceEntries = OMK_SLICE_ENTRIES;  // visitors per slice of such a node, about
+constexpr int kCountSortLone = 2, kCountSortTeam = 1;
+constexpr int kSliceEntries = 192;        // visitors per slice of such a node, about
 constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
@@ -2393,6 +2387,15 @@ __shared__ ChainSlot g_chain_slot[2][kChainWalkers];
 
 // wi: which of the three walking wavefronts this is.  Every block barrier in here is also taken by the owner,
 // which waits the walk out (owner_loop).
+// The statistics of the children one walking wavefront is responsible for, as loaded.
+template <int Q>
+struct ChainKids {
+    int n[Q], vl[Q];
+    float w[Q], p[Q], q2[Q];
+    int2 sp[Q];
+    uint32_t word[Q];  // legality bits
+};
+
 template <int RMAX, bool RAVE>
 __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, int lane, int node, int np, int cb,
                                        int cc, int depth, int m) {
@@ -2412,66 +2415,78 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
     int bars = 0;   // block barriers taken
     int kids = 0, contested = 0, best0 = -1, second = 0;
     uint32_t lk0 = 0u;
-    for (;;) {
-        if (cc <= 0 || depth >= max_depth || level >= kChainMaxLevels) break;
-        const long long tr0 = trace && wi == 0 ? wall_clock64() : 0ll;
-        int nelig = cc;
+    auto eligible = [&](int np_, int cc_) {
+        int e = cc_;
         if (pw) {
-            const int kk = ceil_sqrt_i32(np);
-            nelig = kk < cc ? kk : cc;
+            const int kk = ceil_sqrt_i32(np_);
+            e = kk < cc_ ? kk : cc_;
         }
-        const float ep = c_puct * sqrtf((float)np);
-        const int par = level & 1;
-        // ---- this wavefront's rounds of the children ----
-        int kn[Q], kvl[Q];
-        float kw[Q], kp[Q], kq2[Q];
-        uint32_t k1[Q], k2[Q];
-        bool kin[Q];
-        int2 ksp[Q];
-        {
-            uint32_t word[Q];
+        return e;
+    };
+    // asks for this wavefront's rounds of the children cb_ .. cb_ + nelig_ - 1 (nothing waits for them here)
+    auto issue = [&](ChainKids<Q> &k, int cb_, int nelig_) {
 #pragma unroll
-            for (int q = 0; q < Q; q++) {
-                const int r = wi * Q + q;
-                const int i = r * kWave + lane;
-                const bool in = i < nelig;
-                const int id = cb + i;
-                word[q] = 0xFFFFFFFFu;
-                kn[q] = 0;
-                kw[q] = 0.0f;
-                kp[q] = 0.0f;
-                kvl[q] = 0;
-                kq2[q] = 0.0f;
-                ksp[q] = int2{0, 0};
-                if (r * kWave < nelig) {  // uniform: rounds the node lacks are skipped
-                    if (in && flegal) word[q] = flegal[(uint32_t)id >> 5];
-                    if (in) {
-                        kn[q] = fN[id];
-                        kw[q] = fW[id];
-                        kp[q] = fP[id];
-                        kvl[q] = fVL[id];
-                        if (RAVE) kq2[q] = fq2[id];
-                        ksp[q] = fspan[id];
-                    }
+        for (int q = 0; q < Q; q++) {
+            const int r = wi * Q + q;
+            const int i = r * kWave + lane;
+            const bool in = i < nelig_;
+            const int id = cb_ + i;
+            k.word[q] = 0xFFFFFFFFu;
+            k.n[q] = 0;
+            k.w[q] = 0.0f;
+            k.p[q] = 0.0f;
+            k.vl[q] = 0;
+            k.q2[q] = 0.0f;
+            k.sp[q] = int2{0, 0};
+            if (r * kWave < nelig_) {  // uniform: rounds the node lacks are skipped
+                if (in && flegal) k.word[q] = flegal[(uint32_t)id >> 5];
+                if (in) {
+                    k.n[q] = fN[id];
+                    k.w[q] = fW[id];
+                    k.p[q] = fP[id];
+                    k.vl[q] = fVL[id];
+                    if (RAVE) k.q2[q] = fq2[id];
+                    k.sp[q] = fspan[id];
                 }
             }
+        }
+    };
+    int nelig = eligible(np, cc);
+    bool alive = !(cc <= 0 || depth >= max_depth || level >= kChainMaxLevels);
+    ChainKids<Q> kids_a, kids_b;
+    if (alive) issue(kids_a, cb, nelig);
+    // One level: `cur` holds (or is about to receive) the children of the node the walk stands at; the
+    // children of the child it moves on into are asked for into `nxt` as soon as that child is known, before
+    // the one-winner test, whose arithmetic then runs while they are on their way (they are dropped if the
+    // test fails).  Returns whether the walk goes on.
+    auto step = [&](ChainKids<Q> &cur, ChainKids<Q> &nxt) -> bool {
+        const long long tr0 = trace && wi == 0 ? wall_clock64() : 0ll;
+        const float ep = c_puct * sqrtf((float)np);
+        const int par = level & 1;
+        int (&kn)[Q] = cur.n;
+        int (&kvl)[Q] = cur.vl;
+        float (&kw)[Q] = cur.w;
+        float (&kp)[Q] = cur.p;
+        float (&kq2)[Q] = cur.q2;
+        int2 (&ksp)[Q] = cur.sp;
+        uint32_t k1[Q], k2[Q];
+        bool kin[Q];
 #pragma unroll
-            for (int q = 0; q < Q; q++) {
-                const int r = wi * Q + q;
-                const int i = r * kWave + lane;
-                const int id = cb + i;
-                kin[q] = i < nelig && ((word[q] >> ((uint32_t)id & 31u)) & 1u);
-                k1[q] = k2[q] = 0u;
-                if (r * kWave < nelig) {
-                    if (kin[q]) {
-                        child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
-                    } else {
-                        kn[q] = 0;
-                        kw[q] = 0.0f;
-                        kp[q] = 0.0f;
-                        kvl[q] = 0;
-                        kq2[q] = 0.0f;
-                    }
+        for (int q = 0; q < Q; q++) {
+            const int r = wi * Q + q;
+            const int i = r * kWave + lane;
+            const int id = cb + i;
+            kin[q] = i < nelig && ((cur.word[q] >> ((uint32_t)id & 31u)) & 1u);
+            k1[q] = k2[q] = 0u;
+            if (r * kWave < nelig) {
+                if (kin[q]) {
+                    child_keys<RAVE>(kn[q], kw[q], kp[q], kvl[q], kq2[q], ep, k1[q], k2[q]);
+                } else {
+                    kn[q] = 0;
+                    kw[q] = 0.0f;
+                    kp[q] = 0.0f;
+                    kvl[q] = 0;
+                    kq2[q] = 0.0f;
                 }
             }
         }
@@ -2594,6 +2609,10 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)spos);
         any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
         }  // !SOLO
+        // ---- the children of the child the walk would move on into: on their way during the test ----
+        const int n_nelig = eligible(bn, bsy);
+        const bool n_alive = hk != 0u && !(bsy <= 0 || depth + 1 >= max_depth || level + 1 >= kChainMaxLevels);
+        if (n_alive) issue(nxt, bsx, n_nelig);
         // ---- the one-winner test (single_run) ----
         // (with RAVE and no real first-scan score at all the reference never runs its second scan;
         // select_group knows, and gets no verdict)
@@ -2629,7 +2648,7 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
                         chain_dump<RMAX>(scratch, (wi * Q + q) * kWave + lane, kn[q], kw[q], kp[q], kvl[q], kq2[q], k1[q],
                                          k2[q], kin[q]);
             }
-            break;
+            return false;
         }
         // ---- every visitor takes that child ----
         const int child = cb + best;
@@ -2659,6 +2678,15 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         cc = bsy;
         depth++;
         level++;
+        nelig = n_nelig;
+        alive = n_alive;
+        return n_alive;
+    };
+    if (alive) {
+        for (;;) {
+            if (!step(kids_a, kids_b)) break;
+            if (!step(kids_b, kids_a)) break;
+        }
     }
     if (wi == 0 && lane == 0) {
         g_chain.levels = level;

@@ -69,6 +69,23 @@ struct PtrNode {
     float getRAVEValue() const { return rave_n ? rave_sum / rave_n : 0.0f; }
 };
 
+// the same with the two one-line accessors of the stored sums that flattenTree prefers when they exist
+struct SumNode {
+    std::vector<std::shared_ptr<SumNode>> children;
+    int action = -1, visits = 0, rave_n = 0;
+    float value_sum = 0.0f, prior = 0.0f, rave_sum = 0.0f;
+    std::vector<std::shared_ptr<SumNode>> &getChildren() { return children; }
+    int getAction() const { return action; }
+    int getVisitCount() const { return visits; }
+    float getValue() const { return visits ? value_sum / visits : 0.0f; }
+    float getValueSum() const { return value_sum; }
+    float getPriorProbability() const { return prior; }
+    int getVirtualLoss() const { return 0; }
+    int getRAVECount() const { return rave_n; }
+    float getRAVEValue() const { return rave_n ? rave_sum / rave_n : 0.0f; }
+    float getRAVEValueSum() const { return rave_sum; }
+};
+
 // stands for the reference's own mcts::NetworkOutput (include/mcts/evaluation_types.h:14-17): the search
 // takes the evaluator's output type as it is
 struct RefNetworkOutput {
@@ -168,6 +185,29 @@ static int run_flatten() {
     for (size_t i = 0; i < t.N.size(); i++)
         printf("flat %zu %d %.9g %.9g %d %d %.9g %d %d %d\n", i, t.N[i], t.W[i], t.P[i], t.VL[i], t.rN[i], t.rW[i],
                t.child_begin[i], t.child_count[i], t.action[i]);
+    // value sums that (sum / visits) * visits does not give back in binary32: with the accessors of the stored
+    // sums the arrays hold the sums themselves
+    {
+        SumNode sroot;
+        sroot.visits = 100;
+        int lossy = 0;
+        for (int i = 0; i < 40; i++) {
+            auto c = std::make_shared<SumNode>();
+            c->action = i;
+            c->visits = 3 + i;
+            c->value_sum = 0.1f * (float)(i + 1) + 0.013f;
+            c->rave_n = 7 + i;
+            c->rave_sum = -0.37f * (float)(i + 1);
+            c->prior = 0.025f;
+            if (c->getValue() * (float)c->visits != c->value_sum) lossy++;
+            sroot.children.push_back(c);
+        }
+        omk::FlatTree st = omk::flattenTree(sroot);
+        int exact = 0;
+        for (size_t i = 1; i < st.N.size(); i++)
+            if (st.W[i] == sroot.children[i - 1]->value_sum && st.rW[i] == sroot.children[i - 1]->rave_sum) exact++;
+        printf("sums exact %d of %zu, mean times visits differs from the sum for %d\n", exact, st.N.size() - 1, lossy);
+    }
     // the flattened tree searches on the device
     omk::MCTSSettings s;
     s.max_depth = 4;

@@ -305,3 +305,64 @@ def test_chain_through_narrow_and_wide_nodes(rave, kind, visitors):
     st = select_both(soa, np.zeros(visitors, np.int32), 22, rave=rave, steps=3)
     assert st["replayed_nodes"] == 0, st
 
+
+
+def capacity_chain(fan, depth, at, m, rave, seed=5):
+    """A spine of `depth` nodes, every one of which sends all m visitors into its spine child, except the
+    node at level `at`: there one sibling's prior is the smallest binary32 number with which it is chosen at
+    all, found by bisection on the checker itself, so that the spine child's capacity (the visitors it
+    takes before any other child gets one) is exactly m - 1: the LAST visitor leaves the spine."""
+    rng = np.random.default_rng(seed)
+    N, W, P, cb, cc, act, rN, rW = [10 ** 6], [0.0], [0.0], [0], [0], [-1], [0], [0.0]
+    spine, special = 0, -1
+    for d in range(depth):
+        first = len(N)
+        cb[spine], cc[spine] = first, fan
+        nxt = int(rng.integers(fan))
+        for i in range(fan):
+            if i == nxt:
+                N.append(100000); W.append(90000.0); P.append(0.9)
+                rN.append(50); rW.append(40.0)
+            else:
+                n = int(rng.integers(1, 30))
+                N.append(n); W.append(float(np.float32(-rng.uniform(0, n)))); P.append(0.1 / fan)
+                rN.append(int(rng.integers(0, 9))); rW.append(float(np.float32(-rng.uniform(0, 3))))
+            cb.append(0); cc.append(0); act.append(i)
+        if d == at:
+            special = first + (nxt + 1) % fan
+            N[special], W[special], rN[special], rW[special] = 0, 0.0, 0, 0.0
+        spine = first + nxt
+    soa = dict(N=np.array(N, np.int32), W=np.array(W, np.float32), P=np.array(P, np.float32),
+               VL=np.zeros(len(N), np.int32), child_begin=np.array(cb, np.int32), child_count=np.array(cc, np.int32),
+               action=np.array(act, np.int32))
+    if rave:
+        soa["rN"], soa["rW"] = np.array(rN, np.int32), np.array(rW, np.float32)
+    rp = R.make_params(c_puct=1.4, virtual_loss=3, use_rave=rave, rave_k=1000.0, max_depth=depth + 2)
+    roots = np.zeros(m, np.int32)
+
+    def taken(p):
+        soa["P"][special] = p
+        paths, plen, _, _ = R.RefTree.from_soa(soa).select_batch(roots, rp, near_ties=False)
+        return np.nonzero(paths[:, at + 1] == special)[0]
+
+    lo, hi = np.float32(0.0), np.float32(1.0)
+    assert len(taken(lo)) == 0 and len(taken(hi)) > 0
+    while np.nextafter(lo, np.float32(2.0)) < hi:
+        mid = np.float32((np.float64(lo) + np.float64(hi)) / 2)
+        if len(taken(mid)):
+            hi = mid
+        else:
+            lo = mid
+    who = taken(hi)
+    assert who.tolist() == [m - 1], who       # the last visitor, and nobody else, leaves the spine at that level
+    return soa
+
+
+@pytest.mark.parametrize("fan,rave,m", [(40, False, 200), (300, True, 200), (362, False, 37), (9, True, 900)])
+def test_chain_whose_capacity_is_exceeded_by_one_visitor(fan, rave, m):
+    """25 nodes in a row whose visitors all follow one child; at the 12th the best child takes all visitors
+    but the last one.  The walk down such nodes must stop exactly there, and hand the node over with
+    the right verdict."""
+    soa = capacity_chain(fan, 25, 11, m, rave)
+    st = select_both(soa, np.zeros(m, np.int32), 27, rave=rave, steps=2)
+    assert st["replayed_nodes"] == 0, st

@@ -219,6 +219,9 @@ def test_flatten_tree_lays_a_pointer_tree_out_breadth_first_and_searches_on():
     assert flat[:, 6].tolist() == [1, 4, 0, 6, 0, 0, 0] and flat[:, 7].tolist() == [3, 2, 0, 1, 0, 0, 0]
     assert flat[:, 8].tolist() == [-1, 7, 2, 9, 1, 4, 5]
     assert flat[:, 1].tolist() == [4.0, 8.0, -3.0, 0.5, 2.25, -5.0, 1.5]        # value sums back from the means
+    # a node type with accessors of the stored sums: taken as they are, where mean * visits would lose the last bit
+    sums = next(ln for ln in r.stdout.split("\n") if ln.startswith("sums exact")).replace(",", "").split()
+    assert int(sums[2]) == int(sums[4]) == 40 and int(sums[-1]) > 0, sums
     assert flat[:, 3].tolist() == [0, 0, 3, 0, 0, 0, 0] and flat[:, 4].tolist() == [0, 10, 6, 3, 4, 5, 3]
     ref = R.RefTree(N=flat[:, 0], W=flat[:, 1], P=flat[:, 2], VL=flat[:, 3], child_begin=flat[:, 6], child_count=flat[:, 7],
                     action=flat[:, 8])
