@@ -289,7 +289,7 @@ def traffic_of(workload):
         "kernel; not measured in this run" % tj[workload].get("command", "bench.py --workload %s" % workload))
 
 
-def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parity=True, relaid=False):
+def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parity=True, relaid=False, seeded_repeats=0):
     """Everything bench.py reports about one workload.  relaid: the same forest without the empty
     slots of its board layout (omk_soa_compact_legal), the layout of the reference's own children_
     vectors; everything (byte model, parity, CPU baseline) is then taken on that forest."""
@@ -396,7 +396,7 @@ def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parit
     # uniform value sums; the K steps above drift away from them with every backup): the seeded statistics are
     # uploaded again and the roots set again before every repeat, outside the events; the byte model is
     # taken on the paths of that very selection.  This is what the roofline is quoted on.
-    reps = max(3, min(K, 7))
+    reps = seeded_repeats if seeded_repeats > 0 else max(3, min(K, 7))
     seeded_ms = []
     e0, e1 = ev.create(), ev.create()
     for _ in range(reps):
@@ -520,6 +520,9 @@ def main():
                     help="budget of the CPU baseline leg of --workload (0 = skip); the other configurations get a third")
     ap.add_argument("--scale", type=float, default=1.0, help="scale nodes_per_tree (debugging only)")
     ap.add_argument("--no-parity", action="store_true", help="skip the comparison with the CPU checker")
+    ap.add_argument("--seeded-repeats", type=int, default=0,
+                    help="selections timed on the seeded statistics (each after a fresh upload); 0: min(steps, 7), "
+                         "at least 3")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only run the plain copy kernel over this many MiB, 10 times (to scale profiler "
                          "traffic counters by) and exit")
@@ -544,7 +547,7 @@ def main():
         return
 
     head = measure(omk, synth, args.workload, args.steps, args.warmup, args.seed, args.cpu_seconds, args.scale,
-                   parity=not args.no_parity, relaid=args.head_relaid)
+                   parity=not args.no_parity, relaid=args.head_relaid, seeded_repeats=args.seeded_repeats)
 
     # outside every timed region: three plain copies of 64 MiB, the known-size kernel that a
     # profiler run of this command scales its traffic counters by
@@ -601,7 +604,7 @@ def main():
             r = head
         else:
             r = measure(omk, synth, name, args.steps, args.warmup, args.seed, args.cpu_seconds / 3.0, args.scale,
-                        parity=not args.no_parity)
+                        parity=not args.no_parity, seeded_repeats=args.seeded_repeats)
         per[name] = {
             "workload": r["workload"],
             "select_ms": r["select_ms"],
@@ -667,7 +670,7 @@ def main():
             print("bench.py: %r in --relaid is not a board workload" % name, file=sys.stderr)
             sys.exit(2)
         rel[name] = short(measure(omk, synth, name, args.steps, args.warmup, args.seed, 0.0, args.scale,
-                                  parity=not args.no_parity, relaid=True))
+                                  parity=not args.no_parity, relaid=True, seeded_repeats=args.seeded_repeats))
     if rel:
         out["per_config_relaid"] = rel
     print(json.dumps(out))

@@ -129,6 +129,7 @@ struct omk_batch {
     int32_t *q_ready = nullptr;  // per queue slot: number of the select call that published it
     int32_t *single_ready = nullptr;  // the same per entry of the single-visitor queue
     int32_t *hctx = nullptr;     // contexts of heavy nodes
+    int32_t *hbound = nullptr;   // boundaries between their slices
     int32_t *list_flag = nullptr;  // per visitor-list start: which depth's list is complete
     int32_t hctx_cap = 0;
     int32_t q_cap = 0;
@@ -908,6 +909,9 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     b->q_cap = (int32_t)((B / 2 + B / 16 + 64) * (max_depth + 1));
     b->hctx_cap = (int32_t)std::min<int64_t>(4096, (B / kHeavyMin) * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->hctx, (int64_t)b->hctx_cap * kHeavyCtxInts);
+    if (e == hipSuccess) e = dalloc(&b->hbound, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts);
+    if (e == hipSuccess)
+        e = hipMemset(b->hbound, 0, (size_t)std::max<int64_t>((int64_t)b->hctx_cap * kMaxSlices * kBoundInts, 1) * 4);
     if (e == hipSuccess) e = dalloc(&b->list_flag, B);
     if (e == hipSuccess) e = dalloc(&b->items_q, b->q_cap);
     if (e == hipSuccess) e = dalloc(&b->q_ready, b->q_cap);
@@ -944,7 +948,7 @@ int omk_batch_destroy(omk_batch *b) {
     (void)hipStreamSynchronize(b->f->stream);
     void *ptrs[] = {b->paths,  b->path_len, b->leaf,     b->values, b->items0,   b->items_q,  b->seg0,
                     b->seg[0], b->seg[1],   b->sc_child, b->sc_occ, b->counters, b->out_paths, b->out_actions,
-                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->exp_buf, b->list_flag, b->single_ready};
+                    b->singles0, b->singles_q, b->q_ready, b->hctx, b->hbound, b->exp_buf, b->list_flag, b->single_ready};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     (void)hipGetLastError();
@@ -1050,6 +1054,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
         HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
         HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
+        HIP_TRY(launch_fill_words(b->hbound, 0u, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts, f->stream));
         // the two depth-cap counters take turns by call parity, which this restart breaks once
         HIP_TRY(launch_fill_words(b->counters + kTruncatedWord, 0u, 2, f->stream));
         b->epoch = 0;
@@ -1073,6 +1078,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.fast_singles = 0;
     a.poll_sleep = b->poll_sleep;
     a.hctx = b->hctx;
+    a.hbound = b->hbound;
     a.hctx_n = b->counters + 2 * kSchedStep + 64;
     a.hctx_cap = b->hctx_cap;
     a.list_flag = b->list_flag;

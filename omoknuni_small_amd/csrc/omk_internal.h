@@ -39,6 +39,13 @@ struct Item {
 
 constexpr int kHeavyCtxInts = 16 + 1024;  // 16 + the widest fan-out
 constexpr int kHeavyMin = 1024;          // visitors from which a node is settled by several wavefronts
+constexpr int kMaxSlices = 64;           // slices (and parts of the partition) of such a node, at most
+constexpr int kHeavyFanout = 384;        // widest node settled that way (register budget)
+// What the slices of a heavy node hand to each other: slice s works out the boundary between itself and
+// slice s + 1 and leaves it here for that slice.  Per boundary: [0] == the number of the select call once the
+// rest is written, [1] the threshold key, [2] entries above the boundary, [3] 1 = worked out, 0 = the
+// threshold search failed, [16 + i] entries of child i above the boundary.
+constexpr int kBoundInts = 16 + kHeavyFanout;
 
 struct SelectArgs {
     const Item *items0;    // level-0 items with several visitors, built when the roots are set
@@ -57,6 +64,7 @@ struct SelectArgs {
     int32_t *hctx;         // contexts of heavy nodes, kHeavyCtxInts each: [0] slices still running,
                            // [1] a slice failed a check, [16 + i] visits of child i
     int32_t *hctx_n;       // contexts handed out
+    int32_t *hbound;       // boundaries between the slices of heavy nodes: kMaxSlices x kBoundInts per context
     int32_t *list_flag;    // per visitor-list start: depth of the deepest item whose list, starting there,
                            // is complete (items of kind 3 are published before their list is written)
     int32_t hctx_cap;

@@ -72,11 +72,9 @@ constexpr int kTeamMin = 96;              // batch entries from which the helper
 // a batch of at most this many entries per thread is ordered by counting: a lone wavefront, the block
 constexpr int kCountSortLone = 2, kCountSortTeam = 1;
 constexpr int kSliceEntries = 192;        // visitors per slice of such a node, about
-constexpr int kMaxSlices = 64;
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
-constexpr int kHeavyFanout = 384;         // widest node settled that way (register budget)
 constexpr int kMaxWalkerBlocks = 16;         // blocks of walkers of the persistent launch, at most
 constexpr int kFastSinglesMax = 16384;    // traversals up to which the single-visitor kernel trades bytes for latency
 constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
@@ -578,6 +576,10 @@ struct ChainLds {
 typedef __attribute__((address_space(3))) unsigned char *LdsBytesP;
 // one per block of the multi-visitor kernel
 __shared__ ChainLds g_chain;
+// The timeline, when it is switched on: what a slice of a heavy node did (100 MHz clock): [0] thresholds and
+// exact counts, [1] its batch(es), [2] entries of its first batch, or -1 when it had to search for it, [3] visitors
+// it settled.  One per block.
+__shared__ int g_slice_note[4];
 
 
 // The owner may have left the partition of its previous node with a helper: the block
@@ -1795,16 +1797,17 @@ __device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, floa
         });
 }
 
-// For a slice of a heavy node: the thresholds of the cumulative targets target_hi and
-// target_lo (0 = not wanted) and EXACTLY how many entries of every own child lie at or above
-// each (ct_hi, ct_lo; at most m each).  Every wavefront that asks for the same target of the
-// same node gets the same threshold: the computation is deterministic and depends on the
-// node's state only.  Uses the LDS scratch.
-template <int R, bool RAVE>
+// For a slice of a heavy node: the boundary of the cumulative target `target`: a threshold key T
+// and EXACTLY how many entries of every own child lie above the boundary (ct; at most m each): the
+// entries at or above T, or, where far more entries than the target pile up on T itself, those over T and
+// the first of the pile (see below).  Deterministic, a function of the node's state and the target only.
+// Uses the LDS scratch.
+// TWO: the boundary of a second target as well (target2 > 0; ct2, T2), on the same preparation.
+template <int R, bool RAVE, bool TWO>
 __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const NodeCtx &c, int lane,
                                                  const Kids<R, RAVE> &k, WaveLds<R> &lds, int m, int window,
-                                                 int target_hi, int target_lo, int (&ct_hi)[R], int (&ct_lo)[R],
-                                                 uint32_t &T_hi, uint32_t &T_lo) {
+                                                 int target1, int (&ct1)[R], uint32_t &T1, int target2, int (&ct2)[R],
+                                                 uint32_t &T2) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     OMK_S0();
@@ -1886,37 +1889,94 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     }
     int cta[R];
     OMK_STAMP(9);
-    T_hi = 0xFFFFFFFFu;
-    T_lo = 0u;
-#pragma unroll
-    for (int r = 0; r < R; r++) ct_hi[r] = ct_lo[r] = 0;
-    if (target_hi > 0) {
-        T_hi = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_hi, window, m, lane);
+    auto boundary = [&](int target, int (&ct)[R], uint32_t &T) {
+    // The boundary of one target: the threshold and the exact counts at it.  When far more entries than the
+    // target lie at or above the threshold, they are piled up ON the threshold key (a child whose key does not
+    // move at all over hundreds of visits; no key separates them), and the boundary is put inside the pile:
+    // entries of one key are played child after child by position (first-scan candidates in child order, then
+    // second-scan candidates; comes_before), each child's in visit order, so the first `target - above` of the
+    // pile in that order belong above the boundary, where `above` counts the entries at keys over the threshold
+    // (none of the pile when `above` reaches the target by itself).  The counts that come out add up to
+    // max(target, above); they are still a function of the node and the target alone, and grow with the target:
+    // two targets with one threshold share `above`, and of two thresholds the lower one's `above` holds
+    // everything at or above the higher one.  Whoever uses the counts checks the order they imply like any
+    // other (water_level: the last entry kept must come before every child's next one).
+        T = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target, window, m, lane);
         OMK_STAMP(10);
-        active_counts<R, RAVE>(s, c.ep, uvl, T_hi, m, cta, lane);
+        active_counts<R, RAVE>(s, c.ep, uvl, T, m, cta, lane);
         OMK_STAMP(11);
+        int sum = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) sum += cta[r];
+        const int at_or_above = wave_sum_i32(sum);
+        if (at_or_above - target > window && T < hi_key) {
+            int ctb[R];  // entries at keys over the threshold
+            active_counts<R, RAVE>(s, c.ep, uvl, T + 1u, m, ctb, lane);
+            sum = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) sum += ctb[r];
+            const int above = wave_sum_i32(sum);
+            if (above >= target) {
+                // the key above the threshold has enough already (the search works on estimates): the boundary
+                // goes between the two keys
+#pragma unroll
+                for (int r = 0; r < R; r++) cta[r] = ctb[r];
+            } else {
+                // the pile: e entries of every child at the threshold key, from its visit number ctb on; where
+                // the child stands in the order of the pile
+                int e1[R], e2[R];
+                bool odd = false;
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    e1[r] = e2[r] = 0;
+                    const int e = cta[r] - ctb[r];
+                    if (r < s.rounds && s.c[r] >= 0 && e > 0) {
+                        uint32_t kk, pp;
+                        entry_key<R, RAVE>(s.n[r], s.w[r], s.p[r], s.vl[r], s.q2[r], c.ep, uvl, ctb[r], s.c[r], kk, pp);
+                        if (kk != T) odd = true;
+                        if (pp >= (uint32_t)F) e2[r] = e;
+                        else e1[r] = e;
+                    } else if (e < 0) {
+                        odd = true;
+                    }
+                }
+                if (__ballot(odd) == 0ull) {
+                    int need = target - above;
+                    // the active children are listed in child order: first-scan candidates first, in that order
+                    int carry = 0;
+                    int take[R];
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int inc = wave_inclusive_sum(e1[r], lane);
+                        const int before = carry + inc - e1[r];
+                        const int left = need - before;
+                        take[r] = e1[r] > 0 ? (left <= 0 ? 0 : (left < e1[r] ? left : e1[r])) : 0;
+                        carry += __builtin_amdgcn_readlane(inc, 63);
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int inc = wave_inclusive_sum(e2[r], lane);
+                        const int before = carry + inc - e2[r];
+                        const int left = need - before;
+                        if (e2[r] > 0) take[r] = left <= 0 ? 0 : (left < e2[r] ? left : e2[r]);
+                        carry += __builtin_amdgcn_readlane(inc, 63);
+                    }
+#pragma unroll
+                    for (int r = 0; r < R; r++) cta[r] = ctb[r] + take[r];
+                }
+            }
+        }
 #pragma unroll
         for (int r = 0; r < R; r++)
             if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
         wave_sync_memory();
 #pragma unroll
-        for (int r = 0; r < R; r++) ct_hi[r] = (int)lds.pay[r * kWave + lane];
+        for (int r = 0; r < R; r++) ct[r] = (int)lds.pay[r * kWave + lane];
         wave_sync_memory();
-    }
-    if (target_lo > 0) {
-        T_lo = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target_lo, window, m, lane);
-        OMK_STAMP(10);
-        active_counts<R, RAVE>(s, c.ep, uvl, T_lo, m, cta, lane);
-        OMK_STAMP(11);
-#pragma unroll
-        for (int r = 0; r < R; r++)
-            if (s.c[r] >= 0) lds.pay[s.c[r]] = (uint32_t)cta[r];
-        wave_sync_memory();
-#pragma unroll
-        for (int r = 0; r < R; r++) ct_lo[r] = (int)lds.pay[r * kWave + lane];
-        wave_sync_memory();
-    }
-    if (a.stats && lane == 0) atomicAdd(a.stats + 5, (target_hi > 0) + (target_lo > 0));
+    };
+    boundary(target1, ct1, T1);
+    if (TWO && target2 > 0) boundary(target2, ct2, T2);
+    if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1 + (TWO && target2 > 0 ? 1 : 0));
     return true;
 }
 
@@ -2740,12 +2800,13 @@ struct Continuation {
 //
 // A heavy node (kHeavyMin visitors or more) is cut into slices of its winner order, one
 // queue item each, that wavefronts settle side by side: slice s covers the ranks between
-// the exact entry counts at two score thresholds, T_s and T_s+1, which every slice derives
-// for itself (threshold_counts: same input, same result).  A slice starts the batch loop
-// from the state "child i has had count_i(T_s) visits" and must arrive exactly at
-// count_i(T_s+1); with that check, T_s >= T_s+1, and the batch loop's own checks, slice
-// after slice starts from the true serial state, so the slices together are the serial
-// order.  The slice that reaches the last visitor writes the visits per child; the
+// two boundaries, s and s+1, each a score threshold with the exact entry counts of every child
+// above it (threshold_counts; a boundary may lie inside a pile of entries of one key).  Slice s
+// works out boundary s+1 and leaves it in the node's boundary table, where slice s+1 picks it up:
+// the two neighbours use the same numbers.  A slice starts the batch loop from the state "child i
+// has had count_i(boundary s) visits" and must arrive exactly at count_i(boundary s+1); with that
+// check, T_s >= T_s+1, and the batch loop's own checks, slice after slice starts from the true
+// serial state, so the slices together are the serial order.  The slice that reaches the last visitor writes the visits per child; the
 // wavefront that finishes last (a counter in the node's context) partitions the visitors
 // and walks on, every other returns kStepParked.  Any failed check sends the whole node
 // back to the one-wavefront path.
@@ -2957,16 +3018,84 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             uint32_t T_hi = 0xFFFFFFFFu, T_lo = 0u;
             // the window inside which a threshold search may stop early: narrower than the
             // distance between the targets of two slices
-            ok = threshold_counts<R, RAVE>(a, c, lane, k, lds, m, S >> 2, slice > 0 ? slice * S : 0,
-                                           last ? 0 : (slice + 1) * S, ct_hi, ct_lo, T_hi, T_lo);
+            const long long ts0 = a.trace ? wall_clock64() : 0ll;
+            long long ts1 = ts0;
+            // Every slice works out ONE boundary, the one between itself and the next slice (the last slice: the
+            // threshold of the node's last visitor, with which it knows its one batch like every other slice
+            // instead of searching for it in the batch loop), leaves it in the node's boundary table, and takes
+            // the boundary between the slice before and itself from there: both neighbours use the same numbers
+            // by construction, and nobody searches the same threshold twice.  The slice before was handed out
+            // earlier (slice 0 runs on the wavefront that cut the node), and it writes its boundary before it
+            // waits for anything, so the wait below ends; it is bounded like every other.
+            // A narrow node's boundaries are cheap: every slice works out both of its own (same input, same
+            // result on both sides of a boundary), which costs less than handing them over.
+            constexpr bool kHandOver = R > 1;
+            ok = threshold_counts<R, RAVE, !kHandOver>(a, c, lane, k, lds, m, S >> 2, last ? m : (slice + 1) * S, ct_lo, T_lo,
+                                                       kHandOver ? 0 : slice * S, ct_hi, T_hi);
             if (!ok) OMK_NOTE(20);
-            if (ok && slice > 0) {
+            if (!kHandOver) {
+                if (slice == 0) T_hi = 0xFFFFFFFFu;
+                if (ok && slice > 0) {
+                    int sum = 0;
+#pragma unroll
+                    for (int r = 0; r < R; r++) sum += ct_hi[r];
+                    rank_hi = wave_sum_i32(sum);
+                }
+            }
+            if (kHandOver && !last) {
+                int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)(slice + 1)) * kBoundInts;
                 int sum = 0;
 #pragma unroll
-                for (int r = 0; r < R; r++) sum += ct_hi[r];
-                rank_hi = wave_sum_i32(sum);
+                for (int r = 0; r < R; r++) {
+                    bnd[16 + r * kWave + lane] = ct_lo[r];
+                    sum += ct_lo[r];
+                }
+                sum = wave_sum_i32(sum);
+                if (lane == 0) {
+                    bnd[1] = (int)T_lo;
+                    bnd[2] = sum;
+                    bnd[3] = ok ? 1 : 0;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                if (lane == 0) __hip_atomic_store(bnd + 0, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            if (ok && !last) {
+            if (kHandOver && ok && slice > 0) {
+                const int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)slice) * kBoundInts;
+                bool there = false;
+                for (int spins = 0;; spins++) {
+                    int v = 0, ab = 0;
+                    if (lane == 0) {
+                        v = __hip_atomic_load(bnd + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (v != a.epoch && (spins & 3) == 3)
+                            ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    v = __builtin_amdgcn_readfirstlane(v);
+                    ab = __builtin_amdgcn_readfirstlane(ab);
+                    if (v == a.epoch) {
+                        there = true;
+                        break;
+                    }
+                    if (ab) break;
+                    if (spins >= a.spin_limit) {
+                        if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 3);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(4);
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                if (there) {
+                    T_hi = (uint32_t)__hip_atomic_load(bnd + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    rank_hi = __hip_atomic_load(bnd + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (__hip_atomic_load(bnd + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) ok = false;
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+                        ct_hi[r] = __hip_atomic_load(bnd + 16 + r * kWave + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    ok = false;  // the selection is being given up
+                }
+            }
+            bool preset_ok = !last;
+            if (ok) {
                 int sum = 0;
                 bool bad = false;
 #pragma unroll
@@ -2975,14 +3104,29 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     if (ct_lo[r] < ct_hi[r]) bad = true;
                 }
                 rank_lo = wave_sum_i32(sum);
-                if (T_lo > T_hi || __ballot(bad) != 0ull) {
+                const bool broken = T_lo > T_hi || __ballot(bad) != 0ull;
+                if (last) {
+                    // counts that do not reach the last visitor, or thresholds out of order: the batch loop
+                    // finds the end of the node by itself
+                    preset_ok = !broken && rank_lo >= m;
+                    if (!preset_ok) rank_lo = m;
+                } else if (broken) {
                     ok = false;
                     OMK_NOTE(22);
                 }
             }
+            if (a.trace) ts1 = wall_clock64();
+            if (a.trace && lane == 0) {
+                g_slice_note[2] = -1;
+                g_slice_note[3] = 0;
+            }
             if (ok && rank_hi < m) {
                 const bool closing = last || rank_lo >= m;
                 const int todo = (closing ? m : rank_lo) - rank_hi;
+                if (a.trace && lane == 0) {
+                    g_slice_note[2] = preset_ok ? rank_lo - rank_hi : -1;
+                    g_slice_note[3] = todo;
+                }
                 if (todo > 0) {
                     {
                         int unused_cur;
@@ -2990,7 +3134,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
 #pragma unroll
                         for (int r = 0; r < R; r++) between[r] = ct_lo[r] - ct_hi[r];
                         ok = water_level<R, RAVE>(a, c, lane, k, soff, rank_hi, todo, ct_hi, lds, cnt, false, unused_cur,
-                                                  !last, between, pl.order, pending);
+                                                  preset_ok, between, pl.order, pending);
                     }
                 } else {
 #pragma unroll
@@ -3009,6 +3153,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         OMK_NOTE(23);
                     }
                 }
+            }
+            if (a.trace && lane == 0) {
+                g_slice_note[0] = (int)(ts1 - ts0);
+                g_slice_note[1] = (int)(wall_clock64() - ts1);
             }
             if (!ok && lane == 0) atomicExch(ctx + 1, 1);
             // join: the wavefront that finishes last goes on with the node
@@ -3594,8 +3742,13 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                     for (int q = 0; q < 8; q++)
                         a.trace[12 * ti + 4 + q] = (long long)s_lds.tph[2 * q] | ((long long)s_lds.tph[2 * q + 1] << 32);
 #else
-                    a.trace[12 * ti + 3] = (long long)it.node;
+                    // a slice or a part of a heavy node: its number and their number in the upper half
+                    a.trace[12 * ti + 3] = (long long)it.node | ((long long)(uint32_t)it.pad[2] << 32);
                     for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
+                    if (it.pad[0] == 1 || it.m >= kHeavyMin) {
+                        a.trace[12 * ti + 4] = (long long)(uint32_t)g_slice_note[0] | ((long long)(uint32_t)g_slice_note[1] << 32);
+                        a.trace[12 * ti + 5] = (long long)(uint32_t)g_slice_note[2] | ((long long)(uint32_t)g_slice_note[3] << 32);
+                    }
 #endif
                 }
             }
