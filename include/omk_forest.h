@@ -289,7 +289,7 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * that takes nearly every visitor, [8] when the first block of the persistent launch started,
  * [9] when its last team of wavefronts left, [10] when its last walker left (low 31 bits of the
  * device's 100 MHz clock; these three are kept whether or not the counters are on), [11] the number
- * of walks of lone visitors inside that launch, [12..14] per-phase cycle counts in measurement builds (else 0), [15] nodes cut into
+ * of walks of lone visitors inside that launch, [12..14] unused (0), [15] nodes cut into
  * slices for several wavefronts.  (Nodes taken by the walk down one-winner nodes count in [0]..[2].) */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
 /* The counters above cost one atomic per processed node (and per single-visitor step), all on
@@ -301,15 +301,11 @@ int omk_batch_set_stats(omk_batch *b, int32_t enabled);
  * and end on the GPU's 100 MHz clock, visitors | depth << 32 | kind << 60 (0 a node settled as a
  * whole, 1 a slice of a heavy node, 2 a part of its partition, 3 a node published before its visitor
  * list was complete, 5 a node whose visitors all follow one child, taken by the walk down such nodes,
- * 6 the walk of a lone visitor inside the persistent launch), node | (batches | runs << 8 | entries of
- * the last batch << 16) << 32, then eight words holding two 32-bit phase times each.  The phase
- * times and the counters beside the node are filled by a library built with -DOMK_TRACE only
- * (csrc/Makefile, target `trace`; 0 otherwise): slots 0-7 threshold phase, direct merge: counts and
- * ranks (or 100 x the reason it was refused), evaluation and ordering, emission and checks, loading
- * and scoring the children, the whole settling of the visitors, the partition, direct merge: the
- * dominant child's list; slots 8-15, parts of these: run probe, bounds and active children,
- * threshold search, exact counts, one-winner check, length search of a run, emission of a run, the
- * direct merge as a whole.
+ * 6 the walk of a lone visitor inside the persistent launch), node | number << 32 (number: for a slice
+ * or a part of a heavy node, which one of how many: index | count << 16), then, for a slice of a heavy node,
+ * word 4 = time of its boundaries | time of its batches << 32 (100 MHz clock) and word 5 = entries its
+ * boundaries put in its batch (-1: it searched for the batch itself) | visitors it settled << 32; the other
+ * words are 0.
  * h_trace has room for max_entries records; the records live in the staging memory of
  * omk_batch_read until the next call of it. */
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n);
@@ -373,9 +369,11 @@ int omk_tt_probe_leaves(omk_tt *tt, omk_batch *b, int32_t min_depth, int32_t *d_
  * count and value as they are now); a key that is there keeps its entry unless the new one's
  * replacement score exceeds the old one's by the threshold (:64-74, score = recency * importance,
  * include/mcts/phmap_transposition_table.h:68-72, threshold Config::replacement_threshold = 0.1).
- * Time: the reference stamps entries with a counter shared by its threads, so its values depend on
- * the schedule; here entry i of a call has the time t + i and the table's clock t advances by n per
- * call (lookups likewise).  Among the entries of one call with the same key only the first is
+ * Time (not the reference's: replacement decisions that hinge on recency are not pinned against it):
+ * the reference advances its access counter on a store that finds the key and on a lookup that hits
+ * (:64, :107), from threads that share it, so its stamps depend on the schedule; here entry i of a call
+ * has the time t + i and the table's clock t advances by n per call, misses included (lookups
+ * likewise).  Among the entries of one call with the same key only the first is
  * stored: the serial outcome at the reference's two call sites (a node stored from the traversal
  * has no visits, score 0, and never replaces; the leaves expanded in one step are distinct).
  * An entry with node < 0 is skipped.  h_counts (NULL or [4]): new entries, replacements, entries

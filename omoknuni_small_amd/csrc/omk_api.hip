@@ -1087,9 +1087,6 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.trace = b->trace_on ? (long long *)b->out_paths : nullptr;  // staging that only omk_batch_read uses
     a.trace_n = b->counters + 24;
     a.trace_cap = (int32_t)(b->out_ints / 24);
-#if defined(OMK_PHASE_TIMERS) || defined(OMK_TRACE)
-    a.dbg_grid = getenv("OMK_DBG_GRID") ? atoi(getenv("OMK_DBG_GRID")) : 0;
-#endif
     a.singles0 = b->singles0;
     a.singles_q = b->singles_q;
     a.sc_child = b->sc_child;
@@ -1434,8 +1431,8 @@ int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     return OMK_OK;
 }
 
-// The per-node timeline of the last selection (12 x int64 per processed multi-visitor item), which
-// only a build with -DOMK_TRACE records.
+// The per-node timeline of the last selection (12 x int64 per processed multi-visitor item), recorded when
+// omk_batch_set_trace switched it on before that selection.
 int omk_debug_trace(omk_batch *b, long long *h_trace, int32_t max_entries, int32_t *h_n) {
     if (!b || !h_trace || !h_n || max_entries < 0) return fail(OMK_ERR_INVALID, "omk_debug_trace: bad argument");
     *h_n = 0;

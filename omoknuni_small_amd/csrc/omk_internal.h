@@ -72,10 +72,9 @@ struct SelectArgs {
     int32_t q_cap;
     int32_t epoch;         // number of this select call on the batch, > 0
     long long *trace;      // nullptr, or per processed node: start, end (100 MHz clock), visitors | depth << 32 |
-                           // kind << 60, node, and eight words of phase times (measurement builds only, else 0)
+                           // kind << 60, node | number << 32, and eight words (what a slice of a heavy node did)
     int32_t *trace_n;
     int32_t trace_cap;
-    int32_t dbg_grid;      // cap on the blocks of the multi-visitor kernel (0 = none; measurement builds)
     int32_t *times;        // [0] when the first block of the persistent launch started, [1] when the last team
                            // left, [2] when the last walker left (100 MHz clock, low 31 bits)
     int32_t spin_limit;    // polls of a waiting wavefront before it raises the abort flag

@@ -82,71 +82,6 @@ constexpr int kRunShareMin = 4096;        // a node whose visitors all take one 
 
 enum { kStepLeaf = 0, kStepDescended = 1, kStepParked = 2 };
 
-// Build with -DOMK_PHASE_TIMERS to accumulate shader-clock cycles per phase of the
-// multi-visitor path into statistics slots 8..15 (measurement aid, off by default).
-#if defined(OMK_PHASE_TIMERS) && !defined(OMK_TRACE)
-#define OMK_TRACE
-#endif
-#ifdef OMK_PHASE_TIMERS
-#define OMK_FAIL(code)                                                      \
-    do {                                                                    \
-        if (a.stats && lane == 0) atomicExch(a.stats + 7, (code));          \
-        return false;                                                       \
-    } while (0)
-#define OMK_NOTE(code)                                             \
-    do {                                                           \
-        if (a.stats && lane == 0) atomicExch(a.stats + 7, (code)); \
-    } while (0)
-#define OMK_T0() long long t_phase_ = clock64()
-#define OMK_TICK(slot)                                                              \
-    do {                                                                            \
-        long long now_ = clock64();                                                 \
-        if (a.stats && lane == 0) atomicAdd(a.stats + (slot), (int)((now_ - t_phase_) >> 4)); \
-        t_phase_ = now_;                                                            \
-    } while (0)
-#elif defined(OMK_TRACE)
-// timeline build: the owner wavefront adds up, per node, the time it spends in every phase
-// (100 MHz clock) in the block's LDS scratch; the node's trace record carries the sums
-#define OMK_FAIL(code) return false
-#define OMK_NOTE(code) \
-    do {               \
-    } while (0)
-#define OMK_T0() long long t_phase_ = wall_clock64()
-#define OMK_TICK(slot)                                                       \
-    do {                                                                     \
-        long long now_ = wall_clock64();                                     \
-        if (lane == 0) lds.tph[(slot)-8] += (uint32_t)(now_ - t_phase_);     \
-        t_phase_ = now_;                                                     \
-    } while (0)
-// finer stamps inside a phase, on a timer of their own
-#define OMK_S0() long long t_sub_ = wall_clock64()
-#define OMK_STAMP(slot)                                                  \
-    do {                                                                 \
-        long long now_ = wall_clock64();                                 \
-        if (lane == 0) lds.tph[(slot)] += (uint32_t)(now_ - t_sub_);     \
-        t_sub_ = now_;                                                   \
-    } while (0)
-#else
-#define OMK_FAIL(code) return false
-#define OMK_NOTE(code) \
-    do {               \
-    } while (0)
-#define OMK_T0() \
-    do {         \
-    } while (0)
-#define OMK_TICK(slot) \
-    do {               \
-    } while (0)
-#endif
-#ifndef OMK_S0
-#define OMK_S0() \
-    do {         \
-    } while (0)
-#define OMK_STAMP(slot) \
-    do {                \
-    } while (0)
-#endif
-
 // Register-resident statistics of the children a lane is responsible for: child index
 // i = r * 64 + lane for round r.
 template <int R, bool RAVE>
@@ -206,9 +141,6 @@ template <int R>
 struct WaveLds {
     TeamCmd cmd;
     uint32_t red[4];       // team reductions: smallest / largest inverted key, flags
-#ifdef OMK_TRACE
-    uint32_t tph[16];      // timeline build: time of the node at hand per phase
-#endif
     int wsum[kTeamWaves];  // team prefix scan: totals of the wavefronts
     int offs[R * kWave];   // exclusive prefix of the visit counts in child order
     int st_n[R * kWave];   // statistics of every child, readable by any lane
@@ -1201,7 +1133,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         lds.st_q2[i] = k.q2[r];
     }
 
-    OMK_T0();
     // Set when the threshold search finds the unsettled entries piled up on ONE key in several
     // children and nothing above it (children exactly tied on a plateau): among equal keys the
     // lowest position wins for as long as its key stays there, so the next winners are a run of
@@ -1211,12 +1142,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const int remaining = m - done;
         const int run_min = force_run ? 1 : kRunShortcutMin;
         force_run = false;
-#ifdef OMK_TRACE
-        if (lane == 0) lds.red[3] += 1u;  // batches and runs of this node, for the timeline
-#endif
 
         // ---- 1. threshold and exact per-child counts ----
-        OMK_S0();
         uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -1226,7 +1153,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             }
         uint32_t hi_key, hi_pos;
         wave_best(lbk, lbp, hi_key, hi_pos);
-        if (hi_key == 0u) OMK_FAIL(2);
+        if (hi_key == 0u) return false;
         const int best = (int)(hi_pos >= (uint32_t)F ? hi_pos - (uint32_t)F : hi_pos);
 
         // A slice of a heavy node knows exactly how many entries every child contributes to its
@@ -1310,7 +1237,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     hi_l = new_hi < hi_l ? new_hi : hi_l;
                 }
                 const int L = lo_l;
-                OMK_STAMP(13);
                 // the entry after the run must not come before the run's last one
                 uint32_t nk, np2, lk_, lp_;
                 entry_key<R, RAVE>(bn, bw, bp, bvl, bq2, c.ep, uvl, btk + L, best, nk, np2);
@@ -1355,10 +1281,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     }
                     bad_run = (lds.red[2] & 4u) != 0u;
                 }
-                OMK_STAMP(14);
-#ifdef OMK_TRACE
-                if (!bad_run && lane == 0) lds.red[3] += 0x100u;  // runs emitted without sorting
-#endif
                 if (!bad_run) {
                     if (lane == bl) {
 #pragma unroll
@@ -1374,8 +1296,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 }
             }
         }
-        if (run_min == 1) OMK_FAIL(11);  // the run that had to be there was refused
-        OMK_STAMP(8);
+        if (run_min == 1) return false;  // the run that had to be there was refused
         const int want = remaining < kBatchCap ? remaining : kBatchCap;
         // lower bound of any useful threshold: a child alone has `want` entries at or above the
         // key of its want-th next visit; the best such key over all children (the child that
@@ -1395,7 +1316,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             lo_key = wave_max_u32(lmax);
         }
         if (lo_key == 0u) lo_key = 1u;
-        if (lo_key > hi_key) OMK_FAIL(3);  // scores rose along the best child's list
+        if (lo_key > hi_key) return false;  // scores rose along the best child's list
 
         // Only children whose next entry reaches the lower bound can contribute.  They are
         // listed densely (one per lane and round), so that the work below costs one round per
@@ -1441,7 +1362,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         const int margin = n_act + 8;
         const bool can_finish = remaining + 2 * margin <= kBatchCap;
         int target = can_finish ? remaining + margin : kBatchCap - margin;
-        if (target < 1) OMK_FAIL(4);
+        if (target < 1) return false;
         // No child can win more than the visits that are left: its entries beyond that are
         // never looked at (the batch is cut at `remaining` entries anyway, and such a child's
         // last counted entry lies at or after that cut).
@@ -1449,11 +1370,10 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         int ct[R];
         total = 0;
         int tries = 0;
-        OMK_STAMP(9);
         uint32_t T_forced = 0u;  // threshold imposed for the next round instead of searching one
         bool allow_above = true;
         for (;;) {
-            if (++tries > 8) OMK_FAIL(5);
+            if (++tries > 8) return false;
             const uint32_t T_now = T_forced;  // imposed for this round only
             T_forced = 0u;
             // a threshold with about `target` ESTIMATED entries at or above it (no exact evaluation
@@ -1476,7 +1396,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                     return wave_sum_i32(est);
                 });
             }
-            OMK_STAMP(10);
             uint32_t T = T_now != 0u ? T_now : klo;
             if (T < lo_key) T = lo_key;
             if (T > hi_key) T = hi_key;
@@ -1525,7 +1444,6 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 }
             }
             total = wave_sum_i32(sum);  // at most 64 * R * (capacity + 1)
-            OMK_STAMP(11);
             if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
             // A batch that does not fit is cut at the child with most entries (typically one
             // whose score hardly moves with virtual loss): it contributes fewer entries now,
@@ -1577,10 +1495,10 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             }
             if (can_finish && total < remaining) {
                 target += (remaining - total) + margin;  // not enough to finish: aim lower
-                if (target > kBatchCap) OMK_FAIL(6);
+                if (target > kBatchCap) return false;
                 continue;
             }
-            if (total < 1) OMK_FAIL(7);
+            if (total < 1) return false;
             break;
         }
         if (force_run) continue;
@@ -1590,15 +1508,11 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
             if (ac[r] >= 0) lds.pay[ac[r]] = (uint32_t)ct[r];
         wave_sync_memory();
         }  // !preset_done
-#ifdef OMK_TRACE
-        if (lane == 0) lds.red[3] = (lds.red[3] & 0xFFFFu) | ((uint32_t)total << 16);  // entries of the last batch
-#endif
         int nb[R];  // entries of every own child in this batch
 #pragma unroll
         for (int r = 0; r < R; r++) nb[r] = (int)lds.pay[r * kWave + lane];
         if (capped_child >= 0) capped_last = lds.st_j0[capped_child] + (int)lds.pay[capped_child] - 1;
         wave_sync_memory();
-        OMK_TICK(8);
 
         // ---- 2. evaluate the batch in (child, visit) order ----
         int carry = 0;
@@ -1628,9 +1542,8 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
         } else {
             cur = batch_order<R, RAVE, kWave>(lds, lane, total, c.ep, uvl);
         }
-        if ((lds.red[2] & 4u) != 0u) OMK_FAIL(8);
+        if ((lds.red[2] & 4u) != 0u) return false;
         const uint32_t *skey = lds.key[cur], *spay = lds.pay2[cur];
-        OMK_TICK(10);
 
         // ---- 4. winner order: keep what is needed, check ties across children, emit ----
         int keep = total < remaining ? total : remaining;
@@ -1642,7 +1555,7 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 if ((spay[q] & 0x7FFFFFFFu) == want_pay) qcut = umin32(qcut, (uint32_t)q);
             }
             qcut = wave_min_u32(qcut);
-            if (qcut == 0xFFFFFFFFu) OMK_FAIL(10);
+            if (qcut == 0xFFFFFFFFu) return false;
             if ((int)qcut + 1 < keep) keep = (int)qcut + 1;
         }
         // a node that this one batch settles keeps its winner order in LDS for the partition
@@ -1701,10 +1614,9 @@ __device__ __forceinline__ bool water_level(const SelectArgs &a, const NodeCtx &
                 tk[r] = settled;
             }
         }
-        if (__ballot(bad) != 0ull) OMK_FAIL(9);
+        if (__ballot(bad) != 0ull) return false;
         done += keep;
         wave_sync_memory();
-        OMK_TICK(11);
     }
 #pragma unroll
     for (int r = 0; r < R; r++) cnt[r] = tk[r];
@@ -1810,7 +1722,6 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
                                                  uint32_t &T2) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
-    OMK_S0();
     uint32_t headk[R];
     uint32_t lbk = 0u, lbp = 0xFFFFFFFFu;
 #pragma unroll
@@ -1888,7 +1799,6 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
         }
     }
     int cta[R];
-    OMK_STAMP(9);
     auto boundary = [&](int target, int (&ct)[R], uint32_t &T) {
     // The boundary of one target: the threshold and the exact counts at it.  When far more entries than the
     // target lie at or above the threshold, they are piled up ON the threshold key (a child whose key does not
@@ -1902,9 +1812,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     // everything at or above the higher one.  Whoever uses the counts checks the order they imply like any
     // other (water_level: the last entry kept must come before every child's next one).
         T = active_threshold<R, RAVE>(s, c.ep, uvl, lo_key, hi_key, target, window, m, lane);
-        OMK_STAMP(10);
         active_counts<R, RAVE>(s, c.ep, uvl, T, m, cta, lane);
-        OMK_STAMP(11);
         int sum = 0;
 #pragma unroll
         for (int r = 0; r < R; r++) sum += cta[r];
@@ -2133,16 +2041,6 @@ constexpr int kSparseMax = 64;  // entries of other children a nearly-one-winner
 constexpr int kSparseMin = 8;    // visitors from which that direct merge is tried
 static_assert(2 * kHeavyMin <= kBatchCap, "the (key, position) list of the dominant child fits one sort buffer");
 
-#ifdef OMK_TRACE
-// timeline build: why a direct merge was refused (shown in place of a time, in units of 1 us)
-#define OMK_MERGE_FAIL(code)                           \
-    do {                                               \
-        if (lane == 0) lds.tph[1] = 100u * (code);     \
-        return false;                                  \
-    } while (0)
-#else
-#define OMK_MERGE_FAIL(code) return false
-#endif
 
 // A node where one child wins ALMOST every time: the winner order is that child's list with
 // a few entries of other children merged in.  The child, A, is the one that holds out longest,
@@ -2167,7 +2065,6 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
                                              uint32_t *order, int (&cnt)[R], bool &pending) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
-    OMK_S0();
     // ---- the children that matter, one per lane ----
     int n0 = 0;
     bool listed[R];
@@ -2194,7 +2091,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
         }
         n0 += __popcll(cm);
     }
-    if (n0 < 2 || n0 > kSparseMax) OMK_MERGE_FAIL(1);
+    if (n0 < 2 || n0 > kSparseMax) return false;
     wave_sync_memory();
     int ci = -1, cn = 0, cvl = 0;
     float cw = 0.0f, cp = 0.0f, cq2 = 0.0f;
@@ -2212,9 +2109,9 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     // ---- A: the child that holds out longest ----
     uint32_t lk, lp;
     wave_best(zk, zp, lk, lp);
-    if (lk == 0u) OMK_MERGE_FAIL(7);
+    if (lk == 0u) return false;
     const uint64_t am = __ballot(lane < n0 && zk == lk && zp == lp);
-    if (am == 0ull) OMK_MERGE_FAIL(8);
+    if (am == 0ull) return false;
     const int a_lane = __ffsll((long long)am) - 1;
     const int a_child = __builtin_amdgcn_readlane(ci, a_lane);
     const int a_n = __builtin_amdgcn_readlane(cn, a_lane);
@@ -2224,7 +2121,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     const float a_q2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cq2), a_lane));
     // ---- the others that can get an entry in: next entry before (lk, lp) ----
     const bool is_cand = lane < n0 && lane != a_lane && hk != 0u && comes_before(hk, hp, lk, lp);
-    if (__ballot(is_cand) == 0ull) OMK_MERGE_FAIL(9);
+    if (__ballot(is_cand) == 0ull) return false;
     {
         // Far too many entries by the estimates: leave before anything exact is paid for.  An entry
         // of a child gets in only if fewer than m entries come before it; the child's next entry has
@@ -2241,7 +2138,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
         }
         // (a little below the capacity: the exact counts tend to come out above the estimates, and
         // a refusal after them costs three times what one here does)
-        if (wave_sum_i32(est) > kSparseMax - 4) OMK_MERGE_FAIL(2);
+        if (wave_sum_i32(est) > kSparseMax - 4) return false;
     }
     // ---- A's entries, all m of them, evaluated once into LDS and checked: none may come before its
     // predecessor (its head then stays at or before (lk, lp) throughout) ----
@@ -2267,10 +2164,9 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
             carry_k = (uint32_t)__builtin_amdgcn_readlane((int)kk, 63);
             carry_p = (uint32_t)__builtin_amdgcn_readlane((int)pp, 63);
         }
-        if (__ballot(bad_a) != 0ull) OMK_MERGE_FAIL(5);
+        if (__ballot(bad_a) != 0ull) return false;
     }
     wave_sync_memory();
-    OMK_STAMP(7);
     // how many of A's entries come before the entry (tk, tp): the list is in order, so a bisection
     // on the exact keys
     auto rank_in_a = [&](uint32_t tk, uint32_t tp) {
@@ -2293,12 +2189,12 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     }
     const int inc = wave_inclusive_sum(cc, lane);
     const int total = __builtin_amdgcn_readlane(inc, 63);
-    if (total > kSparseMax) OMK_MERGE_FAIL(3);
+    if (total > kSparseMax) return false;
     const int start = inc - cc;
     // ---- one lane per entry: (lane of its child, visit number) ----
     for (int t = 0; t < cc; t++) lds.hist[start + t] = lane | (t << 8);  // start + cc <= total <= 64
     wave_sync_memory();
-    int bad = 0;  // why the merge is refused (the number only matters to the timeline build)
+    int bad = 0;  // nonzero: the merge is refused
     uint32_t ek = 0u, epos = 0xFFFFFFFFu;
     int e_child = -1, e_t = 0, rank_a = m;
     if (lane < total) {
@@ -2352,9 +2248,8 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
     }
     {
         const int why = (int)wave_max_u32((uint32_t)bad);
-        if (why != 0) OMK_MERGE_FAIL(40 + why);
+        if (why != 0) return false;
     }
-    OMK_STAMP(1);
     // ---- the winner order: the others' entries at their places, A's in between ----
     close_pending(pending);  // the previous node's partition may still read the order buffer
     for (int q = lane; q < m; q += kWave) order[q] = 0u;
@@ -2371,7 +2266,7 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
         if (q < m) order[q] = other ? (v & 0x7FFFFFFFu) : (((uint32_t)a_child << 21) | (uint32_t)(q - below));
         seen += __popcll(om);
     }
-    if (seen != nfv) OMK_MERGE_FAIL(6);  // two entries at one place: cannot happen when the checks hold
+    if (seen != nfv) return false;  // two entries at one place: cannot happen when the checks hold
     // ---- visits per child, back to the lanes that hold the children ----
     if (lane < n0) lds.hist[kSparseMax + lane] = lane == a_lane ? m - nfv : mine_in;
     wave_sync_memory();
@@ -2818,7 +2713,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     // preload: 0 the children are loaded here; 1 two helpers are loading their share (load_ahead); 2 a walk down
     // one-winner nodes stopped at this node and left its children, scored, in the LDS scratch, with the verdict
     bool ahead = preload == 1;
-    OMK_T0();
     const int off = item.off, m = item.m, depth = item.depth;
     // a heavy node is settled and shared out by several wavefronts, which read its visitor
     // list: it must be complete before any of them is called in
@@ -2920,7 +2814,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         lane_best<R, RAVE>(k, lane, bk, bpos);
     }
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
-    OMK_TICK(12);
 
     bool settled = false;
     int st_replay = 0;
@@ -2938,7 +2831,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         for (int r = 0; r < R; r++) cnt[r] = ctx[16 + r * kWave + lane];
         settled = true;
     }
-    OMK_S0();
     bool contested = false;
     int best0 = -1;
     uint32_t lk0 = 0u, lp0 = 0xFFFFFFFFu;
@@ -2951,19 +2843,15 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     } else if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
         settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child, contested, best0,
                                       lk0, lp0);
-    OMK_STAMP(12);
     if (!settled && contested && m >= kSparseMin && m < kHeavyMin) {
         settled = sparse_merge<R, RAVE>(a, c, lane, k, best0, lk0, lp0, m, lds, pl.order, cnt, pending);
         if (settled) {
             lds_cur = 0;
-#ifndef OMK_PHASE_TIMERS
             if (a.stats && lane == 0) atomicAdd(a.stats + 7, 1);
-#endif
         } else {
 #pragma unroll
             for (int r = 0; r < R; r++) cnt[r] = 0;
         }
-        OMK_STAMP(15);
     }
     if (R * kWave <= kHeavyFanout) {
         if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
@@ -2998,9 +2886,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     hid = id;
                     slice = 0;
                     n_slices = K;
-#ifndef OMK_PHASE_TIMERS
                     if (a.stats && lane == 0) atomicAdd(a.stats + 15, 1);
-#endif
                 } else if (lane == 0) {
                     atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
                 }
@@ -3032,7 +2918,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             constexpr bool kHandOver = R > 1;
             ok = threshold_counts<R, RAVE, !kHandOver>(a, c, lane, k, lds, m, S >> 2, last ? m : (slice + 1) * S, ct_lo, T_lo,
                                                        kHandOver ? 0 : slice * S, ct_hi, T_hi);
-            if (!ok) OMK_NOTE(20);
             if (!kHandOver) {
                 if (slice == 0) T_hi = 0xFFFFFFFFu;
                 if (ok && slice > 0) {
@@ -3112,7 +2997,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     if (!preset_ok) rank_lo = m;
                 } else if (broken) {
                     ok = false;
-                    OMK_NOTE(22);
                 }
             }
             if (a.trace) ts1 = wall_clock64();
@@ -3150,7 +3034,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         if (cnt[r] != ct_lo[r]) bad = true;
                     if (__ballot(bad) != 0ull) {
                         ok = false;
-                        OMK_NOTE(23);
                     }
                 }
             }
@@ -3232,7 +3115,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         if (run_child < 0 && seq_lds) lds_cur = 0;
         wave_sync_memory();
     }
-    OMK_TICK(13);
     if (a.stats && lane == 0 && !as_scatter) {
         atomicAdd(a.stats + 0, 1);
         atomicAdd(a.stats + 1, settled ? 1 : 0);
@@ -3281,7 +3163,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         next.span = child_span;
         next.ahead = false;
         next.chain_open = true;
-        OMK_TICK(14);
         return kStepDescended;
     }
     // (1) from the visits per child: the segment of every child, in LDS for all lanes
@@ -3349,7 +3230,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             next.span = keep_span;
             next.ahead = ahead_next;
         }
-        OMK_TICK(14);
         return kStepDescended;
     }
 
@@ -3565,7 +3445,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         if (n_lone > 0 && lane == 0) atomicSub(a.sched_wait, n_lone);
         next.node = -1;
         wave_sync_memory();
-        OMK_TICK(14);
         return kStepDescended;
     }
 
@@ -3622,7 +3501,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     }
     // the next step of the walk reads seg_out and reuses the LDS scratch
     wave_sync_memory();
-    OMK_TICK(14);
     return kStepDescended;
 }
 
@@ -3688,10 +3566,6 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             const int32_t *seg_in = depth == 0 ? a.seg0 : a.seg[(depth - 1) & 1];
             int32_t *seg_out = a.seg[depth & 1];
             const long long tr0 = a.trace ? wall_clock64() : 0ll;  // the timeline, when it is switched on
-#ifdef OMK_TRACE
-            if (lane == 0) s_lds.red[3] = 0u;
-            if (lane < 16) s_lds.tph[lane] = 0u;
-#endif
             NodeCtx c = node_ctx(f, a, it.node, it.np, have_span, pre_span);
             if (chain_open) {
                 // The node settled before sent all its visitors here, and the helpers walk down from this node for
@@ -3737,11 +3611,6 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                     a.trace[12 * ti + 0] = tr0;
                     a.trace[12 * ti + 1] = wall_clock64();
                     a.trace[12 * ti + 2] = (long long)it.m | ((long long)depth << 32) | ((long long)it.pad[0] << 60);
-#ifdef OMK_TRACE
-                    a.trace[12 * ti + 3] = (long long)it.node | ((long long)s_lds.red[3] << 32);
-                    for (int q = 0; q < 8; q++)
-                        a.trace[12 * ti + 4 + q] = (long long)s_lds.tph[2 * q] | ((long long)s_lds.tph[2 * q + 1] << 32);
-#else
                     // a slice or a part of a heavy node: its number and their number in the upper half
                     a.trace[12 * ti + 3] = (long long)it.node | ((long long)(uint32_t)it.pad[2] << 32);
                     for (int q = 0; q < 8; q++) a.trace[12 * ti + 4 + q] = 0;
@@ -3749,7 +3618,6 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
                         a.trace[12 * ti + 4] = (long long)(uint32_t)g_slice_note[0] | ((long long)(uint32_t)g_slice_note[1] << 32);
                         a.trace[12 * ti + 5] = (long long)(uint32_t)g_slice_note[2] | ((long long)(uint32_t)g_slice_note[3] << 32);
                     }
-#endif
                 }
             }
             if (status == kStepParked) break;  // a slice of a heavy node: another wavefront goes on with it
@@ -4178,9 +4046,6 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
         // unit (waiting for work, polling) takes issue slots, cache and LDS bandwidth from it.  Measured
         // on the 4 M-node chess-like tree: 0.247 ms a selection with two blocks per unit, 0.222 with one.
         int capacity = n_cus;
-#ifdef OMK_TRACE
-        if (a0.dbg_grid > 0 && capacity > a0.dbg_grid) capacity = a0.dbg_grid;
-#endif
         if (capacity < 2) capacity = 2;
         int walkers = n_traversals / 64;
         if (walkers > capacity / 4) walkers = capacity / 4;

@@ -74,8 +74,7 @@ class _BatchDev(C.Structure):
 
 
 def library_path():
-    """libomk_forest.so beside this file, or another build of the same ABI named by OMK_FOREST_LIB
-    (the measurement build libomk_forest_trace.so)."""
+    """libomk_forest.so beside this file, or another build of the same ABI named by OMK_FOREST_LIB."""
     return os.environ.get("OMK_FOREST_LIB") or os.path.join(_HERE, "libomk_forest.so")
 
 
@@ -445,7 +444,7 @@ class Batch:
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
                 "replayed_nodes", "threshold_probes", "single_visitor_steps", "merged_nodes", "t_first_block",
-                "t_last_team", "t_last_walker", "walks_in_launch", "cyc_load", "cyc_settle", "cyc_partition",
+                "t_last_team", "t_last_walker", "walks_in_launch", "unused_12", "unused_13", "unused_14",
                 "sliced_nodes")
         return dict(zip(keys, map(int, out)))
 
@@ -455,8 +454,8 @@ class Batch:
 
     def debug_trace(self, max_entries=1 << 16):
         """Timeline of the last select() after enable_trace(): int64 array [n, 12] of
-        (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | counters << 32 and
-        eight words of two 32-bit phase times each (see omk_debug_trace in the header)."""
+        (start, end) on the 100 MHz clock, visitors | depth << 32 | kind << 60, node | number << 32 and
+        eight words, of which a slice of a heavy node fills two (see omk_debug_trace in the header)."""
         buf = np.zeros((int(max_entries), 12), np.int64)
         n = C.c_int32()
         _check(self._lib.omk_debug_trace(self._h, buf.ctypes.data_as(C.c_void_p), C.c_int32(int(max_entries)),
