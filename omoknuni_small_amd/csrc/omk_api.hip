@@ -906,8 +906,11 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     if (e == hipSuccess) e = dalloc(&b->items0, B);
     // a multi-visitor item has at least two visitors, and a level holds each visitor once; a heavy
     // node (kHeavyMin visitors or more) adds at most 63 slice items
-    b->q_cap = (int32_t)((B / 2 + B / 16 + 64) * (max_depth + 1));
-    b->hctx_cap = (int32_t)std::min<int64_t>(4096, (B / kHeavyMin) * (max_depth + 1));
+    // (and as many parts of its partition, and as many boundaries worked out ahead of time)
+    b->q_cap = (int32_t)((B / 2 + B / 4 + 64) * (max_depth + 1));
+    // (a node whose boundaries are worked out ahead of time, and that is then not cut into slices after all, uses
+    // a second context for its partition)
+    b->hctx_cap = (int32_t)std::min<int64_t>(4096, 2 * (B / kHeavyMin) * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->hctx, (int64_t)b->hctx_cap * kHeavyCtxInts);
     if (e == hipSuccess) e = dalloc(&b->hbound, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts);
     if (e == hipSuccess)
@@ -994,6 +997,9 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     HIP_TRY(hipMemcpy(b->seg0, order.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    // every path starts at its root: written here once, not by every selection (the wavefront that takes a
+    // crowded root would spend its first microseconds on thousands of path entries)
+    HIP_TRY(hipMemcpy(b->paths, h_roots, (size_t)n * 4, hipMemcpyHostToDevice));
     if (!items.empty())
         HIP_TRY(hipMemcpy(b->items0, items.data(), items.size() * sizeof(Item), hipMemcpyHostToDevice));
     if (!singles.empty())
@@ -1051,7 +1057,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.items_q = b->items_q;
     a.seg[0] = b->seg[0];
     a.seg[1] = b->seg[1];
-    if (b->epoch == INT32_MAX) {  // ready marks are call numbers: start over before they repeat
+    if (b->epoch >= (1 << 30) - 2) {  // ready marks are call numbers (the boundary table's: twice that): start over before they repeat
         HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
         HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
         HIP_TRY(launch_fill_words(b->hbound, 0u, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts, f->stream));

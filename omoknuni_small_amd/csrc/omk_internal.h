@@ -34,17 +34,19 @@ struct Item {
     int32_t m;      // visitors
     int32_t np;     // N(node) as read by the parent's wavefront
     int32_t depth;  // depth of the node on the visitors' paths
-    int32_t pad[3]; // [0] 0 = node, 1 = slice of a heavy node; [1] context; [2] slice | slices << 16
+    int32_t pad[3]; // [0] 0 = node, 1 = slice of a heavy node, 2 = part of its partition, 3 = node whose visitor
+                    // list is still being written, 4 = one boundary of a node to work out ahead of time;
+                    // [1] context; [2] slice | slices << 16 (kind 4: boundary | slice size << 8)
 };
 
 constexpr int kHeavyCtxInts = 16 + 1024;  // 16 + the widest fan-out
 constexpr int kHeavyMin = 1024;          // visitors from which a node is settled by several wavefronts
 constexpr int kMaxSlices = 64;           // slices (and parts of the partition) of such a node, at most
 constexpr int kHeavyFanout = 384;        // widest node settled that way (register budget)
-// What the slices of a heavy node hand to each other: slice s works out the boundary between itself and
-// slice s + 1 and leaves it here for that slice.  Per boundary: [0] == the number of the select call once the
-// rest is written, [1] the threshold key, [2] entries above the boundary, [3] 1 = worked out, 0 = the
-// threshold search failed, [16 + i] entries of child i above the boundary.
+// The boundaries between the slices of a heavy node: whoever needs one first works it out and leaves it here.
+// Per boundary: [0] 2 * the number of the select call while it is being worked out, that + 1 once the rest is
+// written, [1] the threshold key, [2] entries above the boundary, [3] 1 = worked out, 0 = the threshold search
+// failed, [16 + i] entries of child i above the boundary.
 constexpr int kBoundInts = 16 + kHeavyFanout;
 
 struct SelectArgs {
@@ -62,7 +64,9 @@ struct SelectArgs {
     int32_t *sched_wait;   // [0] visitors still in multi-visitor items, [1] abort flag (a waiting
                            // wavefront gave up, or the queue overflowed)
     int32_t *hctx;         // contexts of heavy nodes, kHeavyCtxInts each: [0] slices still running,
-                           // [1] a slice failed a check, [16 + i] visits of child i
+                           // [1] a slice failed a check, [5] == the number of the select call when the contexts of
+                           // children are listed, [16 + i] visits of child i, [16 + kHeavyFanout + i] context + 1
+                           // of child i whose boundaries are being worked out ahead of time, or 0
     int32_t *hctx_n;       // contexts handed out
     int32_t *hbound;       // boundaries between the slices of heavy nodes: kMaxSlices x kBoundInts per context
     int32_t *list_flag;    // per visitor-list start: depth of the deepest item whose list, starting there,

@@ -1710,16 +1710,15 @@ __device__ __forceinline__ uint32_t active_threshold(const ActiveSet<R> &s, floa
 }
 
 // For a slice of a heavy node: the boundary of the cumulative target `target`: a threshold key T
-// and EXACTLY how many entries of every own child lie above the boundary (ct; at most m each): the
+// and EXACTLY how many entries of every own child lie above the boundary (ct; at most m each, m >= target:
+// a cap on what is looked at, not the node's visitor count, of which a boundary does not depend): the
 // entries at or above T, or, where far more entries than the target pile up on T itself, those over T and
 // the first of the pile (see below).  Deterministic, a function of the node's state and the target only.
 // Uses the LDS scratch.
-// TWO: the boundary of a second target as well (target2 > 0; ct2, T2), on the same preparation.
-template <int R, bool RAVE, bool TWO>
+template <int R, bool RAVE>
 __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const NodeCtx &c, int lane,
                                                  const Kids<R, RAVE> &k, WaveLds<R> &lds, int m, int window,
-                                                 int target1, int (&ct1)[R], uint32_t &T1, int target2, int (&ct2)[R],
-                                                 uint32_t &T2) {
+                                                 int target, int (&ct)[R], uint32_t &T) {
     constexpr int F = R * kWave;
     const uint32_t uvl = (uint32_t)a.vl;
     uint32_t headk[R];
@@ -1799,7 +1798,7 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
         }
     }
     int cta[R];
-    auto boundary = [&](int target, int (&ct)[R], uint32_t &T) {
+    {
     // The boundary of one target: the threshold and the exact counts at it.  When far more entries than the
     // target lie at or above the threshold, they are piled up ON the threshold key (a child whose key does not
     // move at all over hundreds of visits; no key separates them), and the boundary is put inside the pile:
@@ -1881,11 +1880,83 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
 #pragma unroll
         for (int r = 0; r < R; r++) ct[r] = (int)lds.pay[r * kWave + lane];
         wave_sync_memory();
-    };
-    boundary(target1, ct1, T1);
-    if (TWO && target2 > 0) boundary(target2, ct2, T2);
-    if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1 + (TWO && target2 > 0 ? 1 : 0));
+    }
+    if (a.stats && lane == 0) atomicAdd(a.stats + 5, 1);
     return true;
+}
+
+// Visitors per slice of a heavy node: a function of the visitor count in steps (192 up to 12288 visitors, then
+// the next multiple of 64 that keeps the slices at 64), so that whoever knows the count only within a step
+// knows the slice size.
+__device__ __forceinline__ int slice_size(int m) {
+    const int s = ((m + 4095) >> 12) << 6;
+    return s < kSliceEntries ? kSliceEntries : s;
+}
+
+// Boundary number b of a heavy node cut into slices of S visitors (the one between slices b - 1 and b: target
+// rank b * S, window S / 4), through the node's boundary table: whoever asks first works it out and leaves it
+// there (ready word 2 * call number + 1; 2 * call number while it is being worked out), everybody else takes it
+// from there.  One value per boundary whoever computes it: the slices on both sides, and the wavefronts that
+// work boundaries out ahead of time (items of kind 4, published while the node's parent is still being settled:
+// a boundary depends on the node's statistics and its rank only, not on how many visitors the node ends up
+// with).  Whoever holds a claim is running and waits for nothing before it writes, so the bounded wait ends.
+// Returns false when the threshold search failed, or when the selection is being given up.
+template <int R, bool RAVE>
+__device__ __forceinline__ bool slice_boundary(const SelectArgs &a, const NodeCtx &c, int lane, const Kids<R, RAVE> &k,
+                                               WaveLds<R> &lds, int hid, int b, int S, int (&ct)[R], uint32_t &T,
+                                               int &rank) {
+    int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)(b - 1)) * kBoundInts;  // b = 1 .. kMaxSlices
+    const int claimed = 2 * a.epoch, ready = claimed + 1;
+    int state = 0;  // 1 this wavefront works it out, 2 it is there
+    for (int spins = 0;; spins++) {
+        int got = 0, ab = 0;
+        if (lane == 0) {
+            const int v = __hip_atomic_load(bnd + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v == ready) got = 2;
+            else if (v != claimed) got = atomicCAS(bnd + 0, v, claimed) == v ? 1 : 0;
+            else if ((spins & 3) == 3)
+                ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        got = __builtin_amdgcn_readfirstlane(got);
+        ab = __builtin_amdgcn_readfirstlane(ab);
+        if (got) {
+            state = got;
+            break;
+        }
+        if (ab) break;
+        if (spins >= a.spin_limit) {
+            if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 3);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+    if (state == 0) return false;
+    if (state == 1) {
+        const bool ok = threshold_counts<R, RAVE>(a, c, lane, k, lds, b * S + S, S >> 2, b * S, ct, T);
+        int sum = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            bnd[16 + r * kWave + lane] = ct[r];
+            sum += ct[r];
+        }
+        rank = wave_sum_i32(sum);
+        if (lane == 0) {
+            bnd[1] = (int)T;
+            bnd[2] = rank;
+            bnd[3] = ok ? 1 : 0;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (lane == 0) __hip_atomic_store(bnd + 0, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return ok;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    T = (uint32_t)__hip_atomic_load(bnd + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    rank = __hip_atomic_load(bnd + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool ok = __hip_atomic_load(bnd + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        ct[r] = __hip_atomic_load(bnd + 16 + r * kWave + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return ok;
 }
 
 // The commonest crowded node: one child wins every time.  That is the case exactly when
@@ -2677,6 +2748,85 @@ __device__ __noinline__ void chain_finish(KernArgsP ka, int tid3, int n_threads,
 }
 
 // Where the walk goes on after a multi-visitor node whose visitors all chose one child.
+// Called by one slice of a heavy node once it knows a lower bound of every child's visitors (low[]: the child's
+// entries among the first ranks of the node's winner order; at most `slack` more visitors can come).  A child
+// that is sure to get kHeavyMin visitors will be cut into slices of S = slice_size(its visitors), and boundary
+// b of it (rank b * S) depends on the child's own statistics only, which nothing changes before the child
+// itself is shared out.  So the boundaries that are sure to lie within the child's visitors, whatever the final
+// count, become items of the work queue right away (kind 4: pad[1] the child's context, pad[2] = b | S << 8),
+// taken by wavefronts that would otherwise wait; the child's slices find them in the boundary table.  The
+// child's context is handed out here and left in the node's context ([16 + kHeavyFanout + i] = context + 1, 0 =
+// none; [5] = the number of the select call once that is written), where the wavefront that publishes the child
+// picks it up.  Nothing here is a guess: a boundary that turns out not to be needed (the child is settled
+// otherwise) is a wasted computation, never a wrong one.
+template <int R, bool RAVE>
+__device__ __forceinline__ void prefetch_boundaries(const ForestDev &f, const SelectArgs &a, const NodeCtx &c, int lane,
+                                                    const Kids<R, RAVE> &k, const int (&low)[R], int slack, int depth,
+                                                    int *ctx) {
+    int nb[R], sz[R], cid[R];
+    int mine = 0;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        nb[r] = 0;
+        sz[r] = 0;
+        cid[r] = -1;
+        const int L = low[r];
+        if (L >= kHeavyMin && r * kWave + lane < c.nelig) {
+            const int S = slice_size(L);
+            if (S == slice_size(L + slack) && f.span[c.cb + r * kWave + lane].y > 0) {
+                // every boundary the child can need, whatever its final count: the one behind its last slice
+                // included (a boundary does not depend on the count; one too many is a wasted computation)
+                int n = (L + slack + S - 1) / S;
+                n = n < kMaxSlices ? n : kMaxSlices;
+                if (n >= 1) {
+                    const int id = atomicAdd(a.hctx_n, 1);
+                    if (id < a.hctx_cap) {
+                        nb[r] = n;
+                        sz[r] = S;
+                        cid[r] = id;
+                        mine += n;
+                    }
+                }
+            }
+        }
+    }
+    const int inc = wave_inclusive_sum(mine, lane);
+    const int total = __builtin_amdgcn_readlane(inc, 63);
+    int slot0 = 0;
+    if (total > 0) {
+        if (lane == 0) slot0 = atomicAdd(a.sched_tail, total);
+        slot0 = __builtin_amdgcn_readfirstlane(slot0);
+        if (slot0 + total > a.q_cap) {
+            if (lane == 0) atomicExch(a.sched_wait + 1, 2);  // queue overflow: cannot happen on a tree
+            return;
+        }
+    }
+    int at = slot0 + inc - mine;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        ctx[16 + kHeavyFanout + i] = cid[r] + 1;
+        for (int b = 1; b <= nb[r]; b++) {
+            Item it;
+            it.node = c.cb + i;
+            it.off = 0;
+            it.m = low[r];
+            it.np = k.n[r];
+            it.depth = depth + 1;
+            it.pad[0] = 4;
+            it.pad[1] = cid[r];
+            it.pad[2] = b | (sz[r] << 8);
+            a.items_q[at + b - 1] = it;
+        }
+        at += nb[r];
+    }
+    if (lane == 0) ctx[5] = a.epoch;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    at = slot0 + inc - mine;
+    for (int j = 0; j < mine; j++)
+        __hip_atomic_store(a.q_ready + at + j, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 struct Continuation {
     int node;
     int off;
@@ -2823,7 +2973,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
     int run_child = -1, lds_cur = -1;
     bool as_slice = item.pad[0] == 1;
     const bool as_scatter = item.pad[0] == 2;
-    int hid = as_slice || as_scatter ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF, n_slices = (item.pad[2] >> 16) & 0x3FFF;
+    // one boundary of this node, to be worked out ahead of time (prefetch_boundaries): into the table, nothing else
+    const bool just_boundary = item.pad[0] == 4;
+    int hid = as_slice || as_scatter || just_boundary ? item.pad[1] : -1, slice = item.pad[2] & 0xFFFF,
+        n_slices = (item.pad[2] >> 16) & 0x3FFF;
     if (as_scatter) {
         // a part of the partition of a heavy node: the visits per child are in its context
         const int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
@@ -2840,7 +2993,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         best0 = __builtin_amdgcn_readfirstlane(g_chain.e_best0);
         lk0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)g_chain.e_lk0);
         lp0 = (uint32_t)(__builtin_amdgcn_readfirstlane(g_chain.e_second) ? R * kWave + best0 : best0);
-    } else if (!as_slice && !settled && m >= kRunMin && a.vl > 0)
+    } else if (!as_slice && !just_boundary && !settled && m >= kRunMin && a.vl > 0)
         settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child, contested, best0,
                                       lk0, lp0);
     if (!settled && contested && m >= kSparseMin && m < kHeavyMin) {
@@ -2854,12 +3007,13 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         }
     }
     if (R * kWave <= kHeavyFanout) {
-        if (!as_slice && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
+        if (!as_slice && !just_boundary && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
-            const int K = (m + kSliceEntries - 1) / kSliceEntries < kMaxSlices ? (m + kSliceEntries - 1) / kSliceEntries
-                                                                               : kMaxSlices;
+            const int K = (m + slice_size(m) - 1) / slice_size(m);  // at most kMaxSlices
+            // (a node whose boundaries are being worked out ahead of time has its context already)
             int id = a.hctx_cap;
-            if (lane == 0) id = atomicAdd(a.hctx_n, 1);
+            if (item.pad[0] == 3 && item.pad[1] > 0) id = item.pad[1] - 1;
+            else if (lane == 0) id = atomicAdd(a.hctx_n, 1);
             id = __builtin_amdgcn_readfirstlane(id);
             if (id < a.hctx_cap) {
                 int slot0 = 0;
@@ -2892,9 +3046,9 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 }
             }
         }
-        if (as_slice) {
+        if (as_slice || just_boundary) {
             int *ctx = a.hctx + (size_t)hid * kHeavyCtxInts;
-            const int S = (m + n_slices - 1) / n_slices;
+            const int S = just_boundary ? item.pad[2] >> 8 : slice_size(m);
             const bool last = slice == n_slices - 1;
             int ct_hi[R], ct_lo[R];
 #pragma unroll
@@ -2902,83 +3056,40 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             bool ok = true;
             int rank_hi = 0, rank_lo = m;
             uint32_t T_hi = 0xFFFFFFFFu, T_lo = 0u;
-            // the window inside which a threshold search may stop early: narrower than the
-            // distance between the targets of two slices
             const long long ts0 = a.trace ? wall_clock64() : 0ll;
             long long ts1 = ts0;
-            // Every slice works out ONE boundary, the one between itself and the next slice (the last slice: the
-            // threshold of the node's last visitor, with which it knows its one batch like every other slice
-            // instead of searching for it in the batch loop), leaves it in the node's boundary table, and takes
-            // the boundary between the slice before and itself from there: both neighbours use the same numbers
-            // by construction, and nobody searches the same threshold twice.  The slice before was handed out
-            // earlier (slice 0 runs on the wavefront that cut the node), and it writes its boundary before it
-            // waits for anything, so the wait below ends; it is bounded like every other.
-            // A narrow node's boundaries are cheap: every slice works out both of its own (same input, same
-            // result on both sides of a boundary), which costs less than handing them over.
-            constexpr bool kHandOver = R > 1;
-            ok = threshold_counts<R, RAVE, !kHandOver>(a, c, lane, k, lds, m, S >> 2, last ? m : (slice + 1) * S, ct_lo, T_lo,
-                                                       kHandOver ? 0 : slice * S, ct_hi, T_hi);
-            if (!kHandOver) {
-                if (slice == 0) T_hi = 0xFFFFFFFFu;
-                if (ok && slice > 0) {
-                    int sum = 0;
+            // The boundary behind this slice, then the one before it, both through the node's boundary table
+            // (slice_boundary): the neighbours use the same numbers by construction, nobody works the same
+            // boundary out twice, and a boundary worked out ahead of time is simply there.  The boundary behind
+            // the last slice lies at or after the node's last visitor: with it that slice knows its one batch
+            // like every other (it keeps what it needs) instead of searching for it in the batch loop.
+            // (One call site, run twice: the code behind it is the largest of the kernel.)
+#pragma nounroll
+            for (int pass = 0; pass < 2; pass++) {
+                const int b = just_boundary ? (pass == 0 ? (item.pad[2] & 255) : 0) : (pass == 0 ? slice + 1 : slice);
+                if (b == 0 || !ok) continue;
+                int ct[R], rank = 0;
+                uint32_t T = 0u;
+                ok = slice_boundary<R, RAVE>(a, c, lane, k, lds, hid, b, S, ct, T, rank);
+                if (pass == 0) {
 #pragma unroll
-                    for (int r = 0; r < R; r++) sum += ct_hi[r];
-                    rank_hi = wave_sum_i32(sum);
-                }
-            }
-            if (kHandOver && !last) {
-                int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)(slice + 1)) * kBoundInts;
-                int sum = 0;
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    bnd[16 + r * kWave + lane] = ct_lo[r];
-                    sum += ct_lo[r];
-                }
-                sum = wave_sum_i32(sum);
-                if (lane == 0) {
-                    bnd[1] = (int)T_lo;
-                    bnd[2] = sum;
-                    bnd[3] = ok ? 1 : 0;
-                }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-                if (lane == 0) __hip_atomic_store(bnd + 0, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (kHandOver && ok && slice > 0) {
-                const int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)slice) * kBoundInts;
-                bool there = false;
-                for (int spins = 0;; spins++) {
-                    int v = 0, ab = 0;
-                    if (lane == 0) {
-                        v = __hip_atomic_load(bnd + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (v != a.epoch && (spins & 3) == 3)
-                            ab = __hip_atomic_load(a.sched_wait + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                    v = __builtin_amdgcn_readfirstlane(v);
-                    ab = __builtin_amdgcn_readfirstlane(ab);
-                    if (v == a.epoch) {
-                        there = true;
-                        break;
-                    }
-                    if (ab) break;
-                    if (spins >= a.spin_limit) {
-                        if (lane == 0) atomicCAS(a.sched_wait + 1, 0, 3);
-                        break;
-                    }
-                    __builtin_amdgcn_s_sleep(4);
-                }
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-                if (there) {
-                    T_hi = (uint32_t)__hip_atomic_load(bnd + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    rank_hi = __hip_atomic_load(bnd + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (__hip_atomic_load(bnd + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) ok = false;
-#pragma unroll
-                    for (int r = 0; r < R; r++)
-                        ct_hi[r] = __hip_atomic_load(bnd + 16 + r * kWave + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int r = 0; r < R; r++) ct_lo[r] = ct[r];
+                    T_lo = T;
+                    rank_lo = rank;
                 } else {
-                    ok = false;  // the selection is being given up
+#pragma unroll
+                    for (int r = 0; r < R; r++) ct_hi[r] = ct[r];
+                    T_hi = T;
+                    rank_hi = rank;
                 }
             }
+            if (just_boundary) return kStepParked;
+            // The slice before the last knows how many of the first (K - 1) * S visitors every child takes: a
+            // child that takes a thousand of them will be cut into slices itself, and its boundaries depend on
+            // its own statistics only.  They are worked out from now on, by idle wavefronts, while this node's
+            // slices are still being settled (prefetch_boundaries).
+            if (RMAX * kWave <= kHeavyFanout && ok && n_slices >= 2 && slice == n_slices - 2 && depth + 1 < a.max_depth)
+                prefetch_boundaries<R, RAVE>(f, a, c, lane, k, ct_lo, m - rank_lo, depth, ctx);
             bool preset_ok = !last;
             if (ok) {
                 int sum = 0;
@@ -3059,6 +3170,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             if (failed) st_replay = 1;
         }
     }
+    if (just_boundary) return kStepParked;  // (a fan-out class that is never cut into slices)
     if (!settled && m >= kWaterLevelMin && m <= kWaterLevelMaxJ && a.vl > 0) {
         int zero[R];
 #pragma unroll
@@ -3330,6 +3442,9 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                     }
                     int kslot[R];
                     int kbase = slot0 + K2 - 1;
+                    // children whose boundaries are being worked out ahead of time have a context already
+                    const bool ahead_ctx =
+                        __hip_atomic_load(ctx + 5, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.epoch;
 #pragma unroll
                     for (int r = 0; r < R; r++) {
                         const int i = r * kWave + lane;
@@ -3342,7 +3457,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                             it.np = k.n[r];
                             it.depth = depth + 1;
                             it.pad[0] = 3;
-                            it.pad[1] = it.pad[2] = 0;
+                            it.pad[1] = ahead_ctx ? __hip_atomic_load(ctx + 16 + kHeavyFanout + i, __ATOMIC_RELAXED,
+                                                                      __HIP_MEMORY_SCOPE_AGENT)
+                                                  : 0;
+                            it.pad[2] = 0;
                             kslot[r] = kbase + __popcll(kids[r] & ((1ull << lane) - 1ull));
                             a.items_q[kslot[r]] = it;
                         }
@@ -3555,8 +3673,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         Item it = a.items_q[ticket];
         if (it.depth == 0 && it.pad[0] == 0) {
-            it.np = f.N[it.node];
-            for (int j = lane; j < it.m; j += kWave) a.paths[a.seg0[it.off + j]] = it.node;
+            it.np = f.N[it.node];  // (the paths' first entries, the roots, are written when the roots are set)
         }
         bool have_span = false, chain_open = false;
         int preload = 0;  // what select_group finds of the node's children (its argument of that name)
@@ -3591,6 +3708,8 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
             }
             const int preload_now = preload;
             preload = 0;
+            // a boundary to work out ahead of time, of a node that turns out to have no children to choose from
+            if (it.pad[0] == 4 && !(c.cc > 0 && depth < a.max_depth)) break;
             int status = kStepLeaf;
             Continuation next;
             next.node = -1;

@@ -197,7 +197,7 @@ def timeline(workload, warmup=8, levels=()):
           "list was complete; a node cut into slices / scatter parts shows their number and the span from the first "
           "start to the last end)")
     print("%5s %9s %9s %7s %9s %9s %8s  %s" % ("level", "node", "visitors", "kind", "start_us", "end_us", "us", "work"))
-    names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "job", 5: "chain"}
+    names = {0: "node", 1: "slice", 2: "part", 3: "early", 4: "bound", 5: "chain"}
     for d in range(int(depth.max()) + 1):
         at = np.nonzero(depth == d)[0]
         if len(at) == 0:
