@@ -907,7 +907,7 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     // a multi-visitor item has at least two visitors, and a level holds each visitor once; a heavy
     // node (kHeavyMin visitors or more) adds at most 63 slice items
     // (and as many parts of its partition, and as many boundaries worked out ahead of time)
-    b->q_cap = (int32_t)((B / 2 + B / 4 + 64) * (max_depth + 1));
+    b->q_cap = (int32_t)((B + 64) * (max_depth + 1));
     // (a node whose boundaries are worked out ahead of time, and that is then not cut into slices after all, uses
     // a second context for its partition)
     b->hctx_cap = (int32_t)std::min<int64_t>(4096, 2 * (B / kHeavyMin) * (max_depth + 1));

@@ -1885,11 +1885,12 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     return true;
 }
 
-// Visitors per slice of a heavy node: a function of the visitor count in steps (192 up to 12288 visitors, then
-// the next multiple of 64 that keeps the slices at 64), so that whoever knows the count only within a step
-// knows the slice size.
+// Visitors per slice of a heavy node: a function of the visitor count in steps (kSliceEntries up to
+// kSliceEntries * kMaxSlices visitors, then the next multiple of 64 that keeps the slices at kMaxSlices), so that
+// whoever knows the count only within a step knows the slice size.  (128 visitors a slice and up to 128 slices
+// measured the same as 192 and 64: a slice's time is mostly not its entries.)
 __device__ __forceinline__ int slice_size(int m) {
-    const int s = ((m + 4095) >> 12) << 6;
+    const int s = ((m + 64 * kMaxSlices - 1) / (64 * kMaxSlices)) << 6;
     return s < kSliceEntries ? kSliceEntries : s;
 }
 
@@ -1951,6 +1952,34 @@ __device__ __forceinline__ bool slice_boundary(const SelectArgs &a, const NodeCt
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     T = (uint32_t)__hip_atomic_load(bnd + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    rank = __hip_atomic_load(bnd + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool ok = __hip_atomic_load(bnd + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        ct[r] = __hip_atomic_load(bnd + 16 + r * kWave + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return ok;
+}
+
+// A boundary that another wavefront works out, taken from the table once it is there: the counts of every own
+// child and their sum.  Gives up (false) after `polls` polls: only for work that can be left undone.
+template <int R>
+__device__ __forceinline__ bool boundary_read(const SelectArgs &a, int lane, int hid, int b, int polls, int (&ct)[R],
+                                              int &rank) {
+    const int *bnd = a.hbound + ((size_t)hid * kMaxSlices + (size_t)(b - 1)) * kBoundInts;
+    const int ready = 2 * a.epoch + 1;
+    bool there = false;
+    for (int spins = 0; spins < polls; spins++) {
+        int v = 0;
+        if (lane == 0) v = __hip_atomic_load(bnd + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v = __builtin_amdgcn_readfirstlane(v);
+        if (v == ready) {
+            there = true;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+    }
+    if (!there) return false;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     rank = __hip_atomic_load(bnd + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const bool ok = __hip_atomic_load(bnd + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
 #pragma unroll
@@ -3025,17 +3054,16 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                         ctx[0] = K;
                         ctx[1] = 0;
                     }
-                    if (lane < K - 1) {
+                    for (int j = lane; j < K - 1; j += kWave) {
                         Item it = item;
                         it.pad[0] = 1;
                         it.pad[1] = id;
-                        it.pad[2] = (lane + 1) | (K << 16) | (list_ok ? 0 : 1 << 30);
-                        a.items_q[slot0 + lane] = it;
+                        it.pad[2] = (j + 1) | (K << 16) | (list_ok ? 0 : 1 << 30);
+                        a.items_q[slot0 + j] = it;
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-                    if (lane < K - 1)
-                        __hip_atomic_store(a.q_ready + slot0 + lane, a.epoch, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
+                    for (int j = lane; j < K - 1; j += kWave)
+                        __hip_atomic_store(a.q_ready + slot0 + j, a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     as_slice = true;
                     hid = id;
                     slice = 0;
@@ -3084,12 +3112,6 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 }
             }
             if (just_boundary) return kStepParked;
-            // The slice before the last knows how many of the first (K - 1) * S visitors every child takes: a
-            // child that takes a thousand of them will be cut into slices itself, and its boundaries depend on
-            // its own statistics only.  They are worked out from now on, by idle wavefronts, while this node's
-            // slices are still being settled (prefetch_boundaries).
-            if (RMAX * kWave <= kHeavyFanout && ok && n_slices >= 2 && slice == n_slices - 2 && depth + 1 < a.max_depth)
-                prefetch_boundaries<R, RAVE>(f, a, c, lane, k, ct_lo, m - rank_lo, depth, ctx);
             bool preset_ok = !last;
             if (ok) {
                 int sum = 0;
@@ -3151,6 +3173,16 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             if (a.trace && lane == 0) {
                 g_slice_note[0] = (int)(ts1 - ts0);
                 g_slice_note[1] = (int)(wall_clock64() - ts1);
+            }
+            // The boundary before the last slice says how many of the first (K - 1) * S visitors every child takes:
+            // a child that takes a thousand of them will be cut into slices itself, and its boundaries depend on
+            // its own statistics only.  They are worked out from now on, by idle wavefronts, while this node's
+            // slices are still being settled (prefetch_boundaries).  The first slice sees to that: it ends
+            // before the slices in the middle of the order do, and nothing waits for it.
+            if (RMAX * kWave <= kHeavyFanout && ok && slice == 0 && n_slices >= 3 && depth + 1 < a.max_depth) {
+                int ctb[R], rank_b = 0;
+                if (boundary_read<R>(a, lane, hid, n_slices - 1, 512, ctb, rank_b) && rank_b <= m)
+                    prefetch_boundaries<R, RAVE>(f, a, c, lane, k, ctb, m - rank_b, depth, ctx);
             }
             if (!ok && lane == 0) atomicExch(ctx + 1, 1);
             // join: the wavefront that finishes last goes on with the node
@@ -3404,8 +3436,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
                 id = __builtin_amdgcn_readfirstlane(id);
                 if (id < a.hctx_cap) hid = id;
             }
-            const int K2 = (m + kScatterPart - 1) / kScatterPart < kMaxSlices ? (m + kScatterPart - 1) / kScatterPart
-                                                                             : kMaxSlices;
+            const int K2 = (m + kScatterPart - 1) / kScatterPart < kWave ? (m + kScatterPart - 1) / kScatterPart : kWave;
             // The children with several visitors are published together with the parts, before
             // their lists exist (kind 3: they wait for list_flag where they need the list; the
             // parts sit before them in the queue, so whatever a waiting child depends on has
