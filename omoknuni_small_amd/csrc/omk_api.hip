@@ -116,6 +116,7 @@ struct omk_batch {
     float *values = nullptr;
     Item *items0 = nullptr, *items_q = nullptr, *singles0 = nullptr, *singles_q = nullptr;
     int32_t n_singles0 = 0;
+    int32_t n_hctx0 = 0;  // contexts of heavy roots, handed out when the roots are set
     int32_t *seg0 = nullptr, *seg[2] = {nullptr, nullptr};
     int32_t *sc_child = nullptr, *sc_occ = nullptr;
     // [1..16] work statistics, [17] single-visitor queue length, [32] status of omk_batch_leaf_keys,
@@ -994,6 +995,27 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
     }
     // the most crowded roots head the longest chains of work: start them first
     std::stable_sort(items.begin(), items.end(), [](const Item &x, const Item &y) { return x.m > y.m; });
+    // A root that will be cut into slices (kHeavyMin visitors or more): its boundaries depend on its statistics
+    // only, so they are queued right behind the roots (items of kind 4, see prefetch_boundaries in
+    // omk_select.hip) and worked out by other wavefronts while the root's own wavefront still loads its children.
+    int32_t n_hctx0 = 0;
+    {
+        const size_t n_roots = items.size();
+        for (size_t i = 0; i < n_roots && items[i].m >= kHeavyMin && n_hctx0 < b->hctx_cap; i++) {
+            const int32_t S = slice_size(items[i].m), K = (items[i].m + S - 1) / S;
+            if (items.size() + (size_t)K > (size_t)b->stride) break;  // (items0 holds one item per traversal)
+            items[i].pad[1] = n_hctx0 + 1;
+            for (int32_t bnd = 1; bnd <= K; bnd++) {
+                Item it = items[i];
+                it.off = 0;
+                it.pad[0] = 4;
+                it.pad[1] = n_hctx0;
+                it.pad[2] = bnd | (S << 8);
+                items.push_back(it);
+            }
+            n_hctx0++;
+        }
+    }
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     HIP_TRY(hipMemcpy(b->seg0, order.data(), (size_t)n * 4, hipMemcpyHostToDevice));
@@ -1005,6 +1027,7 @@ int omk_batch_set_roots(omk_batch *b, const int32_t *h_roots, int32_t n) {
     if (!singles.empty())
         HIP_TRY(hipMemcpy(b->singles0, singles.data(), singles.size() * sizeof(Item), hipMemcpyHostToDevice));
     b->n_items0 = (int32_t)items.size();
+    b->n_hctx0 = n_hctx0;
     b->n_singles0 = (int32_t)singles.size();
     b->n = n;
     b->generation = f->generation;
@@ -1107,7 +1130,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.c_puct = p->c_puct;
     a.rave_k = p->rave_k;
     HIP_TRY(launch_select(f->dev(), a, b->n_items0, b->n_singles0, b->n, f->max_fanout, p->use_rave != 0, b->n_cus,
-                          f->stream));
+                          b->n_hctx0, f->stream));
     b->selected = true;
     return OMK_OK;
 }

@@ -43,6 +43,16 @@ constexpr int kHeavyCtxInts = 16 + 1024;  // 16 + the widest fan-out
 constexpr int kHeavyMin = 1024;          // visitors from which a node is settled by several wavefronts
 constexpr int kMaxSlices = 64;           // slices (and parts of the partition) of such a node, at most
 constexpr int kHeavyFanout = 384;        // widest node settled that way (register budget)
+constexpr int kSliceEntries = 192;       // visitors per slice of such a node, about
+// Visitors per slice of a heavy node: a function of the visitor count in steps (kSliceEntries up to
+// kSliceEntries * kMaxSlices visitors, then the next multiple of 64 that keeps the slices at kMaxSlices), so that
+// whoever knows the count only within a step knows the slice size.  (128 visitors a slice and up to 128 slices
+// measured the same as 192 and 64: a slice's time is mostly not its entries.)
+__host__ __device__ inline int slice_size(int m) {
+    const int s = ((m + 64 * kMaxSlices - 1) / (64 * kMaxSlices)) << 6;
+    return s < kSliceEntries ? kSliceEntries : s;
+}
+
 // The boundaries between the slices of a heavy node: whoever needs one first works it out and leaves it here.
 // Per boundary: [0] 2 * the number of the select call while it is being worked out, that + 1 once the rest is
 // written, [1] the threshold key, [2] entries above the boundary, [3] 1 = worked out, 0 = the threshold search
@@ -105,7 +115,7 @@ struct SelectArgs {
 };
 
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
-                         int max_fanout, bool rave, int n_cus, hipStream_t s);
+                         int max_fanout, bool rave, int n_cus, int n_hctx0, hipStream_t s);
 
 hipError_t launch_apply_vl(const ForestDev &f, const int32_t *paths, const int32_t *path_len, int n, int stride,
                            int max_len, int vl, hipStream_t s);

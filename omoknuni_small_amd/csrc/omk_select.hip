@@ -71,7 +71,6 @@ constexpr int kTeam = kTeamWaves * 64;
 constexpr int kTeamMin = 96;              // batch entries from which the helpers are called in
 // a batch of at most this many entries per thread is ordered by counting: a lone wavefront, the block
 constexpr int kCountSortLone = 2, kCountSortTeam = 1;
-constexpr int kSliceEntries = 192;        // visitors per slice of such a node, about
 constexpr int kRunShortcutMin = 128;      // entries from which a run of one child is emitted without sorting
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
@@ -1885,15 +1884,6 @@ __device__ __forceinline__ bool threshold_counts(const SelectArgs &a, const Node
     return true;
 }
 
-// Visitors per slice of a heavy node: a function of the visitor count in steps (kSliceEntries up to
-// kSliceEntries * kMaxSlices visitors, then the next multiple of 64 that keeps the slices at kMaxSlices), so that
-// whoever knows the count only within a step knows the slice size.  (128 visitors a slice and up to 128 slices
-// measured the same as 192 and 64: a slice's time is mostly not its entries.)
-__device__ __forceinline__ int slice_size(int m) {
-    const int s = ((m + 64 * kMaxSlices - 1) / (64 * kMaxSlices)) << 6;
-    return s < kSliceEntries ? kSliceEntries : s;
-}
-
 // Boundary number b of a heavy node cut into slices of S visitors (the one between slices b - 1 and b: target
 // rank b * S, window S / 4), through the node's boundary table: whoever asks first works it out and leaves it
 // there (ready word 2 * call number + 1; 2 * call number while it is being worked out), everybody else takes it
@@ -3041,7 +3031,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
             const int K = (m + slice_size(m) - 1) / slice_size(m);  // at most kMaxSlices
             // (a node whose boundaries are being worked out ahead of time has its context already)
             int id = a.hctx_cap;
-            if (item.pad[0] == 3 && item.pad[1] > 0) id = item.pad[1] - 1;
+            if ((item.pad[0] == 3 || (item.pad[0] == 0 && depth == 0)) && item.pad[1] > 0) id = item.pad[1] - 1;
             else if (lane == 0) id = atomicAdd(a.hctx_n, 1);
             id = __builtin_amdgcn_readfirstlane(id);
             if (id < a.hctx_cap) {
@@ -3703,7 +3693,7 @@ __device__ __forceinline__ void owner_loop(const ForestDev &f, const SelectArgs 
         // compute unit every time); one acquire once the item is there
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         Item it = a.items_q[ticket];
-        if (it.depth == 0 && it.pad[0] == 0) {
+        if (it.depth == 0 && (it.pad[0] == 0 || it.pad[0] == 4)) {  // (items the host wrote: a root, a boundary of one)
             it.np = f.N[it.node];  // (the paths' first entries, the roots, are written when the roots are set)
         }
         bool have_span = false, chain_open = false;
@@ -4146,7 +4136,7 @@ __device__ __noinline__ void walkers_loop(ForestDev f, SelectArgs a, int lane) {
 
 // Scheduler state, statistics, the work queue seeded with the items of the roots, and the
 // single-visitor queue seeded with the traversals that are alone at their root.
-__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0, int n_traversals) {
+__global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int open0, int n_traversals, int n_hctx0) {
     const int gid = blockIdx.x * blockDim.x + threadIdx.x;
     const int step = gridDim.x * blockDim.x;
     if (gid == 0) {
@@ -4158,7 +4148,7 @@ __global__ void k_select_reset(SelectArgs a, int n_items0, int n_singles0, int o
         *a.sched_tail = n_items0;
         a.sched_wait[0] = open0;
         a.sched_wait[1] = 0;
-        *a.hctx_n = 0;
+        *a.hctx_n = n_hctx0;  // the contexts of heavy roots are handed out when the roots are set
         *a.trace_n = 0;
     }
     if (a.stats && gid < 16) a.stats[gid] = 0;
@@ -4223,7 +4213,7 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
 }
 
 hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, int n_singles0, int n_traversals,
-                         int max_fanout, bool rave, int n_cus, hipStream_t s) {
+                         int max_fanout, bool rave, int n_cus, int n_hctx0, hipStream_t s) {
     // Every traversal alone at its root (one per tree: leaf-parallel self-play): the single-visitor
     // kernel is the whole select and takes its walkers from the host's list; every walker writes its
     // own leaf and path length, so nothing has to be cleared first (the statistics apart).
@@ -4232,7 +4222,7 @@ hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, 
     if (!alone || a.stats) {
         int reset_blocks = (n_traversals + 255) / 256;
         hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
-                           n_traversals - n_singles0, n_traversals);
+                           n_traversals - n_singles0, n_traversals, n_hctx0);
     }
 #define OMK_DISPATCH(RM)                                                              \
     return rave ? launch_kernels<RM, true>(f, a, n_items0, n_traversals, n_cus, s)    \
