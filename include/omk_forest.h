@@ -300,7 +300,8 @@ int omk_batch_set_stats(omk_batch *b, int32_t enabled);
  * with omk_batch_set_trace before that select.  One record of twelve int64 per piece of work: start
  * and end on the GPU's 100 MHz clock, visitors | depth << 32 | kind << 60 (0 a node settled as a
  * whole, 1 a slice of a heavy node, 2 a part of its partition, 3 a node published before its visitor
- * list was complete, 5 a node whose visitors all follow one child, taken by the walk down such nodes,
+ * list was complete, 4 one boundary between two slices of a heavy node worked out ahead of time, 5 a node
+ * whose visitors all follow one child, taken by the walk down such nodes,
  * 6 the walk of a lone visitor inside the persistent launch), node | number << 32 (number: for a slice
  * or a part of a heavy node, which one of how many: index | count << 16), then, for a slice of a heavy node,
  * word 4 = time of its boundaries | time of its batches << 32 (100 MHz clock) and word 5 = entries its
