@@ -75,6 +75,7 @@ constexpr int kRunShortcutMin = 128;      // entries from which a run of one chi
 constexpr int kScatterPart = 256;         // visitors per part of a heavy node's partition, about
 constexpr int kScatterUnroll = 8;         // chunks of 64 visitors whose loads the partition issues together
 constexpr int kMaxWalkerBlocks = 16;         // blocks of walkers of the persistent launch, at most
+constexpr int kTeamSinglesMaxWaves = 4096;  // wavefronts up to which a batch of lone traversals is walked by blocks (one round of children per wavefront)
 constexpr int kFastSinglesMax = 16384;    // traversals up to which the single-visitor kernel trades bytes for latency
 constexpr int kRunShareMin = 4096;        // a node whose visitors all take one child: visitors from which the scatter
                                           // is shared out like a heavy node's instead of left to one helper
@@ -4065,6 +4066,163 @@ __global__ __launch_bounds__(256) void k_select_singles(ForestDev f, SelectArgs 
     walk_single<RMAX, RAVE, MODE>(f, a, a.singles0[wave], lane);
 }
 
+// The same walk by a whole block, for a batch of few traversals on a wide layout (a legal mask: one slot per
+// action): wavefront w of the block takes round w of every node's children (64 slots), so a level costs the
+// loads and the score arithmetic of ONE round instead of RMAX, one LDS exchange and one block barrier.  A few
+// hundred lone walkers leave the machine empty anyway (one wavefront each on a thousand SIMDs), and what
+// a walk takes is its chain of levels: memory latency plus the instruction issue of the wavefront that scores
+// the children.  Same arithmetic on the same inputs (child_keys), same choice: the first maximum over the
+// first-scan candidates, then the second-scan candidates (comes_before), the second scan only with a real
+// first-scan score, the least visited participating child when no candidate has a real score (wave_pick).
+struct SingleSlot {
+    uint32_t bk, bpos;    // the wavefront's best candidate (key 0 = none)
+    int bn, bsx, bsy;     // that child's visit count and child range
+    uint32_t any1;        // one of its children has a real first-scan key
+    uint32_t fn, fidx;    // its least visited participating child (visit count as an ordered uint; ~0 = none)
+    int fcn, fsx, fsy;    // that child's visit count and child range
+};
+
+template <int RMAX, bool RAVE>
+__global__ __launch_bounds__(RMAX * kWave) void k_select_singles_team(ForestDev f, SelectArgs a, int seeded) {
+    constexpr int F = RMAX * kWave;
+    __shared__ SingleSlot slot[2][RMAX];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *a.n_singles = seeded;
+        *a.truncated_next = 0;
+        a.sched_wait[1] = 0;
+    }
+    if ((int)blockIdx.x >= seeded) return;
+    const Item it = a.singles0[blockIdx.x];
+    int node = it.node, d = it.depth, np = it.np;
+    const int t = it.off;
+    if (d == 0) {
+        np = f.N[node];
+        if (threadIdx.x == 0) a.paths[t] = node;
+    }
+    int2 span = f.span[node];
+    for (int level = 0;; level++) {
+        const int cb = span.x, cc = span.y;
+        int nelig = cc;
+        if (a.pw) {
+            const int kk = ceil_sqrt_i32(np);
+            nelig = kk < cc ? kk : cc;
+        }
+        const float ep = a.c_puct * sqrtf((float)np);
+        int ci = -1, np_child = 0;
+        int2 span_child = int2{0, 0};
+        if (cc > 0 && d < a.max_depth) {
+            // this wavefront's round of the children: everything asked for at once
+            const int i = wv * kWave + lane;
+            const bool in = i < nelig;
+            const int id = cb + i;
+            uint32_t word = 0xFFFFFFFFu;
+            int n = 0, vl = 0;
+            float w = 0.0f, p = 0.0f, q2 = 0.0f;
+            int2 sp = int2{0, 0};
+            if (wv * kWave < nelig) {  // uniform
+                if (in && f.legal) word = f.legal[(uint32_t)id >> 5];
+                if (in) {
+                    n = f.N[id];
+                    w = f.W[id];
+                    p = f.P[id];
+                    vl = f.VL[id];
+                    if (RAVE) q2 = f.q2[id];
+                    sp = f.span[id];
+                }
+            }
+            const bool part = in && ((word >> ((uint32_t)id & 31u)) & 1u);
+            uint32_t k1 = 0u, k2 = 0u;
+            if (part) child_keys<RAVE>(n, w, p, vl, q2, ep, k1, k2);
+            uint32_t bk = k1, bpos = (uint32_t)i;
+            if (k2 > bk) {
+                bk = k2;
+                bpos = (uint32_t)(F + i);
+            }
+            if (bk == 0u) bpos = 0xFFFFFFFFu;
+            uint32_t hk, hp;
+            wave_best(bk, bpos, hk, hp);
+            const uint32_t mn = part ? (uint32_t)n ^ 0x80000000u : 0xFFFFFFFFu;
+            const uint32_t gm = wave_min_u32(mn);
+            const uint32_t gidx = wave_min_u32(part && mn == gm ? (uint32_t)i : 0xFFFFFFFFu);
+            const bool any1 = __ballot(k1 != 0u) != 0ull;
+            const int bl = hk != 0u ? (int)((hp >= (uint32_t)F ? hp - (uint32_t)F : hp) & 63u) : 0;
+            const int fl = gidx != 0xFFFFFFFFu ? (int)(gidx & 63u) : 0;
+            const int bn = __builtin_amdgcn_readlane(n, bl), bsx = __builtin_amdgcn_readlane(sp.x, bl);
+            const int bsy = __builtin_amdgcn_readlane(sp.y, bl);
+            const int fcn = __builtin_amdgcn_readlane(n, fl), fsx = __builtin_amdgcn_readlane(sp.x, fl);
+            const int fsy = __builtin_amdgcn_readlane(sp.y, fl);
+            if (lane == 0) {
+                SingleSlot &sl = slot[level & 1][wv];
+                sl.bk = hk;
+                sl.bpos = hp;
+                sl.bn = bn;
+                sl.bsx = bsx;
+                sl.bsy = bsy;
+                sl.any1 = any1 ? 1u : 0u;
+                sl.fn = gm;
+                sl.fidx = gidx;
+                sl.fcn = fcn;
+                sl.fsx = fsx;
+                sl.fsy = fsy;
+            }
+            __syncthreads();  // (the slots alternate with the level: nobody is a level ahead of a reader)
+            // ---- the same over the wavefronts ----
+            uint32_t gk = 0u, gp = 0xFFFFFFFFu, a1 = 0u, fn = 0xFFFFFFFFu, fi = 0xFFFFFFFFu;
+            int won = 0, fwon = 0;
+#pragma unroll
+            for (int x = 0; x < RMAX; x++) {
+                const SingleSlot &sl = slot[level & 1][x];
+                a1 |= sl.any1;
+                if (sl.bk != 0u && comes_before(sl.bk, sl.bpos, gk, gp)) {
+                    gk = sl.bk;
+                    gp = sl.bpos;
+                    won = x;
+                }
+                if (sl.fn < fn || (sl.fn == fn && sl.fidx < fi)) {
+                    fn = sl.fn;
+                    fi = sl.fidx;
+                    fwon = x;
+                }
+            }
+            if (RAVE && gk != 0u && gp >= (uint32_t)F && a1 == 0u) gk = 0u;  // no second scan without a first-scan score
+            if (gk != 0u) {
+                const SingleSlot &sl = slot[level & 1][won];
+                ci = (int)(gp >= (uint32_t)F ? gp - (uint32_t)F : gp);
+                np_child = sl.bn;
+                span_child = int2{sl.bsx, sl.bsy};
+            } else if (fi != 0xFFFFFFFFu) {
+                const SingleSlot &sl = slot[level & 1][fwon];
+                ci = (int)fi;
+                np_child = sl.fcn;
+                span_child = int2{sl.fsx, sl.fsy};
+            }
+            ci = __builtin_amdgcn_readfirstlane(ci);
+            np_child = __builtin_amdgcn_readfirstlane(np_child);
+            span_child.x = __builtin_amdgcn_readfirstlane(span_child.x);
+            span_child.y = __builtin_amdgcn_readfirstlane(span_child.y);
+        }
+        if (ci < 0) {
+            if (threadIdx.x == 0) {
+                a.leaf[t] = node;
+                a.path_len[t] = d + 1;
+                if (cc > 0 && d >= a.max_depth) atomicAdd(a.truncated, 1);
+            }
+            return;
+        }
+        const int child = cb + ci;
+        if (threadIdx.x == 0) {
+            if (a.stats) atomicAdd(a.stats + 6, 1);
+            if (a.vl > 0) atomicAdd(f.VL + child, a.vl);
+            a.paths[(size_t)(d + 1) * a.stride + t] = child;
+        }
+        node = child;
+        np = np_child;
+        span = span_child;
+        d++;
+    }
+}
+
 // The walkers of the persistent launch: wavefronts of the blocks behind the teams take the lone
 // visitors one by one as the teams create them (a ticket, then the entry's ready word, set after
 // the release fence of whoever wrote the entry), so that a lone visitor walks while the chain of
@@ -4203,7 +4361,10 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
     }
     // every traversal is alone at its root: the walkers are the host's list
     const dim3 grid((n_traversals + 3) / 4), block(256);
-    if (!f.legal)
+    if (RMAX > 1 && f.legal && n_traversals * RMAX <= kTeamSinglesMaxWaves)
+        hipLaunchKernelGGL((k_select_singles_team<RMAX, RAVE>), dim3(n_traversals), dim3(RMAX * kWave), 0, s, f, a0,
+                           n_traversals);
+    else if (!f.legal)
         hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 0>), grid, block, 0, s, f, a0, n_traversals);
     else if (fast)
         hipLaunchKernelGGL((k_select_singles<RMAX, RAVE, 2>), grid, block, 0, s, f, a0, n_traversals);
