@@ -366,3 +366,53 @@ def test_chain_whose_capacity_is_exceeded_by_one_visitor(fan, rave, m):
     soa = capacity_chain(fan, 25, 11, m, rave)
     st = select_both(soa, np.zeros(m, np.int32), 27, rave=rave, steps=2)
     assert st["replayed_nodes"] == 0, st
+
+
+def test_boundaries_of_heavy_children_are_worked_out_ahead_of_time():
+    """A heavy root with heavy children: the children's slice boundaries are queued as items of their own
+    (kind 4 in the timeline) while the root is still being settled, the root's own when the roots are set;
+    the result is the checker's all the same, and nothing is replayed."""
+    import omoknuni_small_amd as omk
+    soa, roots = layered_forest(12, [48, 40])
+    troots = np.zeros(20_000, np.int32)
+    D, vl = 3, 3
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, max_depth=D)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, len(troots), D)
+    b.set_roots(troots)
+    b.enable_stats()
+    b.enable_trace()
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl)
+    rpaths, rlen, rleaf, near = ref.select_batch(troots, rp)
+    b.select(sp)
+    tr = b.debug_trace()
+    gpaths, glen, gleaf, _ = b.read()
+    st = b.stats()
+    assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all()
+    assert st["replayed_nodes"] == 0, st
+    kind = (tr[:, 2] >> 60) & 7
+    depth = (tr[:, 2] >> 32) & 0xFFFFFFF
+    assert ((kind == 4) & (depth == 0)).sum() >= 1, "no boundary of the root was queued"
+    assert ((kind == 4) & (depth == 1)).sum() >= 1, "no boundary of a heavy child was queued ahead of time"
+    assert (kind == 1).sum() >= 1
+
+
+def test_roots_set_again_start_the_paths_anew():
+    """The paths' first entries are written when the roots are set: setting other roots replaces them."""
+    import omoknuni_small_amd as omk
+    soa, roots = layered_forest(13, [30, 10], n_trees=4)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, 600, 3)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=3)
+    for pick in ([0, 1], [2, 3, 1], [3]):
+        troots = roots[np.array(pick)][np.arange(600) % len(pick)].astype(np.int32)
+        ref = R.RefTree.from_soa(soa)
+        rp = R.make_params(c_puct=1.4, virtual_loss=3, max_depth=3)
+        rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp)
+        b.set_roots(troots)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths[:, 0] == troots).all()
+        assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all()
+        f.upload(soa)  # the virtual losses of this selection are dropped with the statistics
