@@ -395,6 +395,38 @@ int omk_tt_set_replacement_threshold(omk_tt *tt, float threshold);
  * call, transpositions reported.  Waits for the stream. */
 int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int32_t cells, const uint64_t *d_player_keys,
                     const uint64_t *d_root_keys, const int32_t *d_root_players, int32_t *d_hits, int32_t *h_counts);
+/* The whole traversal loop with the table on, redirects INCLUDED (mcts_engine_batch_tree_simple.cpp:88-165;
+ * the redirect is :142-156 with MCTSNode::updateChildReference, mcts_node.cpp:617-630): a select for the
+ * batch's roots that, at every step, stores the selected child when it has no visits, looks the position
+ * up, and on a transposition (a node other than the selected one, with visits) takes the virtual loss back
+ * from the selected child, re-points the parent's child slot at the transposition, adds the virtual loss
+ * there and walks on from it.  Off unless called: omk_select_batch never redirects.
+ *   - Exact for the reference run by one thread: the traversals are walked one after the other by a single
+ *     wavefront (a re-pointed slot is seen by every later traversal, as in the serial loop).  Expect
+ *     microseconds per step, not the throughput of omk_select_batch.
+ *   - A re-pointed slot holds another node: selection reads that node's statistics and prior, and the move
+ *     recorded for the step is that node's action (children_[i]->getAction(), :112), as in the reference.
+ *   - Keys are the forest's per-node position keys (omk_soa_view.hash / omk_forest_set_keys): the key of a
+ *     step is that of the node of the tree AS UPLOADED that the recorded moves lead to from the root, which
+ *     is what replaying the moves on the root state gives (:119-124); where no such node exists (a move no
+ *     child slot carries, a node not expanded) the step has no key and the table is not touched.
+ *   - Time stamps: step g of the call stores at clock + 2g and looks up at clock + 2g + 1.
+ *   - d_moves: NULL, or device memory for max_depth * stride ints (omk_batch_dev.stride), level-major like the
+ *     paths (entry (d - 1) * stride + t = the move recorded at step d of traversal t): the move list the
+ *     leaf's state is rebuilt from.  It differs from the actions of the path's nodes exactly at a step that
+ *     redirected.
+ *   - h_counts (NULL or [5]): new entries, replacements, lookups that found an entry, redirects, steps.
+ * Paths, leaves and virtual loss are left as omk_select_batch leaves them (omk_batch_read, omk_backup_batch,
+ * omk_revert_vl work on them).  Once a slot has been re-pointed the forest is a graph until the next
+ * omk_forest_upload: omk_select_batch, omk_backup_rave_batch, omk_forest_add_root_noise and the compactions
+ * refuse it (OMK_ERR_UNSUPPORTED); omk_forest_action_probabilities counts the visits of the nodes the root's
+ * slots hold (mcts_engine_tree.cpp:395-403).  Selection-time progressive widening is refused.  Waits for the
+ * stream. */
+int omk_tt_select_redirect(omk_tt *tt, omk_batch *b, const omk_select_params *params, int32_t *d_moves,
+                           int32_t *h_counts);
+/* h_alias[n_nodes]: the node child slot s holds instead of node s, or -1 (MCTSNode::children_ after
+ * updateChildReference); n_nodes must be the forest's node count. */
+int omk_forest_download_redirects(omk_forest *f, int64_t n_nodes, int32_t *h_alias);
 /* What an entry keeps for the replacement policy, slot by slot beside omk_tt_download. */
 typedef struct omk_tt_meta {
     uint32_t visits;      /* Entry::visits */

@@ -61,6 +61,11 @@ struct omk_forest {
     uint64_t *hash = nullptr;
     bool has_legal = false, has_action = false, has_hash = false;
     void *key_stage = nullptr;  // staging of omk_forest_set_keys: keys, node ids, one status word
+    // Child slots re-pointed at transpositions (omk_tt_select_redirect): alias[s] >= 0 = the node slot s holds
+    // instead of node s.  Allocated by the first such call; `redirected` once a slot has been re-pointed: the
+    // forest is then a graph, and what assumes a tree refuses it until the next upload.
+    int32_t *alias = nullptr;
+    bool redirected = false;
     size_t key_stage_bytes = 0;
     int children = 0;       // live batches and tables created on this forest
     bool released = false;  // omk_forest_destroy was called while children were alive
@@ -196,6 +201,14 @@ static int use_device(const omk_forest *f) {
 
 // Roots, paths and work items of a batch are node ids: stale once the forest was compacted or a
 // different structure uploaded.
+static int tree_only(const char *who, const omk_forest *f) {
+    if (f->redirected)
+        return fail(OMK_ERR_UNSUPPORTED,
+                    "%s: child slots of this forest have been re-pointed at transpositions (omk_tt_select_redirect): "
+                    "it is a graph until the next upload, and this operation needs a tree", who);
+    return OMK_OK;
+}
+
 static int fresh_batch(const char *who, const omk_batch *b) {
     if (b->generation != b->f->generation)
         return fail(OMK_ERR_STATE, "%s: the forest was compacted or uploaded with another structure since this "
@@ -246,7 +259,7 @@ int omk_forest_create(const omk_forest_desc *desc, omk_forest **out) {
 static void forest_free(omk_forest *f) {
     (void)hipSetDevice(f->device);
     if (f->own_stream) (void)hipStreamSynchronize(f->own_stream);
-    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->Q2, f->action, f->legal, f->hash, f->key_stage};
+    void *ptrs[] = {f->span, f->N, f->W, f->P, f->VL, f->rN, f->rW, f->Q2, f->action, f->legal, f->hash, f->key_stage, f->alias};
     for (void *p : ptrs)
         if (p) (void)hipFree(p);
     if (f->own_stream) (void)hipStreamDestroy(f->own_stream);
@@ -377,6 +390,10 @@ int omk_forest_upload(omk_forest *f, const omk_soa_view *v) {
     if (!f->uploaded || f->structure_changed || n != f->n_nodes || ssum != f->structure_sum) f->generation++;
     f->structure_sum = ssum;
     f->structure_changed = false;
+    if (f->redirected) {  // an upload brings a tree: every slot holds its own node again
+        HIP_TRY(launch_fill_words(f->alias, 0xFFFFFFFFu, f->capacity, f->stream));
+        f->redirected = false;
+    }
     f->n_nodes = n;
     f->max_fanout = mf;
     f->prior_sorted = sorted;
@@ -544,6 +561,7 @@ int omk_forest_add_root_noise(omk_forest *f, int32_t root, const float *h_gamma,
     if (!f || !h_gamma) return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: null argument");
     if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_add_root_noise: nothing uploaded");
     if (root < 0 || root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_add_root_noise: root %d", root);
+    if (int rc = tree_only("omk_forest_add_root_noise", f)) return rc;
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     int2 sp;
@@ -605,6 +623,14 @@ int omk_forest_action_probabilities(omk_forest *f, int32_t root, float temperatu
     if (cc <= 0) return OMK_OK;
     std::vector<int32_t> n((size_t)cc), act((size_t)cc);
     HIP_TRY(hipMemcpy(n.data(), f->N + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
+    if (f->redirected) {
+        // the counts are those of the nodes the children vector holds (child->getVisitCount(),
+        // mcts_engine_tree.cpp:401-403), the actions those of the slots (root->getActions(), :395)
+        std::vector<int32_t> al((size_t)cc);
+        HIP_TRY(hipMemcpy(al.data(), f->alias + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
+        for (int32_t i = 0; i < cc; i++)
+            if (al[(size_t)i] >= 0) HIP_TRY(hipMemcpy(&n[(size_t)i], f->N + al[(size_t)i], 4, hipMemcpyDeviceToHost));
+    }
     if (f->has_action) {
         HIP_TRY(hipMemcpy(act.data(), f->action + cb, (size_t)cc * 4, hipMemcpyDeviceToHost));
     } else {
@@ -779,6 +805,7 @@ int omk_forest_compact(omk_forest *f, int32_t new_root, int64_t *h_nodes_after, 
     if (!f) return fail(OMK_ERR_INVALID, "omk_forest_compact: null forest");
     if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact: nothing uploaded");
     if (new_root < 0 || new_root >= f->n_nodes) return fail(OMK_ERR_INVALID, "omk_forest_compact: root %d", new_root);
+    if (int rc = tree_only("omk_forest_compact", f)) return rc;
     if (int rc = use_device(f)) return rc;
     HIP_TRY(hipStreamSynchronize(f->stream));
     const int64_t n = f->n_nodes;
@@ -845,6 +872,7 @@ int omk_forest_compact_static(omk_forest *f, int32_t new_root, int64_t *h_nodes_
     if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_compact_static: nothing uploaded");
     if (new_root < 0 || new_root >= f->n_nodes)
         return fail(OMK_ERR_INVALID, "omk_forest_compact_static: root %d", new_root);
+    if (int rc = tree_only("omk_forest_compact_static", f)) return rc;
     if (f->n_nodes > kStaticCompactNodes)
         return fail(OMK_ERR_CAPACITY,
                     "omk_forest_compact_static: the forest holds %lld nodes, the static scratch memory serves at most "
@@ -1056,11 +1084,28 @@ int omk_batch_device(omk_batch *b, omk_batch_dev *out) {
     return OMK_OK;
 }
 
+// The number of the select call on the batch: ready marks of the queues are call numbers (the boundary table's:
+// twice that), so they start over before they repeat.
+static int next_epoch(omk_batch *b) {
+    omk_forest *f = b->f;
+    if (b->epoch >= (1 << 30) - 2) {
+        HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
+        HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
+        HIP_TRY(launch_fill_words(b->hbound, 0u, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts, f->stream));
+        // the two depth-cap counters take turns by call parity, which this restart breaks once
+        HIP_TRY(launch_fill_words(b->counters + kTruncatedWord, 0u, 2, f->stream));
+        b->epoch = 0;
+    }
+    b->epoch++;
+    return OMK_OK;
+}
+
 int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     if (!b || !p) return fail(OMK_ERR_INVALID, "omk_select_batch: null argument");
     omk_forest *f = b->f;
     if (!f->uploaded || b->n <= 0) return fail(OMK_ERR_STATE, "omk_select_batch: upload a forest and set roots first");
     if (int rc = fresh_batch("omk_select_batch", b)) return rc;
+    if (int rc = tree_only("omk_select_batch", f)) return rc;
     if (p->use_rave && !f->has_rave)
         return fail(OMK_ERR_INVALID, "omk_select_batch: use_rave on a forest created without RAVE arrays");
     if (p->pw && !f->prior_sorted)
@@ -1080,15 +1125,7 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.items_q = b->items_q;
     a.seg[0] = b->seg[0];
     a.seg[1] = b->seg[1];
-    if (b->epoch >= (1 << 30) - 2) {  // ready marks are call numbers (the boundary table's: twice that): start over before they repeat
-        HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
-        HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
-        HIP_TRY(launch_fill_words(b->hbound, 0u, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts, f->stream));
-        // the two depth-cap counters take turns by call parity, which this restart breaks once
-        HIP_TRY(launch_fill_words(b->counters + kTruncatedWord, 0u, 2, f->stream));
-        b->epoch = 0;
-    }
-    b->epoch++;
+    if (int rc = next_epoch(b)) return rc;
     a.q_ready = b->q_ready;
     a.q_cap = b->q_cap;
     a.epoch = b->epoch;
@@ -1154,6 +1191,7 @@ int omk_backup_rave_batch(omk_batch *b) {
     if (!b->selected) return fail(OMK_ERR_STATE, "omk_backup_rave_batch: no selected paths");
     if (int rc = fresh_batch("omk_backup_rave_batch", b)) return rc;
     if (!b->f->has_rave) return fail(OMK_ERR_INVALID, "omk_backup_rave_batch: the forest has no RAVE arrays");
+    if (int rc = tree_only("omk_backup_rave_batch", b->f)) return rc;
     if (int rc = use_device(b->f)) return rc;
     HIP_TRY(launch_rave_backup(b->f->mut(), b->paths, b->path_len, b->values, b->n, b->stride, b->max_depth + 1,
                                b->f->stream));
@@ -1650,6 +1688,82 @@ int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int3
                     status[5], cells);
     status[1] = 0;  // steps that do not exist carry the empty marker on purpose
     return tt_report("omk_tt_traverse", status, h_counts);
+}
+
+int omk_tt_select_redirect(omk_tt *tt, omk_batch *b, const omk_select_params *p, int32_t *d_moves, int32_t *h_counts) {
+    if (!tt || !b || !p) return fail(OMK_ERR_INVALID, "omk_tt_select_redirect: null argument");
+    if (tt->f != b->f) return fail(OMK_ERR_INVALID, "omk_tt_select_redirect: table and batch belong to different forests");
+    omk_forest *f = b->f;
+    if (!f->uploaded || b->n <= 0)
+        return fail(OMK_ERR_STATE, "omk_tt_select_redirect: upload a forest and set roots first");
+    if (int rc = fresh_batch("omk_tt_select_redirect", b)) return rc;
+    if (!f->has_hash)
+        return fail(OMK_ERR_STATE, "omk_tt_select_redirect: the forest has no position keys (upload them, or "
+                    "omk_forest_set_keys)");
+    if (p->use_rave && !f->has_rave)
+        return fail(OMK_ERR_INVALID, "omk_tt_select_redirect: use_rave on a forest created without RAVE arrays");
+    if (p->pw)
+        return fail(OMK_ERR_UNSUPPORTED, "omk_tt_select_redirect: progressive widening at selection time is not "
+                    "part of this loop");
+    if (int rc = use_device(f)) return rc;
+    if (int rc = tt_same_tree(tt)) return rc;
+    hipStream_t s = f->stream;
+    if (!f->alias) {
+        HIP_TRY(dalloc(&f->alias, f->capacity));
+        HIP_TRY(launch_fill_words(f->alias, 0xFFFFFFFFu, f->capacity, s));
+    }
+    if (int rc = next_epoch(b)) return rc;
+    int status[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    HIP_TRY(hipMemcpyAsync(tt->d_status, status, sizeof(status), hipMemcpyHostToDevice, s));
+    RedirectArgs a;
+    memset(&a, 0, sizeof(a));
+    a.alias = f->alias;
+    a.slots = tt->slots;
+    a.meta = tt->meta;
+    a.log2_slots = tt->log2_slots;
+    a.t0 = tt->clock;
+    a.threshold = tt->threshold;
+    a.paths = b->paths;
+    a.path_len = b->path_len;
+    a.leaf = b->leaf;
+    a.moves = d_moves;
+    a.n = b->n;
+    a.stride = b->stride;
+    a.max_depth = b->max_depth;
+    a.vl = p->virtual_loss;
+    a.c_puct = p->c_puct;
+    a.rave_k = p->rave_k;
+    a.counts = tt->d_status;
+    a.truncated = b->counters + kTruncatedWord + (b->epoch & 1);
+    a.truncated_next = b->counters + kTruncatedWord + ((b->epoch + 1) & 1);
+    a.abort_word = b->counters + 3 * kSchedStep + 1;
+    HIP_TRY(launch_select_redirect(f->dev(), a, p->use_rave != 0, s));
+    b->selected = true;
+    HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    tt->clock += 2u * (uint32_t)status[4];
+    if (status[3] > 0) f->redirected = true;
+    if (h_counts)
+        for (int i = 0; i < 5; i++) h_counts[i] = status[i];
+    if (status[5])
+        return fail(OMK_ERR_CAPACITY, "omk_tt_select_redirect: table full, %d entries dropped", status[5]);
+    return OMK_OK;
+}
+
+int omk_forest_download_redirects(omk_forest *f, int64_t n_nodes, int32_t *h_alias) {
+    if (!f || !h_alias) return fail(OMK_ERR_INVALID, "omk_forest_download_redirects: null argument");
+    if (!f->uploaded) return fail(OMK_ERR_STATE, "omk_forest_download_redirects: nothing uploaded");
+    if (n_nodes != f->n_nodes)
+        return fail(OMK_ERR_INVALID, "omk_forest_download_redirects: room for %lld nodes, the forest holds %lld",
+                    (long long)n_nodes, (long long)f->n_nodes);
+    if (!f->alias) {
+        for (int64_t i = 0; i < n_nodes; i++) h_alias[i] = -1;
+        return OMK_OK;
+    }
+    if (int rc = use_device(f)) return rc;
+    HIP_TRY(hipStreamSynchronize(f->stream));
+    HIP_TRY(hipMemcpy(h_alias, f->alias, (size_t)n_nodes * 4, hipMemcpyDeviceToHost));
+    return OMK_OK;
 }
 
 int omk_tt_download_meta(omk_tt *tt, omk_tt_meta *h_meta) {

@@ -725,6 +725,199 @@ hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *
     return hipGetLastError();
 }
 
+// ---- the traversal loop with the transposition table on, redirects included
+// (reference src/mcts/mcts_engine_batch_tree_simple.cpp:88-165: store :116-128, lookup :131-141, redirect
+// :142-156; MCTSNode::updateChildReference src/mcts/mcts_node.cpp:617-630) ----
+//
+// A redirect re-points a child slot of one node at a node that lives under another: the tree becomes a
+// graph, a node's visitors no longer all come through one parent, and what a traversal finds depends on
+// what every earlier one stored, found and re-pointed.  The reference's outcome for one thread is the
+// outcome of the traversals run one after the other, and that is what this kernel does: ONE wavefront
+// walks the traversals in index order, the children of a node spread over its lanes (64 slots a round),
+// the table and the re-pointing done by lane 0.  It is the exact mode for a search that wants the
+// reference's redirects, not a fast one: a step costs a few dependent trips to memory, and nothing
+// overlaps them.
+//
+// alias[s] >= 0: child slot s holds that node instead of node s.  The statistics, the prior and the
+// action that selection and the move record read are those of the node a slot HOLDS
+// (children_[i]->getAction(), :112).  The key of a step is the position key of the node of the
+// ORIGINAL tree (slots, not what they hold) that the recorded moves lead to from the root, which is
+// what replaying the recorded moves on the root state gives (:119-124, :133-137); where no such node
+// exists the step has no key and the table is left alone.
+// Time: step g of the call (counted over all traversals) stores at t0 + 2g and looks up at t0 + 2g + 1.
+
+__device__ __forceinline__ int ld_agent(const int32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ bool slot_legal(const ForestDev &f, int id) {
+    return !f.legal || ((f.legal[(uint32_t)id >> 5] >> ((uint32_t)id & 31u)) & 1u);
+}
+
+// MCTSNode::selectChild over the slots [cb, cb + cc) of `node`; returns the chosen slot or -1.  The
+// same arithmetic (child_keys) and the same choice as the tree kernels: the first maximum of the first
+// scan, a second-scan candidate only when it beats every score before it and only after a first scan
+// that found a child, the least visited child when no score is real.
+template <bool RAVE>
+__device__ __forceinline__ int pick_slot_redirected(const ForestDev &f, const int32_t *alias, int node, int cb, int cc,
+                                                    float c_puct, float rave_k, int lane) {
+    const float ep = c_puct * sqrtf((float)f.N[node]);
+    uint32_t b1 = 0u, p1 = 0xFFFFFFFFu, b2 = 0u, p2 = 0xFFFFFFFFu, fn = 0xFFFFFFFFu, fi = 0xFFFFFFFFu;
+    for (int base = 0; base < cc; base += kWave) {
+        const int i = base + lane;
+        const bool in = i < cc && slot_legal(f, cb + i);
+        if (in) {
+            const int al = ld_agent(alias + cb + i);
+            const int held = al >= 0 ? al : cb + i;
+            const int n = f.N[held];
+            const float w = f.W[held];
+            const int vl = ld_agent(f.VL + held);
+            float q2 = 0.0f;
+            if (RAVE) q2 = combined_value(n, w, f.rN[held], f.rW[held], rave_k);
+            uint32_t k1, k2;
+            child_keys<RAVE>(n, w, f.P[held], vl, q2, ep, k1, k2);
+            if (k1 > b1) { b1 = k1; p1 = (uint32_t)i; }
+            if (k2 > b2) { b2 = k2; p2 = (uint32_t)i; }
+            const uint32_t on = (uint32_t)n ^ 0x80000000u;
+            if (on < fn) { fn = on; fi = (uint32_t)i; }
+        }
+    }
+    const uint32_t m1 = wave_max_u32(b1);
+    if (m1 != 0u) {
+        const uint32_t m2 = wave_max_u32(b2);
+        if (m2 > m1) return cb + (int)wave_min_u32(b2 == m2 ? p2 : 0xFFFFFFFFu);
+        return cb + (int)wave_min_u32(b1 == m1 ? p1 : 0xFFFFFFFFu);
+    }
+    const uint32_t gm = wave_min_u32(fn);
+    const uint32_t idx = wave_min_u32(fn == gm ? fi : 0xFFFFFFFFu);
+    return idx == 0xFFFFFFFFu ? -1 : cb + (int)idx;
+}
+
+template <bool RAVE>
+__global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, RedirectArgs a) {
+    const int lane = threadIdx.x;
+    const uint64_t mask = (1ull << a.log2_slots) - 1ull;
+    int n_new = 0, n_repl = 0, n_found = 0, n_redirect = 0, n_full = 0, n_trunc = 0;
+    uint32_t g = 0u;
+    for (int t = 0; t < a.n; t++) {
+        int cur = a.paths[t];
+        int shadow = cur;
+        int d = 0;
+        for (;;) {
+            const int2 sp = f.span[cur];
+            int slot = -1;
+            if (sp.y > 0 && d < a.max_depth) slot = pick_slot_redirected<RAVE>(f, a.alias, cur, sp.x, sp.y, a.c_puct, a.rave_k, lane);
+            if (slot < 0) {
+                if (lane == 0) {
+                    a.leaf[t] = cur;
+                    a.path_len[t] = d + 1;
+                }
+                if (sp.y > 0 && d >= a.max_depth) n_trunc++;
+                break;
+            }
+            const int al = ld_agent(a.alias + slot);
+            int best = al >= 0 ? al : slot;
+            const int move = f.action ? f.action[best] : best;
+            if (shadow >= 0) {
+                const int2 ss = f.span[shadow];
+                int next = -1;
+                for (int base = 0; base < ss.y && next < 0; base += kWave) {
+                    const int i = base + lane;
+                    const int s = ss.x + i;
+                    const bool hit = i < ss.y && slot_legal(f, s) && (f.action ? f.action[s] : s) == move;
+                    const unsigned long long any = __ballot(hit);
+                    if (any) next = ss.x + base + (__ffsll((long long)any) - 1);
+                }
+                shadow = next;
+            }
+            const unsigned long long key = shadow >= 0 ? f.hash[shadow] : kTTEmpty;
+            if (lane == 0) {
+                if (a.vl > 0) atomicAdd(f.VL + best, a.vl);                       // :109
+                if (a.moves) a.moves[(size_t)d * a.stride + t] = move;            // :112
+                if (key != kTTEmpty) {
+                    uint64_t s = tt_home(key, a.log2_slots);
+                    uint64_t probe = 0;
+                    for (; probe <= mask; probe++, s = (s + 1) & mask) {
+                        const unsigned long long k = a.slots[s].key;
+                        if (k == key || k == kTTEmpty) break;
+                    }
+                    const bool room = probe <= mask;
+                    const bool present = room && a.slots[s].key == key;
+                    const int nv = f.N[best];
+                    if (nv == 0) {                                                // :116-128, store()
+                        if (!room) {
+                            n_full++;
+                        } else {
+                            const int depth = (int)(uint16_t)(d + 1);             // move_sequence.size(); Entry::depth is a uint16_t
+                            bool write = !present;
+                            if (present) {
+                                const uint32_t now = a.t0 + 2u * g;
+                                const float existing = tt_replacement_score(a.meta[s].visits, a.meta[s].value, a.slots[s].depth,
+                                                                            now, a.meta[s].last_access);
+                                const float fresh = tt_replacement_score(0u, 0.0f, depth, now, 0u);
+                                if (fresh > existing * (1.0f + a.threshold)) {
+                                    write = true;
+                                    n_repl++;
+                                }
+                            } else {
+                                n_new++;
+                            }
+                            if (write) {
+                                a.slots[s].key = key;
+                                a.slots[s].node = best;
+                                a.slots[s].depth = depth;
+                                a.meta[s].visits = 0u;
+                                a.meta[s].value = 0.0f;
+                                a.meta[s].last_access = 0u;
+                            }
+                        }
+                    }
+                    int found = -1;
+                    if (room && a.slots[s].key == key) {                          // :141, lookup()
+                        found = a.slots[s].node;
+                        a.meta[s].last_access = a.t0 + 2u * g + 1u;
+                        n_found++;
+                    }
+                    if (found >= 0 && found != best && found < f.n_nodes && f.N[found] > 0) {   // :142
+                        if (a.vl > 0) {
+                            vl_sub_clamp(f.VL + best, a.vl);                      // :146
+                            atomicAdd(f.VL + found, a.vl);                        // :152
+                        }
+                        // :149: the slot selected is the first slot of the node that holds the old child (two slots
+                        // holding one node score alike, and the first of equals is selected)
+                        __hip_atomic_store(a.alias + slot, found, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        best = found;
+                        n_redirect++;
+                    }
+                }
+                a.paths[(size_t)(d + 1) * a.stride + t] = best;
+            }
+            best = __builtin_amdgcn_readfirstlane(best);
+            __threadfence();  // what lane 0 wrote is what every lane reads from here on
+            cur = best;
+            d++;
+            g++;
+        }
+    }
+    if (lane == 0) {
+        a.counts[0] = n_new;
+        a.counts[1] = n_repl;
+        a.counts[2] = n_found;
+        a.counts[3] = n_redirect;
+        a.counts[4] = (int)g;
+        a.counts[5] = n_full;
+        *a.truncated = n_trunc;
+        *a.truncated_next = 0;
+        *a.abort_word = 0;
+    }
+}
+
+hipError_t launch_select_redirect(const ForestDev &f, const RedirectArgs &a, bool rave, hipStream_t s) {
+    if (rave) hipLaunchKernelGGL(k_select_redirect<true>, dim3(1), dim3(kWave), 0, s, f, a);
+    else hipLaunchKernelGGL(k_select_redirect<false>, dim3(1), dim3(kWave), 0, s, f, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
                             const int32_t *depths, int64_t n, int *d_status, hipStream_t s) {
     if (n <= 0) return hipSuccess;

@@ -209,6 +209,25 @@ hipError_t launch_step_keys(const ForestDev &f, const int32_t *paths, const int3
                             int32_t *store_nodes, int32_t *depths, int *d_status, hipStream_t s);
 hipError_t launch_tt_hits(const ForestDev &f, const int32_t *step_nodes, const int32_t *found, int64_t n, int32_t *hit,
                           int *d_status, hipStream_t s);
+// The traversal loop with the table on, redirects included, one traversal after the other (omk_backup.hip).
+struct RedirectArgs {
+    int32_t *alias;
+    TTSlot *slots;
+    TTMeta *meta;
+    int log2_slots;
+    uint32_t t0;
+    float threshold;
+    int32_t *paths;     // level-major [max_depth + 1][stride]; level 0 holds the roots
+    int32_t *path_len;
+    int32_t *leaf;
+    int32_t *moves;     // nullptr, or level-major [max_depth][stride]: the move recorded at every step
+    int n, stride, max_depth, vl;
+    float c_puct, rave_k;
+    int *counts;        // [0] new entries, [1] replacements, [2] lookups that found an entry, [3] redirects,
+                        // [4] steps, [5] stores that found the table full
+    int32_t *truncated, *truncated_next, *abort_word;
+};
+hipError_t launch_select_redirect(const ForestDev &f, const RedirectArgs &a, bool rave, hipStream_t s);
 // d_status[0] += entries that found no free slot, d_status[1] += keys equal to the empty marker
 hipError_t launch_tt_insert(TTSlot *slots, int log2_slots, const uint64_t *keys, const int32_t *nodes,
                             const int32_t *depths, int64_t n, int *d_status, hipStream_t s);

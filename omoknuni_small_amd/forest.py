@@ -28,7 +28,7 @@ EXPORTS = [
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
     "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_set_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
-    "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
+    "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_select_redirect", "omk_forest_download_redirects", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy", "omk_soa_count_legal", "omk_soa_compact_legal",
 ]
 
@@ -252,6 +252,14 @@ class Forest:
         assert len(nodes) == len(keys)
         _check(self._lib.omk_forest_set_keys(self._h, _ptr(nodes, i32p), _ptr(keys, C.POINTER(C.c_uint64)),
                                              C.c_int64(len(nodes))))
+
+    def download_redirects(self):
+        """Per child slot the node it holds instead of its own, or -1 (slots re-pointed by
+        TranspositionTable.select_redirect)."""
+        n, _ = self.node_count()
+        out = np.empty(n, np.int32)
+        _check(self._lib.omk_forest_download_redirects(self._h, C.c_int64(n), _ptr(out, i32p)))
+        return out
 
     def download_structure(self):
         """Returns dict(child_begin, child_count, action) of the current nodes."""
@@ -601,6 +609,33 @@ class TranspositionTable:
             for d in bufs:
                 f.dev_free(d)
         return hits, tuple(int(x) for x in counts)
+
+    def select_redirect(self, batch, params, want_moves=True):
+        """The traversal loop with the table on, redirects included (omk_tt_select_redirect): a select for
+        batch's roots, one traversal after the other, that re-points child slots at transpositions as the
+        reference does.  Returns (moves [n, max_depth] recorded at every step, -1 padded, or None;
+        (new entries, replacements, lookups that found an entry, redirects, steps))."""
+        f = self.forest
+        p = params
+        counts = np.zeros(5, np.int32)
+        n, D = batch.n, batch.max_depth
+        stride = int(batch.device().stride)
+        d_moves = f.dev_alloc(4 * D * stride) if want_moves else 0
+        try:
+            _check(self._lib.omk_tt_select_redirect(self._h, batch._h, C.byref(p), C.c_void_p(d_moves),
+                                                    _ptr(counts, i32p)))
+            moves = None
+            if want_moves:
+                raw = np.empty((D, stride), np.int32)
+                f.d2h(raw, d_moves)
+                plen = np.empty(n, np.int32)
+                _check(self._lib.omk_batch_read(batch._h, None, _ptr(plen, i32p), None, None))
+                moves = np.ascontiguousarray(raw[:, :n].T)
+                moves[np.arange(D)[None, :] >= (plen[:, None] - 1)] = -1
+        finally:
+            if d_moves:
+                f.dev_free(d_moves)
+        return moves, tuple(int(x) for x in counts)
 
     def download_meta(self):
         meta = np.empty(1 << self.log2, dtype=TT_META)

@@ -412,6 +412,127 @@ int64_t ref_tt_lookup_batch(const ref_tt_slot *slots, ref_tt_meta *meta, int32_t
     return hits;
 }
 
+/* ---- the traversal loop with the transposition table switched on, redirects included
+ * (mcts_engine_batch_tree_simple.cpp:88-165; store :116-128, lookup :131-141, redirect :142-156;
+ * MCTSNode::updateChildReference mcts_node.cpp:617-630), one thread, traversals in index order.
+ *
+ * The children vector of a node is the slot range [child_begin, child_begin + child_count); slot s
+ * holds node s until updateChildReference re-points it: alias[s] = the node it holds now, -1 = its own.
+ * The statistics, the prior and the ACTION the loop reads are those of the node a slot holds
+ * (children_[i]->getAction(), :112), so the move recorded for a re-pointed slot is the action of the
+ * node it now holds, as in the reference.  The key of a step is getHash() of the root state with the
+ * recorded moves replayed (:119-124, :133-137): here node_key of the node of the ORIGINAL tree (slots,
+ * not what they hold) that the recorded moves lead to from the root; where that node does not exist
+ * (a move no child slot carries, or a node that is not expanded) the position has no key from there on:
+ * nothing is stored or looked up (the reference would ask the game).
+ * Time: step g of the call (counted over all traversals) stores at t0 + 2g and looks up at t0 + 2g + 1.
+ * counts: [0] new entries, [1] replacements, [2] lookups that found an entry, [3] redirects, [4] steps.
+ * Returns 0, -1 bad root, -2 table full. */
+static int32_t select_slot_redirected(const ref_tree *t, const int32_t *alias, int32_t node, const ref_params *p) {
+    const int32_t cb = t->child_begin[node];
+    const int32_t cc = t->child_count[node];
+    float best_score = -INFINITY;
+    int32_t best = -1;
+    int32_t ncand = 0;
+#define HELD(i) (alias[cb + (i)] >= 0 ? alias[cb + (i)] : cb + (i))
+    for (int32_t i = 0; i < cc; i++) {
+        if (!is_legal(t, cb + i)) continue;
+        float s1, s2;
+        ref_child_scores(t, node, HELD(i), p, &s1, &s2);
+        if (s1 > best_score) { best_score = s1; best = i; }
+        ncand++;
+    }
+    if (best < 0 && ncand > 0) {
+        int min_visits = INT32_MAX;
+        for (int32_t i = 0; i < cc; i++) {
+            if (!is_legal(t, cb + i)) continue;
+            if (t->N[HELD(i)] < min_visits) { min_visits = t->N[HELD(i)]; best = i; }
+        }
+    } else if (best >= 0) {
+        for (int32_t i = 0; i < cc; i++) {
+            if (!is_legal(t, cb + i)) continue;
+            float s1, s2;
+            ref_child_scores(t, node, HELD(i), p, &s1, &s2);
+            if (s2 > best_score) { best_score = s2; best = i; }
+        }
+    }
+#undef HELD
+    return best < 0 ? -1 : cb + best;
+}
+
+int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots, int32_t B, const ref_params *p,
+                              ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, uint32_t t0, float threshold,
+                              const uint64_t *node_key, int32_t *paths, int32_t *path_len, int32_t *leaf,
+                              int32_t *moves, int32_t *counts) {
+    const int32_t stride = p->max_depth + 1;
+    int rc = 0;
+    uint32_t g = 0;
+    for (int j = 0; j < 5; j++) counts[j] = 0;
+    for (int32_t i = 0; i < B; i++) {
+        int32_t *path = paths + (int64_t)i * stride;
+        int32_t *mv = moves ? moves + (int64_t)i * p->max_depth : NULL;
+        for (int32_t d = 0; d < stride; d++) path[d] = -1;
+        for (int32_t d = 0; mv && d < p->max_depth; d++) mv[d] = -1;
+        int32_t current = roots[i];
+        if (current < 0 || current >= t->n_nodes) return -1;
+        int32_t shadow = current;  /* node of the original tree the recorded moves lead to */
+        int32_t len = 0;
+        path[len++] = current;
+        while (t->child_count[current] > 0 && len <= p->max_depth) {
+            const int32_t slot = select_slot_redirected(t, alias, current, p);
+            if (slot < 0) break;
+            int32_t best = alias[slot] >= 0 ? alias[slot] : slot;
+            ref_add_vl(t, best, p->virtual_loss);                                     /* :109 */
+            const int32_t move = t->action ? t->action[best] : best;                 /* :112 */
+            if (mv) mv[len - 1] = move;
+            if (shadow >= 0) {
+                int32_t next = -1;
+                for (int32_t c = 0; c < t->child_count[shadow] && next < 0; c++) {
+                    const int32_t s = t->child_begin[shadow] + c;
+                    if (is_legal(t, s) && (t->action ? t->action[s] : s) == move) next = s;
+                }
+                shadow = next;
+            }
+            const uint64_t key = shadow >= 0 ? node_key[shadow] : REF_TT_EMPTY;
+            if (key != REF_TT_EMPTY) {
+                if (t->N[best] == 0) {                                               /* :116-128 */
+                    int32_t c4[4];
+                    const int32_t depth = len;                                       /* move_sequence.size() */
+                    int r = ref_tt_store_batch(slots, meta, log2_slots, t, &key, &best, &depth, 1, t0 + 2u * g,
+                                               threshold, c4);
+                    if (r == -1) rc = -2;
+                    counts[0] += c4[0];
+                    counts[1] += c4[1];
+                }
+                int32_t found = -1;
+                ref_tt_lookup_batch(slots, meta, log2_slots, &key, 1, 0, t0 + 2u * g + 1u, &found);  /* :141 */
+                if (found >= 0) counts[2]++;
+                if (found >= 0 && found != best && found < t->n_nodes && t->N[found] > 0) {  /* :142 */
+                    ref_remove_vl(t, best, p->virtual_loss);                         /* :146 */
+                    /* :149, updateChildReference: the first slot of `current` that holds the old child */
+                    for (int32_t c = 0; c < t->child_count[current]; c++) {
+                        const int32_t s = t->child_begin[current] + c;
+                        if (is_legal(t, s) && (alias[s] >= 0 ? alias[s] : s) == best) {
+                            alias[s] = found;
+                            break;
+                        }
+                    }
+                    ref_add_vl(t, found, p->virtual_loss);                           /* :152 */
+                    best = found;
+                    counts[3]++;
+                }
+            }
+            g++;
+            current = best;
+            path[len++] = current;
+        }
+        path_len[i] = len;
+        leaf[i] = current;
+    }
+    counts[4] = (int32_t)g;
+    return rc;
+}
+
 /* ---- leaf expansion (mcts_node.cpp:238-436, :512-593; call site
  * mcts_engine_batch_tree_simple.cpp:249-259) ---- */
 /* mcts_node.cpp:296-341: the number of children expand() creates.  The "incremental expansion"

@@ -29,6 +29,8 @@
  *   ref_leaf_keys         src/mcts/mcts_engine_batch_tree_simple.cpp:119-124,133-137 (clone, replay, getHash)
  *   ref_tt_*              call sites src/mcts/mcts_engine_batch_tree_simple.cpp:126,141 and
  *                         src/mcts/phmap_transposition_table.cpp:51-117
+ *   ref_select_redirect_batch  src/mcts/mcts_engine_batch_tree_simple.cpp:88-165 with the table on
+ *                         (redirect :142-156, MCTSNode::updateChildReference src/mcts/mcts_node.cpp:617-630)
  *
  * The node record of include/mcts/mcts_node.h:160-178 is flattened into
  * arrays indexed by node id; the children of a node are the contiguous id
@@ -231,6 +233,15 @@ int ref_tt_insert(ref_tt_slot *slots, int32_t log2_slots, uint64_t key, int32_t 
 /* out_node[i] = node stored under keys[i] with depth >= min_depth, else -1; returns hits */
 int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_t *keys, int64_t n,
                      int32_t min_depth, int32_t *out_node);
+
+/* The traversal loop with the transposition table on, redirects included (see ref_cpu.c): alias[n_nodes]
+ * (-1 = the slot holds its own node) is read and updated; paths [B][max_depth+1], moves [B][max_depth]
+ * (may be NULL); counts[5].  PARITY UNPINNED for the table's arithmetic as above; the loop itself is pinned
+ * by a literal restatement over node objects with children lists (tests/test_oracle_redirect.py). */
+int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots, int32_t B, const ref_params *p,
+                              ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, uint32_t t0, float threshold,
+                              const uint64_t *node_key, int32_t *paths, int32_t *path_len, int32_t *leaf,
+                              int32_t *moves, int32_t *counts);
 
 /* ---- position keys: utils::ZobristHash tables and GomokuState::getHash() of a replayed path ---- */
 typedef struct ref_mt64 {

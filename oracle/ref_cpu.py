@@ -301,6 +301,35 @@ class RefTree:
         assert n >= 0, "sample count does not match the number of children"
         return int(n)
 
+    def select_redirect_batch(self, roots, params, tt, node_key, alias=None):
+        """The traversal loop with the transposition table on, redirects included (see ref_cpu.c).
+        alias (int32 per node, -1 = the slot holds its own node) is updated in place; returns
+        (paths, path_len, leaf, moves, counts) with counts = new entries, replacements, lookups that found
+        an entry, redirects, steps; tt's clock advances by two per step."""
+        roots = np.ascontiguousarray(roots, dtype=np.int32)
+        node_key = np.ascontiguousarray(node_key, dtype=np.uint64)
+        assert len(node_key) == self.n
+        if alias is None:
+            alias = np.full(self.n, -1, np.int32)
+        assert alias.dtype == np.int32 and len(alias) == self.n and alias.flags.c_contiguous
+        B = len(roots)
+        stride = params.max_depth + 1
+        paths = np.empty((B, stride), dtype=np.int32)
+        path_len = np.empty(B, dtype=np.int32)
+        leaf = np.empty(B, dtype=np.int32)
+        moves = np.empty((B, params.max_depth), dtype=np.int32)
+        counts = np.zeros(5, np.int32)
+        fn = lib().ref_select_redirect_batch
+        fn.restype = C.c_int
+        rc = fn(C.byref(self._c), _ptr(alias, i32p), _ptr(roots, i32p), C.c_int32(B), C.byref(params),
+                C.c_void_p(tt.slots.ctypes.data), C.c_void_p(tt.meta.ctypes.data), C.c_int32(tt.log2),
+                C.c_uint32(tt.clock & 0xFFFFFFFF), C.c_float(tt.threshold), _ptr(node_key, u64p), _ptr(paths, i32p),
+                _ptr(path_len, i32p), _ptr(leaf, i32p), _ptr(moves, i32p), _ptr(counts, i32p))
+        if rc != 0:
+            raise ValueError("ref_select_redirect_batch: %d" % rc)
+        tt.clock += 2 * int(counts[4])
+        return paths, path_len, leaf, moves, counts
+
     def gather_actions(self, paths, path_len):
         paths, path_len, B, stride = self._paths_args(paths, path_len)
         out = np.empty((B, stride - 1), dtype=np.int32)

@@ -1,0 +1,145 @@
+"""GPU parity of the traversal loop with the transposition table on, redirects included
+(omk_tt_select_redirect; reference src/mcts/mcts_engine_batch_tree_simple.cpp:88-165, the redirect
+:142-156) against the CPU checker, which tests/test_oracle_redirect.py pins against a literal
+restatement over node objects: paths, leaves, recorded moves, the node every child slot holds, virtual
+loss, visit counts and the table's content bit for bit, search step after search step.  Games: the
+reference's own collision fixture (tests/mcts/transposition_table_test.cpp:15-232, move lists [0, 1]
+and [1, 0] share a key) and a stone-placing game whose key ignores the order of a side's stones."""
+import numpy as np
+import pytest
+
+from oracle import ref_cpu as R
+from tests.test_gpu_tt_policy import same_tables
+from tests.test_oracle_redirect import fixture_tree, stones_tree
+
+pytestmark = pytest.mark.gpu
+
+
+def as_soa(g, rng, rave=False, mask_frac=0.0):
+    n = g["n"]
+    soa = dict(N=np.zeros(n, np.int32), W=np.zeros(n, np.float32), P=g["P"], VL=np.zeros(n, np.int32),
+               child_begin=g["cb"], child_count=g["cc"], action=g["action"], hash=g["keys"])
+    if rave:
+        soa["rN"] = rng.integers(0, 30, n).astype(np.int32)
+        soa["rW"] = (rng.uniform(-1, 1, n) * soa["rN"]).astype(np.float32)
+    if mask_frac:
+        bits = rng.random(n) >= mask_frac
+        bits[0] = True
+        pad = np.zeros((n + 31) // 32 * 32, np.uint8)
+        pad[:n] = bits
+        soa["legal"] = np.packbits(pad.reshape(-1, 32), axis=1, bitorder="little").view("<u4").reshape(-1).copy()
+    return soa
+
+
+def search_both(g, seed, batches, B, vl=3, max_depth=8, rave=False, mask_frac=0.0, log2=12):
+    import omoknuni_small_amd as omk
+    rng = np.random.default_rng(seed)
+    soa = as_soa(g, rng, rave, mask_frac)
+    n = g["n"]
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    tt, ref_tt = omk.TranspositionTable(f, log2), R.RefTT(log2)
+    alias = np.full(n, -1, np.int32)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=300.0)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=300.0, max_depth=max_depth)
+    b = omk.Batch(f, B, max_depth)
+    roots = np.zeros(B, np.int32)
+    total = np.zeros(5, np.int64)
+    for step in range(batches):
+        what = "seed %d step %d" % (seed, step)
+        b.set_roots(roots)
+        moves, counts = tt.select_redirect(b, sp)
+        paths, plen, leaf, _ = b.read()
+        rpaths, rplen, rleaf, rmoves, rcounts = ref.select_redirect_batch(roots, rp, ref_tt, g["keys"], alias)
+        assert (plen == rplen).all(), what
+        assert (paths == rpaths).all() and (leaf == rleaf).all(), what
+        assert (moves == rmoves).all(), what
+        assert counts == tuple(int(x) for x in rcounts), what
+        total += rcounts
+        assert (f.download_redirects() == alias).all(), what
+        assert (f.download()["VL"] == ref.VL).all(), what
+        same_tables(tt, ref_tt, what)
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        b.set_values(values)
+        b.backup(vl)
+        ref.backup_batch(rpaths, rplen, values, vl)
+        dev = f.download()
+        assert (dev["N"] == ref.N).all() and (dev["VL"] == ref.VL).all(), what
+        # the device adds a node's values of one step in another order than the serial loop
+        assert np.allclose(dev["W"], ref.W, rtol=0, atol=1e-5 * max(1.0, np.sqrt(B))), what
+        ref.W[:] = dev["W"]
+    return f, ref, alias, total, (b, sp, tt)
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_collision_fixture_of_the_reference(seed):
+    g = fixture_tree(np.random.default_rng(seed))
+    f, ref, alias, total, _ = search_both(g, seed, batches=12, B=8)
+    assert total[3] >= 1 and (alias >= 0).any()
+
+
+@pytest.mark.parametrize("seed,vl,rave,mask", [(11, 3, False, 0.0), (12, 1, True, 0.0), (13, 0, False, 0.0),
+                                               (14, 3, False, 0.25), (15, 2, True, 0.2)])
+def test_stone_game_with_many_transpositions(seed, vl, rave, mask):
+    g = stones_tree(np.random.default_rng(seed), cells=6, plies=4)
+    f, ref, alias, total, _ = search_both(g, seed, batches=20, B=32, vl=vl, max_depth=6, rave=rave, mask_frac=mask)
+    assert total[3] >= 5, total
+
+
+def test_wide_nodes_and_a_depth_bound():
+    # 70 children at the root and 69 under each: more than one round of 64 slots per node; paths cut at 2 steps
+    g = stones_tree(np.random.default_rng(21), cells=70, plies=2)
+    f, ref, alias, total, _ = search_both(g, 21, batches=6, B=96, max_depth=2, log2=14)
+    assert total[4] == 6 * 96 * 2
+    g = stones_tree(np.random.default_rng(22), cells=6, plies=4)
+    search_both(g, 22, batches=8, B=16, max_depth=2)
+
+
+def test_a_redirected_forest_is_a_graph_until_the_next_upload():
+    import omoknuni_small_amd as omk
+    rng = np.random.default_rng(31)
+    g = stones_tree(rng, cells=5, plies=4)
+    f, ref, alias, total, (b, sp, tt) = search_both(g, 31, batches=25, B=16, max_depth=6)
+    assert total[3] > 0
+    # what needs a tree says so
+    b.set_roots(np.zeros(16, np.int32))
+    with pytest.raises(omk.OmkError, match="re-pointed"):
+        b.select(sp)
+    with pytest.raises(omk.OmkError, match="re-pointed"):
+        f.compact(0)
+    # the root's action probabilities count the visits of the nodes its slots hold
+    held = np.where(alias >= 0, alias, np.arange(g["n"])).astype(np.int32)
+    seen = R.RefTree(N=ref.N[held], W=ref.W, P=ref.P, VL=ref.VL, child_begin=g["cb"], child_count=g["cc"],
+                     action=g["action"])
+    for root in [0] + [int(i) for i in np.nonzero(alias >= 0)[0][:3] if g["cc"][i] > 0]:
+        got, k = f.action_probabilities(root, 1.0, 5)
+        want, rk = seen.action_probabilities(root, 1.0, 5)
+        assert k == rk and got.tobytes() == want.tobytes()
+    # an upload brings a tree back
+    soa = as_soa(g, rng)
+    f.upload(soa)
+    assert (f.download_redirects() == -1).all()
+    b.set_roots(np.zeros(16, np.int32))
+    b.select(sp)
+    paths, plen, leaf, _ = b.read()
+    rpaths, rplen, rleaf, _ = R.RefTree.from_soa(soa).select_batch(np.zeros(16, np.int32), R.make_params(max_depth=6))
+    assert (paths == rpaths).all() and (plen == rplen).all()
+
+
+def test_without_position_keys_or_with_widening_it_refuses():
+    import omoknuni_small_amd as omk
+    g = fixture_tree(np.random.default_rng(41))
+    soa = as_soa(g, np.random.default_rng(41))
+    del soa["hash"]
+    f = omk.Forest.from_soa(soa)
+    tt = omk.TranspositionTable(f, 8)
+    b = omk.Batch(f, 4, 4)
+    b.set_roots(np.zeros(4, np.int32))
+    with pytest.raises(omk.OmkError, match="position keys"):
+        tt.select_redirect(b, omk.SelectParams())
+    f2 = omk.Forest.from_soa(as_soa(g, np.random.default_rng(41)))
+    tt2 = omk.TranspositionTable(f2, 8)
+    b2 = omk.Batch(f2, 4, 4)
+    b2.set_roots(np.zeros(4, np.int32))
+    with pytest.raises(omk.OmkError, match="widening"):
+        tt2.select_redirect(b2, omk.SelectParams(pw=True))
