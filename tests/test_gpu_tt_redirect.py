@@ -31,7 +31,7 @@ def as_soa(g, rng, rave=False, mask_frac=0.0):
     return soa
 
 
-def search_both(g, seed, batches, B, vl=3, max_depth=8, rave=False, mask_frac=0.0, log2=12):
+def search_both(g, seed, batches, B, vl=3, max_depth=8, rave=False, mask_frac=0.0, log2=12, roots=None, revert_every=0):
     import omoknuni_small_amd as omk
     rng = np.random.default_rng(seed)
     soa = as_soa(g, rng, rave, mask_frac)
@@ -43,7 +43,7 @@ def search_both(g, seed, batches, B, vl=3, max_depth=8, rave=False, mask_frac=0.
     sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=300.0)
     rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=300.0, max_depth=max_depth)
     b = omk.Batch(f, B, max_depth)
-    roots = np.zeros(B, np.int32)
+    roots = np.zeros(B, np.int32) if roots is None else np.ascontiguousarray(roots, np.int32)
     total = np.zeros(5, np.int64)
     for step in range(batches):
         what = "seed %d step %d" % (seed, step)
@@ -59,6 +59,12 @@ def search_both(g, seed, batches, B, vl=3, max_depth=8, rave=False, mask_frac=0.
         assert (f.download_redirects() == alias).all(), what
         assert (f.download()["VL"] == ref.VL).all(), what
         same_tables(tt, ref_tt, what)
+        if revert_every and step % revert_every == revert_every - 1:
+            # a batch that is given up: the virtual losses come off again, nothing is backed up
+            b.revert_vl(vl)
+            ref.revert_vl_paths(rpaths, rplen, vl)
+            assert (f.download()["VL"] == ref.VL).all(), what
+            continue
         values = rng.uniform(-1, 1, B).astype(np.float32)
         b.set_values(values)
         b.backup(vl)
@@ -93,6 +99,31 @@ def test_wide_nodes_and_a_depth_bound():
     assert total[4] == 6 * 96 * 2
     g = stones_tree(np.random.default_rng(22), cells=6, plies=4)
     search_both(g, 22, batches=8, B=16, max_depth=2)
+
+
+def test_a_transposition_to_an_ancestor_makes_paths_that_loop_up_to_the_depth_bound():
+    # the position three plies down carries the key of the position one ply down (a repetition): once the
+    # latter has visits the former's slot is re-pointed at it, and a path that comes that way goes round
+    # until the depth bound ends it; a node then occurs several times on one path, and the backup counts
+    # every occurrence, as the reference's loop over the path does
+    g = fixture_tree(np.random.default_rng(51))
+    for a, b in (([0, 0, 0], [0]), ([1, 1, 0], [1]), ([0, 1, 1], [0])):
+        g["keys"][g["hist"].index(a)] = g["keys"][g["hist"].index(b)]
+    f, ref, alias, total, _ = search_both(g, 51, batches=14, B=8, max_depth=9)
+    assert total[3] >= 1
+    looped = [int(s) for s in np.nonzero(alias >= 0)[0] if len(g["hist"][alias[s]]) < len(g["hist"][s])]
+    assert looped, alias
+    assert total[4] > 14 * 8 * 4          # paths longer than the game is deep
+
+
+def test_several_roots_positions_without_a_key_and_batches_given_up():
+    rng = np.random.default_rng(61)
+    g = stones_tree(rng, cells=6, plies=4)
+    g["keys"][rng.random(g["n"]) < 0.15] = np.uint64(0xFFFFFFFFFFFFFFFF)      # positions the host never keyed
+    # traversals that start at the root and at two of its children (searches of three positions side by side)
+    roots = np.array([0, 1, 2] * 8, np.int32)
+    f, ref, alias, total, _ = search_both(g, 61, batches=24, B=24, max_depth=5, roots=roots, revert_every=5)
+    assert total[3] >= 3, total
 
 
 def test_a_redirected_forest_is_a_graph_until_the_next_upload():
