@@ -16,6 +16,7 @@ ForestEngine::ForestEngine(InferenceFunction inference_fn, const MCTSSettings &s
 }
 
 ForestEngine::~ForestEngine() {
+    if (d_moves_) omk_dev_free(forest_, d_moves_);
     if (table_) omk_tt_destroy(table_);
     if (batch_) omk_batch_destroy(batch_);
     if (forest_) omk_forest_destroy(forest_);
@@ -57,13 +58,39 @@ void ForestEngine::selectLeafBatch(const std::vector<int32_t> &roots, std::vecto
     p.use_rave = (settings_.use_rave && has_rave_) ? 1 : 0;
     p.rave_k = settings_.rave_constant;
     p.pw = settings_.selection_prior_widening ? 1 : 0;
-    check(omk_select_batch(batch_, &p), "omk_select_batch");
     const int D = settings_.max_depth;
+    const bool follow = followsTranspositions();
+    int stride = 0;
+    if (follow) {
+        ensureTable();
+        omk_batch_dev dev;
+        check(omk_batch_device(batch_, &dev), "omk_batch_device");
+        stride = dev.stride;
+        const int64_t want = (int64_t)D * stride;
+        if (want > d_moves_ints_) {
+            if (d_moves_) check(omk_dev_free(forest_, d_moves_), "omk_dev_free");
+            d_moves_ = nullptr;
+            check(omk_dev_alloc(forest_, want * 4, &d_moves_), "omk_dev_alloc");
+            d_moves_ints_ = want;
+        }
+        check(omk_tt_select_redirect(table_, batch_, &p, (int32_t *)d_moves_, redirect_counts_.data()),
+              "omk_tt_select_redirect");
+    } else {
+        check(omk_select_batch(batch_, &p), "omk_select_batch");
+    }
     h_paths_.resize((size_t)n * (D + 1));
     h_len_.resize((size_t)n);
     h_leaf_.resize((size_t)n);
     h_actions_.resize((size_t)n * D);
     check(omk_batch_read(batch_, h_paths_.data(), h_len_.data(), h_leaf_.data(), h_actions_.data()), "omk_batch_read");
+    if (follow) {
+        // the recorded moves, level-major on the device: row d holds step d + 1 of every traversal
+        h_moves_.resize((size_t)D * stride);
+        check(omk_dev_d2h(forest_, h_moves_.data(), d_moves_, (int64_t)D * stride * 4), "omk_dev_d2h");
+        for (int i = 0; i < n; i++)
+            for (int d = 0; d + 1 < h_len_[(size_t)i]; d++)
+                h_actions_[(size_t)i * D + d] = h_moves_[(size_t)d * stride + i];
+    }
     leaves.clear();
     leaves.resize((size_t)n);
     for (int i = 0; i < n; i++) {
@@ -101,13 +128,16 @@ void ForestEngine::setPositionKeys(const std::vector<int32_t> &nodes, const std:
     check(omk_forest_set_keys(forest_, nodes.data(), keys.data(), (int64_t)nodes.size()), "omk_forest_set_keys");
 }
 
+void ForestEngine::ensureTable() {
+    if (table_) return;
+    // 32 bytes per slot; the largest power of two that fits the configured size, 2^10 .. 2^26 slots
+    int log2 = 10;
+    while (log2 < 26 && (size_t(64) << log2) <= settings_.transposition_table_size_mb * (size_t(1) << 20)) log2++;
+    check(omk_tt_create(forest_, log2, &table_), "omk_tt_create");
+}
+
 std::array<int32_t, 4> ForestEngine::traverseTranspositionTable() {
-    if (!table_) {
-        // 32 bytes per slot; the largest power of two that fits the configured size, 2^10 .. 2^26 slots
-        int log2 = 10;
-        while (log2 < 26 && (size_t(64) << log2) <= settings_.transposition_table_size_mb * (size_t(1) << 20)) log2++;
-        check(omk_tt_create(forest_, log2, &table_), "omk_tt_create");
-    }
+    ensureTable();
     std::array<int32_t, 4> counts{0, 0, 0, 0};
     check(omk_tt_traverse(table_, batch_, nullptr, 0, nullptr, nullptr, nullptr, nullptr, counts.data()), "omk_tt_traverse");
     return counts;
@@ -125,7 +155,8 @@ void ForestEngine::downloadStructure(int64_t n_nodes, int32_t *child_begin, int3
 }
 
 int64_t ForestEngine::expandLeafBatch(const std::vector<std::vector<int>> &legal_moves,
-                                      const std::vector<NetworkOutput> &outputs, int action_space) {
+                                      const std::vector<NetworkOutput> &outputs, int action_space,
+                                      std::vector<int32_t> *first_child) {
     if ((int)legal_moves.size() != last_n_) throw std::runtime_error("expandLeafBatch: one move list per simulation");
     const bool have_policy = outputs.size() == legal_moves.size();
     std::vector<int32_t> begin(legal_moves.size() + 1, 0), moves, pbegin(legal_moves.size() + 1, 0);
@@ -147,8 +178,9 @@ int64_t ForestEngine::expandLeafBatch(const std::vector<std::vector<int>> &legal
     p.progressive_widening_c = settings_.progressive_widening_c;
     p.progressive_widening_k = settings_.progressive_widening_k;
     const int64_t before = nodeCount();
+    if (first_child) first_child->assign(legal_moves.size(), -1);
     check(omk_expand_batch_ex(batch_, begin.data(), moves.data(), with_policy ? pbegin.data() : nullptr,
-                              with_policy ? policy.data() : nullptr, &p, nullptr),
+                              with_policy ? policy.data() : nullptr, &p, first_child ? first_child->data() : nullptr),
           "omk_expand_batch_ex");
     return nodeCount() - before;
 }

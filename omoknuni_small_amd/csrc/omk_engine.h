@@ -56,6 +56,12 @@ struct MCTSSettings {
     // the table of positions (reference :97-98; the slots here are 32 bytes with their policy fields)
     bool use_transposition_table = true;
     size_t transposition_table_size_mb = 128;
+    // Not a field of the reference, whose traversal always follows a transposition it finds (reference
+    // src/mcts/mcts_engine_batch_tree_simple.cpp:142-156).  Off: transpositions are counted and the tree stays a
+    // tree (the fast selection).  On (with use_transposition_table): every batch is selected by the loop that
+    // follows and re-points them as the reference does, one traversal after the other (omk_tt_select_redirect:
+    // exact for the reference run by one thread, microseconds per step).
+    bool follow_transpositions = false;
     // Not in the reference: only the ceil(sqrt(N_parent)) children of highest prior take part in a
     // selection (omk_select_params::pw; needs children stored by descending prior)
     bool selection_prior_widening = false;
@@ -97,8 +103,9 @@ class ForestEngine {
     // output's own policy (by action when it has action_space entries, by child when it has as
     // many as children, uniform otherwise or when empty).  action_space <= 0: the size of the
     // first policy that is not empty.  Returns the nodes added.
+    // first_child (optional): per simulation the id of the first child created from its move list, or -1.
     int64_t expandLeafBatch(const std::vector<std::vector<int>> &legal_moves, const std::vector<NetworkOutput> &outputs,
-                            int action_space = 0);
+                            int action_space = 0, std::vector<int32_t> *first_child = nullptr);
     void setLegalMovesFunction(LegalMovesFunction fn) { legal_moves_fn_ = std::move(fn); }
     // SearchResult.probabilities (reference MCTSEngine::getActionProbabilities,
     // src/mcts/mcts_engine_tree.cpp:388-465): visit counts of root's children, temperature.
@@ -116,6 +123,13 @@ class ForestEngine {
     // up, transpositions counted (never followed).  The table is created on first use with about
     // settings.transposition_table_size_mb.  Returns {new entries, replacements, duplicates, transpositions}.
     std::array<int32_t, 4> traverseTranspositionTable();
+    // With settings.follow_transpositions the selection itself is the loop with the table (reference :88-165):
+    // what the last selectLeafBatch counted, {new entries, replacements, lookups that found an entry, redirects,
+    // steps}.  The leaves' move_sequence is then the list of RECORDED moves (the action of the node each selected
+    // slot held), which is what the reference replays; it differs from the actions of the path's nodes at a
+    // step that redirected.
+    std::array<int32_t, 5> lastRedirectCounts() const { return redirect_counts_; }
+    bool followsTranspositions() const { return settings_.use_transposition_table && settings_.follow_transpositions; }
     int64_t nodeCount() const;
     void downloadStructure(int64_t n_nodes, int32_t *child_begin, int32_t *child_count, int32_t *action);
 
@@ -129,6 +143,7 @@ class ForestEngine {
    private:
     void check(int status, const char *what) const;
     void ensureBatch(int n);
+    void ensureTable();
 
     InferenceFunction inference_fn_;
     LegalMovesFunction legal_moves_fn_;
@@ -139,7 +154,10 @@ class ForestEngine {
     int batch_capacity_ = 0;
     int last_n_ = 0;
     bool has_rave_ = false;
-    std::vector<int32_t> h_paths_, h_len_, h_leaf_, h_actions_, h_roots_;
+    std::vector<int32_t> h_paths_, h_len_, h_leaf_, h_actions_, h_roots_, h_moves_;
+    void *d_moves_ = nullptr;  // recorded moves of the last selection that followed transpositions
+    int64_t d_moves_ints_ = 0;
+    std::array<int32_t, 5> redirect_counts_{0, 0, 0, 0, 0};
 };
 
 }  // namespace omk

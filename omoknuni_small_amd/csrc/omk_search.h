@@ -43,7 +43,8 @@ struct SearchResult {
     int64_t nodes = 0;
     // the table of positions over the whole search (settings.use_transposition_table): entries stored,
     // and lookups that found ANOTHER visited node for the position reached: what the reference would
-    // redirect to (src/mcts/mcts_engine_batch_tree_simple.cpp:141-157); counted, never followed
+    // redirect to (src/mcts/mcts_engine_batch_tree_simple.cpp:141-157): counted, and followed only with
+    // settings.follow_transpositions (then `transpositions` counts the redirects made)
     int64_t table_entries = 0, transpositions = 0;
 };
 
@@ -188,6 +189,10 @@ class GPUForestMCTSEngine {
         v.legal = nullptr;
         v.hash = nullptr;
         engine_.uploadTree(v);
+        if constexpr (detail::has_hash<State>::value) {
+            // the loop that follows transpositions goes by the nodes' own keys: the root's is the first
+            if (engine_.followsTranspositions()) engine_.setPositionKeys({0}, {(uint64_t)state.getHash()});
+        }
 
         std::vector<StatePtr> states;
         std::vector<float> values;
@@ -203,8 +208,16 @@ class GPUForestMCTSEngine {
             states.clear();
             states.reserve(pending.size());
             for (auto &pe : pending) states.push_back(std::move(pe.state));
+            bool follow = false;
+            if constexpr (detail::has_hash<State>::value) follow = engine_.followsTranspositions();
+            if (follow) {
+                // the selection was the loop with the table itself (store, lookup, redirect)
+                const std::array<int32_t, 5> c = engine_.lastRedirectCounts();
+                result.table_entries += c[0];
+                result.transpositions += c[3];
+            }
             if constexpr (detail::has_hash<State>::value) {
-                if (st.use_transposition_table) {
+                if (st.use_transposition_table && !follow) {
                     // the keys of the positions reached, from the game itself, then the table's part of the
                     // traversal (:116-162) over the paths just selected
                     key_nodes_.clear();
@@ -236,7 +249,10 @@ class GPUForestMCTSEngine {
                 if (st.shuffle_moves) shuffleMoves(legal[i]);
                 values[i] = out[i].value;
             }
-            engine_.expandLeafBatch(legal, out, action_space);  // phase 3, first half (:249-259)
+            engine_.expandLeafBatch(legal, out, action_space, follow ? &first_child_ : nullptr);  // phase 3, first half (:249-259)
+            if constexpr (detail::has_hash<State>::value) {
+                if (follow) keyNewChildren(states, legal);
+            }
             if (!root_expanded) {
                 root_expanded = true;
                 if (st.add_dirichlet_noise) addDirichletNoise();
@@ -295,6 +311,32 @@ class GPUForestMCTSEngine {
     }
 
    private:
+    // The loop that follows transpositions stores a child under the key of its position the first time the
+    // child is selected (reference :116-128), and gets that key by replaying the moves on a clone of the root
+    // state.  With the tree on the device the key has to be there before the selection: every child created by
+    // this batch's expansions is keyed now, from the leaf state the host already holds (one clone + makeMove +
+    // getHash per child).  The children of a leaf are the first of its move list, in that order; new ids are
+    // handed out in simulation order, so a leaf's children end where the next expanded leaf's begin.
+    void keyNewChildren(const std::vector<StatePtr> &states, const std::vector<std::vector<int>> &legal) {
+        key_nodes_.clear();
+        key_values_.clear();
+        const int64_t n_after = engine_.nodeCount();
+        for (size_t i = 0; i < states.size(); i++) {
+            const int32_t first = first_child_[i];
+            if (first < 0) continue;
+            int64_t end = n_after;
+            for (size_t j = 0; j < states.size(); j++)
+                if (first_child_[j] > first && first_child_[j] < end) end = first_child_[j];
+            for (int64_t c = first; c < end; c++) {
+                StatePtr s = states[i]->clone();
+                s->makeMove(legal[i][(size_t)(c - first)]);
+                key_nodes_.push_back((int32_t)c);
+                key_values_.push_back((uint64_t)s->getHash());
+            }
+        }
+        if (!key_nodes_.empty()) engine_.setPositionKeys(key_nodes_, key_values_);
+    }
+
     // Fisher-Yates from the last place down, one raw 32-bit output of the generator per place
     // (j = output mod (k + 1)): spelled out rather than std::shuffle, whose use of the generator is
     // the standard library's own, so that a test can restate it
@@ -343,7 +385,7 @@ class GPUForestMCTSEngine {
     std::mt19937 random_engine_;
     std::mt19937 shuffle_engine_;  // its own stream: noise and the move drawn do not depend on the tree's size
     std::vector<LeafItem> leaves_;
-    std::vector<int32_t> key_nodes_;
+    std::vector<int32_t> key_nodes_, first_child_;
     std::vector<uint64_t> key_values_;
 };
 

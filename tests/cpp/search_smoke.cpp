@@ -93,7 +93,7 @@ struct RefNetworkOutput {
     float value = 0.0f;
 };
 
-static int run_search(int sims, int batch, bool widening, bool noise, float temperature, int searches) {
+static int run_search(int sims, int batch, bool widening, bool noise, float temperature, int searches, bool follow) {
     omk::MCTSSettings s;
     s.num_simulations = sims;
     s.batch_size = batch;
@@ -103,6 +103,7 @@ static int run_search(int sims, int batch, bool widening, bool noise, float temp
     s.temperature = temperature;
     s.max_depth = 16;
     s.transposition_table_size_mb = 1;  // 2^15 slots
+    s.follow_transpositions = follow;
     using Engine = omk::GPUForestMCTSEngine<RingState, RefNetworkOutput>;
     long evaluated = 0;
     Engine::InferenceFunction evaluator = [&](const std::vector<std::unique_ptr<RingState>> &states) {
@@ -232,7 +233,7 @@ int main(int argc, char **argv) {
     try {
         if (argc >= 7 && !strcmp(argv[1], "search"))
             return run_search(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]) != 0, atoi(argv[5]) != 0, (float)atof(argv[6]),
-                              argc >= 8 ? atoi(argv[7]) : 1);
+                              argc >= 8 ? atoi(argv[7]) : 1, argc >= 9 && atoi(argv[8]) != 0);
         if (argc >= 2 && !strcmp(argv[1], "flatten")) return run_flatten();
     } catch (const std::exception &e) {
         fprintf(stderr, "search_smoke: %s\n", e.what());

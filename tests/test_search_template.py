@@ -78,17 +78,17 @@ def shuffle_moves(moves, gen):
     return moves
 
 
-def replay_search(sims, batch, widening, seed=5489, searches=1):
+def replay_search(sims, batch, widening, seed=5489, searches=1, follow=False):
     """`searches` searches one after the other on one engine (the generator of the shuffles runs on, the
     tree and the table of positions start empty every time: a table entry dies with the tree its node
     belongs to); the last one is returned."""
     gen = Mt19937(seed + 1)
     for _ in range(searches):
-        ref = replay_one_search(sims, batch, widening, gen)
+        ref = replay_one_search(sims, batch, widening, gen, follow)
     return ref
 
 
-def replay_one_search(sims, batch, widening, gen):
+def replay_one_search(sims, batch, widening, gen, follow=False):
     root_state = Ring()
     root_state.make(3)
     z = np.zeros(1, np.int32)
@@ -101,12 +101,23 @@ def replay_one_search(sims, batch, widening, gen):
     no_key = np.uint64(0xFFFFFFFFFFFFFFFF)
     entries = transpositions = 0
     done, first = 0, True
+    # settings.follow_transpositions: the selection is the loop with the table, redirects included; every node
+    # has its key from the moment it is created (keyNewChildren), and slots get re-pointed (alias)
+    keys, alias = np.full(1, no_key, np.uint64), np.full(1, -1, np.int32)
     while done < sims:
         n = 1 if first else min(batch, sims - done)
         first = False
         roots = np.zeros(n, np.int32)
-        paths, plen, leaf, _ = ref.select_batch(roots, rp)
-        acts = ref.gather_actions(paths, plen)
+        if follow:
+            grow = ref.n - len(keys)
+            keys = np.concatenate([keys, np.full(grow, no_key, np.uint64)])
+            alias = np.concatenate([alias, np.full(grow, -1, np.int32)])
+            paths, plen, leaf, acts, counts = ref.select_redirect_batch(roots, rp, table, keys, alias)
+            entries += int(counts[0])
+            transpositions += int(counts[3])
+        else:
+            paths, plen, leaf, _ = ref.select_batch(roots, rp)
+            acts = ref.gather_actions(paths, plen)
         begin, moves, pb, pol, values = [0], [], [0], [], []
         states = []
         for t in range(n):
@@ -115,11 +126,12 @@ def replay_one_search(sims, batch, widening, gen):
                 s.make(int(a))
             states.append(s)
             key_of[int(leaf[t])] = np.uint64(s.hash())
-        step_keys = np.array([[key_of.get(int(paths[t, d]), no_key) if d < plen[t] else no_key
-                               for d in range(1, paths.shape[1])] for t in range(n)], np.uint64).reshape(n, -1)
-        _, counts = table.traverse(ref, paths, plen, step_keys)
-        entries += counts[0]
-        transpositions += counts[3]
+        if not follow:
+            step_keys = np.array([[key_of.get(int(paths[t, d]), no_key) if d < plen[t] else no_key
+                                   for d in range(1, paths.shape[1])] for t in range(n)], np.uint64).reshape(n, -1)
+            _, counts = table.traverse(ref, paths, plen, step_keys)
+            entries += counts[0]
+            transpositions += counts[3]
         for t in range(n):
             s = states[t]
             v, p = evaluate(s)
@@ -129,11 +141,23 @@ def replay_one_search(sims, batch, widening, gen):
             begin.append(len(moves))
             pol.extend(p.tolist())
             pb.append(len(pol))
-        ref.expand_batch(leaf, begin, np.array(moves if moves else [0], np.int32), policy=np.array(pol, np.float32),
-                         action_space=CELLS, policy_begin=pb, widening=(2.0, 0.5) if widening else None)
+        first_child = ref.expand_batch(leaf, begin, np.array(moves if moves else [0], np.int32),
+                                       policy=np.array(pol, np.float32), action_space=CELLS, policy_begin=pb,
+                                       widening=(2.0, 0.5) if widening else None)
+        if follow:
+            grow = ref.n - len(keys)
+            keys = np.concatenate([keys, np.full(grow, no_key, np.uint64)])
+            alias = np.concatenate([alias, np.full(grow, -1, np.int32)])
+            for t in range(n):
+                if first_child[t] >= 0:
+                    for j in range(int(ref.child_count[leaf[t]])):
+                        s = states[t].clone()
+                        s.make(int(moves[begin[t] + j]))
+                        keys[first_child[t] + j] = np.uint64(s.hash())
         ref.backup_batch(paths, plen, np.array(values, np.float32), 3)
         done += n
     ref.table_counts = (entries, transpositions)
+    ref.alias = alias
     return ref
 
 
@@ -176,6 +200,39 @@ def test_search_with_the_reference_signatures_matches_the_checker(widening):
         assert ref.child_count[0] == 11
     # a terminal state is answered without a search: the side to move has lost
     assert lines[-1] == "terminal action -1 value -1 probabilities 12"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("widening", [0, 1])
+def test_search_that_follows_transpositions_matches_the_checker(widening):
+    """settings.follow_transpositions: every batch is selected by the loop that stores, looks up and REDIRECTS
+    (reference mcts_engine_batch_tree_simple.cpp:88-165), every new child keyed by the game's own hash when it
+    is created; the mock game's key does not depend on the order of the moves, so transpositions abound.  The
+    whole search replayed through the checker: every node, the redirects counted, the move probabilities."""
+    sims, batch = 300, 16
+    r = subprocess.run([EXE, "search", str(sims), str(batch), str(widening), "0", "0", "1", "1"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().split("\n")
+    head = lines[0].split()
+    probs = np.array([float(x) for x in next(ln for ln in lines if ln.startswith("probabilities")).split()[1:]], np.float32)
+    table = next(ln for ln in lines if ln.startswith("table entries")).split()
+    nodes = np.array([[float(x) for x in ln.split()[2:]] for ln in lines if ln.startswith("node ")])
+    ref = replay_search(sims, batch, widening, follow=True)
+    assert (int(table[2]), int(table[4])) == ref.table_counts, (table, ref.table_counts)
+    assert ref.table_counts[1] > 0 and (ref.alias >= 0).any()          # slots were re-pointed
+    assert int(head[7]) == ref.n == len(nodes)
+    assert (nodes[:, 0] == ref.N).all() and (nodes[:, 3] == ref.VL).all()
+    assert (nodes[:, 4] == ref.child_begin).all() and (nodes[:, 5] == ref.child_count).all()
+    assert (nodes[:, 6] == ref.action).all()
+    assert np.abs(nodes[:, 1] - ref.W).max() <= 1e-5 * max(1.0, np.abs(ref.W).max())
+    assert ref.N[0] == sims
+    # the probabilities count the visits of the nodes the root's slots hold
+    held = np.where(ref.alias >= 0, ref.alias, np.arange(ref.n)).astype(np.int32)
+    seen = R.RefTree(N=ref.N[held], W=ref.W, P=ref.P, VL=ref.VL, child_begin=ref.child_begin, child_count=ref.child_count,
+                     action=ref.action)
+    want, children = seen.action_probabilities(0, 0.0, CELLS)
+    assert children == ref.child_count[0] and (probs == want).all()
 
 
 @pytest.mark.gpu
