@@ -426,7 +426,13 @@ def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parit
     # single-visitor kernel; the roofline is quoted for the kernel that carries the work, with the
     # whole selection phase (HIP events around it on the forest's stream) as its launch duration
     has_groups = len(np.unique(troots)) < B
-    dominant = "k_select_groups" if has_groups else "k_select_singles"
+    # (the library walks a small batch of lone traversals on a wide layout with a legal mask by blocks, one round
+    # of 64 child slots per wavefront: the same rule as its launch code)
+    fan = int(np.max(soa["child_count"]))
+    rounds = 1 if fan <= 64 else 4 if fan <= 256 else 6 if fan <= 384 else 16
+    singles = ("k_select_singles_team" if rounds > 1 and soa.get("legal") is not None and B * rounds <= 4096
+               else "k_select_singles")
+    dominant = "k_select_groups" if has_groups else singles
     sel_ms_step = sel_ms / K
     bak_ms_step = bak_ms / K
     achieved_timed = sel_bytes / (sel_ms * 1e-3) / 1e9
@@ -473,7 +479,7 @@ def measure(omk, synth, name, steps, warmup, seed, cpu_seconds, scale=1.0, parit
             "launch_covers": "the whole selection, HIP events around it on the forest's stream: " +
                              ("k_select_reset + k_select_groups (teams and walkers in one persistent launch)"
                               if has_groups else
-                              "k_select_singles alone (no reset launch when every traversal is alone at its root)")
+                              singles + " alone (no reset launch when every traversal is alone at its root)")
                              + "; rocprofv3's per-kernel averages add up to it",
             # the same figures over the K timed steps, whose statistics drift with every backup (they depend on
             # --steps / --warmup; kept as information)
