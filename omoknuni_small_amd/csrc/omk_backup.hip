@@ -793,6 +793,28 @@ __device__ __forceinline__ int pick_slot_redirected(const ForestDev &f, const in
     return idx == 0xFFFFFFFFu ? -1 : cb + (int)idx;
 }
 
+// The winning slot of one round of candidates (see pick_slot_redirected): index among the slots, or ~0.
+__device__ __forceinline__ uint32_t pick_of_round(uint32_t b1, uint32_t p1, uint32_t b2, uint32_t p2, uint32_t fn,
+                                                 uint32_t fi) {
+    const uint32_t m1 = wave_max_u32(b1);
+    if (m1 != 0u) {
+        const uint32_t m2 = wave_max_u32(b2);
+        if (m2 > m1) return wave_min_u32(b2 == m2 ? p2 : 0xFFFFFFFFu);
+        return wave_min_u32(b1 == m1 ? p1 : 0xFFFFFFFFu);
+    }
+    const uint32_t gm = wave_min_u32(fn);
+    return wave_min_u32(fn == gm ? fi : 0xFFFFFFFFu);
+}
+
+// A step is a chain of dependent trips to memory and nothing overlaps them, so the walk asks for as much as it
+// can in one trip.  A node of at most 64 slots (one per lane): alias, legality word, statistics, action, position
+// key and child range of every slot come together, read as if no slot were re-pointed; the few lanes whose slot
+// IS re-pointed read their node's again.  What the step needs next is then in registers: the chosen node's
+// visit count (the next node's N_parent, and the store's "no visits yet"), its action, its child range, and,
+// while the recorded moves still lead along the nodes walked (shadow == cur), the key of the position reached,
+// which is the key of the slot that carries the recorded move.  Two dependent trips a step are left: the
+// children, then the table's slot.  Wider nodes and paths whose recorded moves have left the nodes walked take
+// the plain sequence of loads.
 template <bool RAVE>
 __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, RedirectArgs a) {
     const int lane = threadIdx.x;
@@ -803,10 +825,91 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
         int cur = a.paths[t];
         int shadow = cur;
         int d = 0;
+        int2 sp = f.span[cur];
+        int np = f.N[cur];
         for (;;) {
-            const int2 sp = f.span[cur];
-            int slot = -1;
-            if (sp.y > 0 && d < a.max_depth) slot = pick_slot_redirected<RAVE>(f, a.alias, cur, sp.x, sp.y, a.c_puct, a.rave_k, lane);
+            int slot = -1, best = -1, nbest = 0, move = 0, shadow_next = -1;
+            int2 nsp = int2{0, 0};
+            unsigned long long key = kTTEmpty;
+            bool key_known = false;
+            if (sp.y > 0 && d < a.max_depth) {
+                if (sp.y <= kWave) {
+                    const int s = sp.x + lane;
+                    const bool in_range = lane < sp.y;
+                    uint32_t word = 0xFFFFFFFFu;
+                    int al = -1, n = 0, vl = 0, act = s, rn = 0;
+                    float w = 0.0f, p = 0.0f, rw = 0.0f;
+                    int2 csp = int2{0, 0};
+                    unsigned long long hk = kTTEmpty;
+                    if (in_range) {
+                        if (f.legal) word = f.legal[(uint32_t)s >> 5];
+                        al = ld_agent(a.alias + s);
+                        n = f.N[s];
+                        w = f.W[s];
+                        p = f.P[s];
+                        vl = ld_agent(f.VL + s);
+                        if (f.action) act = f.action[s];
+                        hk = f.hash[s];
+                        csp = f.span[s];
+                        if (RAVE) {
+                            rn = f.rN[s];
+                            rw = f.rW[s];
+                        }
+                    }
+                    const bool in = in_range && ((word >> ((uint32_t)s & 31u)) & 1u);
+                    const int act_slot = act;  // the move this slot stands for in the tree as uploaded
+                    int held = s;
+                    if (in && al >= 0) {  // a re-pointed slot: the node it holds
+                        held = al;
+                        n = f.N[held];
+                        w = f.W[held];
+                        p = f.P[held];
+                        vl = ld_agent(f.VL + held);
+                        act = f.action ? f.action[held] : held;
+                        csp = f.span[held];
+                        if (RAVE) {
+                            rn = f.rN[held];
+                            rw = f.rW[held];
+                        }
+                    }
+                    uint32_t k1 = 0u, k2 = 0u, on = 0xFFFFFFFFu;
+                    if (in) {
+                        const float q2 = RAVE ? combined_value(n, w, rn, rw, a.rave_k) : 0.0f;
+                        child_keys<RAVE>(n, w, p, vl, q2, a.c_puct * sqrtf((float)np), k1, k2);
+                        on = (uint32_t)n ^ 0x80000000u;
+                    }
+                    const uint32_t idx = pick_of_round(k1, (uint32_t)lane, k2, (uint32_t)lane, on, in ? (uint32_t)lane : 0xFFFFFFFFu);
+                    if (idx != 0xFFFFFFFFu) {
+                        const int L = (int)idx;
+                        slot = sp.x + L;
+                        best = __builtin_amdgcn_readlane(held, L);
+                        nbest = __builtin_amdgcn_readlane(n, L);
+                        move = __builtin_amdgcn_readlane(act, L);
+                        nsp.x = __builtin_amdgcn_readlane(csp.x, L);
+                        nsp.y = __builtin_amdgcn_readlane(csp.y, L);
+                        if (shadow == cur) {
+                            const unsigned long long any = __ballot(in && act_slot == move);
+                            if (any) {
+                                const int l2 = __ffsll((long long)any) - 1;
+                                shadow_next = sp.x + l2;
+                                const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)hk, l2);
+                                const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(hk >> 32), l2);
+                                key = ((unsigned long long)hi << 32) | lo;
+                            }
+                            key_known = true;
+                        }
+                    }
+                } else {
+                    slot = pick_slot_redirected<RAVE>(f, a.alias, cur, sp.x, sp.y, a.c_puct, a.rave_k, lane);
+                    if (slot >= 0) {
+                        const int al = ld_agent(a.alias + slot);
+                        best = al >= 0 ? al : slot;
+                        nbest = f.N[best];
+                        move = f.action ? f.action[best] : best;
+                        nsp = f.span[best];
+                    }
+                }
+            }
             if (slot < 0) {
                 if (lane == 0) {
                     a.leaf[t] = cur;
@@ -815,22 +918,20 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
                 if (sp.y > 0 && d >= a.max_depth) n_trunc++;
                 break;
             }
-            const int al = ld_agent(a.alias + slot);
-            int best = al >= 0 ? al : slot;
-            const int move = f.action ? f.action[best] : best;
-            if (shadow >= 0) {
-                const int2 ss = f.span[shadow];
-                int next = -1;
-                for (int base = 0; base < ss.y && next < 0; base += kWave) {
-                    const int i = base + lane;
-                    const int s = ss.x + i;
-                    const bool hit = i < ss.y && slot_legal(f, s) && (f.action ? f.action[s] : s) == move;
-                    const unsigned long long any = __ballot(hit);
-                    if (any) next = ss.x + base + (__ffsll((long long)any) - 1);
+            if (!key_known) {
+                if (shadow >= 0) {
+                    const int2 ss = f.span[shadow];
+                    for (int base = 0; base < ss.y && shadow_next < 0; base += kWave) {
+                        const int i = base + lane;
+                        const int s = ss.x + i;
+                        const bool hit = i < ss.y && slot_legal(f, s) && (f.action ? f.action[s] : s) == move;
+                        const unsigned long long any = __ballot(hit);
+                        if (any) shadow_next = ss.x + base + (__ffsll((long long)any) - 1);
+                    }
                 }
-                shadow = next;
+                if (shadow_next >= 0) key = f.hash[shadow_next];
             }
-            const unsigned long long key = shadow >= 0 ? f.hash[shadow] : kTTEmpty;
+            int redirected = 0;
             if (lane == 0) {
                 if (a.vl > 0) atomicAdd(f.VL + best, a.vl);                       // :109
                 if (a.moves) a.moves[(size_t)d * a.stride + t] = move;            // :112
@@ -843,8 +944,7 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
                     }
                     const bool room = probe <= mask;
                     const bool present = room && a.slots[s].key == key;
-                    const int nv = f.N[best];
-                    if (nv == 0) {                                                // :116-128, store()
+                    if (nbest == 0) {                                             // :116-128, store()
                         if (!room) {
                             n_full++;
                         } else {
@@ -887,14 +987,25 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
                         // holding one node score alike, and the first of equals is selected)
                         __hip_atomic_store(a.alias + slot, found, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         best = found;
+                        redirected = 1;
                         n_redirect++;
                     }
                 }
                 a.paths[(size_t)(d + 1) * a.stride + t] = best;
             }
             best = __builtin_amdgcn_readfirstlane(best);
-            __threadfence();  // what lane 0 wrote is what every lane reads from here on
+            redirected = __builtin_amdgcn_readfirstlane(redirected);
+            // what lane 0 wrote is what every lane reads from here on: one wavefront, whose accesses to an address
+            // reach the cache in program order; virtual loss and aliases are read past the first-level cache
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            if (redirected) {
+                nsp = f.span[best];
+                nbest = f.N[best];
+            }
             cur = best;
+            sp = nsp;
+            np = nbest;
+            shadow = shadow_next;
             d++;
             g++;
         }
