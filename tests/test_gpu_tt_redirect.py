@@ -101,6 +101,19 @@ def test_wide_nodes_and_a_depth_bound():
     search_both(g, 22, batches=8, B=16, max_depth=2)
 
 
+def test_wide_nodes_with_transpositions():
+    # the same wide tree with the positions [a, b] and [b, a] given one key: slots of nodes of more than 64
+    # slots get re-pointed, and later selections read through them (the walk's path for wide nodes)
+    g = stones_tree(np.random.default_rng(23), cells=70, plies=2)
+    at = {tuple(h): i for i, h in enumerate(g["hist"])}
+    for (x, y), i in [(k, v) for k, v in at.items() if len(k) == 2]:
+        if x > y:
+            g["keys"][i] = g["keys"][at[(y, x)]]
+    f, ref, alias, total, _ = search_both(g, 23, batches=14, B=128, max_depth=2, log2=14)
+    assert total[3] >= 10, total
+    assert (alias >= 0).sum() >= 10
+
+
 def test_a_transposition_to_an_ancestor_makes_paths_that_loop_up_to_the_depth_bound():
     # the position three plies down carries the key of the position one ply down (a repetition): once the
     # latter has visits the former's slot is re-pointed at it, and a path that comes that way goes round
