@@ -941,6 +941,10 @@ int omk_batch_create(omk_forest *f, int32_t max_traversals, int32_t max_depth, o
     // a second context for its partition)
     b->hctx_cap = (int32_t)std::min<int64_t>(4096, 2 * (B / kHeavyMin) * (max_depth + 1));
     if (e == hipSuccess) e = dalloc(&b->hctx, (int64_t)b->hctx_cap * kHeavyCtxInts);
+    // (a context says by the number of the select call that its children's contexts are listed: memory that an
+    // earlier batch left behind would say so for this batch's first calls, whose numbers start again at 1)
+    if (e == hipSuccess)
+        e = hipMemset(b->hctx, 0, (size_t)std::max<int64_t>((int64_t)b->hctx_cap * kHeavyCtxInts, 1) * 4);
     if (e == hipSuccess) e = dalloc(&b->hbound, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts);
     if (e == hipSuccess)
         e = hipMemset(b->hbound, 0, (size_t)std::max<int64_t>((int64_t)b->hctx_cap * kMaxSlices * kBoundInts, 1) * 4);
@@ -1092,6 +1096,7 @@ static int next_epoch(omk_batch *b) {
         HIP_TRY(launch_fill_words(b->q_ready, 0u, b->q_cap, f->stream));
         HIP_TRY(launch_fill_words(b->single_ready, 0u, b->max_traversals, f->stream));
         HIP_TRY(launch_fill_words(b->hbound, 0u, (int64_t)b->hctx_cap * kMaxSlices * kBoundInts, f->stream));
+        HIP_TRY(launch_fill_words(b->hctx, 0u, (int64_t)b->hctx_cap * kHeavyCtxInts, f->stream));
         // the two depth-cap counters take turns by call parity, which this restart breaks once
         HIP_TRY(launch_fill_words(b->counters + kTruncatedWord, 0u, 2, f->stream));
         b->epoch = 0;

@@ -12,7 +12,10 @@ from tests.test_gpu_scheduler import chain_forest, layered_forest, select_both
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+# (seed 6: its 58th forest once lost a visitor, because the contexts of heavy nodes of a NEW batch were memory an
+# earlier batch of the process had left behind, and a context says by the number of the select call, which
+# starts again at 1 with every batch, that the contexts of its children are listed)
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 6])
 def test_random_forests_and_crowds(seed):
     rng = np.random.default_rng(seed)
     replayed = []
