@@ -4380,7 +4380,7 @@ hipError_t launch_select(const ForestDev &f, const SelectArgs &a, int n_items0, 
     // own leaf and path length, so nothing has to be cleared first (the statistics apart).
     // Otherwise the reset launch.
     const bool alone = n_items0 == 0 && n_singles0 == n_traversals;
-    if (!alone || a.stats) {
+    if (!alone || a.stats || a.trace) {  // (the statistics and the timeline start at zero)
         int reset_blocks = (n_traversals + 255) / 256;
         hipLaunchKernelGGL(k_select_reset, dim3(reset_blocks), dim3(256), 0, s, a, n_items0, n_singles0,
                            n_traversals - n_singles0, n_traversals, n_hctx0);
