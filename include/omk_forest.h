@@ -230,7 +230,8 @@ int omk_forest_compact_static(omk_forest *f, int32_t new_root, int64_t *h_nodes_
  * h_moves[h_move_begin[t] .. h_move_begin[t+1]) of its leaf state (the state it replayed from
  * omk_batch_read); an empty list means a terminal state, the node stays a leaf.  A leaf
  * reached by several simulations is expanded once, with the list of the first of them in
- * index order that offers moves; a node that already has children is left alone; at most
+ * index order that offers moves; a node that already has children (the selection stopped at it
+ * because of the depth bound) is left alone and takes no ids; at most
  * 1000 moves are used (the reference's limit).  One child per move in the order given (the
  * reference shuffles with a random seed: every order is one of its outcomes), zero
  * statistics, action = the move.  Priors: h_policy NULL -> 1 / children (expand's uniform

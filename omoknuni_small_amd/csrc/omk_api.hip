@@ -1300,24 +1300,39 @@ int omk_expand_batch_ex(omk_batch *b, const int32_t *h_move_begin, const int32_t
         for (size_t i = 0; i < order.size(); i++)
             if (i == 0 || order[i].first != order[i - 1].first) winners.push_back(order[i].second);
         std::sort(winners.begin(), winners.end());  // ids are handed out in traversal order
-        // progressive widening reads the visit count of every leaf that is about to be expanded
+        // A leaf that has children already (the selection stopped at it because of the depth bound) is left alone
+        // and takes no ids: its child range is read first.  Progressive widening reads the visit count of every
+        // leaf that is about to be expanded: it comes in the same trip.
         std::vector<int32_t> visits(winners.size(), 0);
-        if (params->use_progressive_widening && !winners.empty()) {
+        if (!winners.empty()) {
             const size_t nw = winners.size();
-            if (nw * 8 > b->exp_bytes) {
+            if (nw * 16 > b->exp_bytes) {
                 if (b->exp_buf) HIP_TRY(hipFree(b->exp_buf));
                 b->exp_buf = nullptr;
                 b->exp_bytes = 0;
-                HIP_TRY(hipMalloc(&b->exp_buf, nw * 16));
-                b->exp_bytes = nw * 16;
+                HIP_TRY(hipMalloc(&b->exp_buf, nw * 32));
+                b->exp_bytes = nw * 32;
             }
             std::vector<int32_t> ids(nw);
+            std::vector<int2> spans(nw);
             for (size_t i = 0; i < nw; i++) ids[i] = leaf[(size_t)winners[i]];
             int32_t *d_ids = (int32_t *)b->exp_buf, *d_n = d_ids + nw;
+            uint64_t *d_span = (uint64_t *)(d_ids + 2 * nw);
             HIP_TRY(hipMemcpyAsync(d_ids, ids.data(), nw * 4, hipMemcpyHostToDevice, s));
             HIP_TRY(launch_gather_words((uint32_t *)d_n, (const uint32_t *)f->N, d_ids, (int64_t)nw, s));
+            HIP_TRY(launch_gather_dwords(d_span, (const uint64_t *)f->span, d_ids, (int64_t)nw, s));
             HIP_TRY(hipMemcpyAsync(visits.data(), d_n, nw * 4, hipMemcpyDeviceToHost, s));
+            HIP_TRY(hipMemcpyAsync(spans.data(), d_span, nw * 8, hipMemcpyDeviceToHost, s));
             HIP_TRY(hipStreamSynchronize(s));
+            size_t kept = 0;
+            for (size_t i = 0; i < nw; i++) {
+                if (spans[i].y != 0) continue;
+                winners[kept] = winners[i];
+                visits[kept] = visits[i];
+                kept++;
+            }
+            winners.resize(kept);
+            visits.resize(kept);
         }
         int64_t cursor = f->n_nodes;
         bool sorted = true;

@@ -185,9 +185,10 @@ __global__ void k_expand_mask(uint32_t *legal, int64_t old_nodes, int64_t new_no
 }
 
 // One wavefront per leaf.  The children are written first, the leaf's child range last: a
-// node is a leaf exactly while its child count is 0.  A leaf that already has children
-// (the selection stopped at it because of the depth bound) is left alone; the ids reserved
-// for it become unreachable nodes with zero statistics.
+// node is a leaf exactly while its child count is 0.  The host offers no job for a leaf that
+// already has children (the selection stopped at it because of the depth bound: it reads the
+// child ranges first, so that such a leaf takes no ids); should one come all the same it is left
+// alone.
 __global__ __launch_bounds__(64) void k_expand(ForestMut f, const ExpandJob *jobs, int n_jobs, const int32_t *moves,
                                                const float *priors, int32_t *status) {
     const int j = blockIdx.x;

@@ -79,6 +79,43 @@ def test_tree_grows_on_the_device(rave, B):
     assert ref.n > 1000
 
 
+def test_leaves_at_the_depth_bound_are_left_alone_and_take_no_ids():
+    """With a short depth bound the selection soon stops at nodes that have children already; the host still
+    offers their states' moves.  Such a node stays as it is and no ids are spent on it: the ids of the nodes
+    that ARE created stay those of the checker, step after step."""
+    import omoknuni_small_amd as omk
+    A, B, D, vl = 64, 600, 3, 3
+    soa = dict(N=np.zeros(1, np.int32), W=np.zeros(1, np.float32), P=np.ones(1, np.float32), VL=np.zeros(1, np.int32),
+               child_begin=np.zeros(1, np.int32), child_count=np.zeros(1, np.int32), action=np.full(1, -1, np.int32))
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa, capacity=400_000)
+    b = omk.Batch(f, B, D)
+    roots = np.zeros(B, np.int32)
+    b.set_roots(roots)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, max_depth=D)
+    rng = np.random.default_rng(8)
+    capped = 0
+    for step in range(12):
+        rpaths, rlen, rleaf, _ = ref.select_batch(roots, rp)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths == rpaths).all() and (gleaf == rleaf).all()
+        capped += int((ref.child_count[rleaf] > 0).sum())
+        begin, moves, policy = offers(rng, rleaf, A, max_moves=20)
+        rfirst = ref.expand_batch(rleaf, begin, moves, policy=policy, action_space=A)
+        gfirst = b.expand(begin, moves, policy=policy, action_space=A)
+        assert (gfirst == rfirst).all(), "step %d: new ids differ" % step
+        assert f.node_count()[0] == ref.n
+        values = rng.uniform(-1, 1, B).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, values, vl)
+        b.set_values(values)
+        b.backup(vl)
+        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        ref.W[:] = st["W"]
+    assert capped > 100          # the bound was hit at nodes that have children
+
+
 def test_tree_grows_with_progressive_widening_and_ragged_policies():
     """The reference's default settings (use_progressive_widening, c = 2, k = 0.5): only the first
     min(legal, max(8, 2 sqrt(N + 1))) offered moves become children; policies of every length
