@@ -2538,10 +2538,11 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         }
         // ---- its best candidate, and the best candidate of its other children ----
         uint32_t bk = 0u, bpos = 0xFFFFFFFFu;
-        bool has1 = false;
+        bool has1 = false, odd1 = false;
 #pragma unroll
         for (int q = 0; q < Q; q++) {
             has1 |= k1[q] != 0u;
+            if (RAVE) odd1 |= kin[q] && !(fabsf(kw[q]) <= 3.0e38f);
             if (k1[q] > bk) { bk = k1[q]; bpos = (uint32_t)((wi * Q + q) * kWave + lane); }
         }
 #pragma unroll
@@ -2565,7 +2566,7 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         wave_best(ok_, opos, sk, spos);
         int bn, bvl, bsx, bsy;
         float bw, bp, bq2;
-        bool any1;
+        bool any1, odd_any = false;
         if (SOLO) {
             int tn = kn[0], tvl = kvl[0], tsx = ksp[0].x, tsy = ksp[0].y;
             float tw = kw[0], tp = kp[0], tq2 = kq2[0];
@@ -2578,6 +2579,7 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
             bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tp), ml));
             bq2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq2), ml));
             any1 = __ballot(has1) != 0ull;
+            if (RAVE) odd_any = __ballot(odd1) != 0ull;
         } else {
         {
             int tn = 0, tvl = 0, tsx = 0, tsy = 0;
@@ -2596,6 +2598,7 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
             }
             // the lane that holds the wavefront's best child writes the slot (one lane, one pass)
             const bool any1w = __ballot(has1) != 0ull;
+            const bool odd1w = RAVE && __ballot(odd1) != 0ull;
             if (lane == (int)(mine == 0xFFFFFFFFu ? 0u : (mine & 63u))) {
                 ChainSlot &sl = g_chain_slot[par][wi];
                 sl.bk = hk;
@@ -2609,7 +2612,7 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
                 sl.q2 = tq2;
                 sl.sx = tsx;
                 sl.sy = tsy;
-                sl.any1 = any1w ? 1u : 0u;
+                sl.any1 = (any1w ? 1u : 0u) | (odd1w ? 2u : 0u);
             }
         }
         __syncthreads();
@@ -2653,7 +2656,8 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         hp = (uint32_t)__builtin_amdgcn_readfirstlane((int)hp);
         sk = (uint32_t)__builtin_amdgcn_readfirstlane((int)sk);
         spos = (uint32_t)__builtin_amdgcn_readfirstlane((int)spos);
-        any1 = __builtin_amdgcn_readfirstlane((int)a1) != 0;
+        any1 = (__builtin_amdgcn_readfirstlane((int)a1) & 1) != 0;
+        odd_any = (__builtin_amdgcn_readfirstlane((int)a1) & 2) != 0;
         }  // !SOLO
         // ---- the children of the child the walk would move on into: on their way during the test ----
         const int n_nelig = eligible(bn, bsy);
@@ -2662,7 +2666,8 @@ __device__ __noinline__ int chain_walk(KernArgsP ka, LdsBytesP scratch, int wi, 
         // ---- the one-winner test (single_run) ----
         // (with RAVE and no real first-scan score at all the reference never runs its second scan;
         // select_group knows, and gets no verdict)
-        bool one = hk != 0u && (!RAVE || any1);
+        // (a child whose value sum is not finite: the node is settled one visitor after the other, select_group)
+        bool one = hk != 0u && (!RAVE || (any1 && !odd_any));
         const int best = (int)(hp >= (uint32_t)F ? hp - (uint32_t)F : hp);
         if (one) {
             uint32_t lk, lp;
@@ -2984,6 +2989,20 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         lane_best<R, RAVE>(k, lane, bk, bpos);
     }
     const uint32_t uvl = a.vl > 0 ? (uint32_t)a.vl : 0u;
+    // The parallel paths merge the children's entries of both scans by key.  The reference runs its second scan
+    // only at a visit whose first scan found a child, and that holds for every visit of the node when it holds for
+    // the first, as long as the value sums are finite (a first-scan score is then real at every visit).  A child
+    // without visits whose value sum is NOT finite scores 0 + exploration at its first visit and -inf or NaN from
+    // then on, while its RAVE blend, which ignores the value sum of an unvisited node, stays real: the first scan
+    // can run dry in the middle of the node's visitors.  Such a node is settled one visitor after the other
+    // (wave_pick applies the rule at every visit).
+    bool odd = false;
+    if (RAVE) {
+        bool o = false;
+#pragma unroll
+        for (int r = 0; r < R; r++) o |= k.part[r] && !(fabsf(k.w[r]) <= 3.0e38f);
+        odd = __ballot(o) != 0ull;
+    }
 
     bool settled = false;
     int st_replay = 0;
@@ -3013,10 +3032,10 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         best0 = __builtin_amdgcn_readfirstlane(g_chain.e_best0);
         lk0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)g_chain.e_lk0);
         lp0 = (uint32_t)(__builtin_amdgcn_readfirstlane(g_chain.e_second) ? R * kWave + best0 : best0);
-    } else if (!as_slice && !just_boundary && !settled && m >= kRunMin && a.vl > 0)
+    } else if (!as_slice && !just_boundary && !settled && m >= kRunMin && a.vl > 0 && !odd)
         settled = single_run<R, RAVE>(a, c, lane, k, bk, bpos, soff, m, m >= kRunShareMin, cnt, run_child, contested, best0,
                                       lk0, lp0);
-    if (!settled && contested && m >= kSparseMin && m < kHeavyMin) {
+    if (!settled && contested && m >= kSparseMin && m < kHeavyMin && !odd) {
         settled = sparse_merge<R, RAVE>(a, c, lane, k, best0, lk0, lp0, m, lds, pl.order, cnt, pending);
         if (settled) {
             lds_cur = 0;
@@ -3027,7 +3046,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         }
     }
     if (R * kWave <= kHeavyFanout) {
-        if (!as_slice && !just_boundary && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0) {
+        if (!as_slice && !just_boundary && !settled && m >= kHeavyMin && m <= kWaterLevelMaxJ && a.vl > 0 && !odd) {
             // cut the node into slices: the others go to the queue, this wavefront takes the first
             const int K = (m + slice_size(m) - 1) / slice_size(m);  // at most kMaxSlices
             // (a node whose boundaries are being worked out ahead of time has its context already)
@@ -3194,7 +3213,7 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         }
     }
     if (just_boundary) return kStepParked;  // (a fan-out class that is never cut into slices)
-    if (!settled && m >= kWaterLevelMin && m <= kWaterLevelMaxJ && a.vl > 0) {
+    if (!settled && m >= kWaterLevelMin && m <= kWaterLevelMaxJ && a.vl > 0 && !odd) {
         int zero[R];
 #pragma unroll
         for (int r = 0; r < R; r++) zero[r] = 0;

@@ -53,3 +53,43 @@ def test_random_forests_and_crowds(seed):
     # exact either way), but it must stay the exception
     print("replayed:", replayed)
     assert sum(r[2] for r in replayed) <= 3, replayed
+
+
+@pytest.mark.parametrize("first", [0, 25])
+def test_values_that_are_not_finite_with_crowds(first):
+    """NaN priors, value sums of -inf, NaN or 3e38, exact ties at zero, virtual loss 0 and 1000, under crowds
+    of up to 9000 visitors, with and without RAVE.  (Seed 29: an unvisited child whose value sum is -inf scores
+    0 + exploration once and -inf from then on while its RAVE blend stays real, so the reference's first scan
+    runs dry in the middle of a node's visitors and the least visited child takes the rest: a node with such a
+    child is settled one visitor after the other.)"""
+    for seed in range(first, first + 25):
+        rng = np.random.default_rng(seed)
+        rave = bool(rng.integers(2))
+        if rng.random() < 0.5:
+            soa, _ = random_tree(int(rng.integers(1 << 30)), n_expand=int(rng.integers(5, 200)),
+                                 fanout=(1, int(rng.integers(2, 300))), max_depth=int(rng.integers(2, 8)), rave=rave,
+                                 mask_frac=float(rng.choice([0.0, 0.3])), vl_frac=0.2, tie_frac=0.2,
+                                 n_max=int(rng.integers(2, 500)))
+            D = 9
+        else:
+            lay = [int(rng.integers(4, 380)), int(rng.integers(4, 30)), int(rng.integers(2, 6))]
+            soa, _ = layered_forest(int(rng.integers(1 << 30)), lay, rave=rave)
+            D = 4
+        n = len(soa["N"])
+        soa["P"], soa["W"], soa["N"] = soa["P"].copy(), soa["W"].copy(), soa["N"].copy()
+        kind = int(rng.integers(5))
+        idx = rng.random(n) < float(rng.choice([0.02, 0.2, 0.9]))
+        idx[0] = False
+        if kind == 0:
+            soa["P"][idx] = np.nan
+        elif kind == 1:
+            soa["W"][idx] = -np.inf
+        elif kind == 2:
+            soa["W"][idx] = np.nan
+        elif kind == 3:
+            soa["P"][idx], soa["N"][idx], soa["W"][idx] = 0.0, 0, 0.0
+        else:
+            soa["W"][idx] = np.float32(3e38)
+        vl = int(rng.choice([0, 0, 1, 3, 1000]))
+        B = int(rng.integers(2, 9000))
+        select_both(soa, np.zeros(B, np.int32), D, rave=rave, steps=2, vl=vl)
