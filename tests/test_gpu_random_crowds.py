@@ -93,3 +93,62 @@ def test_values_that_are_not_finite_with_crowds(first):
         vl = int(rng.choice([0, 0, 1, 3, 1000]))
         B = int(rng.integers(2, 9000))
         select_both(soa, np.zeros(B, np.int32), D, rave=rave, steps=2, vl=vl)
+
+
+def test_the_widest_fan_out_class_with_crowds():
+    """Nodes of 385 to 1024 children (never cut into slices: one wavefront settles them batch after batch), one
+    to three trees, up to 12000 visitors."""
+    for seed in range(15):
+        rng = np.random.default_rng(seed)
+        lay = [int(rng.integers(385, 1025)), int(rng.integers(2, 30))]
+        if rng.random() < 0.4:
+            lay.append(int(rng.integers(2, 6)))
+        rave = bool(rng.integers(2))
+        plateau = rave and bool(rng.integers(2)) and min(lay) >= 3
+        soa, roots = layered_forest(int(rng.integers(1 << 30)), lay, n_trees=int(rng.integers(1, 4)), rave=rave,
+                                    plateau=plateau)
+        B = int(rng.integers(2, 12000))
+        tr = np.sort(rng.integers(0, len(roots), B)).astype(np.int32)
+        select_both(soa, roots[tr], len(lay) + 1, rave=rave, steps=2, vl=int(rng.integers(1, 5)))
+
+
+def test_selection_time_widening_with_crowds():
+    """omk_select_params::pw (only the ceil(sqrt(N_parent)) children of highest prior take part) on forests
+    whose children are stored by descending prior, parents of few and of many visits, crowds up to 12000."""
+    import omoknuni_small_amd as omk
+    from oracle import ref_cpu as R
+    for seed in range(15):
+        rng = np.random.default_rng(seed)
+        lay = [int(rng.integers(4, 380)), int(rng.integers(4, 40)), int(rng.integers(2, 8))]
+        rave = bool(rng.integers(2))
+        soa, roots = layered_forest(int(rng.integers(1 << 30)), lay, n_trees=int(rng.integers(1, 4)), rave=rave)
+        P = soa["P"].copy()
+        for node in np.nonzero(soa["child_count"] > 0)[0]:
+            cb, cc = soa["child_begin"][node], soa["child_count"][node]
+            P[cb:cb + cc] = np.sort(P[cb:cb + cc])[::-1]
+        soa["P"] = P
+        soa["N"] = soa["N"].copy()
+        small = (rng.random(len(P)) < 0.3) & (soa["child_count"] > 0)
+        soa["N"][small] = rng.integers(0, 50, int(small.sum()))
+        B, D, vl = int(rng.integers(2, 12000)), 4, int(rng.integers(1, 5))
+        troots = roots[np.sort(rng.integers(0, len(roots), B))].astype(np.int32)
+        ref = R.RefTree.from_soa(soa)
+        rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0, pw=True, max_depth=D)
+        f = omk.Forest.from_soa(soa)
+        b = omk.Batch(f, B, D)
+        b.set_roots(troots)
+        sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0, pw=True)
+        for step in range(2):
+            rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
+            b.select(sp)
+            gpaths, glen, gleaf, _ = b.read()
+            assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all(), (seed, step)
+            vals = rng.uniform(-1, 1, B).astype(np.float32)
+            ref.backup_batch(rpaths, rlen, vals, vl)
+            b.set_values(vals)
+            b.backup(vl)
+            st = f.download()
+            assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all(), (seed, step)
+            ref.W[:] = st["W"]
+        b.close()
+        f.close()
