@@ -111,7 +111,12 @@ def test_leaves_at_the_depth_bound_are_left_alone_and_take_no_ids():
         ref.backup_batch(rpaths, rlen, values, vl)
         b.set_values(values)
         b.backup(vl)
-        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        st, sx = f.download(), f.download_structure()
+        assert (sx["child_begin"] == ref.child_begin).all() and (sx["child_count"] == ref.child_count).all()
+        assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all() and st["P"].tobytes() == ref.P.tobytes()
+        # (600 values a step meet at the root, added in another order than the serial loop's)
+        err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
+        assert err.max() <= 1e-5 * np.sqrt(B), step
         ref.W[:] = st["W"]
     assert capped > 100          # the bound was hit at nodes that have children
 
