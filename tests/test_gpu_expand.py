@@ -1,6 +1,8 @@
 """GPU parity of leaf expansion (omk_expand_batch) and of search steps on a tree that grows on
 the device: select -> leaf gather -> expand -> backup, every array against the CPU checker
-after every phase.  Structure, priors, actions, N and virtual loss bit-exact; W within 1e-5."""
+after every phase.  Structure, priors, actions, N and virtual loss bit-exact; W within 1e-5 (relative to
+max(|W|, 1); where hundreds of values meet at a node in one step, the bound grows with the square root of
+their number, as in the full-size tests: the device adds them in another order than the serial loop)."""
 import numpy as np
 import pytest
 
@@ -10,7 +12,9 @@ from tests.helpers import random_tree
 pytestmark = pytest.mark.gpu
 
 
-def assert_same_forest(f, ref, what):
+def assert_same_forest(f, ref, what, k=1):
+    """k: values a node may have taken in the step just backed up (the device adds them in another order than
+    the serial loop; the bound grows with sqrt(k), as in the full-size tests)."""
     st = f.download()
     sx = f.download_structure()
     assert len(st["N"]) == ref.n, what
@@ -19,7 +23,7 @@ def assert_same_forest(f, ref, what):
     assert st["P"].tobytes() == ref.P.tobytes(), what
     assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all(), what
     err = np.abs(st["W"].astype(np.float64) - ref.W) / np.maximum(np.abs(ref.W), 1.0)
-    assert err.max() <= 1e-5, what
+    assert err.max() <= 1e-5 * max(1.0, np.sqrt(k) / 8.0), what
     return st
 
 
@@ -74,7 +78,7 @@ def test_tree_grows_on_the_device(rave, B):
         ref.backup_batch(rpaths, rlen, values, vl)
         b.set_values(values)
         b.backup(vl)
-        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        st = assert_same_forest(f, ref, "after backup, step %d" % step, B)
         ref.W[:] = st["W"]
     assert ref.n > 1000
 
@@ -163,7 +167,7 @@ def test_tree_grows_with_progressive_widening_and_ragged_policies():
         ref.backup_batch(rpaths, rlen, values, vl)
         b.set_values(values)
         b.backup(vl)
-        st = assert_same_forest(f, ref, "after backup, step %d" % step)
+        st = assert_same_forest(f, ref, "after backup, step %d" % step, B)
         ref.W[:] = st["W"]
     assert kinds_seen == {0, 1, 2, 3} and ref.n > 500
     # widening at work: no node has more children than its visit count allowed when it was expanded
