@@ -171,3 +171,48 @@ def test_two_batches_on_one_forest(first):
 def test_a_tree_that_grows_and_is_reused(first):
     for seed in range(first, first + 15):
         growing_tree_session(seed)
+
+
+def test_selections_that_give_up_in_mid_session():
+    """Tiny spin limits make waiting wavefronts give up (the kernels still end normally): the library says so,
+    and once the statistics are put back the same batch selects correctly again, time after time."""
+    import omoknuni_small_amd as omk
+    gave_up = 0
+    for seed in range(12):
+        rng = np.random.default_rng(seed)
+        lay = [int(rng.integers(4, 300)), int(rng.integers(4, 30)), int(rng.integers(2, 8))]
+        rave = bool(rng.integers(2))
+        soa, roots = layered_forest(int(rng.integers(1 << 30)), lay, n_trees=int(rng.integers(1, 4)), rave=rave)
+        B, D, vl = int(rng.integers(200, 12000)), 4, 3
+        troots = roots[np.sort(rng.integers(0, len(roots), B))].astype(np.int32)
+        ref = R.RefTree.from_soa(soa)
+        f = omk.Forest.from_soa(soa)
+        b = omk.Batch(f, B, D)
+        b.set_roots(troots)
+        sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0)
+        rp = R.make_params(c_puct=1.4, virtual_loss=vl, use_rave=rave, rave_k=1000.0, max_depth=D)
+        for op in range(5):
+            if rng.random() < 0.5:
+                cur = dict(soa)
+                cur["N"], cur["W"], cur["VL"] = ref.N.copy(), ref.W.copy(), ref.VL.copy()
+                b.set_spin_limit(int(rng.choice([0, 1, 2, 5, 20, 100])))
+                b.select(sp)
+                try:
+                    b.read()
+                except omk.OmkError as e:
+                    assert e.code == -6, e       # OMK_ERR_STATE: the selection gave up
+                    gave_up += 1
+                f.upload(cur)                    # whatever virtual loss the incomplete selection left is gone
+                b.set_spin_limit(1 << 22)
+            rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
+            b.select(sp)
+            gpaths, glen, gleaf, _ = b.read()
+            assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all(), (seed, op)
+            vals = rng.uniform(-1, 1, B).astype(np.float32)
+            ref.backup_batch(rpaths, rlen, vals, vl)
+            b.set_values(vals)
+            b.backup(vl)
+            same_statistics(f, ref, "seed %d operation %d" % (seed, op), B)
+        b.close()
+        f.close()
+    assert gave_up >= 5
