@@ -321,6 +321,13 @@ int omk_batch_set_trace(omk_batch *b, int32_t enabled);
  * one).  The default (about four million polls, seconds) is never reached in normal
  * operation; tests of the error path set a tiny limit.  No counterpart in the reference. */
 int omk_batch_set_spin_limit(omk_batch *b, int32_t polls);
+/* The ready marks of the scheduler's queues are the number of the select call on the batch, which starts
+ * over (all marks cleared) shortly before 2^30 calls: some days of continuous search.  A test cannot wait
+ * for that; this sets the number of the call made last (0 <= count < 2^30), so that the next calls cross
+ * the point.  Only between a batch's selections (the marks in memory belong to earlier numbers: moving the
+ * count BACK to a number already used leaves stale marks that look fresh, so go forward only).  No
+ * counterpart in the reference. */
+int omk_debug_set_select_count(omk_batch *b, int32_t count);
 
 /* ---- transposition table: the lookup/store call sites of
  *      mcts_engine_batch_tree_simple.cpp:126,141 (PHMapTranspositionTable::store / lookup,

@@ -1504,6 +1504,21 @@ int omk_batch_set_spin_limit(omk_batch *b, int32_t polls) {
     return OMK_OK;
 }
 
+int omk_debug_set_select_count(omk_batch *b, int32_t count) {
+    if (!b) return fail(OMK_ERR_INVALID, "omk_debug_set_select_count: null batch");
+    if (count < b->epoch || count >= (1 << 30))
+        return fail(OMK_ERR_INVALID, "omk_debug_set_select_count: count %d (the last call was number %d; forward only, "
+                    "below 2^30)", count, b->epoch);
+    // the two depth-cap counters take turns by call parity: keep the parity, so that the counter the next call
+    // starts from is the one the last call cleared
+    if ((count & 1) != (b->epoch & 1)) {
+        if (count + 1 >= (1 << 30)) return fail(OMK_ERR_INVALID, "omk_debug_set_select_count: count %d", count);
+        count++;
+    }
+    b->epoch = count;
+    return OMK_OK;
+}
+
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16) {
     int32_t *h_stats8 = h_stats16;
     if (!b || !h_stats8) return fail(OMK_ERR_INVALID, "omk_batch_stats: null argument");

@@ -27,7 +27,7 @@ EXPORTS = [
     "omk_sync", "omk_batch_create", "omk_batch_destroy",
     "omk_batch_set_roots", "omk_batch_set_values", "omk_batch_device", "omk_select_batch", "omk_backup_batch",
     "omk_revert_vl", "omk_backup_rave_batch", "omk_apply_vl_paths", "omk_revert_vl_paths", "omk_backup_paths", "omk_batch_read",
-    "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_set_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
+    "omk_batch_leaf_keys", "omk_debug_trace", "omk_batch_set_trace", "omk_batch_truncated", "omk_batch_stats", "omk_batch_set_stats", "omk_batch_set_spin_limit", "omk_debug_set_select_count", "omk_tt_create", "omk_tt_destroy", "omk_tt_clear", "omk_tt_insert", "omk_tt_probe",
     "omk_tt_probe_leaves", "omk_tt_store", "omk_tt_set_replacement_threshold", "omk_tt_traverse", "omk_tt_select_redirect", "omk_forest_download_redirects", "omk_tt_download_meta", "omk_tt_upload", "omk_tt_download", "omk_dev_alloc", "omk_dev_free", "omk_dev_h2d",
     "omk_dev_d2h", "omk_dev_copy", "omk_soa_count_legal", "omk_soa_compact_legal",
 ]
@@ -446,6 +446,11 @@ class Batch:
     def set_spin_limit(self, polls):
         """Bound of the waits inside the persistent selection kernel (error-path tests)."""
         _check(self._lib.omk_batch_set_spin_limit(self._h, C.c_int32(int(polls))))
+
+    def debug_set_select_count(self, count):
+        """Test hook: the number of the select call made last (forward only), to cross the point where the
+        call numbers start over without making 2^30 calls."""
+        _check(self._lib.omk_debug_set_select_count(self._h, C.c_int32(int(count))))
 
     def stats(self):
         out = np.zeros(16, np.int32)

@@ -416,3 +416,41 @@ def test_roots_set_again_start_the_paths_anew():
         assert (gpaths[:, 0] == troots).all()
         assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all()
         f.upload(soa)  # the virtual losses of this selection are dropped with the statistics
+
+
+def test_call_numbers_start_over_without_a_trace():
+    """The queues' ready marks are call numbers, which start over shortly before 2^30 calls (all marks, the
+    boundary table and the heavy nodes' contexts cleared): selections on both sides of that point, with heavy
+    nodes, slices, boundaries worked out ahead of time, lone walkers and the depth-cap counter, stay exact."""
+    import omoknuni_small_amd as omk
+    soa, roots = layered_forest(21, [150, 30, 6], n_trees=2)
+    B, D, vl = 9000, 3, 3              # the depth bound cuts every path at a node with children
+    troots = roots[np.sort(np.arange(B) % 2)].astype(np.int32)
+    ref = R.RefTree.from_soa(soa)
+    rp = R.make_params(c_puct=1.4, virtual_loss=vl, max_depth=D)
+    f = omk.Forest.from_soa(soa)
+    b = omk.Batch(f, B, D)
+    b.set_roots(troots)
+    b.enable_stats()
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=vl)
+    rng = np.random.default_rng(2)
+    sliced = 0
+    for step in range(10):
+        if step == 2:
+            b.debug_set_select_count((1 << 30) - 6)       # four calls before the numbers start over
+        rpaths, rlen, rleaf, _ = ref.select_batch(troots, rp, near_ties=False)
+        b.select(sp)
+        gpaths, glen, gleaf, _ = b.read()
+        assert (gpaths == rpaths).all() and (glen == rlen).all() and (gleaf == rleaf).all(), step
+        assert b.truncated() == int(((ref.child_count[rleaf] > 0) & (rlen == D + 1)).sum()), step
+        sliced += b.stats()["sliced_nodes"]
+        vals = rng.uniform(-1, 1, B).astype(np.float32)
+        ref.backup_batch(rpaths, rlen, vals, vl)
+        b.set_values(vals)
+        b.backup(vl)
+        st = f.download()
+        assert (st["N"] == ref.N).all() and (st["VL"] == ref.VL).all(), step
+        ref.W[:] = st["W"]
+    assert sliced >= 10
+    with pytest.raises(omk.OmkError):
+        b.debug_set_select_count(1)                        # forward only
