@@ -1147,7 +1147,11 @@ int omk_select_batch(omk_batch *b, const omk_select_params *p) {
     a.n_trav = b->n;
     a.n_team_blocks = 0;
     a.fast_singles = 0;
-    a.poll_sleep = b->poll_sleep;
+    // A waiting wavefront sleeps about a microsecond between two polls, so that hundreds of them leave the memory
+    // system to those that work.  A small batch has few wavefronts waiting and a short chain of crowded nodes, every
+    // hand-over of which pays that sleep: they poll without it (measured on 64 traversals: 0.095 -> 0.092 ms; on
+    // 4096, with the sleep off: 0.216 -> 0.221).
+    a.poll_sleep = b->n <= 256 ? 0 : b->poll_sleep;
     a.hctx = b->hctx;
     a.hbound = b->hbound;
     a.hctx_n = b->counters + 2 * kSchedStep + 64;
