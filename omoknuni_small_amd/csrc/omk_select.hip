@@ -4367,7 +4367,7 @@ static hipError_t launch_kernels(const ForestDev &f, const SelectArgs &a0, int n
         int walkers = n_traversals / 64;
         if (walkers > capacity / 4) walkers = capacity / 4;
         if (walkers > kMaxWalkerBlocks) walkers = kMaxWalkerBlocks;  // idle walkers poll: more of them slow the teams
-        if (walkers < 1) walkers = 1;
+        if (walkers < 4) walkers = 4;  // (a small batch ends with a handful of lone walks: enough walkers to take them at once)
         int teams = capacity - walkers;
         const int most = n_traversals / 2;
         if (teams > most) teams = most;
