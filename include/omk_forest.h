@@ -418,7 +418,8 @@ int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int3
  *     step is that of the node of the tree AS UPLOADED that the recorded moves lead to from the root, which
  *     is what replaying the moves on the root state gives (:119-124); where no such node exists (a move no
  *     child slot carries, a node not expanded) the step has no key and the table is not touched.
- *   - Time stamps: step g of the call stores at clock + 2g and looks up at clock + 2g + 1.
+ *   - Time stamps: the table's clock advances here as the reference's access counter does on one thread: by
+ *     one on a store that finds its key (phmap_transposition_table.cpp:65) and on a lookup that hits (:107).
  *   - d_moves: NULL, or device memory for max_depth * stride ints (omk_batch_dev.stride), level-major like the
  *     paths (entry (d - 1) * stride + t = the move recorded at step d of traversal t): the move list the
  *     leaf's state is rebuilt from.  It differs from the actions of the path's nodes exactly at a step that

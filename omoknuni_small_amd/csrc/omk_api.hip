@@ -1780,7 +1780,7 @@ int omk_tt_select_redirect(omk_tt *tt, omk_batch *b, const omk_select_params *p,
     b->selected = true;
     HIP_TRY(hipMemcpyAsync(status, tt->d_status, sizeof(status), hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
-    tt->clock += 2u * (uint32_t)status[4];
+    tt->clock += (uint32_t)status[6];  // the ticks of the access counter
     if (status[3] > 0) f->redirected = true;
     if (h_counts)
         for (int i = 0; i < 5; i++) h_counts[i] = status[i];

@@ -745,7 +745,8 @@ hipError_t launch_tt_probe(const TTSlot *slots, int log2_slots, const uint64_t *
 // ORIGINAL tree (slots, not what they hold) that the recorded moves lead to from the root, which is
 // what replaying the recorded moves on the root state gives (:119-124, :133-137); where no such node
 // exists the step has no key and the table is left alone.
-// Time: step g of the call (counted over all traversals) stores at t0 + 2g and looks up at t0 + 2g + 1.
+// Time: the reference's access counter as one thread advances it, from t0 on: it ticks on a store that
+// finds its key (phmap_transposition_table.cpp:65) and on a lookup that hits (:107), not otherwise.
 
 __device__ __forceinline__ int ld_agent(const int32_t *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -822,6 +823,7 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
     const uint64_t mask = (1ull << a.log2_slots) - 1ull;
     int n_new = 0, n_repl = 0, n_found = 0, n_redirect = 0, n_full = 0, n_trunc = 0;
     uint32_t g = 0u;
+    uint32_t clk = a.t0;  // the table's access counter (lane 0 keeps it)
     for (int t = 0; t < a.n; t++) {
         int cur = a.paths[t];
         int shadow = cur;
@@ -952,7 +954,7 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
                             const int depth = (int)(uint16_t)(d + 1);             // move_sequence.size(); Entry::depth is a uint16_t
                             bool write = !present;
                             if (present) {
-                                const uint32_t now = a.t0 + 2u * g;
+                                const uint32_t now = clk++;                       // :65
                                 const float existing = tt_replacement_score(a.meta[s].visits, a.meta[s].value, a.slots[s].depth,
                                                                             now, a.meta[s].last_access);
                                 const float fresh = tt_replacement_score(0u, 0.0f, depth, now, 0u);
@@ -976,7 +978,7 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
                     int found = -1;
                     if (room && a.slots[s].key == key) {                          // :141, lookup()
                         found = a.slots[s].node;
-                        a.meta[s].last_access = a.t0 + 2u * g + 1u;
+                        a.meta[s].last_access = clk++;                            // :107
                         n_found++;
                     }
                     if (found >= 0 && found != best && found < f.n_nodes && f.N[found] > 0) {   // :142
@@ -1018,6 +1020,7 @@ __global__ __launch_bounds__(kWave) void k_select_redirect(ForestDev f, Redirect
         a.counts[3] = n_redirect;
         a.counts[4] = (int)g;
         a.counts[5] = n_full;
+        a.counts[6] = (int)(clk - a.t0);
         *a.truncated = n_trunc;
         *a.truncated_next = 0;
         *a.abort_word = 0;

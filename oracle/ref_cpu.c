@@ -425,9 +425,10 @@ int64_t ref_tt_lookup_batch(const ref_tt_slot *slots, ref_tt_meta *meta, int32_t
  * not what they hold) that the recorded moves lead to from the root; where that node does not exist
  * (a move no child slot carries, or a node that is not expanded) the position has no key from there on:
  * nothing is stored or looked up (the reference would ask the game).
- * Time: step g of the call (counted over all traversals) stores at t0 + 2g and looks up at t0 + 2g + 1.
- * counts: [0] new entries, [1] replacements, [2] lookups that found an entry, [3] redirects, [4] steps.
- * Returns 0, -1 bad root, -2 table full. */
+ * Time: the reference's access counter on one thread, starting at t0: it ticks on a store that finds its key
+ * (phmap_transposition_table.cpp:65) and on a lookup that hits (:107), and not otherwise.
+ * counts: [0] new entries, [1] replacements, [2] lookups that found an entry, [3] redirects, [4] steps,
+ * [5] ticks of the counter.  Returns 0, -1 bad root, -2 table full. */
 static int32_t select_slot_redirected(const ref_tree *t, const int32_t *alias, int32_t node, const ref_params *p) {
     const int32_t cb = t->child_begin[node];
     const int32_t cc = t->child_count[node];
@@ -467,7 +468,8 @@ int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots,
     const int32_t stride = p->max_depth + 1;
     int rc = 0;
     uint32_t g = 0;
-    for (int j = 0; j < 5; j++) counts[j] = 0;
+    uint32_t clock = t0;  /* access_counter_: ticks on a store that finds its key (:65) and on a lookup that hits (:107) */
+    for (int j = 0; j < 6; j++) counts[j] = 0;
     for (int32_t i = 0; i < B; i++) {
         int32_t *path = paths + (int64_t)i * stride;
         int32_t *mv = moves ? moves + (int64_t)i * p->max_depth : NULL;
@@ -498,15 +500,18 @@ int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots,
                 if (t->N[best] == 0) {                                               /* :116-128 */
                     int32_t c4[4];
                     const int32_t depth = len;                                       /* move_sequence.size() */
-                    int r = ref_tt_store_batch(slots, meta, log2_slots, t, &key, &best, &depth, 1, t0 + 2u * g,
-                                               threshold, c4);
+                    int r = ref_tt_store_batch(slots, meta, log2_slots, t, &key, &best, &depth, 1, clock, threshold, c4);
                     if (r == -1) rc = -2;
+                    else if (c4[0] == 0) clock++;                                    /* the key was there: :65 */
                     counts[0] += c4[0];
                     counts[1] += c4[1];
                 }
                 int32_t found = -1;
-                ref_tt_lookup_batch(slots, meta, log2_slots, &key, 1, 0, t0 + 2u * g + 1u, &found);  /* :141 */
-                if (found >= 0) counts[2]++;
+                ref_tt_lookup_batch(slots, meta, log2_slots, &key, 1, 0, clock, &found);         /* :141 */
+                if (found >= 0) {
+                    counts[2]++;
+                    clock++;                                                         /* :107 */
+                }
                 if (found >= 0 && found != best && found < t->n_nodes && t->N[found] > 0) {  /* :142 */
                     ref_remove_vl(t, best, p->virtual_loss);                         /* :146 */
                     /* :149, updateChildReference: the first slot of `current` that holds the old child */
@@ -530,6 +535,7 @@ int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots,
         leaf[i] = current;
     }
     counts[4] = (int32_t)g;
+    counts[5] = (int32_t)(clock - t0);
     return rc;
 }
 

@@ -236,8 +236,10 @@ int64_t ref_tt_probe(const ref_tt_slot *slots, int32_t log2_slots, const uint64_
 
 /* The traversal loop with the transposition table on, redirects included (see ref_cpu.c): alias[n_nodes]
  * (-1 = the slot holds its own node) is read and updated; paths [B][max_depth+1], moves [B][max_depth]
- * (may be NULL); counts[5].  PARITY UNPINNED for the table's arithmetic as above; the loop itself is pinned
- * by a literal restatement over node objects with children lists (tests/test_oracle_redirect.py). */
+ * (may be NULL); counts[6].  The table's clock is the reference's on one thread (it ticks on a store that
+ * finds its key and on a lookup that hits); with several threads the reference's stamps depend on the
+ * schedule.  The loop, the clock included, is pinned by a literal restatement over node objects with
+ * children lists and a dictionary as the table (tests/test_oracle_redirect.py). */
 int ref_select_redirect_batch(ref_tree *t, int32_t *alias, const int32_t *roots, int32_t B, const ref_params *p,
                               ref_tt_slot *slots, ref_tt_meta *meta, int32_t log2_slots, uint32_t t0, float threshold,
                               const uint64_t *node_key, int32_t *paths, int32_t *path_len, int32_t *leaf,

@@ -305,7 +305,7 @@ class RefTree:
         """The traversal loop with the transposition table on, redirects included (see ref_cpu.c).
         alias (int32 per node, -1 = the slot holds its own node) is updated in place; returns
         (paths, path_len, leaf, moves, counts) with counts = new entries, replacements, lookups that found
-        an entry, redirects, steps; tt's clock advances by two per step."""
+        an entry, redirects, steps; tt's clock advances as the reference's access counter does on one thread."""
         roots = np.ascontiguousarray(roots, dtype=np.int32)
         node_key = np.ascontiguousarray(node_key, dtype=np.uint64)
         assert len(node_key) == self.n
@@ -318,7 +318,7 @@ class RefTree:
         path_len = np.empty(B, dtype=np.int32)
         leaf = np.empty(B, dtype=np.int32)
         moves = np.empty((B, params.max_depth), dtype=np.int32)
-        counts = np.zeros(5, np.int32)
+        counts = np.zeros(6, np.int32)
         fn = lib().ref_select_redirect_batch
         fn.restype = C.c_int
         rc = fn(C.byref(self._c), _ptr(alias, i32p), _ptr(roots, i32p), C.c_int32(B), C.byref(params),
@@ -327,8 +327,8 @@ class RefTree:
                 _ptr(path_len, i32p), _ptr(leaf, i32p), _ptr(moves, i32p), _ptr(counts, i32p))
         if rc != 0:
             raise ValueError("ref_select_redirect_batch: %d" % rc)
-        tt.clock += 2 * int(counts[4])
-        return paths, path_len, leaf, moves, counts
+        tt.clock += int(counts[5])
+        return paths, path_len, leaf, moves, counts[:5]
 
     def gather_actions(self, paths, path_len):
         paths, path_len, B, stride = self._paths_args(paths, path_len)

@@ -133,7 +133,10 @@ def literal_select_child(tree, node, params):
 
 
 def literal_batch(tree, nodes, root, B, params, table, clock, game_hash):
-    """mcts_engine_batch_tree_simple.cpp:88-165 for B traversals, one after the other."""
+    """mcts_engine_batch_tree_simple.cpp:88-165 for B traversals, one after the other.  The table's access
+    counter starts at `clock` and ticks where the reference's does: on a store that finds its key
+    (phmap_transposition_table.cpp:65) and on a lookup that returns an entry (:107).  Returns the counter
+    as its last element."""
     vl = params.virtual_loss
     out_paths, out_moves, redirects, g = [], [], 0, 0
     for _ in range(B):
@@ -148,8 +151,11 @@ def literal_batch(tree, nodes, root, B, params, table, clock, game_hash):
             h = game_hash(moves)                                       # :119-124, :133-137
             if h is not None:
                 if tree.N[best.id] == 0:                               # :116
-                    table.store(tree, h, best.id, len(moves), clock + 2 * g)
-                tt = table.lookup(h, 0, clock + 2 * g + 1)             # :141
+                    if table.store(tree, h, best.id, len(moves), clock) != "new":
+                        clock += 1
+                tt = table.lookup(h, 0, clock)                         # :141
+                if tt >= 0:
+                    clock += 1
                 if tt >= 0 and tt != best.id and tree.N[tt] > 0:       # :142
                     tree.remove_vl(best.id, vl)                        # :146
                     idx = [c is best for c in current.children].index(True)   # updateChildReference: first match
@@ -162,7 +168,7 @@ def literal_batch(tree, nodes, root, B, params, table, clock, game_hash):
             path.append(current.id)
         out_paths.append(path)
         out_moves.append(moves)
-    return out_paths, out_moves, redirects, g
+    return out_paths, out_moves, redirects, g, clock
 
 
 def run_search(g, seed, batches, B, vl=3, c_puct=1.4, max_depth=8):
@@ -180,8 +186,8 @@ def run_search(g, seed, batches, B, vl=3, c_puct=1.4, max_depth=8):
     for _ in range(batches):
         t0 = tt.clock
         paths, plen, leaf, moves, counts = flat.select_redirect_batch(np.zeros(B, np.int32), params, tt, g["keys"], alias)
-        lp, lm, lr, lg = literal_batch(lit, nodes, 0, B, params, table, t0, g["game_hash"])
-        assert counts[4] == lg and tt.clock == t0 + 2 * lg
+        lp, lm, lr, lg, lclock = literal_batch(lit, nodes, 0, B, params, table, t0, g["game_hash"])
+        assert counts[4] == lg and tt.clock == lclock
         for i in range(B):
             assert paths[i, :plen[i]].tolist() == lp[i], (i, paths[i], lp[i])
             assert (paths[i, plen[i]:] == -1).all() and leaf[i] == lp[i][-1]
