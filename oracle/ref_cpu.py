@@ -325,6 +325,13 @@ class RefTree:
                 C.c_void_p(tt.slots.ctypes.data), C.c_void_p(tt.meta.ctypes.data), C.c_int32(tt.log2),
                 C.c_uint32(tt.clock & 0xFFFFFFFF), C.c_float(tt.threshold), _ptr(node_key, u64p), _ptr(paths, i32p),
                 _ptr(path_len, i32p), _ptr(leaf, i32p), _ptr(moves, i32p), _ptr(counts, i32p))
+        if rc == -2:
+            # the table ran full: every traversal was still made (without the entries that found no room);
+            # the error carries what they did
+            tt.clock += int(counts[5])
+            err = ValueError("ref_select_redirect_batch: table full")
+            err.result = (paths, path_len, leaf, moves, counts[:5])
+            raise err
         if rc != 0:
             raise ValueError("ref_select_redirect_batch: %d" % rc)
         tt.clock += int(counts[5])

@@ -139,6 +139,61 @@ def test_several_roots_positions_without_a_key_and_batches_given_up():
     assert total[3] >= 3, total
 
 
+def test_a_table_that_runs_full_is_reported_and_the_traversals_are_made_all_the_same():
+    # 16 slots for a game with far more positions: entries that find no room are dropped (and counted), the
+    # traversals go on without them; the call reports the table as full after it has done everything else,
+    # so the batch can be read, backed up or given up as after any other selection
+    import omoknuni_small_amd as omk
+    rng = np.random.default_rng(71)
+    g = stones_tree(rng, cells=6, plies=3)
+    soa = as_soa(g, rng)
+    ref = R.RefTree.from_soa(soa)
+    f = omk.Forest.from_soa(soa)
+    tt, ref_tt = omk.TranspositionTable(f, 4), R.RefTT(4)
+    alias = np.full(g["n"], -1, np.int32)
+    sp = omk.SelectParams(c_puct=1.4, virtual_loss=2)
+    rp = R.make_params(c_puct=1.4, virtual_loss=2, max_depth=5)
+    B = 24
+    b = omk.Batch(f, B, 5)
+    roots = np.zeros(B, np.int32)
+    full = 0
+    for step in range(6):
+        what = "step %d" % step
+        b.set_roots(roots)
+        dev_full = ref_full = False
+        try:
+            tt.select_redirect(b, sp)
+        except omk.OmkError as e:
+            assert "table full" in str(e), e
+            dev_full = True
+        try:
+            rpaths, rplen, rleaf, rmoves, rcounts = ref.select_redirect_batch(roots, rp, ref_tt, g["keys"], alias)
+        except ValueError as e:
+            ref_full = True
+            rpaths, rplen, rleaf, rmoves, rcounts = e.result
+        assert dev_full == ref_full, what
+        full += dev_full
+        paths, plen, leaf, _ = b.read()
+        assert (plen == rplen).all() and (paths == rpaths).all() and (leaf == rleaf).all(), what
+        assert (f.download_redirects() == alias).all(), what
+        assert (f.download()["VL"] == ref.VL).all(), what
+        same_tables(tt, ref_tt, what)
+        if step % 2:
+            b.revert_vl(2)
+            ref.revert_vl_paths(rpaths, rplen, 2)
+        else:
+            values = rng.uniform(-1, 1, B).astype(np.float32)
+            b.set_values(values)
+            b.backup(2)
+            ref.backup_batch(rpaths, rplen, values, 2)
+            dev = f.download()
+            assert (dev["N"] == ref.N).all(), what
+            assert np.allclose(dev["W"], ref.W, rtol=0, atol=1e-5 * max(1.0, np.sqrt(B))), what
+            ref.W[:] = dev["W"]
+        assert (f.download()["VL"] == ref.VL).all(), what
+    assert full >= 3, full
+
+
 def test_a_redirected_forest_is_a_graph_until_the_next_upload():
     import omoknuni_small_amd as omk
     rng = np.random.default_rng(31)
