@@ -425,6 +425,10 @@ int omk_tt_traverse(omk_tt *tt, omk_batch *b, const uint64_t *d_piece_keys, int3
  *     leaf's state is rebuilt from.  It differs from the actions of the path's nodes exactly at a step that
  *     redirected.
  *   - h_counts (NULL or [5]): new entries, replacements, lookups that found an entry, redirects, steps.
+ *   - A table without room for a new entry drops it and the traversals go on without it; the call then
+ *     returns OMK_ERR_CAPACITY AFTER everything else is done (h_counts filled, the batch selected: read it,
+ *     back it up or revert it as after any selection).  The reference's table evicts instead
+ *     (enforceMemoryLimit, phmap_transposition_table.cpp:77-79): size the table for the search.
  * Paths, leaves and virtual loss are left as omk_select_batch leaves them (omk_batch_read, omk_backup_batch,
  * omk_revert_vl work on them).  Once a slot has been re-pointed the forest is a graph until the next
  * omk_forest_upload: omk_select_batch, omk_backup_rave_batch, omk_forest_add_root_noise and the compactions
