@@ -290,8 +290,9 @@ int omk_batch_truncated(omk_batch *b, int32_t *h_count);
  * that takes nearly every visitor, [8] when the first block of the persistent launch started,
  * [9] when its last team of wavefronts left, [10] when its last walker left (low 31 bits of the
  * device's 100 MHz clock; these three are kept whether or not the counters are on), [11] the number
- * of walks of lone visitors inside that launch, [12..14] unused (0), [15] nodes cut into
- * slices for several wavefronts.  (Nodes taken by the walk down one-winner nodes count in [0]..[2].) */
+ * of walks of lone visitors inside that launch, [12] nodes of more than 64 child slots settled through
+ * the few children that can be chosen at all, one per lane (RAVE layouts), [13..14] unused (0), [15] nodes
+ * cut into slices for several wavefronts.  (Nodes taken by the walk down one-winner nodes count in [0]..[2].) */
 int omk_batch_stats(omk_batch *b, int32_t *h_stats16);
 /* The counters above cost one atomic per processed node (and per single-visitor step), all on
  * the same few addresses, so they are off unless switched on here (enabled != 0); with

@@ -2372,6 +2372,112 @@ __device__ __forceinline__ bool sparse_merge(const SelectArgs &a, const NodeCtx 
 }
 
 
+// A wide node (more than 64 child slots) whose visitors split, settled as a narrow one.  Of all its
+// children only those can be chosen whose next entry comes before the entry (lk0, lp0) that the child
+// with the best next entry, B, shows its LAST visitor, provided B's entries are in order: B's head is
+// then at or before (lk0, lp0) at every step, so a child whose head does not come before that entry is
+// never the best.  Where B's order is provable (keys_provably_monotone) and these children are at most
+// 64, they are moved to one lane each, in child order (positions keep their order, and every first-scan
+// candidate still comes before every second-scan one), and the water level of the narrow class settles
+// them: its probes walk one round of children instead of R.  The winner order comes back with the
+// children's own indices, the visits per child to the lanes that hold them.  Returns false with nothing
+// the caller relies on changed (cnt[] zero).
+template <int R, bool RAVE>
+__device__ __forceinline__ bool narrow_water_level(const SelectArgs &a, const NodeCtx &c, int lane,
+                                                   const Kids<R, RAVE> &k, int soff, int best0, uint32_t lk0,
+                                                   uint32_t lp0, int m, WaveLds<R> &lds, int (&cnt)[R], int &lds_cur,
+                                                   uint32_t *order, bool &pending) {
+    static_assert(R > 1, "a narrow node is settled as it is");
+    constexpr int F = R * kWave;
+    const uint32_t uvl = (uint32_t)a.vl;
+    int n0 = 0;
+    bool listed[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = r * kWave + lane;
+        uint32_t hk = k.k1[r], hp = (uint32_t)i;
+        if (k.k2[r] > k.k1[r]) {
+            hk = k.k2[r];
+            hp = (uint32_t)(F + i);
+        }
+        listed[r] = hk != 0u && (i == best0 || comes_before(hk, hp, lk0, lp0));
+        const uint64_t cm = __ballot(listed[r]);
+        if (listed[r]) {
+            const int cl = n0 + __popcll(cm & ((1ull << lane) - 1ull));
+            if (cl < kWave) {
+                lds.st_j0[cl] = i;
+                lds.st_n[cl] = k.n[r];
+                lds.st_w[cl] = k.w[r];
+                lds.st_p[cl] = k.p[r];
+                lds.st_vl[cl] = k.vl[r];
+                lds.st_q2[cl] = k.q2[r];
+            }
+        }
+        n0 += __popcll(cm);
+    }
+    if (n0 < 2 || n0 > kWave) return false;
+    wave_sync_memory();
+    Kids<1, RAVE> kc;
+    int orig = -1;
+    kc.part[0] = lane < n0;
+    kc.n[0] = 0;
+    kc.w[0] = 0.0f;
+    kc.p[0] = 0.0f;
+    kc.vl[0] = 0;
+    kc.q2[0] = 0.0f;
+    if (lane < n0) {
+        orig = lds.st_j0[lane];
+        kc.n[0] = lds.st_n[lane];
+        kc.w[0] = lds.st_w[lane];
+        kc.p[0] = lds.st_p[lane];
+        kc.vl[0] = lds.st_vl[lane];
+        kc.q2[0] = lds.st_q2[lane];
+    }
+    score_round<1, RAVE>(kc, 0, c.ep);
+    {
+        const bool b_ok = orig == best0 && keys_provably_monotone<RAVE>(kc.n[0], kc.w[0], kc.p[0], kc.vl[0], kc.q2[0],
+                                                                       c.ep, uvl, m - 1);
+        if (__ballot(b_ok) == 0ull) return false;
+    }
+    wave_sync_memory();  // every lane has read its child: the scratch changes hands
+    WaveLds<1> &l1 = reinterpret_cast<WaveLds<1> &>(lds);
+    NodeCtx c1 = c;
+    c1.cc = n0;
+    c1.nelig = n0;
+    int cnt1[1] = {0};
+    const int zero1[1] = {0};
+    int cur = -1;
+    if (!water_level<1, RAVE>(a, c1, lane, kc, soff, 0, m, zero1, l1, cnt1, true, cur, false, zero1, order, pending))
+        return false;
+    // ---- back to the node's own child indices ----
+    // (every lane takes part in the exchange, whether it has an entry in this pass or not)
+    if (cur >= 0) {
+        for (int base = 0; base < m; base += kWave) {
+            const int q = base + lane;
+            const uint32_t v = q < m ? order[q] : 0u;
+            const int i = __shfl(orig, (int)((v >> 21) & 63u), kWave);
+            if (q < m) order[q] = (v & 0x80000000u) | ((uint32_t)i << 21) | (v & 0x1FFFFFu);
+        }
+    } else {
+        for (int base = 0; base < m; base += kWave) {
+            const int q = base + lane;
+            const int cl = q < m ? a.sc_child[soff + q] : 0;
+            const int i = __shfl(orig, cl & 63, kWave);
+            if (q < m) a.sc_child[soff + q] = i;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) lds.st_j0[r * kWave + lane] = 0;
+    wave_sync_memory();
+    if (lane < n0) lds.st_j0[orig] = cnt1[0];
+    wave_sync_memory();
+#pragma unroll
+    for (int r = 0; r < R; r++) cnt[r] = lds.st_j0[r * kWave + lane];
+    lds_cur = cur;
+    wave_sync_memory();
+    return true;
+}
+
 // ---- Chains of nodes whose visitors all follow one child ----
 // Most crowded nodes below the top of a tree are of that kind, often a dozen in a row (a whole
 // selection of the Go workload with 16 visitors per tree starts with a chain of them), and on such a
@@ -3213,6 +3319,21 @@ __device__ __forceinline__ int select_group(const ForestDev &f, const SelectArgs
         }
     }
     if (just_boundary) return kStepParked;  // (a fan-out class that is never cut into slices)
+    // (with RAVE, where every probe of the water level scores two scans per child; without it the path's code
+    // costs the kernel more than its shorter probes save)
+    if constexpr (R > 1 && RAVE) {
+        if (!settled && contested && m >= kWaterLevelMin && m < kHeavyMin && a.vl > 0 && !odd && !as_slice &&
+            !as_scatter) {
+            settled = narrow_water_level<R, RAVE>(a, c, lane, k, soff, best0, lk0, lp0, m, lds, cnt, lds_cur, pl.order,
+                                                  pending);
+            if (settled && a.stats && lane == 0) atomicAdd(a.stats + 12, 1);
+            if (!settled) {
+                lds_cur = -1;
+#pragma unroll
+                for (int r = 0; r < R; r++) cnt[r] = 0;
+            }
+        }
+    }
     if (!settled && m >= kWaterLevelMin && m <= kWaterLevelMaxJ && a.vl > 0 && !odd) {
         int zero[R];
 #pragma unroll

@@ -457,7 +457,7 @@ class Batch:
         _check(self._lib.omk_batch_stats(self._h, _ptr(out, i32p)))
         keys = ("group_nodes", "water_level_nodes", "settled_by_water_level", "settled_one_by_one",
                 "replayed_nodes", "threshold_probes", "single_visitor_steps", "merged_nodes", "t_first_block",
-                "t_last_team", "t_last_walker", "walks_in_launch", "unused_12", "unused_13", "unused_14",
+                "t_last_team", "t_last_walker", "walks_in_launch", "narrowed_nodes", "unused_13", "unused_14",
                 "sliced_nodes")
         return dict(zip(keys, map(int, out)))
 

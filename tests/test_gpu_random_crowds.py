@@ -112,6 +112,40 @@ def test_the_widest_fan_out_class_with_crowds():
         select_both(soa, roots[tr], len(lay) + 1, rave=rave, steps=2, vl=int(rng.integers(1, 5)))
 
 
+def test_wide_nodes_with_rave_settled_through_the_children_that_can_be_chosen():
+    """With RAVE, a node of more than 64 child slots whose 24 to 1023 visitors split is settled through the few
+    children that can be chosen at all, moved to one lane each (the counter says how often).  Forests with the
+    statistics of the Go workload (a few children dominate a node) at several sizes of crowd, and random shapes
+    of 65 to 380 slots with masks, plateaus and pre-existing virtual loss."""
+    from omoknuni_small_amd import synth
+    narrowed = 0
+    for seed, B in enumerate((2000, 5000, 9000, 16000)):
+        soa, roots, meta = synth.generate("c4", seed=40 + seed, nodes_per_tree=600_000)
+        st = select_both(soa, synth.traversal_roots(roots, B), int(meta["max_depth"]), rave=True, steps=3,
+                         vl=int(meta["virtual_loss"]) if seed % 2 else 1, rave_k=float(meta.get("rave_k", 3000.0)))
+        narrowed += st["narrowed_nodes"]
+    print("nodes settled that way:", narrowed)
+    assert narrowed >= 5, narrowed  # (the full-size Go workload has 20 to 30 such nodes a selection)
+    for seed in range(12):
+        rng = np.random.default_rng(1000 + seed)
+        if seed % 3 == 2:
+            soa, _ = random_tree(int(rng.integers(1 << 30)), n_expand=int(rng.integers(20, 120)),
+                                 fanout=(65, int(rng.integers(70, 380))), max_depth=int(rng.integers(3, 7)), rave=True,
+                                 mask_frac=float(rng.choice([0.0, 0.3])), vl_frac=0.2, tie_frac=0.1,
+                                 n_max=int(rng.integers(50, 4000)))
+            D = 8
+            roots = np.zeros(int(rng.integers(24, 3000)), np.int32)
+        else:
+            lay = [int(rng.integers(65, 380)), int(rng.integers(65, 200)), int(rng.integers(3, 7))]
+            soa, r = layered_forest(int(rng.integers(1 << 30)), lay, n_trees=int(rng.integers(1, 3)), rave=True,
+                                    plateau=bool(rng.integers(2)))
+            D = 4
+            B = int(rng.integers(24, 4000))
+            roots = r[np.sort(rng.integers(0, len(r), B))].astype(np.int32)
+        select_both(soa, roots, D, rave=True, steps=3, vl=int(rng.integers(1, 4)),
+                    rave_k=float(rng.choice([300.0, 1000.0, 3000.0])))
+
+
 def test_selection_time_widening_with_crowds():
     """omk_select_params::pw (only the ceil(sqrt(N_parent)) children of highest prior take part) on forests
     whose children are stored by descending prior, parents of few and of many visits, crowds up to 12000."""
